@@ -1,0 +1,396 @@
+"""CPU oracle for the mixed-precision MoE GroupGEMM path.  TEST INFRASTRUCTURE ONLY.
+
+This module is a numpy restatement of the reference algorithm.  It is the checker for the HIP
+path: only ``tests/``, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py``
+may import it; nothing under ``mxmoe_amd/`` does, and the product never falls back to it.
+
+Every function cites the reference lines it follows (paths relative to the reference root).
+
+What pins each function (so that a dropped term, wrong sign, wrong index or transposed operand
+fails a test in ``tests/test_oracle_*.py``):
+
+* ``quant_minmax`` / ``dequant`` / ``fake_quant``  — hand-computed known answers incl. ties
+  (round-half-even after clamp), a sweep over every finite fp16 value against a float64 closed
+  form, invariants (|q| <= upper, absmax -> +-upper, group min -> 0, max -> 2^b-1).
+* ``int_gemm``            — exact integer arithmetic vs a python-int brute force.
+* ``epilogue_wxax``       — closed form incl. the sa = sb = 1 special case (int -> fp16 convert).
+* ``sylvester_fwht``      — scipy.linalg.hadamard dense product, involution, H e_0, Parseval.
+* ``had_table``           — H H^T = K I and all entries +-1.
+* ``online_hadamard``     — dense kron(H_K, H_{n/K}) / sqrt(n) in float64.
+* ``route_topk``          — textbook softmax / top-k, weights sum to one.
+* ``permute_by_expert``   — brute force against a dict-of-lists.
+* ``tile_to_problem``     — every (problem, tile_m, tile_n) visited exactly once.
+* ``silu_mul``            — float64 ``x*sigmoid(x)*u`` within one fp16 ulp.
+
+Parity unpinned (see also the header of ``online_hadamard``): the reference's online rotation
+calls the third-party ``fast_hadamard_transform`` CUDA package (Dao-AILab, version unpinned,
+empty submodule in the reference) and an fp16 ``hadK @ x`` matmul whose accumulation order is
+backend dependent.  None of the reference's files pins their last fp16 bit.  The order used here
+is this build's own deterministic definition; agreement with the reference at that boundary is
+"equal up to fp16 rounding of the rotated activation".
+"""
+from __future__ import annotations
+
+from pathlib import Path
+
+import numpy as np
+
+F16 = np.float16
+F32 = np.float32
+
+_HAD_FILE = Path(__file__).resolve().parent.parent / "mxmoe_amd" / "data" / "had_tables.npz"
+
+
+# --------------------------------------------------------------------------------------------
+# Quantiser  (mxmoe/quant/quant.py:40-109; second statement mxmoe/kernels/src/include/quantize.cuh:218-279)
+# --------------------------------------------------------------------------------------------
+def quant_minmax(t: np.ndarray, bits: int, gsize: int, sym: bool, clip=(1.0, 1.0), zero_guard: bool = True):
+    """Dynamic min/max quantisation along the last dim, in the dtype of ``t`` (fp16 in the path).
+
+    Follows quant.py:61-84: groups are ``reshape(-1, gsize)``; sym: ``upper = 2^(b-1)-1``,
+    ``scale = absmax / upper``, ``zp = 0``; asym: ``upper = 2^b-1``, ``scale = (max*c1 - min*c0) / upper``,
+    ``zp = min*c0`` (a float zero point); ``q = round(clamp((x - zp) / scale, lower, upper))`` with
+    clamp BEFORE the round-half-even.  Every operation rounds to ``t.dtype``.
+
+    ``zero_guard`` follows quantize.cuh:258 (``scale == 0 -> 1``); quant.py has no guard and yields
+    NaN for a constant-zero group.  Returns ``(q (t.shape, t.dtype), scale [G,1], zp [G,1])``.
+    """
+    dt = t.dtype
+    g = t.shape[-1] if gsize == -1 else gsize
+    r = t.reshape(-1, g)
+    if sym:
+        upper = float((1 << (bits - 1)) - 1)
+        lower = -upper
+        gmax = np.abs(r).max(axis=1, keepdims=True)
+        scale = (gmax / dt.type(upper)).astype(dt)
+        zp = np.zeros_like(scale)
+    else:
+        upper = float((1 << bits) - 1)
+        lower = 0.0
+        gmin = (r.min(axis=1, keepdims=True) * dt.type(clip[0])).astype(dt)
+        gmax = (r.max(axis=1, keepdims=True) * dt.type(clip[1])).astype(dt)
+        scale = ((gmax - gmin).astype(dt) / dt.type(upper)).astype(dt)
+        zp = gmin
+    if zero_guard:
+        scale = np.where(scale == 0, dt.type(1), scale).astype(dt)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        x = (r - zp).astype(dt)
+        x = (x / scale).astype(dt)
+    x = np.clip(x, dt.type(lower), dt.type(upper))
+    q = np.rint(x).astype(dt)  # numpy rint == torch.round == round-half-to-even
+    return q.reshape(t.shape), scale, zp
+
+
+def dequant(q: np.ndarray, scale: np.ndarray, zp: np.ndarray, gsize: int) -> np.ndarray:
+    """quant.py:99-102: ``q.reshape(-1, g) * scale + zp`` — two roundings in ``q.dtype``."""
+    dt = q.dtype
+    g = q.shape[-1] if gsize == -1 else gsize
+    r = q.reshape(-1, g)
+    return ((r * scale).astype(dt) + zp).astype(dt).reshape(q.shape)
+
+
+def fake_quant(t: np.ndarray, bits: int, gsize: int, sym: bool, clip=(1.0, 1.0)) -> np.ndarray:
+    """quant.py:104-106 (``bits == 16`` passes through, quant.py:95,100,105)."""
+    if bits >= 16:
+        return t
+    q, s, z = quant_minmax(t, bits, gsize, sym, clip)
+    return dequant(q, s, z, gsize)
+
+
+# --------------------------------------------------------------------------------------------
+# GEMMs and epilogues
+# --------------------------------------------------------------------------------------------
+def int_gemm(qa: np.ndarray, qb: np.ndarray) -> np.ndarray:
+    """Integer accumulators of the w8a8 / w4a4 mainloop (cta_gemm.cuh:557-598): ``acc[m,n] = sum_k qa[m,k] qb[n,k]``.
+
+    Computed exactly (float64 matmul of small integers is exact below 2^53) and returned as int32;
+    asserts the int32 range the kernels accumulate in is not exceeded.
+    """
+    a = np.asarray(qa, dtype=np.float64)
+    b = np.asarray(qb, dtype=np.float64)
+    acc = a @ b.T
+    assert np.abs(acc).max(initial=0) < 2**31
+    return acc.astype(np.int64).astype(np.int32)
+
+
+def epilogue_wxax(acc: np.ndarray, sa: np.ndarray, sb: np.ndarray) -> np.ndarray:
+    """w-a epilogue (mm_tile.cuh:468-496 then :642-646): ``half(float(acc) * float(half(sa[m] * sb[n])))``.
+
+    ``sa`` [M] per-token and ``sb`` [N] per-channel fp16 scales; their product is rounded to fp16
+    first, widened to fp32, multiplied with the converted accumulator in fp32, rounded to fp16.
+    """
+    s = (sa.astype(F16).reshape(-1, 1) * sb.astype(F16).reshape(1, -1)).astype(F16)
+    return (acc.astype(F32) * s.astype(F32)).astype(F16)
+
+
+def gemm_fakequant(xq: np.ndarray, wq: np.ndarray) -> np.ndarray:
+    """The fake-quant linear (quant.py:126-130 hook + ``F.linear``): ``xq @ wq.T`` on fp16 values.
+
+    fp16 storage, float64 accumulation (the tightest reading of "what the mathematics fixes"),
+    rounded once to fp16.  This is the value the 1e-2 max-abs-rel criterion compares against.
+    """
+    return (xq.astype(np.float64) @ wq.astype(np.float64).T).astype(F16)
+
+
+def gemm_fp16(x: np.ndarray, w: np.ndarray) -> np.ndarray:
+    """fp16 x fp16 -> fp32 accumulate -> fp16 (cta_gemm.cuh:8-107); float64 here, compared at 1e-2."""
+    return gemm_fakequant(x, w)
+
+
+# --------------------------------------------------------------------------------------------
+# SiLU * up  (input of the down projection)
+# --------------------------------------------------------------------------------------------
+_LOG2E = F32(1.4426950408889634)
+_LN2_HI = F32(0.693145751953125)          # 0x3f317200, low mantissa bits zero
+_LN2_LO = F32(1.428606765330187e-06)      # ln2 - LN2_HI
+_EXP_C = [F32(c) for c in (1.0, 1.0, 0.5, 0.16666667, 0.041666668, 0.008333334, 0.0013888889, 0.0001984127)]
+
+
+def exp_f32_fixed(t: np.ndarray) -> np.ndarray:
+    """exp(t) in fp32 as a FIXED sequence of individually rounded fp32 mul/add ops (no FMA).
+
+    ``k = rint(t*log2e)``, ``r = (t - k*LN2_HI) - k*LN2_LO``, degree-7 Horner polynomial, exact
+    scaling by 2^k.  The HIP kernels run the identical op sequence (contraction off), which is
+    what makes ``silu_mul`` bit-reproducible between CPU and GPU.  Relative error < 2e-7.
+    """
+    t = np.clip(t.astype(F32), F32(-87.0), F32(87.0))
+    k = np.rint((t * _LOG2E).astype(F32)).astype(F32)
+    r = (t - (k * _LN2_HI).astype(F32)).astype(F32)
+    r = (r - (k * _LN2_LO).astype(F32)).astype(F32)
+    p = np.full_like(r, _EXP_C[7])
+    for c in _EXP_C[6::-1]:
+        p = ((p * r).astype(F32) + c).astype(F32)
+    return np.ldexp(p, k.astype(np.int32)).astype(F32)
+
+
+def silu_mul(gate_up: np.ndarray) -> np.ndarray:
+    """``silu(gate) * up`` on a fused ``[rows, 2I]`` fp16 tensor, first half = gate, second = up.
+
+    Contract of the reference's ``silu_mul_then_quant_kernel`` launch (ref_bind.cu:691-716; kernel
+    source absent from the reference).  fp32: ``s = g / (1 + exp(-g))``, ``y = s * u``, one fp16 rounding.
+    """
+    i = gate_up.shape[-1] // 2
+    g = gate_up[..., :i].astype(F32)
+    u = gate_up[..., i:].astype(F32)
+    e = exp_f32_fixed(-g)
+    s = (g / (F32(1.0) + e).astype(F32)).astype(F32)
+    return (s * u).astype(F32).astype(F16)
+
+
+# --------------------------------------------------------------------------------------------
+# Hadamard rotation  (mxmoe/quant/hadamard_utils.py:5-106, rotation.py:403-421)
+# --------------------------------------------------------------------------------------------
+_HAD_ORDER = (176, 172, 156, 140, 108, 60, 52, 36, 28, 40, 20, 12)  # hadamard_utils.py:7-56 test order
+
+
+def had_table(k: int) -> np.ndarray:
+    """K x K +-1 matrix (int8) — hadamard_utils.py:162-4379 tables, stored bit-packed."""
+    z = np.load(_HAD_FILE)
+    bits = np.unpackbits(z[f"had{k}"])[: k * k].reshape(k, k)
+    return (1 - 2 * bits.astype(np.int8)).astype(np.int8)
+
+
+def _is_pow2(n: int) -> bool:
+    return n > 0 and (n & (n - 1)) == 0
+
+
+def get_hadK(n: int):
+    """hadamard_utils.py:5-59: first K in the reference's test order with ``n % K == 0`` and ``n/K`` a power of two."""
+    for k in _HAD_ORDER:
+        if n % k == 0:
+            assert _is_pow2(n // k)
+            return had_table(k), k
+    assert _is_pow2(n)
+    return None, 1
+
+
+def sylvester_fwht(x: np.ndarray) -> np.ndarray:
+    """Unnormalised Walsh-Hadamard transform along the last dim (length 2^m), Sylvester order.
+
+    Stages in ASCENDING stride h = 1, 2, 4, ...: ``(a, b) -> (a + b, a - b)`` for index pairs
+    ``(i, i + h)`` with bit ``h`` of ``i`` clear.  Each op rounds in ``x.dtype``; with fp32 input
+    every output is a fixed binary tree of fp32 adds, which the HIP kernel reproduces bit for bit.
+    """
+    n = x.shape[-1]
+    assert _is_pow2(n)
+    y = x.copy()
+    h = 1
+    while h < n:
+        v = y.reshape(*y.shape[:-1], n // (2 * h), 2, h)
+        a = v[..., 0, :].copy()
+        b = v[..., 1, :].copy()
+        v[..., 0, :] = a + b
+        v[..., 1, :] = a - b
+        h *= 2
+    return y
+
+
+def had_scale(n: int) -> np.float32:
+    """``1.0 / torch.tensor(n).sqrt()`` (hadamard_utils.py:99,103): fp32 sqrt, fp32 reciprocal."""
+    return F32(1.0) / np.sqrt(F32(n))
+
+
+def online_hadamard(x: np.ndarray) -> np.ndarray:
+    """Online rotation of fp16 rows: ``y = (H_K kron H_{n/K}) x / sqrt(n)``, index ``p = k*(n/K) + j``.
+
+    Follows ``matmul_hadU_cuda`` (hadamard_utils.py:96-106): view ``[K, n/K]``, Sylvester transform
+    of each length-``n/K`` row scaled by ``1/sqrt(n)`` and returned in fp16, then ``hadK @ .`` in fp16.
+    PARITY UNPINNED at the last fp16 bit (third-party kernel + backend matmul order, see module
+    header).  This build's definition: fp32 ``sylvester_fwht`` (ascending strides), one fp32 multiply by
+    ``had_scale(n)``, round to fp16; K > 1: ``y[k] = sum_{k'} H[k,k'] v[k']`` accumulated in fp32
+    sequentially over ``k' = 0..K-1`` starting from 0, rounded to fp16.
+    """
+    assert x.dtype == F16
+    n = x.shape[-1]
+    hk, k = get_hadK(n)
+    m = n // k
+    v = x.astype(F32).reshape(-1, k, m)
+    v = (sylvester_fwht(v) * had_scale(n)).astype(F32).astype(F16)
+    if k == 1:
+        return v.reshape(x.shape)
+    vf = v.astype(F32)
+    acc = np.zeros_like(vf)
+    for kp in range(k):  # fixed sequential order
+        sgn = hk[:, kp].astype(F32).reshape(1, k, 1)
+        acc = (acc + sgn * vf[:, kp : kp + 1, :]).astype(F32)
+    return acc.astype(F16).reshape(x.shape)
+
+
+def matmul_hadU_f64(x: np.ndarray) -> np.ndarray:
+    """float64 restatement of the pure-torch ``matmul_hadU`` (hadamard_utils.py:62-83), for cross-checks.
+
+    Its butterfly pairs ADJACENT elements and concatenates sums then differences at every level
+    (the ``view(.., n/2, 2, .)`` at :68-73), stopping at length K, then applies ``hadK @`` and ``/ sqrt(n)``.
+    """
+    n = x.shape[-1]
+    hk, k = get_hadK(n)
+    inp = x.astype(np.float64).reshape(-1, n, 1)
+    while inp.shape[1] > k:
+        b, l, w = inp.shape
+        v = inp.reshape(b, l // 2, 2, w)
+        inp = np.concatenate([v[:, :, 0, :] + v[:, :, 1, :], v[:, :, 0, :] - v[:, :, 1, :]], axis=-1)
+    if k > 1:
+        inp = hk.astype(np.float64)[None] @ inp
+    return inp.reshape(x.shape) / np.sqrt(np.float64(n))
+
+
+# --------------------------------------------------------------------------------------------
+# Routing, permutation, offsets
+# --------------------------------------------------------------------------------------------
+def route_topk(logits: np.ndarray, topk: int):
+    """moe_tracer.py:79-86: ``softmax(logits, fp32) -> topk -> renormalise``.  Returns (ids int32 [T,k], weights fp32)."""
+    z = logits.astype(F32)
+    z = z - z.max(axis=1, keepdims=True)
+    p = np.exp(z)
+    p = p / p.sum(axis=1, keepdims=True)
+    ids = np.argsort(-p, axis=1, kind="stable")[:, :topk]
+    w = np.take_along_axis(p, ids, axis=1)
+    w = w / w.sum(axis=1, keepdims=True)
+    return ids.astype(np.int32), w.astype(F32)
+
+
+def permute_by_expert(topk_ids: np.ndarray, num_experts: int):
+    """ref_bind.cu:47-64,449-453: sort the flattened expert ids, ``perm = idx // topk``, ``bincount``.
+
+    The reference's sort is unstable (order inside an expert unspecified); this build fixes the STABLE order.
+    Returns ``(dst_exp_sorted int32 [R], perm_indices int64 [R] (source token of each sorted row),
+    src_slot int64 [R] (flattened (token, slot) index), recv_tokens_per_exp int64 [E])``.
+    """
+    flat = topk_ids.reshape(-1).astype(np.int64)
+    order = np.argsort(flat, kind="stable")
+    k = topk_ids.shape[1]
+    return flat[order].astype(np.int32), (order // k).astype(np.int64), order.astype(np.int64), np.bincount(flat, minlength=num_experts).astype(np.int64)
+
+
+def act_tag(a_bits: int, gsize: int) -> int:
+    """ref_bind.cu:461-473: 0 fp16, 1 int8 per-token, 2 int4 per-token, 3 int4 group-128, -1 unsupported."""
+    if a_bits >= 16:
+        return 0
+    if a_bits == 8 and gsize == -1:
+        return 1
+    if a_bits == 4 and gsize == -1:
+        return 2
+    if a_bits == 4 and gsize == 128:
+        return 3
+    return -1
+
+
+def act_offsets(recv: np.ndarray, num_tokens: int, qparams_per_exp, k_dim: int, has_shared: bool, shared_k_dim: int | None = None):
+    """Per-expert exclusive offsets of the packed activation / scale stores (ref_bind.cu:475-505, 635-671).
+
+    Units are fp16 elements, as in the reference: row strides ``K``, ``K/2``, ``K/4`` halves for tags
+    0/1/2(3); scale strides 0 / 1 / 1 / ``K/128``.  The shared expert is index E with ``num_tokens`` rows.
+    Returns dict of int64 arrays ``tag, start_row, inp_off, scale_off, inp_size, scale_size`` (length E(+1)).
+    """
+    e_tot = len(recv) + (1 if has_shared else 0)
+    out = {k: np.zeros(e_tot, dtype=np.int64) for k in ("tag", "start_row", "inp_off", "scale_off", "inp_size", "scale_size")}
+    rows = io = so = 0
+    for e in range(e_tot):
+        a_bits, _w, g, _s = qparams_per_exp[e]
+        tag = act_tag(a_bits, g)
+        kd = k_dim if (e < len(recv) or shared_k_dim is None) else shared_k_dim
+        ld = kd if tag == 0 else (kd // 2 if tag == 1 else kd // 4)
+        sld = 0 if tag == 0 else (1 if tag in (1, 2) else kd // 128)
+        n = num_tokens if e == len(recv) else int(recv[e])
+        out["tag"][e], out["start_row"][e], out["inp_off"][e], out["scale_off"][e] = tag, rows, io, so
+        out["inp_size"][e], out["scale_size"][e] = ld * n, sld * n
+        rows += n
+        io += ld * n
+        so += sld * n
+    return out
+
+
+# --------------------------------------------------------------------------------------------
+# Tile scheduler  (mxmoe/kernels/src/include/tile_scheduler.cuh:5-50, kernel_sketch.py:87-101)
+# --------------------------------------------------------------------------------------------
+def tile_prefix(problem_mn, tile_mn):
+    """Inclusive prefix sum of ``ceil(M/BM) * ceil(N/BN)`` per problem (kernel_sketch.py:89-101)."""
+    tot, out = 0, []
+    for (m, n), (bm, bn) in zip(problem_mn, tile_mn):
+        tot += -(-m // bm) * -(-n // bn)
+        out.append(tot)
+    return out
+
+
+def tile_to_problem(tile_idx: int, prefix, problem_mn, tile_mn):
+    """tile_scheduler.cuh:25-49: first problem with ``prefix[i] > tile_idx``; local index -> (idx // grid_n, idx % grid_n).
+
+    Returns ``(-1, 0, 0)`` past the end, else ``(problem, tile_m, tile_n)`` (x = row tile, y = column tile).
+    """
+    if not prefix or tile_idx >= prefix[-1]:
+        return -1, 0, 0
+    p = next(i for i, s in enumerate(prefix) if tile_idx < s)
+    local = tile_idx - (prefix[p - 1] if p else 0)
+    grid_n = -(-problem_mn[p][1] // tile_mn[p][1])
+    return p, local // grid_n, local % grid_n
+
+
+# --------------------------------------------------------------------------------------------
+# Whole-layer fake-quant path (what the CPU baseline times) and the integer path next to it
+# --------------------------------------------------------------------------------------------
+def quant_weight(w: np.ndarray, w_bits: int, gsize: int, sym: bool):
+    """RTN weight quantisation = ``quant_minmax`` on the ``[N, K]`` weight rows (quant.py:913 / quantize.cuh:218-279)."""
+    return quant_minmax(w, w_bits, gsize, sym)
+
+
+def linear_block(x: np.ndarray, w: np.ndarray, qp, rotate: bool):
+    """One linear block of one expert in one format ``qp = (a_bits, w_bits, gsize, sym)``.
+
+    Returns ``(out_kernel fp16, out_fakequant fp16, acc int32 | None)``:
+    * w-a formats (a_bits < 16): activations optionally rotated (``online_hadamard``), per-token sym
+      quantised; weights per-channel sym RTN; ``acc = int_gemm``; ``out_kernel = epilogue_wxax``;
+      ``out_fakequant = gemm_fakequant(dequant(xq), dequant(wq))`` (quant.py:126-130 path).
+    * weight-only (a_bits == 16, w_bits < 16): ``out = x @ fake_quant(w).T``; fp16: plain GEMM.
+    """
+    a_bits, w_bits, g, sym = qp
+    if a_bits < 16:
+        xr = online_hadamard(x) if rotate else x
+        qa, sa, _ = quant_minmax(xr, a_bits, -1, True)
+        qb, sb, _ = quant_minmax(w, w_bits, -1, True)
+        acc = int_gemm(qa, qb)
+        out_k = epilogue_wxax(acc, sa.reshape(-1), sb.reshape(-1))
+        out_f = gemm_fakequant(dequant(qa, sa, 0 * sa, -1), dequant(qb, sb, 0 * sb, -1))
+        return out_k, out_f, acc
+    wq = fake_quant(w, w_bits, g, sym) if w_bits < 16 else w
+    out = gemm_fakequant(x, wq)
+    return out, out, None

@@ -1,0 +1,65 @@
+"""Pins the oracle's routing, permutation, offsets and tile scheduler by brute force."""
+import numpy as np
+
+from oracle import mxmoe_oracle as O
+
+
+def test_route_topk_textbook():
+    rng = np.random.default_rng(0)
+    logits = rng.standard_normal((50, 9)).astype(np.float32)
+    ids, w = O.route_topk(logits, 3)
+    p = np.exp(logits.astype(np.float64)); p /= p.sum(1, keepdims=True)
+    for t in range(50):
+        best = sorted(range(9), key=lambda e: -p[t, e])[:3]
+        assert ids[t].tolist() == best
+        assert np.allclose(w[t], p[t, best] / p[t, best].sum(), rtol=1e-5)
+    assert np.allclose(w.sum(1), 1, atol=1e-6)
+
+
+def test_permutation_bruteforce_and_stability():
+    rng = np.random.default_rng(1)
+    E, T, k = 7, 40, 3
+    ids = np.stack([rng.permutation(E)[:k] for _ in range(T)]).astype(np.int32)
+    ids[ids == 4] = 5                                                      # leave expert 4 empty (may duplicate 5 in a row)
+    dst, perm, slot, recv = O.permute_by_expert(ids, E)
+    buckets = {e: [] for e in range(E)}
+    for t in range(T):
+        for s in range(k):
+            buckets[int(ids[t, s])].append((t, t * k + s))
+    exp_perm = [t for e in range(E) for t, _ in buckets[e]]
+    exp_slot = [s for e in range(E) for _, s in buckets[e]]
+    assert perm.tolist() == exp_perm and slot.tolist() == exp_slot         # stable order inside an expert
+    assert recv.tolist() == [len(buckets[e]) for e in range(E)] and recv[4] == 0
+    assert dst.tolist() == sorted(ids.reshape(-1).tolist())
+
+
+def test_act_offsets_strides_and_shared():
+    recv = np.array([3, 0, 2, 5])
+    qp = [(16, 4, 128, False), (8, 8, -1, True), (4, 4, -1, True), (8, 8, -1, True), (4, 4, 128, True)]
+    o = O.act_offsets(recv, num_tokens=6, qparams_per_exp=qp, k_dim=256, has_shared=True)
+    assert o["tag"].tolist() == [0, 1, 2, 1, 3]
+    assert o["start_row"].tolist() == [0, 3, 3, 5, 10]
+    assert o["inp_size"].tolist() == [3 * 256, 0, 2 * 64, 5 * 128, 6 * 64]  # K, K/2, K/4 halves per row
+    assert o["scale_size"].tolist() == [0, 0, 2, 5, 6 * 2]                  # 0 / 1 / 1 / K/128
+    assert o["inp_off"].tolist() == [0, 768, 768, 896, 1536]
+    assert o["scale_off"].tolist() == [0, 0, 0, 2, 7]
+    assert [O.act_tag(2, -1), O.act_tag(8, 128)] == [-1, -1]
+
+
+def test_tile_scheduler_visits_every_tile_once():
+    rng = np.random.default_rng(2)
+    for _ in range(20):
+        p = int(rng.integers(1, 9))
+        mn = [(int(rng.integers(1, 700)), int(rng.integers(1, 6)) * 128) for _ in range(p)]
+        tiles = [(int(rng.choice([16, 32, 64, 128, 256])), int(rng.choice([64, 128, 256]))) for _ in range(p)]
+        prefix = O.tile_prefix(mn, tiles)
+        seen = set()
+        for t in range(prefix[-1]):
+            pi, tm, tn = O.tile_to_problem(t, prefix, mn, tiles)
+            assert 0 <= pi < p
+            bm, bn = tiles[pi]
+            assert tm * bm < mn[pi][0] and tn * bn < mn[pi][1]
+            assert (pi, tm, tn) not in seen
+            seen.add((pi, tm, tn))
+        assert len(seen) == sum(-(-m // bm) * -(-n // bn) for (m, n), (bm, bn) in zip(mn, tiles))
+        assert O.tile_to_problem(prefix[-1], prefix, mn, tiles)[0] == -1

@@ -1,0 +1,149 @@
+"""Pins oracle.quant_minmax / dequant / epilogue / int_gemm / silu_mul by known answers, closed forms and brute force."""
+import numpy as np
+import pytest
+
+from oracle import mxmoe_oracle as O
+
+F16 = np.float16
+
+
+def test_sym_int4_known_answers_with_ties():
+    # absmax 7 -> scale exactly 1; x/scale ties go to even AFTER the clamp (quant.py:82).
+    x = np.array([[7, 0.5, 1.5, 2.5, 6.5, -0.5, -1.5, -2.5, -6.5, 3.49, -7, 100 * 0]], dtype=F16)
+    q, s, z = O.quant_minmax(x, 4, -1, True)
+    assert s.item() == 1.0 and z.item() == 0
+    assert q.tolist() == [[7, 0, 2, 2, 6, -0, -2, -2, -6, 3, -7, 0]]
+
+
+def test_sym_int8_known_answers():
+    x = np.array([[127, -127, 63.5, 64.5, 1, -1]], dtype=F16)
+    q, s, _ = O.quant_minmax(x, 8, -1, True)
+    assert s.item() == 1.0
+    assert q.tolist() == [[127, -127, 64, 64, 1, -1]]
+    # a scale that is not a power of two: absmax 2 -> scale = fp16(2/127)
+    x = np.array([[2.0, 1.0, -0.25]], dtype=F16)
+    q, s, _ = O.quant_minmax(x, 8, -1, True)
+    sc = F16(F16(2.0) / F16(127))
+    assert s.item() == sc
+    exp = [np.rint(np.clip(F16(v / sc), -127, 127)) for v in x[0]]
+    assert q[0].tolist() == exp and q[0, 0] == 127
+
+
+def test_clamp_happens_before_round():
+    # x/scale = 7.5 would round to 8 if rounded first; clamp-then-round gives 7.
+    x = np.array([[7.0, 7.5 * 0 + 7.0]], dtype=F16)
+    q, _, _ = O.quant_minmax(x, 4, -1, True)
+    assert q.max() == 7
+    # asym: value above max cannot occur, but the closed form must still clamp to 2^b-1
+    x = np.array([[0.0, 15.0, 7.5, 8.5]], dtype=F16)
+    q, s, z = O.quant_minmax(x, 4, -1, False)
+    assert s.item() == 1.0 and z.item() == 0.0
+    assert q.tolist() == [[0, 15, 8, 8]]
+
+
+def test_asym_group_known_answers():
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((6, 256)).astype(F16)
+    for bits in (4, 3):
+        q, s, z = O.quant_minmax(x, bits, 128, False)
+        g = x.reshape(-1, 128)
+        qg = q.reshape(-1, 128)
+        up = (1 << bits) - 1
+        assert s.shape == (12, 1) and z.shape == (12, 1)
+        assert np.array_equal(z[:, 0], g.min(axis=1))                      # float zero-point = group min
+        assert np.array_equal(s[:, 0], ((g.max(1) - g.min(1)).astype(F16) / F16(up)).astype(F16))
+        assert qg.min() >= 0 and qg.max() <= up
+        assert np.all(qg[np.arange(12), g.argmin(1)] == 0)                 # min -> 0
+        assert np.all(qg[np.arange(12), g.argmax(1)] >= up - 1)            # max -> 2^b-1 (up to fp16 rounding of the ratio)
+        deq = O.dequant(q, s, z, 128)
+        err = np.abs(deq.astype(np.float64) - x.astype(np.float64)).reshape(-1, 128)
+        assert np.all(err <= s.astype(np.float64) * 0.5 * 1.01 + 2e-3)
+
+
+def test_zero_group_guard_and_reference_nan():
+    x = np.zeros((2, 8), dtype=F16)
+    q, s, _ = O.quant_minmax(x, 4, -1, True)                               # quantize.cuh:258 guard
+    assert np.all(s == 1) and np.all(q == 0)
+    q, s, _ = O.quant_minmax(x, 4, -1, True, zero_guard=False)             # quant.py: 0/0 -> NaN
+    assert np.all(np.isnan(q))
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_sym_sweep_all_fp16_against_float64_closed_form(bits):
+    # every finite fp16 value v paired with an absmax element A, one row each: q(v) must equal
+    # RNE(clamp(fp16(v / fp16(A/upper)))) evaluated independently in float64 with explicit fp16 roundings.
+    allv = np.arange(0, 1 << 16, dtype=np.uint16).view(F16)
+    allv = allv[np.isfinite(allv)]
+    up = (1 << (bits - 1)) - 1
+    for A in (F16(1.0), F16(3.3), F16(0.0117), F16(1000.0)):
+        v = allv[np.abs(allv) <= A]
+        rows = np.stack([v, np.full_like(v, A)], axis=1)
+        q, s, _ = O.quant_minmax(rows, bits, -1, True)
+        sc = np.float64(F16(np.float64(A) / up))                           # one fp16 rounding
+        assert np.all(s[:, 0] == F16(sc))
+        ratio = (v.astype(np.float64) / sc).astype(F16).astype(np.float64) # one fp16 rounding (exact quotient -> fp16)
+        exp = np.rint(np.clip(ratio, -up, up))
+        assert np.array_equal(q[:, 0].astype(np.float64), exp)
+        assert np.all(q[:, 1] == up)                                       # absmax element -> +upper
+        assert np.all(np.abs(q) <= up)
+
+
+def test_int_gemm_matches_python_int_bruteforce():
+    rng = np.random.default_rng(1)
+    a = rng.integers(-127, 128, size=(5, 37))
+    b = rng.integers(-127, 128, size=(7, 37))
+    acc = O.int_gemm(a, b)
+    for m in range(5):
+        for n in range(7):
+            assert int(acc[m, n]) == sum(int(a[m, k]) * int(b[n, k]) for k in range(37))
+    assert acc.dtype == np.int32 and acc.shape == (5, 7)                   # [M, N], not transposed
+    # worst-case magnitude at the largest BASELINE K stays inside int32
+    k = 14336
+    assert O.int_gemm(np.full((1, k), 127), np.full((1, k), -127))[0, 0] == -127 * 127 * k
+
+
+def test_epilogue_closed_forms():
+    acc = np.array([[3, -70000], [2**24 + 1, 5]], dtype=np.int32)
+    one = np.ones(2, dtype=F16)
+    out = O.epilogue_wxax(acc, one, one)                                   # sa=sb=1: int -> fp32 -> fp16 conversion
+    assert out[0, 0] == 3 and np.isinf(out[0, 1]) and out[1, 1] == 5
+    sa = np.array([0.1, 0.013], dtype=F16)
+    sb = np.array([0.02, 0.5], dtype=F16)
+    out = O.epilogue_wxax(acc, sa, sb)
+    for m in range(2):
+        for n in range(2):
+            s16 = F16(sa[m] * sb[n])                                       # product rounded to fp16 FIRST
+            assert out[m, n] == F16(np.float32(acc[m, n]) * np.float32(s16))
+    # sa indexes rows (tokens), sb columns (channels): swapping them must change the result
+    assert not np.array_equal(out, O.epilogue_wxax(acc, sb, sa))
+
+
+def test_fakequant_path_agrees_with_integer_path_within_tolerance():
+    rng = np.random.default_rng(2)
+    x = rng.standard_normal((33, 256)).astype(F16)
+    w = (rng.standard_normal((48, 256)) * 0.02).astype(F16)
+    for qp in [(4, 4, -1, True), (8, 8, -1, True)]:
+        ok, of, acc = O.linear_block(x, w, qp, rotate=True)
+        rel = np.abs(ok.astype(np.float64) - of.astype(np.float64)).max() / np.abs(of.astype(np.float64)).max()
+        assert rel < 1e-2 and acc.dtype == np.int32
+
+
+def test_exp_fixed_and_silu_mul():
+    t = np.linspace(-87, 87, 20001).astype(np.float32)
+    rel = np.abs(O.exp_f32_fixed(t).astype(np.float64) / np.exp(t.astype(np.float64)) - 1)
+    assert rel.max() < 3e-7
+    rng = np.random.default_rng(3)
+    gu = (rng.standard_normal((17, 64)) * 3).astype(F16)
+    gu[0, :4] = [F16(-60000), F16(60000), F16(0), F16(-0.0)]
+    y = O.silu_mul(gu)
+    g = gu[:, :32].astype(np.float64)
+    u = gu[:, 32:].astype(np.float64)
+    with np.errstate(over="ignore"):
+        ref = g / (1 + np.exp(-g)) * u
+    assert y.shape == (17, 32)
+    fin = np.abs(ref) < 65504
+    ulp = np.maximum(2.0 ** np.floor(np.log2(np.maximum(np.abs(ref), 1e-30))) * 2.0**-10, 2.0**-24)
+    assert np.all(np.abs(y.astype(np.float64) - ref)[fin] <= 0.501 * ulp[fin])  # one correctly rounded fp16 result
+    assert np.all(np.isinf(y[~fin]))
+    # first half is the gate: swapping halves changes the answer
+    assert not np.array_equal(y, O.silu_mul(np.concatenate([gu[:, 32:], gu[:, :32]], axis=1)))
