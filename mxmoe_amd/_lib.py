@@ -1,0 +1,58 @@
+"""ctypes loader of libmxmoe_amd.so.  There is no CPU fallback: a missing library is an error."""
+from __future__ import annotations
+
+import ctypes as C
+from pathlib import Path
+
+LIB_PATH = Path(__file__).resolve().parent / "libmxmoe_amd.so"
+
+
+class Dim3(C.Structure):
+    _fields_ = [("x", C.c_uint32), ("y", C.c_uint32), ("z", C.c_uint32)]
+
+
+class QParams(C.Structure):
+    _fields_ = [("a_bits", C.c_int32), ("w_bits", C.c_int32), ("gsize", C.c_int32), ("sym", C.c_uint8), ("_pad", C.c_uint8 * 3)]
+
+
+_P = C.c_void_p
+_I = C.c_int
+
+# name -> (restype, argtypes); mirrors include/mxmoe_amd.h declaration by declaration
+SIGNATURES = {
+    "mxmoe_last_error": (C.c_char_p, []),
+    "mxmoe_num_kernels": (_I, []),
+    "mxmoe_kernel_name": (C.c_char_p, [_I]),
+    "mxmoe_find_kernel": (_I, [C.c_char_p]),
+    "mxmoe_kernel_num_branches": (_I, [_I]),
+    "mxmoe_kernel_branch": (_I, [_I, _I, C.POINTER(C.c_int32)]),
+    "mxmoe_group_gemm": (_I, [_I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, C.POINTER(Dim3), _P, C.POINTER(QParams), _I, _P, _P]),
+    "mxmoe_group_gemm_plan": (_I, [_I, C.POINTER(Dim3), C.POINTER(QParams), _I, C.POINTER(C.c_int32), C.POINTER(C.c_int32)]),
+}
+
+_cached = {}
+
+
+def load(path: str | Path | None = None) -> C.CDLL:
+    """Load the library (or a generated one at `path`) and attach the C-ABI signatures."""
+    p = Path(path) if path is not None else LIB_PATH
+    key = str(p)
+    if key in _cached:
+        return _cached[key]
+    if not p.exists():
+        raise RuntimeError(
+            f"{p} is missing: build it with `python -m mxmoe_amd.build` (hipcc, gfx950). "
+            "mxmoe_amd has no CPU fallback for its kernels."
+        )
+    lib = C.CDLL(str(p))
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _cached[key] = lib
+    return lib
+
+
+def check(lib: C.CDLL, rc: int) -> None:
+    if rc != 0:
+        raise RuntimeError(lib.mxmoe_last_error().decode())

@@ -1,0 +1,283 @@
+// Fused one-launch GroupGEMM: tile scheduler, per-problem branch dispatch, host launcher and kernel registry.
+//
+// Mirrors the reference's generated `groupgemm_hz_fused_<i>` pair (kernel + host launcher,
+// mxmoe/kernels/compose_kernel.py:150-295, mxmoe/kernels/kernel_sketch.py:82-145) with these differences:
+//  * one workgroup per tile instead of a persistent grid: the hardware dispatcher hands out tiles as
+//    workgroups retire, which balances the mixed tile costs of a mixed-precision launch;
+//  * the tile prefix sum and the per-problem branch index travel in the kernel-argument segment, so a launch
+//    performs no allocation, no host-to-device copy and no synchronisation (the reference does
+//    cudaMalloc + cudaMemcpy + cudaFree per call, kernel_sketch.py:102-104,142-143);
+//  * workgroup ids are remapped so that each of the 8 XCDs (one L2 each; workgroups are dealt round-robin)
+//    receives one contiguous run of the tile list, i.e. whole experts, and re-reads of an expert's weights
+//    and activations by neighbouring tiles stay inside one L2;
+//  * a qcfg may own several tile shapes; the host picks one per problem from its row count.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "mxmoe_tiles.hpp"
+#include "mxmoe_wo_tiles.hpp"
+
+namespace mxmoe {
+
+constexpr int kMaxProblems = 256;  // per launch; longer problem lists are split into several launches
+constexpr int kNumXcd = 8;
+
+struct FusedArgs {
+  const uint8_t* const* As;
+  const uint8_t* const* Bs;
+  const _Float16* const* sa;
+  const _Float16* const* sb;
+  _Float16* const* Cs;
+  int32_t* const* acc;  // optional accumulator dumps (null, or per-problem pointers which may themselves be null)
+  const mxmoe_dim3* sizes;
+  int problem_offset;   // first problem of this launch inside the arrays above
+  int num_problems;
+  int total_tiles;
+  int chunk;                      // tiles per XCD = ceil(total_tiles / 8)
+  int prefix[kMaxProblems];       // inclusive prefix sum of tiles per problem
+  uint8_t branch[kMaxProblems];   // which tile type runs each problem
+};
+
+template <int I, class... Tiles>
+struct Dispatch;
+template <int I>
+struct Dispatch<I> {
+  __device__ static __forceinline__ void go(int, TileArgs&, int, uint8_t*) {}
+};
+template <int I, class T, class... Rest>
+struct Dispatch<I, T, Rest...> {
+  __device__ static __forceinline__ void go(int branch, TileArgs& t, int local, uint8_t* smem) {
+    if (branch == I) {
+      // tile_scheduler.cuh:40-49: local index -> (row tile, column tile), column tile fastest
+      const int grid_n = (t.N + T::BN - 1) / T::BN;
+      t.tile_m = local / grid_n;
+      t.tile_n = local - t.tile_m * grid_n;
+      T::run(t, smem);
+    } else {
+      Dispatch<I + 1, Rest...>::go(branch, t, local, smem);
+    }
+  }
+};
+
+template <class... Tiles>
+__global__ void __launch_bounds__(kThreads, 2) fused_group_gemm_kernel(const FusedArgs args) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  const int wg = blockIdx.x;
+  const int tile = (wg % kNumXcd) * args.chunk + wg / kNumXcd;
+  if (tile >= args.total_tiles) return;
+  // tile_scheduler.cuh:25-37 — first problem whose inclusive prefix exceeds the tile index (binary search here)
+  int lo = 0, hi = args.num_problems - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi) >> 1;
+    if (tile < args.prefix[mid]) hi = mid; else lo = mid + 1;
+  }
+  const int p = lo;
+  const int local = tile - (p ? args.prefix[p - 1] : 0);
+  const int gp = args.problem_offset + p;
+  const mxmoe_dim3 sz = args.sizes[gp];
+  TileArgs t;
+  t.A = args.As[gp];
+  t.B = args.Bs[gp];
+  t.sa = args.sa ? args.sa[gp] : nullptr;
+  t.sb = args.sb ? args.sb[gp] : nullptr;
+  t.C = args.Cs[gp];
+  t.acc_dump = args.acc ? args.acc[gp] : nullptr;
+  t.M = (int)sz.x;
+  t.N = (int)sz.y;
+  t.K = (int)sz.z;
+  t.tile_m = t.tile_n = 0;
+  Dispatch<0, Tiles...>::go(args.branch[p], t, local, smem);
+}
+
+// ------------------------------------------------------------------ host side ------------------------------------------------------------------
+
+enum class Fmt { FP16, W8A8, W4A4, W4A16, W3A16, UNSUPPORTED };
+
+inline Fmt classify(const mxmoe_qparams& q) {
+  if (q.a_bits >= 16 && q.w_bits >= 16) return Fmt::FP16;
+  if (q.a_bits == 8 && q.w_bits == 8 && q.gsize == -1 && q.sym) return Fmt::W8A8;
+  if (q.a_bits == 4 && q.w_bits == 4 && q.gsize == -1 && q.sym) return Fmt::W4A4;
+  if (q.a_bits >= 16 && q.w_bits == 4 && q.gsize == 128) return Fmt::W4A16;
+  if (q.a_bits >= 16 && q.w_bits == 3 && q.gsize == 128) return Fmt::W3A16;
+  return Fmt::UNSUPPORTED;
+}
+
+inline const char* fmt_name(Fmt f, bool sym) {
+  switch (f) {
+    case Fmt::FP16: return "fp16";
+    case Fmt::W8A8: return "w8a8_g-1_sym";
+    case Fmt::W4A4: return "w4a4_g-1_sym";
+    case Fmt::W4A16: return sym ? "w4a16_g128_sym" : "w4a16_g128_asym";
+    case Fmt::W3A16: return sym ? "w3a16_g128_sym" : "w3a16_g128_asym";
+    default: return "unsupported";
+  }
+}
+
+struct BranchInfo {
+  Fmt fmt;
+  int BM, BN, BK, WGM, WGN;
+  int lds_bytes;
+  int k_multiple;  // K must be a multiple of this
+  int max_m;       // largest M this branch accepts (skinny weight-only tiles), or 0 = any
+};
+
+template <class T>
+struct BranchOf;
+template <Op OP, int BM, int BN, int WGM, int WGN>
+struct BranchOf<MfmaTile<OP, BM, BN, WGM, WGN>> {
+  static BranchInfo get() {
+    using T = MfmaTile<OP, BM, BN, WGM, WGN>;
+    const Fmt f = OP == Op::I8 ? Fmt::W8A8 : (OP == Op::I4 ? Fmt::W4A4 : Fmt::FP16);
+    return BranchInfo{f, BM, BN, T::BK, WGM, WGN, T::kLdsBytes, T::BK, 0};
+  }
+};
+template <int WBITS, int BN>
+struct BranchOf<SkinnyWoTile<WBITS, BN>> {
+  static BranchInfo get() {
+    using T = SkinnyWoTile<WBITS, BN>;
+    return BranchInfo{WBITS == 4 ? Fmt::W4A16 : Fmt::W3A16, T::BM, BN, 128, 1, 4, T::kLdsBytes, 128, 0};
+  }
+};
+
+using LaunchFn = hipError_t (*)(const FusedArgs&, int grid, int lds, hipStream_t);
+
+struct FusedKernel {
+  std::string name;  // "[qcfg: (BM,BN,BK) (WGM,WGN,1) 2], ...<fn name>" — same shape as registry.cuh:42-70
+  std::vector<BranchInfo> branches;
+  int lds_bytes;
+  LaunchFn launch;
+};
+
+inline std::vector<FusedKernel>& registry() {
+  static std::vector<FusedKernel> r;
+  return r;
+}
+
+inline std::string& last_error() {
+  static thread_local std::string e;
+  return e;
+}
+
+template <class... Tiles>
+hipError_t launch_fused(const FusedArgs& a, int grid, int lds, hipStream_t s) {
+  hipLaunchKernelGGL((fused_group_gemm_kernel<Tiles...>), dim3(grid), dim3(kThreads), lds, s, a);
+  return hipGetLastError();
+}
+
+template <class... Tiles>
+int register_fused(const char* fn_name) {
+  FusedKernel k;
+  k.branches = {BranchOf<Tiles>::get()...};
+  k.lds_bytes = 0;
+  std::string n;
+  for (const auto& b : k.branches) {
+    char buf[160];
+    snprintf(buf, sizeof buf, "[%s: (%d,%d,%d) (%d,%d,1) 2], ", fmt_name(b.fmt, b.fmt == Fmt::W8A8 || b.fmt == Fmt::W4A4), b.BM, b.BN, b.BK, b.WGM, b.WGN);
+    n += buf;
+    k.lds_bytes = std::max(k.lds_bytes, b.lds_bytes);
+  }
+  k.name = n + fn_name;
+  k.launch = &launch_fused<Tiles...>;
+  if (k.lds_bytes > 64 * 1024) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&fused_group_gemm_kernel<Tiles...>), hipFuncAttributeMaxDynamicSharedMemorySize, k.lds_bytes);
+  }
+  registry().push_back(k);
+  return (int)registry().size() - 1;
+}
+
+// Pick the branch of `k` that runs a problem: same format, then fewest padded rows, then the larger tile.
+inline int pick_branch(const FusedKernel& k, Fmt f, int M) {
+  int best = -1;
+  long best_pad = 0;
+  for (int i = 0; i < (int)k.branches.size(); ++i) {
+    const auto& b = k.branches[i];
+    if (b.fmt != f) continue;
+    const long pad = (long)((M + b.BM - 1) / b.BM) * b.BM;
+    if (best < 0 || pad < best_pad || (pad == best_pad && b.BM > k.branches[best].BM)) {
+      best = i;
+      best_pad = pad;
+    }
+  }
+  return best;
+}
+
+// A kernel can run a problem list when it has a branch for every format in it.
+inline bool kernel_covers(const FusedKernel& k, const mxmoe_qparams* q, int count) {
+  for (int i = 0; i < count; ++i) {
+    const Fmt f = classify(q[i]);
+    if (f == Fmt::UNSUPPORTED || pick_branch(k, f, 1) < 0) return false;
+  }
+  return true;
+}
+
+// Host launcher.  Array arguments as in the reference FuncType (registry.cuh:28-39): every pointer array and
+// d_sizes / d_q live in device memory, h_sizes / h_q are their host mirrors.  ld* and d_q are accepted and unused.
+inline int group_gemm(int kernel_id, const void* const* As, const void* const* Bs, const void* const* sa, const void* const* sb, void* const* Cs,
+                      int32_t* const* acc, const mxmoe_dim3* d_sizes, const mxmoe_dim3* h_sizes, const mxmoe_qparams* h_q, int count, hipStream_t stream) {
+  if (count <= 0) return 0;
+  auto& reg = registry();
+  if (kernel_id < 0) {
+    for (int i = 0; i < (int)reg.size() && kernel_id < 0; ++i)
+      if (kernel_covers(reg[i], h_q, count)) kernel_id = i;
+    if (kernel_id < 0) {
+      last_error() = "quant type not supported";  // same message as the reference launcher (compose_kernel.py:433)
+      return 1;
+    }
+  }
+  if (kernel_id >= (int)reg.size()) {
+    last_error() = "kernel id out of range";
+    return 2;
+  }
+  const FusedKernel& k = reg[kernel_id];
+  for (int base = 0; base < count; base += kMaxProblems) {
+    const int n = std::min(kMaxProblems, count - base);
+    FusedArgs a;
+    std::memset(&a, 0, sizeof a);
+    a.As = reinterpret_cast<const uint8_t* const*>(As);
+    a.Bs = reinterpret_cast<const uint8_t* const*>(Bs);
+    a.sa = reinterpret_cast<const _Float16* const*>(sa);
+    a.sb = reinterpret_cast<const _Float16* const*>(sb);
+    a.Cs = reinterpret_cast<_Float16* const*>(Cs);
+    a.acc = acc;
+    a.sizes = d_sizes;
+    a.problem_offset = base;
+    a.num_problems = n;
+    int total = 0;
+    for (int i = 0; i < n; ++i) {
+      const mxmoe_dim3& sz = h_sizes[base + i];
+      const Fmt f = classify(h_q[base + i]);
+      const int b = f == Fmt::UNSUPPORTED ? -1 : pick_branch(k, f, (int)sz.x);
+      if (b < 0) {
+        last_error() = "quant type not supported";
+        return 1;
+      }
+      const BranchInfo& bi = k.branches[b];
+      if (sz.z == 0 || sz.z % bi.k_multiple != 0 || sz.y % 4 != 0 || (bi.fmt != Fmt::FP16 && bi.fmt != Fmt::W8A8 && bi.fmt != Fmt::W4A4 && sz.y % 16 != 0)) {
+        char buf[200];
+        snprintf(buf, sizeof buf, "problem %d: shape [%u,%u,%u] not supported by tile %s (K %% %d, N %% 4)", base + i, sz.x, sz.y, sz.z, fmt_name(bi.fmt, true), bi.k_multiple);
+        last_error() = buf;
+        return 3;
+      }
+      total += (int)((sz.x + bi.BM - 1) / bi.BM) * (int)((sz.y + bi.BN - 1) / bi.BN);  // M == 0 contributes no tiles
+      a.prefix[i] = total;
+      a.branch[i] = (uint8_t)b;
+    }
+    if (total == 0) continue;
+    a.total_tiles = total;
+    a.chunk = (total + kNumXcd - 1) / kNumXcd;
+    const hipError_t e = k.launch(a, a.chunk * kNumXcd, k.lds_bytes, stream);
+    if (e != hipSuccess) {
+      last_error() = std::string("kernel launch failed: ") + hipGetErrorString(e);
+      return 4;
+    }
+  }
+  return 0;
+}
+
+}  // namespace mxmoe

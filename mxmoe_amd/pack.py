@@ -1,0 +1,65 @@
+"""Offline packers: quantised integers -> the gfx950 operand layouts the kernels read.
+
+Role of the reference's host packers `pack_wxax`, `permute_weight`, `pack_weightonly`, `permute_scale`
+(mxmoe/kernels/src/include/quantize.cuh:299-475).  The layouts are this library's own (nothing else reads the
+reference's), chosen for 64-lane waves: see csrc/include/mxmoe_tiles.hpp and mxmoe_wo_tiles.hpp.
+All functions are pure torch and run on whatever device their input lives on.
+"""
+from __future__ import annotations
+
+import torch
+
+# element e (0..7) of a dword's eight values sits in nibble (e >> 1) + 4 * (e & 1)
+_NIBBLE_OF_ELEM = [(e >> 1) + 4 * (e & 1) for e in range(8)]
+
+
+def pack_int4_k(q: torch.Tensor) -> torch.Tensor:
+    """Signed int4 values [R, K] (in [-8, 7]) -> uint8 [R, K/2]; element 2j in the low nibble of byte j.
+
+    Used for both operands of w4a4 (activations per token, weights per channel), K contiguous as in the
+    reference's `pack_wxax` (quantize.cuh:424-475), but with little-endian nibble order.
+    """
+    assert q.shape[-1] % 2 == 0
+    v = q.to(torch.int16) & 0xF
+    return (v[..., 0::2] | (v[..., 1::2] << 4)).to(torch.uint8).contiguous()
+
+
+def unpack_int4_k(p: torch.Tensor) -> torch.Tensor:
+    """Inverse of `pack_int4_k` -> int8 [R, K]."""
+    lo = (p.to(torch.int16) & 0xF)
+    hi = (p.to(torch.int16) >> 4) & 0xF
+    v = torch.stack([lo, hi], dim=-1).reshape(*p.shape[:-1], p.shape[-1] * 2)
+    return torch.where(v >= 8, v - 16, v).to(torch.int8)
+
+
+def pack_weight_only(q: torch.Tensor, bits: int) -> torch.Tensor:
+    """Unsigned weight codes [N, K] (0 .. 2^bits - 1) -> int32 [N/16, K/128, 64, bits] (flattened to 1-D).
+
+    Lane l of block (nb, kb) carries channel nb*16 + (l & 15), k = kb*128 + (l >> 4)*32 + 0..31.
+    bits == 4: dword j holds values 8j..8j+7, value e in nibble (e >> 1) + 4*(e & 1).
+    bits == 3: dwords 0..2 hold values 0..23 in the low three bits of their nibbles; bit 3 of nibble p of
+    dword d holds bit d of value 24 + e(p).
+    """
+    assert bits in (3, 4)
+    n, k = q.shape
+    assert n % 16 == 0 and k % 128 == 0
+    v = q.to(torch.int64).reshape(n // 16, 16, k // 128, 4, 32)       # [nb, row, kb, g, e32]
+    v = v.permute(0, 2, 3, 1, 4).reshape(n // 16, k // 128, 64, 32)    # lane = g*16 + row
+    shifts = torch.tensor([4 * p for p in _NIBBLE_OF_ELEM], dtype=torch.int64, device=q.device)
+    ndw = 4 if bits == 4 else 3
+    main = v[..., : ndw * 8].reshape(*v.shape[:-1], ndw, 8)
+    dw = (main << shifts).sum(dim=-1)                                  # [nb, kb, 64, ndw]
+    if bits == 3:
+        extra = v[..., 24:32]                                          # values 24..31
+        for d in range(3):
+            dw[..., d] |= (((extra >> d) & 1) << (shifts + 3)).sum(dim=-1)
+    dw = torch.where(dw >= 2**31, dw - 2**32, dw).to(torch.int32)
+    return dw.reshape(-1).contiguous()
+
+
+def pack_weight_only_scales(scale: torch.Tensor, zero: torch.Tensor) -> torch.Tensor:
+    """Group scale / zero [N, K/128] fp16 -> fp16 [N/16, K/128, 16, 2] flattened (scale, zero interleaved)."""
+    n, g = scale.shape
+    assert n % 16 == 0
+    sz = torch.stack([scale.to(torch.float16), zero.to(torch.float16)], dim=-1)  # [N, G, 2]
+    return sz.reshape(n // 16, 16, g, 2).permute(0, 2, 1, 3).reshape(-1).contiguous()

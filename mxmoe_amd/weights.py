@@ -1,0 +1,54 @@
+"""Quantise + pack one weight matrix [N, K] for a format; the result is what `Bs[p]` / `scale_b[p]` point to."""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+
+from . import pack
+from .quant import quant_minmax
+
+
+@dataclass
+class PackedWeight:
+    data: torch.Tensor            # packed weights in the kernel's layout
+    scale: torch.Tensor | None    # per-channel scales [N] (w-a) or group (scale, zero) table (weight-only)
+    qparams: tuple                # (a_bits, w_bits, gsize, sym)
+    n: int
+    k: int
+    q: torch.Tensor | None = None  # integer codes [N, K] (kept only when asked; tests)
+
+    @property
+    def nbytes(self) -> int:
+        return self.data.numel() * self.data.element_size() + (0 if self.scale is None else self.scale.numel() * self.scale.element_size())
+
+
+def quantize_and_pack(w: torch.Tensor, qparams, keep_codes: bool = False) -> PackedWeight:
+    """RTN-quantise `w` [N, K] fp16 for `(a_bits, w_bits, gsize, sym)` and pack it.
+
+    fp16: kept as is.  w8a8 / w4a4: per-channel symmetric codes, int8 [N, K] / packed nibbles [N, K/2], fp16 scale [N].
+    w4a16 / w3a16 group-128: unsigned codes in the wave-interleaved layout with a (scale, zero) table; symmetric
+    variants are stored offset-binary with zero = -2^(b-1) * scale (exact).
+    """
+    a_bits, w_bits, gsize, sym = qparams
+    n, k = w.shape
+    if w_bits >= 16:
+        return PackedWeight(w.contiguous(), None, tuple(qparams), n, k)
+    q, scale, zp = quant_minmax(w, w_bits, gsize, sym)
+    if a_bits < 16:
+        assert gsize == -1 and sym, "w-a formats are per-channel symmetric"
+        qi = q.to(torch.int8)
+        data = qi.contiguous() if w_bits == 8 else pack.pack_int4_k(qi)
+        return PackedWeight(data, scale.reshape(n).contiguous(), tuple(qparams), n, k, qi if keep_codes else None)
+    assert gsize == 128, "weight-only kernels implement group size 128"
+    g = k // gsize
+    scale = scale.reshape(n, g)
+    zp = zp.reshape(n, g)
+    codes = q.reshape(n, k)
+    if sym:
+        off = 1 << (w_bits - 1)
+        codes = codes + off
+        zp = (-off * scale).to(scale.dtype)
+    codes = codes.to(torch.uint8)
+    return PackedWeight(pack.pack_weight_only(codes, w_bits), pack.pack_weight_only_scales(scale, zp), tuple(qparams), n, k,
+                        codes if keep_codes else None)

@@ -1,0 +1,114 @@
+"""GPU parity of the fused GroupGEMM (through the C-ABI) against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import mxmoe_oracle as O
+
+pytestmark = pytest.mark.gpu
+F16 = np.float16
+DEV = "cuda"
+
+
+def _rel(a, b):
+    a = a.astype(np.float64)
+    b = b.astype(np.float64)
+    return np.abs(a - b).max() / max(np.abs(b).max(), 1e-6)
+
+
+def _wxax_problem(rng, m, n, k, bits, rotate=False):
+    from mxmoe_amd import pack
+
+    x = rng.standard_normal((m, k)).astype(F16)
+    w = (rng.standard_normal((n, k)) * 0.02).astype(F16)
+    qa, sa, _ = O.quant_minmax(x, bits, -1, True)
+    qb, sb, _ = O.quant_minmax(w, bits, -1, True)
+    ta, tb = torch.from_numpy(qa.astype(np.int8)), torch.from_numpy(qb.astype(np.int8))
+    if bits == 4:
+        ta, tb = pack.pack_int4_k(ta), pack.pack_int4_k(tb)
+    acc = O.int_gemm(qa, qb)
+    return dict(A=ta.to(DEV), B=tb.to(DEV), sa=torch.from_numpy(sa.reshape(-1)).to(DEV), sb=torch.from_numpy(sb.reshape(-1)).to(DEV),
+                acc=acc, out=O.epilogue_wxax(acc, sa.reshape(-1), sb.reshape(-1)),
+                fq=O.gemm_fakequant(O.dequant(qa, sa, 0 * sa, -1), O.dequant(qb, sb, 0 * sb, -1)),
+                size=(m, n, k), q=(bits, bits, -1, True))
+
+
+def _launch(probs, kernel_id=-1, dump=True):
+    from mxmoe_amd.group_gemm import GroupGemmLaunch
+
+    Cs = [torch.full((p["size"][0], p["size"][1]), float("nan"), dtype=torch.float16, device=DEV) for p in probs]
+    accs = [torch.zeros((p["size"][0], p["size"][1]), dtype=torch.int32, device=DEV) for p in probs] if dump else None
+    g = GroupGemmLaunch([p["A"] for p in probs], [p["B"] for p in probs], [p.get("sa") for p in probs], [p.get("sb") for p in probs],
+                        Cs, [p["size"] for p in probs], [p["q"] for p in probs], kernel_id=kernel_id, acc=accs)
+    g.run()
+    torch.cuda.synchronize()
+    return g, [c.cpu().numpy() for c in Cs], ([a.cpu().numpy() for a in accs] if dump else None)
+
+
+def test_wxax_mixed_launch_bit_exact_accumulators():
+    rng = np.random.default_rng(0)
+    shapes = [(1, 256, 128, 4), (31, 512, 256, 8), (33, 384, 1408, 4), (130, 256, 256, 8), (300, 768, 384, 4),
+              (64, 2816, 2048, 4), (129, 2048, 1408, 8), (17, 260, 128, 8)]
+    probs = [_wxax_problem(rng, m, n, k, b) for (m, n, k, b) in shapes]
+    g, outs, accs = _launch(probs)
+    kid, branches, tiles = g.plan()
+    print("kernel", kid, "branches", branches, "tiles", tiles)
+    for p, out, acc in zip(probs, outs, accs):
+        assert np.array_equal(acc, p["acc"]), f"int32 accumulators differ for {p['size']} {p['q']}"
+        assert np.array_equal(out.view(np.uint16), p["out"].view(np.uint16)), f"fp16 epilogue differs for {p['size']}"
+        assert _rel(out, p["fq"]) <= 1e-2                                  # tolerance of the fake-quant comparison
+
+
+def test_wxax_empty_and_single_row_problems():
+    rng = np.random.default_rng(1)
+    probs = [_wxax_problem(rng, m, 256, 128, b) for (m, b) in [(5, 8), (1, 4)]]
+    empty = dict(probs[0])
+    empty.update(A=torch.zeros((0, 128), dtype=torch.int8, device=DEV), sa=torch.zeros(0, dtype=torch.float16, device=DEV), size=(0, 256, 128))
+    g, outs, accs = _launch([probs[0], empty, probs[1]])
+    assert np.array_equal(accs[0], probs[0]["acc"]) and np.array_equal(accs[2], probs[1]["acc"])
+    assert outs[1].shape == (0, 256)
+
+
+def test_fp16_group_gemm():
+    rng = np.random.default_rng(2)
+    probs = []
+    for (m, n, k) in [(34, 2816, 2048), (7, 512, 64), (200, 256, 1408), (128, 260, 32)]:
+        x = rng.standard_normal((m, k)).astype(F16)
+        w = (rng.standard_normal((n, k)) * 0.02).astype(F16)
+        probs.append(dict(A=torch.from_numpy(x).to(DEV), B=torch.from_numpy(w).to(DEV), ref=O.gemm_fp16(x, w), size=(m, n, k), q=(16, 16, -1, True)))
+    _, outs, _ = _launch(probs, dump=False)
+    for p, out in zip(probs, outs):
+        assert _rel(out, p["ref"]) <= 1e-2, p["size"]
+        assert _rel(out, p["ref"]) <= 2e-3                                 # fp32 accumulation: far inside the tolerance
+
+
+def test_weight_only_skinny():
+    from mxmoe_amd.weights import quantize_and_pack
+
+    rng = np.random.default_rng(3)
+    probs = []
+    for (m, n, k, bits, sym) in [(3, 2816, 2048, 4, False), (1, 256, 128, 3, False), (16, 128, 1408, 3, False), (32, 5632, 2048, 4, False),
+                                 (5, 2048, 1408, 4, True), (19, 144, 256, 3, True)]:
+        x = rng.standard_normal((m, k)).astype(F16)
+        w = (rng.standard_normal((n, k)) * 0.02).astype(F16)
+        pw = quantize_and_pack(torch.from_numpy(w), (16, bits, 128, sym), keep_codes=True)
+        q, s, z = O.quant_minmax(w, bits, 128, sym)
+        codes = q.reshape(n, k) + ((1 << (bits - 1)) if sym else 0)
+        assert np.array_equal(pw.q.numpy(), codes.astype(np.uint8))        # torch quantiser == oracle quantiser
+        ref = O.gemm_fakequant(x, O.dequant(q, s, z, 128))
+        probs.append(dict(A=torch.from_numpy(x).to(DEV), B=pw.data.to(DEV), sb=pw.scale.to(DEV), ref=ref, size=(m, n, k), q=(16, bits, 128, sym)))
+    _, outs, _ = _launch(probs, dump=False)
+    for p, out in zip(probs, outs):
+        assert _rel(out, p["ref"]) <= 1e-2, (p["size"], p["q"], _rel(out, p["ref"]))
+
+
+def test_unsupported_format_raises_reference_message():
+    rng = np.random.default_rng(4)
+    p = _wxax_problem(rng, 4, 256, 128, 8)
+    p["q"] = (8, 4, -1, True)
+    with pytest.raises(RuntimeError, match="quant type not supported"):
+        _launch([p])
+    p = _wxax_problem(rng, 4, 256, 128, 8)
+    p["size"] = (4, 256, 100)
+    with pytest.raises(RuntimeError, match="not supported by tile"):
+        _launch([p])

@@ -1,0 +1,66 @@
+"""Host checks of the packed layouts: a numpy model of the kernels' in-register unpack must invert the packers."""
+import numpy as np
+import torch
+
+from mxmoe_amd import pack
+
+NIB = [(e >> 1) + 4 * (e & 1) for e in range(8)]
+
+
+def _cvt8(d, mask_bits):
+    """Model of SkinnyWoTile::cvt8: (d & LO), (d & HI), then the same on d >> 8 -> 8 values in k order."""
+    d = d.astype(np.uint64)
+    lo = (1 << mask_bits) - 1
+    out = np.zeros(d.shape + (8,), dtype=np.int64)
+    for half, src in enumerate((d, d >> 8)):
+        out[..., 4 * half + 0] = src & lo                    # low half of (x & MASK_LO)
+        out[..., 4 * half + 1] = (src >> 16) & lo            # high half
+        out[..., 4 * half + 2] = (src >> 4) & lo             # low half of (x & MASK_HI), weight 16 folded by the 64.0 magic
+        out[..., 4 * half + 3] = (src >> 20) & lo
+    return out
+
+
+def _unpack_model(dw, bits):
+    dw = dw.astype(np.int64) & 0xFFFFFFFF
+    if bits == 4:
+        return np.concatenate([_cvt8(dw[..., j], 4) for j in range(4)], axis=-1)
+    t = ((dw[..., 0] >> 3) & 0x11111111) | ((dw[..., 1] >> 2) & 0x22222222) | ((dw[..., 2] >> 1) & 0x44444444)
+    return np.concatenate([_cvt8(dw[..., j], 3) for j in range(3)] + [_cvt8(t, 3)], axis=-1)
+
+
+def test_int4_k_pack_roundtrip_and_nibble_order():
+    q = torch.randint(-8, 8, (7, 64), dtype=torch.int8)
+    p = pack.pack_int4_k(q)
+    assert p.shape == (7, 32) and p.dtype == torch.uint8
+    assert torch.equal(pack.unpack_int4_k(p), q)
+    one = torch.zeros(1, 4, dtype=torch.int8)
+    one[0, 0], one[0, 1] = 3, -2
+    assert pack.pack_int4_k(one)[0, 0].item() == (3 | (14 << 4))       # element 0 low nibble, element 1 high nibble
+    # kernel-side widening: (x << 4) & 0xF0 and x & 0xF0 as int8 equal 16 * value
+    b = p.numpy().astype(np.uint8)
+    even = ((b.astype(np.uint16) << 4) & 0xF0).astype(np.uint8).view(np.int8)
+    odd = (b & 0xF0).view(np.int8)
+    assert np.array_equal(even, 16 * q.numpy()[:, 0::2]) and np.array_equal(odd, 16 * q.numpy()[:, 1::2])
+
+
+def test_weight_only_pack_matches_kernel_unpack_model():
+    for bits in (4, 3):
+        n, k = 48, 384
+        codes = torch.randint(0, 1 << bits, (n, k), dtype=torch.uint8)
+        dw = pack.pack_weight_only(codes, bits).numpy().reshape(n // 16, k // 128, 64, bits)
+        vals = _unpack_model(dw, bits)                               # [nb, kb, lane, 32]
+        for nb in range(n // 16):
+            for kb in range(k // 128):
+                for lane in (0, 1, 15, 16, 37, 63):
+                    row = nb * 16 + (lane & 15)
+                    k0 = kb * 128 + (lane >> 4) * 32
+                    assert np.array_equal(vals[nb, kb, lane], codes[row, k0:k0 + 32].numpy())
+        assert dw.size * 4 == n * k * bits // 8                         # exactly `bits` bits per weight
+
+
+def test_weight_only_scale_table_layout():
+    n, g = 32, 3
+    s = torch.arange(n * g, dtype=torch.float16).reshape(n, g)
+    z = -s
+    t = pack.pack_weight_only_scales(s, z).reshape(n // 16, g, 16, 2)
+    assert t[1, 2, 5, 0] == s[16 + 5, 2] and t[1, 2, 5, 1] == z[16 + 5, 2]
