@@ -8,6 +8,7 @@
  * Each entry point names the reference interface it replaces (paths relative to the reference repository).
  */
 #pragma once
+#include <stddef.h>
 #include <stdint.h>
 
 #include "../mxmoe_amd/csrc/include/mxmoe_types.h"
@@ -59,6 +60,37 @@ int mxmoe_group_gemm(int kernel_id, const void* const* As, const void* const* Bs
 /* Tile count and branch choice the launcher would make, without launching: fills branch_out[p] and returns the total
  * number of tiles through *tiles_out.  Host-only; used by the scheduler tests and the kernel-profile table. */
 int mxmoe_group_gemm_plan(int kernel_id, const mxmoe_dim3* h_sizes, const mxmoe_qparams* h_q, int problem_count, int32_t* branch_out, int32_t* tiles_out);
+
+/* ---- token permutation: replaces gg_permute_inp and the sort / bincount prologue of quant_inp_act
+ *      (mxmoe/kernels/src/ref_bind.cu:47-64, 449-453) ----
+ *
+ * topk_ids [num_tokens, topk] int32 (device).  Writes, in STABLE order (by expert, then by flattened (token, slot) index):
+ * dst_exp_sorted [R] int32, perm_indices [R] int64 (source token of each sorted row), src_slot [R] int64 (flattened
+ * (token, slot) index; may be NULL) and recv_tokens_per_exp [E] int64 (device), R = num_tokens * topk.
+ * `workspace` is device scratch of mxmoe_permute_workspace_bytes(R, E) bytes.  Ids outside [0, E) are dropped. */
+size_t mxmoe_permute_workspace_bytes(int total_rows, int num_experts);
+int mxmoe_build_permutation(const int32_t* topk_ids, int num_tokens, int topk, int num_experts, int32_t* dst_exp_sorted, int64_t* perm_indices,
+                            int64_t* src_slot, int64_t* recv_tokens_per_exp, void* workspace, void* stream);
+
+/* ---- activation quantisers: replace the launches of quant_act_kernel and silu_mul_then_quant_kernel
+ *      (mxmoe/kernels/src/ref_bind.cu:524-544 and 691-716; their source, act_kernel.cuh, is absent from the reference) ----
+ *
+ * One workgroup per destination row; rows 0..R-1 are the routed rows in sorted order, rows R..R+T-1 (when has_shared) the
+ * always-on shared expert, stored as expert index E.  exp_table is a DEVICE int64 [4][E(+1)] table: tag (0 fp16 copy,
+ * 1 int8 per token, 2 int4 per token), first row, offset into inp_store and offset into scale_store, both offsets in fp16
+ * elements exactly as ref_bind.cu:475-505 computes them (row strides K, K/2, K/4 halves; one scale per row).
+ * rotate: 0 no rotation, 1 rotate rows of quantised experts, 2 rotate every row, with y = (H_k kron H_{n/k}) x / sqrt(n)
+ * (mxmoe/quant/hadamard_utils.py:96-106).  had_k = 1 for power-of-two rows; otherwise H_k = S_f kron B and had_signs is a
+ * DEVICE float [(k/f)^2] array holding B as +-1.0 (mxmoe/quant/hadamard_utils.py:162-4379 tables).
+ *
+ * mxmoe_quant_act gathers row perm_indices[r] of hidden [T, K] (shared rows read token r - R).
+ * mxmoe_silu_mul_quant reads gate_up [R, 2N] (first half gate, second half up; shared rows from gate_up_shared [T, 2*N_shared]),
+ * computes silu(gate) * up in fp32 rounded once to fp16, then rotates / quantises / packs like mxmoe_quant_act. */
+int mxmoe_quant_act(const void* hidden, void* inp_store, void* scale_store, const int32_t* dst_exp_sorted, const int64_t* perm_indices, const int64_t* exp_table,
+                    int K, int rows_routed, int num_tokens, int num_experts, int has_shared, int rotate, int had_k, int had_f, const float* had_signs, void* stream);
+int mxmoe_silu_mul_quant(const void* gate_up, const void* gate_up_shared, void* inp_store, void* scale_store, const int32_t* dst_exp_sorted, const int64_t* exp_table,
+                         int N, int N_shared, int rows_routed, int num_tokens, int num_experts, int has_shared, int rotate, int had_k, int had_f,
+                         const float* had_signs, void* stream);
 
 #ifdef __cplusplus
 }

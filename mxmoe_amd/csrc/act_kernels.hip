@@ -1,0 +1,524 @@
+// Prologue kernels of the MoE layer on gfx950:
+//   * stable token permutation by expert (histogram -> scan -> ranked scatter);
+//   * gather + online Hadamard rotation + per-token quantisation + packing      (quant_act);
+//   * SiLU(gate) * up + online Hadamard rotation + per-token quantisation + packing (silu_mul_then_quant).
+//
+// The reference launches `quant_act_kernel` / `silu_mul_then_quant_kernel` (mxmoe/kernels/src/ref_bind.cu:531-544,
+// 701-716) whose source file (act_kernel.cuh) is absent from the reference; the contracts implemented here are the
+// launch arguments and the host offset builder of ref_bind.cu:461-505, 635-671: one workgroup per destination row,
+// rows grouped by expert, per-expert tag {0 fp16 copy, 1 int8, 2 int4}, row strides K, K/2, K/4 halves, one fp16
+// scale per row.  The permutation replaces torch::sort + bincount of ref_bind.cu:47-64,449-453 with a STABLE order.
+//
+// Arithmetic is the exact operation sequence of the fp16 quantiser (mxmoe/quant/quant.py:68-84: absmax / upper,
+// x / scale, clamp, round-half-even, all rounded to fp16) and of a fixed-order fp32 Hadamard transform, so integer
+// codes are reproducible bit for bit on a CPU; this file must be compiled with FMA contraction off.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <cmath>
+#include <string>
+
+#include "../../include/mxmoe_amd.h"
+#include "include/mxmoe_launch.hpp"
+
+namespace mxmoe {
+
+// ------------------------------------------------------------------------------------------------------------
+// Stable permutation by expert
+// ------------------------------------------------------------------------------------------------------------
+constexpr int kPermChunk = 256;  // flattened (token, slot) entries per single-wave workgroup
+
+// lanes of the wave that hold the same expert id as this lane (ids < 2^16)
+__device__ __forceinline__ uint64_t match_same(int e, int nbits) {
+  uint64_t m = ~0ull;
+  for (int b = 0; b < nbits; ++b) {
+    const uint64_t bal = __ballot((e >> b) & 1);
+    m &= ((e >> b) & 1) ? bal : ~bal;
+  }
+  return m;
+}
+
+__global__ void __launch_bounds__(64) perm_hist_kernel(const int32_t* __restrict__ ids, int total, int E, int32_t* __restrict__ hist /*[blocks][E]*/) {
+  extern __shared__ int32_t cnt[];
+  for (int e = threadIdx.x; e < E; e += 64) cnt[e] = 0;
+  __syncthreads();
+  const int base = blockIdx.x * kPermChunk;
+  for (int i = threadIdx.x; i < kPermChunk; i += 64) {
+    const int idx = base + i;
+    if (idx < total) {
+      const int e = ids[idx];
+      if (e >= 0 && e < E) atomicAdd(&cnt[e], 1);
+    }
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += 64) hist[blockIdx.x * E + e] = cnt[e];
+}
+
+// one workgroup: per expert, exclusive scan over blocks; expert offsets; counts as int64
+__global__ void __launch_bounds__(256) perm_scan_kernel(int32_t* __restrict__ hist, int blocks, int E, int64_t* __restrict__ recv, int32_t* __restrict__ expert_off) {
+  extern __shared__ int32_t tot[];
+  for (int e = threadIdx.x; e < E; e += 256) {
+    int run = 0;
+    for (int b = 0; b < blocks; ++b) {
+      const int v = hist[b * E + e];
+      hist[b * E + e] = run;
+      run += v;
+    }
+    tot[e] = run;
+    recv[e] = run;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int run = 0;
+    for (int e = 0; e < E; ++e) {
+      expert_off[e] = run;
+      run += tot[e];
+    }
+  }
+}
+
+__global__ void __launch_bounds__(64) perm_scatter_kernel(const int32_t* __restrict__ ids, int total, int E, int topk, int nbits, const int32_t* __restrict__ hist,
+                                                          const int32_t* __restrict__ expert_off, int32_t* __restrict__ dst_exp_sorted, int64_t* __restrict__ perm,
+                                                          int64_t* __restrict__ src_slot) {
+  extern __shared__ int32_t run[];  // next free rank per expert for this block
+  for (int e = threadIdx.x; e < E; e += 64) run[e] = expert_off[e] + hist[blockIdx.x * E + e];
+  __syncthreads();
+  const int lane = threadIdx.x;
+  const int base = blockIdx.x * kPermChunk;
+  for (int i = 0; i < kPermChunk; i += 64) {  // sub-chunks in order keep the sort stable
+    const int idx = base + i + lane;
+    const bool ok = idx < total;
+    int e = ok ? ids[idx] : -1;
+    if (e < 0 || e >= E) e = E;  // parked on a dummy id, never written
+    const uint64_t same = match_same(e, nbits);
+    const int before = __popcll(same & ((1ull << lane) - 1));
+    int first = 0;
+    if (e < E) first = run[e];
+    __syncthreads();
+    if (e < E) {
+      const int pos = first + before;
+      dst_exp_sorted[pos] = e;
+      perm[pos] = idx / topk;
+      if (src_slot) src_slot[pos] = idx;
+      if (before == 0) run[e] = first + __popcll(same);
+    }
+    __syncthreads();
+  }
+}
+
+// ------------------------------------------------------------------------------------------------------------
+// Row kernels
+// ------------------------------------------------------------------------------------------------------------
+struct RotPlan {
+  int n;        // row length
+  int m;        // length of the Sylvester part (n = K * m), power of two >= 8
+  int f;        // H_K = S_f kron B
+  int kb;       // order of B (1 when K == 1)
+  float scale;  // 1 / sqrt(n), computed in fp32 on the host
+};
+
+struct RowArgs {
+  const _Float16* src;
+  const _Float16* src_shared;
+  uint8_t* inp_store;
+  _Float16* scale_store;
+  const int32_t* dst_exp;
+  const int64_t* perm;
+  const int64_t* table;  // [4][Et]: tag, start_row, inp_off, scale_off (offsets in fp16 elements)
+  const float* signs;    // B as +-1.0f, [kb][kb], or null
+  int R, T, E, Et;
+  int rows;
+  int rotate;  // 0 never, 1 rows of quantised experts, 2 every row
+  RotPlan plan, plan_shared;
+};
+
+// fixed fp32 op sequence for exp(t), identical to the CPU restatement
+__device__ __forceinline__ float exp_fixed(float t) {
+  t = fminf(fmaxf(t, -87.0f), 87.0f);
+  const float k = rintf(t * 1.4426950408889634f);
+  float r = t - k * 0.693145751953125f;
+  r = r - k * 1.428606765330187e-06f;
+  float p = 0.0001984127f;
+  p = p * r + 0.0013888889f;
+  p = p * r + 0.008333334f;
+  p = p * r + 0.041666668f;
+  p = p * r + 0.16666667f;
+  p = p * r + 0.5f;
+  p = p * r + 1.0f;
+  p = p * r + 1.0f;
+  return ldexpf(p, (int)k);
+}
+
+__device__ __forceinline__ float round_h(float v) { return (float)(_Float16)v; }
+
+template <int MAXC, bool SILU>
+__global__ void __launch_bounds__(256) row_quant_kernel(const RowArgs a) {
+  extern __shared__ __align__(16) float lds[];
+  const int tid = threadIdx.x;
+  const int nmax = max(a.plan.n, a.plan_shared.n);
+  float* x = lds;                  // [nmax]
+  float* sg = lds + nmax;          // [kb*kb]
+  float* red = sg + a.plan.kb * a.plan.kb;  // [8]
+  if (a.signs) {
+    for (int i = tid; i < a.plan.kb * a.plan.kb; i += 256) sg[i] = a.signs[i];
+  }
+
+  for (int row = blockIdx.x; row < a.rows; row += gridDim.x) {
+    const bool shared_row = row >= a.R;
+    const int e = shared_row ? a.E : a.dst_exp[row];
+    const RotPlan pl = shared_row ? a.plan_shared : a.plan;
+    const int n = pl.n;
+    const int nchunks = n >> 3;
+    const int tag = (int)a.table[e];
+    const long start_row = a.table[a.Et + e];
+    const long inp_off = a.table[2 * a.Et + e];
+    const long scale_off = a.table[3 * a.Et + e];
+    const long lrow = row - start_row;
+    const bool rot = a.rotate == 2 || (a.rotate == 1 && tag != 0);
+
+    const _Float16* srow;
+    if (SILU) {
+      srow = shared_row ? a.src_shared + (long)(row - a.R) * 2 * n : a.src + (long)row * 2 * n;
+    } else {
+      srow = a.src + (shared_row ? (long)(row - a.R) : (long)a.perm[row]) * n;
+    }
+
+    float v[MAXC][8];
+    __syncthreads();  // previous row fully consumed (and the sign table staged)
+#pragma unroll
+    for (int i = 0; i < MAXC; ++i) {
+      const int c = tid + i * 256;
+      if (c < nchunks) {
+        const v8h g = *reinterpret_cast<const v8h*>(srow + c * 8);
+        if (SILU) {
+          const v8h u = *reinterpret_cast<const v8h*>(srow + n + c * 8);
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const float gf = (float)g[j];
+            const float s = gf / (1.0f + exp_fixed(-gf));
+            v[i][j] = round_h(keep_f32(s * (float)u[j]));
+          }
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) v[i][j] = (float)g[j];
+        }
+        if (rot) {
+          // Sylvester strides 1, 2, 4 inside the chunk
+#pragma unroll
+          for (int h = 1; h < 8; h <<= 1) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+              if (!(j & h)) {
+                const float p = v[i][j], q = v[i][j + h];
+                v[i][j] = p + q;
+                v[i][j + h] = p - q;
+              }
+            }
+          }
+#pragma unroll
+          for (int j = 0; j < 8; ++j) x[c * 8 + j] = v[i][j];
+        }
+      }
+    }
+
+    if (rot) {
+      // Sylvester strides 8 .. m/2 through LDS (ascending)
+      for (int h = 8; h < pl.m; h <<= 1) {
+        const int hc = h >> 3;
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < MAXC; ++i) {
+          const int c = tid + i * 256;
+          if (c < nchunks) {
+            const float* o = x + (c ^ hc) * 8;
+            const bool upper = c & hc;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[i][j] = upper ? o[j] - v[i][j] : v[i][j] + o[j];
+          }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < MAXC; ++i) {
+          const int c = tid + i * 256;
+          if (c < nchunks) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) x[c * 8 + j] = v[i][j];
+          }
+        }
+      }
+      // scale, round to fp16
+#pragma unroll
+      for (int i = 0; i < MAXC; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[i][j] = round_h(keep_f32(v[i][j] * pl.scale));
+
+      if (pl.kb > 1) {
+        const int mc = pl.m >> 3;  // chunks per k row
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < MAXC; ++i) {
+          const int c = tid + i * 256;
+          if (c < nchunks) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) x[c * 8 + j] = v[i][j];
+          }
+        }
+        __syncthreads();
+        // dense B stage: t[b] = sum_{b'} B[b][b'] v[b'], b' ascending, starting from 0
+#pragma unroll
+        for (int i = 0; i < MAXC; ++i) {
+          const int c = tid + i * 256;
+          if (c < nchunks) {
+            const int k = c / mc, jc = c - k * mc;
+            const int blk = k / pl.kb, b = k - blk * pl.kb;
+            const float* vb = x + ((long)blk * pl.kb * mc + jc) * 8;
+            const float* sr = sg + b * pl.kb;
+            float acc[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) acc[j] = 0.0f;
+            for (int bp = 0; bp < pl.kb; ++bp) {
+              const float s = sr[bp];
+              const float* vv = vb + (long)bp * mc * 8;
+#pragma unroll
+              for (int j = 0; j < 8; ++j) acc[j] = acc[j] + s * vv[j];
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[i][j] = acc[j];
+          }
+        }
+        // S_f butterflies across blocks of kb rows (ascending)
+        for (int hh = 1; hh < pl.f; hh <<= 1) {
+          const int hc = hh * pl.kb * mc;
+          __syncthreads();
+#pragma unroll
+          for (int i = 0; i < MAXC; ++i) {
+            const int c = tid + i * 256;
+            if (c < nchunks) {
+#pragma unroll
+              for (int j = 0; j < 8; ++j) x[c * 8 + j] = v[i][j];
+            }
+          }
+          __syncthreads();
+#pragma unroll
+          for (int i = 0; i < MAXC; ++i) {
+            const int c = tid + i * 256;
+            if (c < nchunks) {
+              const bool upper = ((c / (pl.kb * mc)) & hh) != 0;
+              const float* o = x + (long)(upper ? c - hc : c + hc) * 8;
+#pragma unroll
+              for (int j = 0; j < 8; ++j) v[i][j] = upper ? o[j] - v[i][j] : v[i][j] + o[j];
+            }
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < MAXC; ++i)
+#pragma unroll
+          for (int j = 0; j < 8; ++j) v[i][j] = round_h(v[i][j]);
+      }
+    }
+
+    // ---- store: fp16 copy or per-token symmetric quantisation ----
+    if (tag == 0) {
+      _Float16* out = reinterpret_cast<_Float16*>(a.inp_store) + inp_off + lrow * n;
+#pragma unroll
+      for (int i = 0; i < MAXC; ++i) {
+        const int c = tid + i * 256;
+        if (c < nchunks) {
+          v8h o;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) o[j] = (_Float16)v[i][j];
+          *reinterpret_cast<v8h*>(out + c * 8) = o;
+        }
+      }
+      continue;
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < MAXC; ++i) {
+      const int c = tid + i * 256;
+      if (c < nchunks) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[i][j]));
+      }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
+    __syncthreads();
+    if ((tid & 63) == 0) red[tid >> 6] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    const float upper = tag == 1 ? 127.0f : 7.0f;
+    float scale = round_h(amax / upper);   // fp16 division: fp32 quotient of two fp16 values, rounded to fp16
+    if (scale == 0.0f) scale = 1.0f;       // quantize.cuh:258
+    if (tid == 0) a.scale_store[scale_off + lrow] = (_Float16)scale;
+    uint8_t* out = a.inp_store + 2 * (inp_off + lrow * (tag == 1 ? n / 2 : n / 4));
+#pragma unroll
+    for (int i = 0; i < MAXC; ++i) {
+      const int c = tid + i * 256;
+      if (c < nchunks) {
+        int q[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float r = round_h(v[i][j] / scale);
+          q[j] = (int)rintf(fminf(fmaxf(r, -upper), upper));
+        }
+        if (tag == 1) {
+          uint2 w;
+          w.x = (q[0] & 0xFF) | ((q[1] & 0xFF) << 8) | ((q[2] & 0xFF) << 16) | ((unsigned)(q[3] & 0xFF) << 24);
+          w.y = (q[4] & 0xFF) | ((q[5] & 0xFF) << 8) | ((q[6] & 0xFF) << 16) | ((unsigned)(q[7] & 0xFF) << 24);
+          *reinterpret_cast<uint2*>(out + c * 8) = w;
+        } else {
+          unsigned w = 0;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) w |= (unsigned)(q[j] & 0xF) << (4 * j);
+          *reinterpret_cast<unsigned*>(out + c * 4) = w;
+        }
+      }
+    }
+  }
+}
+
+static int make_plan(int n, int had_k, int had_f, RotPlan* p) {
+  p->n = n;
+  p->scale = 1.0f / sqrtf((float)n);
+  p->kb = 1;
+  p->f = 1;
+  p->m = n;
+  if (had_k > 1) {
+    if (n % had_k) return 1;
+    p->m = n / had_k;
+    p->f = had_f;
+    p->kb = had_k / had_f;
+  }
+  if (p->m < 8 || (p->m & (p->m - 1))) return 1;
+  return 0;
+}
+
+template <bool SILU>
+static int launch_rows(const RowArgs& a, int lds_bytes, hipStream_t s) {
+  const int nmax = a.plan.n > a.plan_shared.n ? a.plan.n : a.plan_shared.n;
+  const int chunks = (nmax / 8 + 255) / 256;
+  int dev = 0, cus = 256;
+  (void)hipGetDevice(&dev);
+  (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+  const int grid = a.rows < cus * 8 ? a.rows : cus * 8;
+  if (lds_bytes > 64 * 1024) {
+    last_error() = "row too long for the activation kernels";
+    return 3;
+  }
+  if (chunks <= 1) hipLaunchKernelGGL((row_quant_kernel<1, SILU>), dim3(grid), dim3(256), lds_bytes, s, a);
+  else if (chunks <= 2) hipLaunchKernelGGL((row_quant_kernel<2, SILU>), dim3(grid), dim3(256), lds_bytes, s, a);
+  else if (chunks <= 3) hipLaunchKernelGGL((row_quant_kernel<3, SILU>), dim3(grid), dim3(256), lds_bytes, s, a);
+  else if (chunks <= 7) hipLaunchKernelGGL((row_quant_kernel<7, SILU>), dim3(grid), dim3(256), lds_bytes, s, a);
+  else {
+    last_error() = "row too long for the activation kernels";
+    return 3;
+  }
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    last_error() = std::string("kernel launch failed: ") + hipGetErrorString(e);
+    return 4;
+  }
+  return 0;
+}
+
+}  // namespace mxmoe
+
+using namespace mxmoe;
+
+extern "C" {
+
+size_t mxmoe_permute_workspace_bytes(int total, int num_experts) {
+  const size_t blocks = (size_t)(total + kPermChunk - 1) / kPermChunk;
+  return (blocks * num_experts + num_experts) * sizeof(int32_t);
+}
+
+int mxmoe_build_permutation(const int32_t* topk_ids, int num_tokens, int topk, int num_experts, int32_t* dst_exp_sorted, int64_t* perm_indices,
+                            int64_t* src_slot, int64_t* recv_tokens_per_exp, void* workspace, void* stream) {
+  const int total = num_tokens * topk;
+  if (total <= 0 || num_experts <= 0 || num_experts > 4096) {
+    last_error() = "bad permutation size";
+    return 3;
+  }
+  hipStream_t s = (hipStream_t)stream;
+  const int blocks = (total + kPermChunk - 1) / kPermChunk;
+  int32_t* hist = reinterpret_cast<int32_t*>(workspace);
+  int32_t* expert_off = hist + (size_t)blocks * num_experts;
+  int nbits = 1;
+  while ((1 << nbits) <= num_experts) ++nbits;  // ids 0..E (E = parked lanes)
+  const size_t lds = (size_t)num_experts * sizeof(int32_t);
+  hipLaunchKernelGGL(perm_hist_kernel, dim3(blocks), dim3(64), lds, s, topk_ids, total, num_experts, hist);
+  hipLaunchKernelGGL(perm_scan_kernel, dim3(1), dim3(256), lds, s, hist, blocks, num_experts, recv_tokens_per_exp, expert_off);
+  hipLaunchKernelGGL(perm_scatter_kernel, dim3(blocks), dim3(64), lds, s, topk_ids, total, num_experts, topk, nbits, hist, expert_off, dst_exp_sorted, perm_indices,
+                     src_slot);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    last_error() = std::string("kernel launch failed: ") + hipGetErrorString(e);
+    return 4;
+  }
+  return 0;
+}
+
+static int fill_common(RowArgs& a, int n, int n_shared, int had_k, int had_f, const float* signs) {
+  if (n % 8 || (n_shared % 8)) {
+    last_error() = "row length must be a multiple of 8";
+    return 3;
+  }
+  if (make_plan(n, had_k, had_f, &a.plan) || make_plan(n_shared > 0 ? n_shared : n, had_k, had_f, &a.plan_shared)) {
+    last_error() = "row length is not (Hadamard order) x (power of two >= 8)";
+    return 3;
+  }
+  a.signs = a.plan.kb > 1 ? signs : nullptr;
+  if (a.plan.kb > 1 && !signs) {
+    last_error() = "missing Hadamard sign table";
+    return 3;
+  }
+  return 0;
+}
+
+int mxmoe_quant_act(const void* hidden, void* inp_store, void* scale_store, const int32_t* dst_exp_sorted, const int64_t* perm_indices, const int64_t* exp_table,
+                    int K, int rows_routed, int num_tokens, int num_experts, int has_shared, int rotate, int had_k, int had_f, const float* had_signs, void* stream) {
+  RowArgs a{};
+  a.src = a.src_shared = reinterpret_cast<const _Float16*>(hidden);
+  a.inp_store = reinterpret_cast<uint8_t*>(inp_store);
+  a.scale_store = reinterpret_cast<_Float16*>(scale_store);
+  a.dst_exp = dst_exp_sorted;
+  a.perm = perm_indices;
+  a.table = exp_table;
+  a.R = rows_routed;
+  a.T = num_tokens;
+  a.E = num_experts;
+  a.Et = num_experts + (has_shared ? 1 : 0);
+  a.rows = rows_routed + (has_shared ? num_tokens : 0);
+  a.rotate = rotate;
+  if (a.rows == 0) return 0;
+  if (const int rc = fill_common(a, K, K, rotate ? had_k : 1, rotate ? had_f : 1, had_signs)) return rc;
+  const int lds = (K + a.plan.kb * a.plan.kb + 8) * (int)sizeof(float);
+  return launch_rows<false>(a, lds, (hipStream_t)stream);
+}
+
+int mxmoe_silu_mul_quant(const void* gate_up, const void* gate_up_shared, void* inp_store, void* scale_store, const int32_t* dst_exp_sorted, const int64_t* exp_table,
+                         int N, int N_shared, int rows_routed, int num_tokens, int num_experts, int has_shared, int rotate, int had_k, int had_f,
+                         const float* had_signs, void* stream) {
+  RowArgs a{};
+  a.src = reinterpret_cast<const _Float16*>(gate_up);
+  a.src_shared = reinterpret_cast<const _Float16*>(gate_up_shared);
+  a.inp_store = reinterpret_cast<uint8_t*>(inp_store);
+  a.scale_store = reinterpret_cast<_Float16*>(scale_store);
+  a.dst_exp = dst_exp_sorted;
+  a.perm = nullptr;
+  a.table = exp_table;
+  a.R = rows_routed;
+  a.T = num_tokens;
+  a.E = num_experts;
+  a.Et = num_experts + (has_shared ? 1 : 0);
+  a.rows = rows_routed + (has_shared ? num_tokens : 0);
+  a.rotate = rotate;
+  if (a.rows == 0) return 0;
+  if (const int rc = fill_common(a, N, has_shared ? N_shared : N, rotate ? had_k : 1, rotate ? had_f : 1, had_signs)) return rc;
+  const int nmax = N > a.plan_shared.n ? N : a.plan_shared.n;
+  const int lds = (nmax + a.plan.kb * a.plan.kb + 8) * (int)sizeof(float);
+  return launch_rows<true>(a, lds, (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -195,9 +195,11 @@ int register_fused(const char* fn_name) {
 inline int pick_branch(const FusedKernel& k, Fmt f, int M) {
   int best = -1;
   long best_pad = 0;
+  static const int force_bm = getenv("MXMOE_FORCE_BM") ? atoi(getenv("MXMOE_FORCE_BM")) : 0;
   for (int i = 0; i < (int)k.branches.size(); ++i) {
     const auto& b = k.branches[i];
     if (b.fmt != f) continue;
+    if (force_bm && b.BM != force_bm) continue;
     const long pad = (long)((M + b.BM - 1) / b.BM) * b.BM;
     if (best < 0 || pad < best_pad || (pad == best_pad && b.BM > k.branches[best].BM)) {
       best = i;

@@ -48,6 +48,14 @@ struct TileArgs {
   int tile_m, tile_n;
 };
 
+// Keeps a freshly computed fp32 value opaque to the optimiser.  Without it the compiler folds "fp32 multiply, then convert to
+// fp16" into one v_fma_mixlo_f16, which rounds the exact product once; the reference arithmetic (and its CPU restatement) rounds
+// to fp32 first and to fp16 second, and the two differ on ties.
+__device__ __forceinline__ float keep_f32(float v) {
+  asm volatile("" : "+v"(v));
+  return v;
+}
+
 // LDS byte offset of 16-byte chunk `c` (0..3) of tile row `r`.  Rows are 64 bytes; the chunk index is XORed with
 // bits 1..2 of the row so rows r, r+1 (which share a 128-byte bank line) and the next three row pairs all land
 // on different 16-byte groups.
@@ -231,7 +239,7 @@ struct MfmaTile {
               if constexpr (OP == Op::I4) a >>= 8;  // exact: the accumulator is 256 * sum
               // reference epilogue (mm_tile.cuh:490-493, 642-646): float(acc) * float(half(sa * sb)), rounded to half
               const _Float16 s = s_a * s_b[e];
-              o[e] = (_Float16)((float)a * (float)s);
+              o[e] = (_Float16)keep_f32((float)a * (float)s);
               if (t.acc_dump) t.acc_dump[(long)m * N + n + e] = a;
             }
           }

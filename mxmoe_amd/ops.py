@@ -1,0 +1,268 @@
+"""The five operators of the reference's `mxmoe_ops` extension (mxmoe/kernels/src/ref_bind.cu:759-768), same names,
+argument order and return tuples, running on the gfx950 kernels behind the C-ABI.
+
+Differences a caller can see, all deliberate:
+  * rows of one expert keep their original (token, slot) order (the reference's torch::sort is unstable);
+  * packed activations use this library's layouts (int4: two values per byte, even element in the low nibble);
+  * failures raise RuntimeError instead of exit(EXIT_FAILURE) (mxmoe/kernels/src/include/helper.h:186-193);
+  * `quant_inp_act` / `silu_mul_then_quant` accept `rotate=` (0 none, 1 rows of quantised experts, 2 all rows) for the
+    online Hadamard rotation that the reference applies from Python (mxmoe/quant/rotation.py:403-421).
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+from .group_gemm import GroupGemmLaunch
+from .hadamard import device_signs
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def act_tag(a_bits: int, gsize: int) -> int:
+    """ref_bind.cu:461-473."""
+    if a_bits >= 16:
+        return 0
+    if a_bits == 8 and gsize == -1:
+        return 1
+    if a_bits == 4 and gsize == -1:
+        return 2
+    if a_bits == 4 and gsize == 128:
+        return 3
+    return -1
+
+
+def gg_permute_inp(hidden: torch.Tensor, topk_ids: torch.Tensor, E: int):
+    """ref_bind.cu:47-64 -> (num_problems, inp_buffer [R, K], perm_indices [R], recv_tokens_per_exp [E] int64 CPU)."""
+    dst, perm, _slot, recv = build_permutation(topk_ids, E)
+    recv_cpu = recv.cpu()
+    return int((recv_cpu != 0).sum()), hidden.index_select(0, perm), perm, recv_cpu
+
+
+def build_permutation(topk_ids: torch.Tensor, num_experts: int):
+    """Stable sort of the flattened expert ids on the device -> (dst_exp_sorted int32 [R], perm_indices int64 [R],
+    src_slot int64 [R], recv_tokens_per_exp int64 [E] on the device)."""
+    lib = _lib.load()
+    ids = topk_ids.to(torch.int32).contiguous()
+    t, k = ids.shape
+    r = t * k
+    dev = ids.device
+    dst = torch.empty(r, dtype=torch.int32, device=dev)
+    perm = torch.empty(r, dtype=torch.int64, device=dev)
+    slot = torch.empty(r, dtype=torch.int64, device=dev)
+    recv = torch.empty(num_experts, dtype=torch.int64, device=dev)
+    ws = torch.empty(lib.mxmoe_permute_workspace_bytes(r, num_experts), dtype=torch.uint8, device=dev)
+    _lib.check(lib, lib.mxmoe_build_permutation(ids.data_ptr(), t, k, num_experts, dst.data_ptr(), perm.data_ptr(), slot.data_ptr(), recv.data_ptr(), ws.data_ptr(), _stream()))
+    return dst, perm, slot, recv
+
+
+def _offsets(recv_cpu, num_tokens: int, num_experts: int, has_shared: bool, qparams_per_exp, ld: int, ld_shared: int):
+    """Host offset builder of ref_bind.cu:475-505 / 635-671 (units: fp16 elements)."""
+    et = num_experts + (1 if has_shared else 0)
+    if len(qparams_per_exp) < et:
+        raise RuntimeError(f"qparams_per_exp has {len(qparams_per_exp)} entries, need {et}")
+    rows = []
+    table = torch.zeros((4, et), dtype=torch.int64)
+    inp_sizes, scale_sizes, lds = [], [], []
+    acc = io = so = 0
+    for e in range(et):
+        a_bits, _w, g, _s = qparams_per_exp[e]
+        tag = act_tag(int(a_bits), int(g))
+        if tag not in (0, 1, 2):
+            raise RuntimeError("quant type not supported")
+        width = ld_shared if e == num_experts else ld
+        qld = width if tag == 0 else (width // 2 if tag == 1 else width // 4)
+        sld = 0 if tag == 0 else 1
+        n = num_tokens if e == num_experts else int(recv_cpu[e])
+        table[0, e], table[1, e], table[2, e], table[3, e] = tag, acc, io, so
+        rows.append(n)
+        inp_sizes.append(qld * n)
+        scale_sizes.append(sld * n)
+        lds.append(qld)
+        acc += n
+        io += qld * n
+        so += sld * n
+    return table, rows, inp_sizes, scale_sizes, lds, io, so
+
+
+def _views(store, scale_store, table, rows, inp_sizes, scale_sizes, lds):
+    inp_list, scale_list = [], []
+    for e, n in enumerate(rows):
+        if n == 0:
+            continue
+        off = int(table[2, e])
+        inp_list.append(store[off:off + inp_sizes[e]].view(n, lds[e]))
+        soff = int(table[3, e])
+        scale_list.append(scale_store[soff:soff + scale_sizes[e]])
+    return inp_list, scale_list
+
+
+def quant_inp_act(hidden, topk_ids, num_experts: int, N: int, num_shared_experts: int, qparams_per_exp, verbose: bool = False, rotate: int = 0):
+    """ref_bind.cu:434-592.  Returns (inp_list, scale_list, out_list, inp_store, scale_store, out_store,
+    recv_tokens_per_exp (int64 CPU), perm_indices, dst_exp_sorted).  The lists are views into the stores, one per
+    non-empty problem (shared expert last); out_list[p] is the [M_p, 2N] (shared: [T, 2N * num_shared]) gate_up output buffer."""
+    lib = _lib.load()
+    assert hidden.dim() == 2 and hidden.dtype == torch.float16 and hidden.is_cuda
+    hidden = hidden.contiguous()
+    t, k = hidden.shape
+    topk = topk_ids.shape[1]
+    has_shared = num_shared_experts > 0
+    dst, perm, _slot, recv = build_permutation(topk_ids, num_experts)
+    recv_cpu = recv.cpu()                                   # one small D2H copy, as ref_bind.cu:451
+    table, rows, inp_sizes, scale_sizes, lds, io, so = _offsets(recv_cpu, t, num_experts, has_shared, qparams_per_exp, k, k)
+    dev = hidden.device
+    inp_store = torch.empty(io, dtype=torch.float16, device=dev)
+    scale_store = torch.empty(so, dtype=torch.float16, device=dev)
+    out_store = torch.empty((num_shared_experts + topk) * t * N * 2, dtype=torch.float16, device=dev)
+    d_table = table.to(dev)
+    hk, hf, signs = device_signs(k, dev) if rotate else (1, 1, None)
+    _lib.check(lib, lib.mxmoe_quant_act(hidden.data_ptr(), inp_store.data_ptr(), scale_store.data_ptr(), dst.data_ptr(), perm.data_ptr(), d_table.data_ptr(),
+                                        k, t * topk, t, num_experts, int(has_shared), rotate, hk, hf, None if signs is None else signs.data_ptr(), _stream()))
+    inp_list, scale_list = _views(inp_store, scale_store, table, rows, inp_sizes, scale_sizes, lds)
+    out_list, off = [], 0
+    for e, n in enumerate(rows):
+        if n == 0:
+            continue
+        ld = N * 2 * num_shared_experts if e == num_experts else N * 2
+        out_list.append(out_store[off:off + n * ld].view(n, ld))
+        off += n * ld
+    if verbose:
+        for e, n in enumerate(rows):
+            print(f"exp: {e} tokens: {n} qinp_size: {inp_sizes[e]} qinp_scale_size: {scale_sizes[e]}")
+    return inp_list, scale_list, out_list, inp_store, scale_store, out_store, recv_cpu, perm, dst
+
+
+def silu_mul_then_quant(inp, num_problems: int, num_experts: int, K: int, N: int, num_shared_experts: int, num_tokens: int, topk: int,
+                        values_sorted, recv_tokens_per_exp, qparams_per_exp, rotate: int = 0):
+    """ref_bind.cu:595-757.  `inp` is the flat gate_up output store ([R, 2N] routed rows then [T, 2N*num_shared] shared rows),
+    `values_sorted` the sorted expert ids.  Returns (inp_list, scale_list, out_list, inp_store, scale_store, out_store) where
+    out_list[p] is the [M_p, K] buffer of the down projection."""
+    lib = _lib.load()
+    has_shared = num_shared_experts > 0
+    r = num_tokens * topk
+    dev = inp.device
+    recv_cpu = recv_tokens_per_exp.cpu()
+    table, rows, inp_sizes, scale_sizes, lds, io, so = _offsets(recv_cpu, num_tokens, num_experts, has_shared, qparams_per_exp, N, N * max(num_shared_experts, 1))
+    inp_store = torch.empty(io, dtype=torch.float16, device=dev)
+    scale_store = torch.empty(so, dtype=torch.float16, device=dev)
+    out_store = torch.empty((1 + topk) * num_tokens * K, dtype=torch.float16, device=dev)
+    d_table = table.to(dev)
+    flat = inp.reshape(-1)
+    n_sh = N * num_shared_experts
+    hk, hf, signs = device_signs(N, dev) if rotate else (1, 1, None)
+    if rotate and has_shared and device_signs(n_sh, dev)[0] != hk:
+        raise RuntimeError("routed and shared intermediate sizes need the same Hadamard order")
+    shared_ptr = flat.data_ptr() + r * N * 2 * 2
+    _lib.check(lib, lib.mxmoe_silu_mul_quant(flat.data_ptr(), shared_ptr, inp_store.data_ptr(), scale_store.data_ptr(), values_sorted.data_ptr(), d_table.data_ptr(),
+                                             N, n_sh, r, num_tokens, num_experts, int(has_shared), rotate, hk, hf, None if signs is None else signs.data_ptr(), _stream()))
+    inp_list, scale_list = _views(inp_store, scale_store, table, rows, inp_sizes, scale_sizes, lds)
+    out_list, off = [], 0
+    for e, n in enumerate(rows):
+        if n == 0:
+            continue
+        out_list.append(out_store[off:off + n * K].view(n, K))
+        off += n * K
+    return inp_list, scale_list, out_list, inp_store, scale_store, out_store
+
+
+def _problem_lists(num_experts: int, experts, recv_cpu, num_tokens: int):
+    has_shared = len(experts) > num_experts
+    for e in range(num_experts + (1 if has_shared else 0)):
+        n = num_tokens if e == num_experts else int(recv_cpu[e])
+        if n:
+            yield e, n
+
+
+def gg_mxmoe_share_fused(inp, experts, scale_zp_a, scale_zp_b, output, N: int, K: int, shared_N: int, shared_K: int, qparams_per_exp,
+                         recv_tokens_per_exp, verbose: bool = False, kernel_id: int = -1, acc_dump=None):
+    """ref_bind.cu:312-431: one fused launch over every non-empty expert (+ the shared expert as problem index E).
+
+    `inp`, `scale_zp_a`, `output` are indexed by PROBLEM, `experts`, `scale_zp_b`, `qparams_per_exp` by EXPERT
+    (ref_bind.cu:362-371).  Returns `output`."""
+    plan = prepare_gg(inp, experts, scale_zp_a, scale_zp_b, output, N, K, shared_N, shared_K, qparams_per_exp, recv_tokens_per_exp, kernel_id, acc_dump)
+    if verbose:
+        print(f"num_problems: {plan.count}")
+        for i, (s, q) in enumerate(zip(plan.sizes, plan.qparams)):
+            print(f"problem {i}: {list(s)} qparams: {q}")
+    plan.run()
+    return output
+
+
+def prepare_gg(inp, experts, scale_zp_a, scale_zp_b, output, N, K, shared_N, shared_K, qparams_per_exp, recv_tokens_per_exp, kernel_id: int = -1, acc_dump=None) -> GroupGemmLaunch:
+    """The pointer-table part of `gg_mxmoe_share_fused`, reusable across launches (CUDA-graph friendly)."""
+    recv_cpu = recv_tokens_per_exp.cpu()
+    e_cnt = recv_cpu.shape[0]
+    num_tokens = inp[-1].shape[0] if len(inp) else 0
+    As, Bs, sa, sb, Cs, sizes, qps = [], [], [], [], [], [], []
+    for p, (e, n) in enumerate(_problem_lists(e_cnt, experts, recv_cpu, num_tokens)):
+        As.append(inp[p])
+        Bs.append(experts[e])
+        sa.append(scale_zp_a[p] if scale_zp_a is not None and p < len(scale_zp_a) else None)
+        sb.append(scale_zp_b[e] if scale_zp_b is not None else None)
+        Cs.append(output[p])
+        sizes.append((n, shared_N, shared_K) if e == e_cnt else (n, N, K))
+        qps.append(tuple(qparams_per_exp[e]))
+    if len(As) != len(inp):
+        raise RuntimeError(f"{len(inp)} inputs for {len(As)} non-empty problems")
+    g = GroupGemmLaunch(As, Bs, sa, sb, Cs, sizes, qps, kernel_id=kernel_id, acc=acc_dump)
+    g.qparams = qps
+    return g
+
+
+def gg_cutlass(inp, experts, topk_ids, output, num_problems=None, inp_buffer=None, perm_indices=None, recv_tokens_per_exp=None):
+    """ref_bind.cu:68-182: fp16 grouped GEMM `output[rows of e] = inp[perm rows] @ experts[e].T` (the reference's CUTLASS baseline;
+    here the fp16 MFMA branch of the same fused kernel).  experts [E, N, K] fp16, output [T*topk, N]."""
+    if inp.dim() != 2:
+        raise RuntimeError("hidden must be 2D")
+    if not (inp.is_cuda and experts.is_cuda):
+        raise RuntimeError("dev must be on cuda")
+    e_cnt, n, k = experts.shape
+    if perm_indices is None:
+        num_problems, inp_buffer, perm_indices, recv_tokens_per_exp = gg_permute_inp(inp, topk_ids, e_cnt)
+    recv_cpu = recv_tokens_per_exp.cpu()
+    As, Bs, Cs, sizes = [], [], [], []
+    st = 0
+    for e in range(e_cnt):
+        m = int(recv_cpu[e])
+        if m == 0:
+            continue
+        As.append(inp_buffer[st:st + m])
+        Bs.append(experts[e])
+        Cs.append(output[st:st + m])
+        sizes.append((m, n, k))
+        st += m
+    GroupGemmLaunch(As, Bs, None, None, Cs, sizes, [(16, 16, -1, True)] * len(As)).run()
+    return output
+
+
+def gg_cutlass_share_fused(inp, experts, shared_experts, topk_ids, output, shared_output, num_problems=None, inp_buffer=None, perm_indices=None,
+                           recv_tokens_per_exp=None):
+    """ref_bind.cu:184-310: as `gg_cutlass` plus one more problem `shared_output = inp @ shared_experts.T` in the same launch."""
+    if inp.dim() != 2:
+        raise RuntimeError("hidden must be 2D")
+    if not (inp.is_cuda and experts.is_cuda):
+        raise RuntimeError("dev must be on cuda")
+    e_cnt, n, k = experts.shape
+    n_sh, k_sh = shared_experts.shape
+    if perm_indices is None:
+        num_problems, inp_buffer, perm_indices, recv_tokens_per_exp = gg_permute_inp(inp, topk_ids, e_cnt)
+    recv_cpu = recv_tokens_per_exp.cpu()
+    As, Bs, Cs, sizes = [], [], [], []
+    st = 0
+    for e in range(e_cnt):
+        m = int(recv_cpu[e])
+        if m == 0:
+            continue
+        As.append(inp_buffer[st:st + m])
+        Bs.append(experts[e])
+        Cs.append(output[st:st + m])
+        sizes.append((m, n, k))
+        st += m
+    As.append(inp)
+    Bs.append(shared_experts)
+    Cs.append(shared_output)
+    sizes.append((inp.shape[0], n_sh, k_sh))
+    GroupGemmLaunch(As, Bs, None, None, Cs, sizes, [(16, 16, -1, True)] * len(As)).run()
+    return output

@@ -17,6 +17,7 @@ fails a test in ``tests/test_oracle_*.py``):
 * ``sylvester_fwht``      — scipy.linalg.hadamard dense product, involution, H e_0, Parseval.
 * ``had_table``           — H H^T = K I and all entries +-1.
 * ``online_hadamard``     — dense kron(H_K, H_{n/K}) / sqrt(n) in float64.
+* ``had_factor``          — kron(S_f, B) rebuilt and compared with the table.
 * ``route_topk``          — textbook softmax / top-k, weights sum to one.
 * ``permute_by_expert``   — brute force against a dict-of-lists.
 * ``tile_to_problem``     — every (problem, tile_m, tile_n) visited exactly once.
@@ -230,15 +231,39 @@ def had_scale(n: int) -> np.float32:
     return F32(1.0) / np.sqrt(F32(n))
 
 
+def had_factor(k: int):
+    """Split ``H_K = S_f kron B`` with ``S_f`` the Sylvester matrix of the largest power of two ``f`` for which it holds.
+
+    had176 of the reference's table is ``S_4 kron B_44``; had28 has no such factor (f = 1).  Returns ``(f, Kb, B int8)``.
+    """
+    h = had_table(k)
+    f = 1
+    while k % (2 * f) == 0:
+        g = 2 * f
+        b = k // g
+        blk = h[:b, :b]
+        ok = all(
+            np.array_equal(h[i * b:(i + 1) * b, j * b:(j + 1) * b], ((-1) ** bin(i & j).count("1")) * blk)
+            for i in range(g) for j in range(g)
+        )
+        if not ok:
+            break
+        f = g
+    kb = k // f
+    return f, kb, h[:kb, :kb].copy()
+
+
 def online_hadamard(x: np.ndarray) -> np.ndarray:
     """Online rotation of fp16 rows: ``y = (H_K kron H_{n/K}) x / sqrt(n)``, index ``p = k*(n/K) + j``.
 
     Follows ``matmul_hadU_cuda`` (hadamard_utils.py:96-106): view ``[K, n/K]``, Sylvester transform
     of each length-``n/K`` row scaled by ``1/sqrt(n)`` and returned in fp16, then ``hadK @ .`` in fp16.
     PARITY UNPINNED at the last fp16 bit (third-party kernel + backend matmul order, see module
-    header).  This build's definition: fp32 ``sylvester_fwht`` (ascending strides), one fp32 multiply by
-    ``had_scale(n)``, round to fp16; K > 1: ``y[k] = sum_{k'} H[k,k'] v[k']`` accumulated in fp32
-    sequentially over ``k' = 0..K-1`` starting from 0, rounded to fp16.
+    header).  This build's definition, which the HIP kernels reproduce bit for bit:
+      1. fp32 ``sylvester_fwht`` along ``n/K`` (ascending strides), one fp32 multiply by ``had_scale(n)``, round to fp16;
+      2. K > 1, with ``H_K = S_f kron B`` (``had_factor``): inside each of the f blocks of Kb rows,
+         ``t[b] = sum_{b'} B[b,b'] v[b']`` accumulated in fp32 from 0 over ``b' = 0..Kb-1`` in order; then the
+         ``S_f`` butterflies across blocks in fp32 (ascending strides); one rounding to fp16.
     """
     assert x.dtype == F16
     n = x.shape[-1]
@@ -248,11 +273,14 @@ def online_hadamard(x: np.ndarray) -> np.ndarray:
     v = (sylvester_fwht(v) * had_scale(n)).astype(F32).astype(F16)
     if k == 1:
         return v.reshape(x.shape)
-    vf = v.astype(F32)
+    f, kb, b = had_factor(k)
+    vf = v.astype(F32).reshape(-1, f, kb, m)
     acc = np.zeros_like(vf)
-    for kp in range(k):  # fixed sequential order
-        sgn = hk[:, kp].astype(F32).reshape(1, k, 1)
-        acc = (acc + sgn * vf[:, kp : kp + 1, :]).astype(F32)
+    for bp in range(kb):  # fixed sequential order
+        sgn = b[:, bp].astype(F32).reshape(1, 1, kb, 1)
+        acc = (acc + sgn * vf[:, :, bp:bp + 1, :]).astype(F32)
+    # S_f butterflies across the block index (axis 1): move it last, transform, move back
+    acc = np.moveaxis(sylvester_fwht(np.ascontiguousarray(np.moveaxis(acc, 1, -1))), -1, 1)
     return acc.astype(F16).reshape(x.shape)
 
 

@@ -1,0 +1,133 @@
+"""GPU parity of the prologue kernels (permutation, act-quant with Hadamard, SiLU*up-quant) and of the whole layer
+chained through the `mxmoe_ops`-style operators, against the CPU oracle.  Integer codes and scales must be bit-exact."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import mxmoe_oracle as O
+
+pytestmark = pytest.mark.gpu
+F16 = np.float16
+DEV = "cuda"
+
+
+def _ids(rng, t, e, k):
+    return np.stack([rng.permutation(e)[:k] for _ in range(t)]).astype(np.int32)
+
+
+def test_permutation_matches_oracle_and_is_stable():
+    from mxmoe_amd import ops
+
+    rng = np.random.default_rng(0)
+    for (t, e, k) in [(1, 4, 2), (37, 7, 3), (300, 60, 4), (2048, 64, 6), (513, 8, 2)]:
+        ids = _ids(rng, t, e, k)
+        if e > 5:
+            ids[ids == 3] = 5 if k == 1 else ids[ids == 3]                  # keep ids valid
+        dst, perm, slot, recv = ops.build_permutation(torch.from_numpy(ids).to(DEV), e)
+        torch.cuda.synchronize()
+        o_dst, o_perm, o_slot, o_recv = O.permute_by_expert(ids, e)
+        assert np.array_equal(dst.cpu().numpy(), o_dst)
+        assert np.array_equal(perm.cpu().numpy(), o_perm)
+        assert np.array_equal(slot.cpu().numpy(), o_slot)
+        assert np.array_equal(recv.cpu().numpy(), o_recv)
+
+
+def _unpack(store_view, tag, n):
+    raw = store_view.contiguous().view(torch.uint8).cpu().numpy().reshape(store_view.shape[0], -1)
+    if tag == 1:
+        return raw.view(np.int8)
+    lo = (raw & 0xF).astype(np.int8)
+    hi = (raw >> 4).astype(np.int8)
+    q = np.stack([lo, hi], axis=-1).reshape(raw.shape[0], -1)
+    return np.where(q >= 8, q - 16, q).astype(np.int8)
+
+
+@pytest.mark.parametrize("k,rotate", [(2048, 1), (4096, 1), (256, 0), (2048, 2)])
+def test_quant_inp_act_bit_exact(k, rotate):
+    from mxmoe_amd import ops
+
+    rng = np.random.default_rng(k + rotate)
+    t, e, topk, n_sh = 48, 6, 2, 1
+    x = rng.standard_normal((t, k)).astype(F16)
+    x[3] = 0                                                               # all-zero token: scale guard
+    ids = _ids(rng, t, e, topk)
+    ids[ids == 4] = 5 if False else ids[ids == 4]
+    qp = [(4, 4, -1, True), (8, 8, -1, True), (16, 4, 128, False), (4, 4, -1, True), (8, 8, -1, True), (16, 16, -1, True), (8, 8, -1, True)]
+    res = ops.quant_inp_act(torch.from_numpy(x).to(DEV), torch.from_numpy(ids).to(DEV), e, 1408, n_sh, qp, rotate=rotate)
+    inp_list, scale_list, out_list, inp_store, scale_store, out_store, recv, perm, dst = res
+    torch.cuda.synchronize()
+    o_dst, o_perm, _, o_recv = O.permute_by_expert(ids, e)
+    assert np.array_equal(recv.numpy(), o_recv)
+    p = 0
+    st = 0
+    for ex in range(e + 1):
+        m = t if ex == e else int(o_recv[ex])
+        if m == 0:
+            continue
+        rows = x if ex == e else x[o_perm[st:st + m]]
+        if ex < e:
+            st += m
+        a_bits = qp[ex][0]
+        tag = O.act_tag(a_bits, qp[ex][2])
+        rot = rotate == 2 or (rotate == 1 and tag != 0)
+        xr = O.online_hadamard(rows) if rot else rows
+        got = inp_list[p]
+        assert out_list[p].shape == (m, 2 * 1408 * (n_sh if ex == e else 1))
+        if tag == 0:
+            assert np.array_equal(got.cpu().numpy().view(np.uint16), xr.view(np.uint16)), f"expert {ex} fp16 rows"
+        else:
+            q, s, _ = O.quant_minmax(xr, a_bits, -1, True)
+            assert np.array_equal(scale_list[p].cpu().numpy().view(np.uint16), s.reshape(-1).view(np.uint16)), f"expert {ex} scales"
+            assert np.array_equal(_unpack(got, tag, k), q.astype(np.int8)), f"expert {ex} codes"
+        p += 1
+    assert p == len(inp_list)
+
+
+@pytest.mark.parametrize("n,n_sh,rotate", [(1408, 2, 2), (2048, 0, 1), (14336, 0, 1), (512, 1, 0)])
+def test_silu_mul_then_quant_bit_exact(n, n_sh, rotate):
+    from mxmoe_amd import ops
+
+    rng = np.random.default_rng(n)
+    t, e, topk = 12, 4, 2
+    ids = _ids(rng, t, e, topk)
+    o_dst, o_perm, _, o_recv = O.permute_by_expert(ids, e)
+    r = t * topk
+    gu = (rng.standard_normal((r, 2 * n)) * 2).astype(F16)
+    gu_sh = (rng.standard_normal((t, 2 * n * max(n_sh, 1))) * 2).astype(F16)
+    flat = np.concatenate([gu.reshape(-1), gu_sh.reshape(-1)]) if n_sh else gu.reshape(-1)
+    qp = [(4, 4, -1, True), (8, 8, -1, True), (16, 4, 128, False), (4, 4, -1, True), (8, 8, -1, True)]
+    res = ops.silu_mul_then_quant(torch.from_numpy(flat).to(DEV), int((o_recv != 0).sum()), e, 2048, n, n_sh, t, topk,
+                                  torch.from_numpy(o_dst).to(DEV), torch.from_numpy(o_recv), qp, rotate=rotate)
+    inp_list, scale_list, out_list = res[:3]
+    torch.cuda.synchronize()
+    p = st = 0
+    for ex in range(e + (1 if n_sh else 0)):
+        m = t if ex == e else int(o_recv[ex])
+        if m == 0:
+            continue
+        src = gu_sh if ex == e else gu[st:st + m]
+        if ex < e:
+            st += m
+        y = O.silu_mul(src)
+        a_bits = qp[ex][0]
+        tag = O.act_tag(a_bits, qp[ex][2])
+        if rotate == 2 or (rotate == 1 and tag != 0):
+            y = O.online_hadamard(y)
+        got = inp_list[p]
+        assert out_list[p].shape == (m, 2048)
+        if tag == 0:
+            assert np.array_equal(got.cpu().numpy().view(np.uint16), y.view(np.uint16)), f"expert {ex} fp16 rows"
+        else:
+            q, s, _ = O.quant_minmax(y, a_bits, -1, True)
+            assert np.array_equal(scale_list[p].cpu().numpy().view(np.uint16), s.reshape(-1).view(np.uint16)), f"expert {ex} scales"
+            assert np.array_equal(_unpack(got, tag, y.shape[1]), q.astype(np.int8)), f"expert {ex} codes"
+        p += 1
+
+
+def test_unsupported_activation_format():
+    from mxmoe_amd import ops
+
+    x = torch.zeros((4, 256), dtype=torch.float16, device=DEV)
+    ids = torch.zeros((4, 1), dtype=torch.int32, device=DEV)
+    with pytest.raises(RuntimeError, match="quant type not supported"):
+        ops.quant_inp_act(x, ids, 2, 128, 0, [(2, 2, -1, True), (8, 8, -1, True)])

@@ -55,3 +55,11 @@ def test_online_hadamard_equals_dense_kron(n):
 def test_had_scale_is_fp32_reciprocal_sqrt():
     assert O.had_scale(2048) == np.float32(1.0) / np.sqrt(np.float32(2048))
     assert O.had_scale(4096) == np.float32(1 / 64)
+
+
+def test_had_factor_rebuilds_the_table():
+    f, kb, b = O.had_factor(176)
+    assert (f, kb) == (4, 44)
+    assert np.array_equal(np.kron(hadamard(4), b.astype(np.int64)), O.had_table(176).astype(np.int64))
+    f, kb, b = O.had_factor(28)
+    assert (f, kb) == (1, 28) and np.array_equal(b, O.had_table(28))
