@@ -1,0 +1,198 @@
+#!/usr/bin/env python3
+"""GroupGEMM benchmark of the mixed-precision MoE layer on one MI355X.
+
+One "step" = the two fused GroupGEMM launches of one MoE layer (gate_up, then down) over one batch of synthetic,
+HBM-resident, already permuted + quantised inputs — the region the reference times with cudaEvents around its launcher
+(mxmoe/kernels/src/test.cu:101-158, mxmoe/kernels/src/test_utils.h:97-191), metric TOPS = sum(2*M*N*K) / time.
+
+Prints ONE JSON line.  `roofline` prices the dominant kernel (the gate_up launch) against the MI355X peak with its launch
+duration measured by HIP events on the launch stream inside the timed region; `cpu_baseline` times the CPU restatement of
+the reference's fake-quant path on a bounded sample of the same workload on this box's host cores.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+PEAK = {"int8": 5000.0, "fp16": 2500.0, "hbm": 8000.0}  # MI355X: TOP/s dense int8 MFMA, TFLOP/s dense fp16 MFMA, GB/s HBM3E
+
+
+def build_layer(name: str, tokens: int | None):
+    import torch
+
+    from mxmoe_amd import synth
+    from mxmoe_amd.layer import MxMoELayer
+
+    cfg = synth.get_config(name, tokens)
+    hidden = synth.make_hidden(cfg)
+    ids, _ = synth.make_routing(cfg)
+    layer = MxMoELayer(cfg)
+    layer.prepare(hidden, ids)
+    layer.gate_up()
+    layer.act()
+    layer.down()
+    torch.cuda.synchronize()
+    return cfg, layer
+
+
+def time_layer(layer, steps: int, warmup: int):
+    """K steps of (gate_up launch, down launch); returns (ms_per_step, avg gate_up ms, avg down ms)."""
+    import torch
+
+    st = layer.state
+    g1, g2 = st["gg1"], st["gg2"]
+    for _ in range(warmup):
+        g1.run()
+        g2.run()
+    torch.cuda.synchronize()
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for a, b, c in ev:
+        a.record()
+        g1.run()
+        b.record()
+        g2.run()
+        c.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3
+    up = sum(a.elapsed_time(b) for a, b, _ in ev) / steps
+    dn = sum(b.elapsed_time(c) for _, b, c in ev) / steps
+    return wall / steps, up, dn
+
+
+def roofline_of(cfg, layer, up_ms: float, dn_ms: float):
+    """Roofline entry of the dominant launch.  Compute-bound layers (w-a formats at thousands of tokens): ops of the
+    gate_up launch against the int8 (or fp16) MFMA peak.  Skinny weight-only layers: algorithmic bytes against HBM."""
+    st = layer.state
+    by = layer.algorithmic_bytes()
+    name, ms, plan = ("gate_up", up_ms, st["gg1"]) if up_ms >= dn_ms else ("down", dn_ms, st["gg2"])
+    fmts = {q[:2] for q in plan.qparams}
+    compute_bound = cfg.tokens * cfg.topk / cfg.num_experts >= 128
+    if compute_bound:
+        peak = PEAK["fp16"] if all(a >= 16 for a, _ in fmts) else PEAK["int8"]
+        ach = plan.ops / (ms * 1e-3) / 1e12
+        return {"kernel": f"fused_group_gemm[{name}]", "bound": "mfma", "achieved": round(ach, 2), "peak": peak, "unit": "TFLOP/s",
+                "frac": round(ach / peak, 4), "traffic": None, "launch_us": round(ms * 1e3, 2), "algorithmic_bytes": by[name]["total"]}
+    ach = by[name]["total"] / (ms * 1e-3) / 1e9
+    return {"kernel": f"fused_group_gemm[{name}]", "bound": "hbm", "achieved": round(ach, 1), "peak": PEAK["hbm"], "unit": "GB/s",
+            "frac": round(ach / PEAK["hbm"], 4), "traffic": None, "launch_us": round(ms * 1e3, 2), "algorithmic_bytes": by[name]["total"]}
+
+
+def cpu_baseline(cfg, budget_s: float = 20.0):
+    """The fake-quant path (per expert: fake_quant(x) @ fake_quant(W13)^T -> SiLU*up -> fake_quant(.) @ fake_quant(W2)^T,
+    fp16 storage, fp32 matmul) from the CPU oracle, on as many experts of this workload as fit the time budget."""
+    import numpy as np
+
+    from mxmoe_amd import synth
+    from oracle import mxmoe_oracle as O
+
+    hidden = synth.make_hidden(cfg).numpy()
+    ids, _ = synth.make_routing(cfg)
+    _, perm, _, recv = O.permute_by_expert(ids.numpy(), cfg.num_experts)
+    formats = synth.draw_formats(cfg)
+    starts = np.concatenate([[0], np.cumsum(recv)])
+    ops = 0
+    spent = 0.0
+    used = []
+    f32 = np.float32
+    for e in np.argsort(-recv):  # busiest experts first
+        m = int(recv[e])
+        if m == 0 or spent > budget_s:
+            break
+        w13, w2 = (w.numpy() for w in synth.expert_weights(cfg, int(e)))
+        (a1, wb1, g1, s1), (a2, wb2, g2, s2) = formats[e]
+        w13q = O.fake_quant(w13, wb1, g1, s1).astype(f32)  # offline in the reference (quant.py:913): not timed
+        w2q = O.fake_quant(w2, wb2, g2, s2).astype(f32)
+        x = hidden[perm[starts[e]:starts[e + 1]]]
+        t0 = time.perf_counter()
+        xq = O.fake_quant(O.online_hadamard(x) if (cfg.rotate and a1 < 16) else x, a1, -1, True) if a1 < 16 else x
+        mid = (xq.astype(f32) @ w13q.T).astype(np.float16)
+        y = O.silu_mul(mid)
+        yq = O.fake_quant(O.online_hadamard(y) if (cfg.rotate and a2 < 16) else y, a2, -1, True) if a2 < 16 else y
+        out = (yq.astype(f32) @ w2q.T).astype(np.float16)
+        spent += time.perf_counter() - t0
+        assert out.shape == (m, cfg.hidden)
+        ops += 2 * m * (2 * cfg.inter * cfg.hidden + cfg.hidden * cfg.inter)
+        used.append(int(e))
+    cores = os.cpu_count() or 1
+    return {"value": round(ops / spent / 1e12, 5), "unit": "TOPS", "cores": cores, "kind": "port",
+            "sample": f"{len(used)} busiest experts of {cfg.name} ({sum(int(recv[e]) for e in used)} of {cfg.rows} routed rows), "
+                      f"activation fake-quant + fp32 matmuls + SiLU timed, {spent:.1f} s"}
+
+
+def run_workload(name: str, steps: int, warmup: int, tokens=None):
+    cfg, layer = build_layer(name, tokens)
+    ms, up, dn = time_layer(layer, steps, warmup)
+    ops = layer.gemm_ops()
+    st = layer.state
+    return cfg, layer, {
+        "workload": name, "tops": round(ops / (ms * 1e-3) / 1e12, 2), "ms_per_step": round(ms, 4),
+        "gate_up_us": round(up * 1e3, 2), "down_us": round(dn * 1e3, 2),
+        "gate_up_tops": round(st["gg1"].ops / (up * 1e-3) / 1e12, 2), "down_tops": round(st["gg2"].ops / (dn * 1e-3) / 1e12, 2),
+        "ops": ops, "roofline": roofline_of(cfg, layer, up, dn),
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--also", default="c3,c4", help="comma-separated extra workloads reported under 'also' (empty to skip)")
+    ap.add_argument("--tokens", type=int, default=None)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (the layer would shard by expert; see DESIGN.md). Use --gpus 1.", file=sys.stderr)
+        return 2
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (no CPU fallback exists for the HIP kernels)", file=sys.stderr)
+        return 2
+    from mxmoe_amd import synth
+
+    cfg, layer, main_res = run_workload(args.workload, args.steps, args.warmup, args.tokens)
+    also = {}
+    del layer
+    torch.cuda.empty_cache()
+    for extra in [w for w in args.also.split(",") if w and w != args.workload]:
+        _, lay, res = run_workload(extra, max(10, args.steps // 2), max(5, args.warmup // 2))
+        also[extra] = res
+        del lay
+        torch.cuda.empty_cache()
+
+    fm = sorted({synth.qcfg_str(q) for f in synth.draw_formats(cfg) for q in f})
+    out = {
+        "metric": "GroupGEMM TOPS, Qwen1.5-MoE layer bs=8192" if args.workload in ("c2", "c3") else f"GroupGEMM TOPS, {cfg.description}",
+        "value": main_res["tops"],
+        "unit": "TOPS",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": main_res["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8" if any(q != "fp16" and "a16" not in q for q in fm) else "f16",
+        "data": "synthetic",
+        "config": {"workload": f"{args.workload}: {cfg.description}", "experts": cfg.num_experts, "topk": cfg.topk, "hidden": cfg.hidden,
+                   "intermediate": cfg.inter, "tokens": cfg.tokens, "formats": fm, "step": "gate_up GroupGEMM launch + down GroupGEMM launch"},
+        "roofline": main_res["roofline"],
+        "detail": {k: main_res[k] for k in ("gate_up_us", "down_us", "gate_up_tops", "down_tops", "ops")},
+        "also": also,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(cfg)
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -378,7 +378,7 @@ __global__ void __launch_bounds__(256) row_quant_kernel(const RowArgs a) {
   }
 }
 
-static int make_plan(int n, int had_k, int had_f, RotPlan* p) {
+static int make_plan(int n, int had_k, int had_f, bool rotate, RotPlan* p) {
   p->n = n;
   p->scale = 1.0f / sqrtf((float)n);
   p->kb = 1;
@@ -390,7 +390,7 @@ static int make_plan(int n, int had_k, int had_f, RotPlan* p) {
     p->f = had_f;
     p->kb = had_k / had_f;
   }
-  if (p->m < 8 || (p->m & (p->m - 1))) return 1;
+  if (rotate && (p->m < 8 || (p->m & (p->m - 1)))) return 1;
   return 0;
 }
 
@@ -460,11 +460,12 @@ int mxmoe_build_permutation(const int32_t* topk_ids, int num_tokens, int topk, i
 }
 
 static int fill_common(RowArgs& a, int n, int n_shared, int had_k, int had_f, const float* signs) {
+  const bool rot = a.rotate != 0;
   if (n % 8 || (n_shared % 8)) {
     last_error() = "row length must be a multiple of 8";
     return 3;
   }
-  if (make_plan(n, had_k, had_f, &a.plan) || make_plan(n_shared > 0 ? n_shared : n, had_k, had_f, &a.plan_shared)) {
+  if (make_plan(n, had_k, had_f, rot, &a.plan) || make_plan(n_shared > 0 ? n_shared : n, had_k, had_f, rot, &a.plan_shared)) {
     last_error() = "row length is not (Hadamard order) x (power of two >= 8)";
     return 3;
   }

@@ -237,9 +237,11 @@ struct MfmaTile {
             for (int e = 0; e < 4; ++e) {
               int a = acc[i][j][q * 4 + e];
               if constexpr (OP == Op::I4) a >>= 8;  // exact: the accumulator is 256 * sum
-              // reference epilogue (mm_tile.cuh:490-493, 642-646): float(acc) * float(half(sa * sb)), rounded to half
-              const _Float16 s = s_a * s_b[e];
-              o[e] = (_Float16)keep_f32((float)a * (float)s);
+              // float(acc) * (sa * sb) rounded to half, as the reference epilogue (mm_tile.cuh:490-493, 642-646) except that the
+              // scale product stays in fp32, where it is exact: the reference rounds it to fp16 first, which turns subnormal
+              // (a few significant bits) for typical int8 scales and breaks the 1e-2 agreement with the fake-quant path.
+              const float s = (float)s_a * (float)s_b[e];
+              o[e] = (_Float16)keep_f32((float)a * s);
               if (t.acc_dump) t.acc_dump[(long)m * N + n + e] = a;
             }
           }

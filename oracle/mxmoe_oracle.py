@@ -114,14 +114,20 @@ def int_gemm(qa: np.ndarray, qb: np.ndarray) -> np.ndarray:
     return acc.astype(np.int64).astype(np.int32)
 
 
-def epilogue_wxax(acc: np.ndarray, sa: np.ndarray, sb: np.ndarray) -> np.ndarray:
-    """w-a epilogue (mm_tile.cuh:468-496 then :642-646): ``half(float(acc) * float(half(sa[m] * sb[n])))``.
+def epilogue_wxax(acc: np.ndarray, sa: np.ndarray, sb: np.ndarray, scale_product: str = "fp32") -> np.ndarray:
+    """w-a epilogue (mm_tile.cuh:468-496 then :642-646): ``half(float(acc) * (sa[m] * sb[n]))``.
 
-    ``sa`` [M] per-token and ``sb`` [N] per-channel fp16 scales; their product is rounded to fp16
-    first, widened to fp32, multiplied with the converted accumulator in fp32, rounded to fp16.
+    ``sa`` [M] per-token and ``sb`` [N] per-channel fp16 scales.  The reference kernel rounds the scale product to
+    fp16 (``T(r_sa * r_sb)`` on halves, mm_tile.cuh:490) before widening; for int8 scales that product is an fp16
+    subnormal (~1e-6) and loses most of its mantissa, which alone exceeds the 1e-2 tolerance against the fake-quant
+    path.  ``scale_product="fp32"`` (what the HIP kernels do) keeps the product of the two fp16 scales in fp32, where it
+    is exact; ``"fp16"`` restates the reference kernel literally.  Then: fp32 multiply with the converted accumulator,
+    one rounding to fp32, one to fp16.
     """
-    s = (sa.astype(F16).reshape(-1, 1) * sb.astype(F16).reshape(1, -1)).astype(F16)
-    return (acc.astype(F32) * s.astype(F32)).astype(F16)
+    a = sa.astype(F16).reshape(-1, 1)
+    b = sb.astype(F16).reshape(1, -1)
+    s = (a * b).astype(F16).astype(F32) if scale_product == "fp16" else (a.astype(F32) * b.astype(F32)).astype(F32)
+    return (acc.astype(F32) * s).astype(F32).astype(F16)
 
 
 def gemm_fakequant(xq: np.ndarray, wq: np.ndarray) -> np.ndarray:

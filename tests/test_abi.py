@@ -1,0 +1,80 @@
+"""CPU checks of the C-ABI boundary: the library loads, exports every symbol the header declares, and its host-only
+entry points (registry, launch planning, error paths) behave.  No kernel is launched here."""
+import ctypes as C
+import re
+from pathlib import Path
+
+import pytest
+
+ROOT = Path(__file__).resolve().parent.parent
+
+
+def test_header_symbols_are_exported_and_bound(lib):
+    from mxmoe_amd import _lib
+
+    header = (ROOT / "include" / "mxmoe_amd.h").read_text()
+    declared = set(re.findall(r"\b(mxmoe_[a-z0-9_]+)\s*\(", header))
+    declared -= {"mxmoe_dim3", "mxmoe_qparams"}
+    assert declared, "no declarations found"
+    for name in sorted(declared):
+        assert hasattr(lib, name), f"{name} declared in include/mxmoe_amd.h but not exported"
+        assert name in _lib.SIGNATURES, f"{name} has no ctypes signature"
+    assert set(_lib.SIGNATURES) == declared
+
+
+def test_struct_layouts_match_the_reference_sizes():
+    from mxmoe_amd import _lib
+
+    assert C.sizeof(_lib.QParams) == 16 and C.sizeof(_lib.Dim3) == 12      # QParams quantize.cuh:14-25, dim3
+
+
+def test_registry_names_follow_the_reference_format(lib):
+    n = lib.mxmoe_num_kernels()
+    assert n >= 4
+    names = [lib.mxmoe_kernel_name(i).decode() for i in range(n)]
+    assert any(re.match(r"\[w4a4_g-1_sym: \(\d+,\d+,\d+\) \(\d,\d,1\) \d\], ", s) for s in names)
+    assert lib.mxmoe_find_kernel(b"groupgemm_hz_fused_wxax") == 0
+    assert lib.mxmoe_find_kernel(b"nope") == -1
+    out = (C.c_int32 * 8)()
+    assert lib.mxmoe_kernel_branch(0, 0, out) == 0 and out[1] % 32 == 0 and out[2] % 64 == 0
+    assert lib.mxmoe_kernel_branch(0, 99, out) != 0 and b"branch" in lib.mxmoe_last_error()
+
+
+def _plan(lib, kernel, probs):
+    from mxmoe_amd import _lib
+
+    sizes = (_lib.Dim3 * len(probs))(*[_lib.Dim3(*p[0]) for p in probs])
+    qs = (_lib.QParams * len(probs))(*[_lib.QParams(p[1][0], p[1][1], p[1][2], int(p[1][3])) for p in probs])
+    br = (C.c_int32 * len(probs))()
+    tiles = C.c_int32()
+    rc = lib.mxmoe_group_gemm_plan(kernel, sizes, qs, len(probs), br, C.byref(tiles))
+    return rc, list(br), tiles.value
+
+
+def test_plan_counts_tiles_like_the_reference_launcher(lib):
+    # kernel_sketch.py:89-101: total += cdiv(M, BM) * cdiv(N, BN) per problem with the tile of its qcfg
+    probs = [((546, 2816, 2048), (4, 4, -1, True)), ((0, 2816, 2048), (8, 8, -1, True)), ((20, 2048, 1408), (8, 8, -1, True))]
+    rc, br, tiles = _plan(lib, -1, probs)
+    assert rc == 1000                                                     # first registered kernel covers w4a4 + w8a8
+    out = (C.c_int32 * 8)()
+    exp = 0
+    for (m, n, _k), b in zip([p[0] for p in probs], br):
+        lib.mxmoe_kernel_branch(0, b, out)
+        exp += -(-m // out[1]) * -(-n // out[2])
+    assert tiles == exp
+    lib.mxmoe_kernel_branch(0, br[2], out)
+    assert out[0] == 1 and out[1] == 32                                  # 20 rows of w8a8 -> the 32-row w8a8 tile
+
+
+def test_unsupported_format_message(lib):
+    rc, _, _ = _plan(lib, -1, [((8, 256, 128), (8, 4, -1, True))])
+    assert rc == 1 and lib.mxmoe_last_error() == b"quant type not supported"   # compose_kernel.py:433
+    rc, _, _ = _plan(lib, -1, [((8, 256, 128), (16, 4, 128, False)), ((8, 256, 128), (4, 4, -1, True)), ((8, 256, 128), (16, 16, -1, True))])
+    assert rc >= 1000 and b"fused_all" in lib.mxmoe_kernel_name(rc - 1000)
+
+
+def test_missing_library_fails_loudly(tmp_path):
+    from mxmoe_amd import _lib
+
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        _lib.load(tmp_path / "libmissing.so")

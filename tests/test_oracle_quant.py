@@ -110,12 +110,22 @@ def test_epilogue_closed_forms():
     sa = np.array([0.1, 0.013], dtype=F16)
     sb = np.array([0.02, 0.5], dtype=F16)
     out = O.epilogue_wxax(acc, sa, sb)
+    lit = O.epilogue_wxax(acc, sa, sb, scale_product="fp16")
     for m in range(2):
         for n in range(2):
-            s16 = F16(sa[m] * sb[n])                                       # product rounded to fp16 FIRST
-            assert out[m, n] == F16(np.float32(acc[m, n]) * np.float32(s16))
+            s32 = np.float32(sa[m]) * np.float32(sb[n])                    # exact in fp32 (11 + 11 significant bits)
+            assert float(s32) == float(sa[m]) * float(sb[n])
+            assert out[m, n] == F16(np.float32(acc[m, n]) * s32)
+            s16 = F16(sa[m] * sb[n])                                       # the reference kernel rounds the product to fp16 first
+            assert lit[m, n] == F16(np.float32(acc[m, n]) * np.float32(s16))
     # sa indexes rows (tokens), sb columns (channels): swapping them must change the result
     assert not np.array_equal(out, O.epilogue_wxax(acc, sb, sa))
+    # typical int8 scales: the fp16 product is subnormal and off by percents, the fp32 product is not
+    sa8, sb8 = np.array([0.001], dtype=F16), np.array([0.0007], dtype=F16)
+    exact = 1000 * float(sa8[0]) * float(sb8[0])
+    a1000 = np.array([[1000]], dtype=np.int32)
+    assert abs(float(O.epilogue_wxax(a1000, sa8, sb8)[0, 0]) / exact - 1) < 1e-3
+    assert abs(float(O.epilogue_wxax(a1000, sa8, sb8, "fp16")[0, 0]) / exact - 1) > 5e-3
 
 
 def test_fakequant_path_agrees_with_integer_path_within_tolerance():
