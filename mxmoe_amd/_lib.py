@@ -37,8 +37,13 @@ SIGNATURES = {
 _cached = {}
 
 
+GEMM_ONLY = ("mxmoe_last_error", "mxmoe_num_kernels", "mxmoe_kernel_name", "mxmoe_find_kernel", "mxmoe_kernel_num_branches", "mxmoe_kernel_branch",
+             "mxmoe_group_gemm", "mxmoe_group_gemm_plan")
+
+
 def load(path: str | Path | None = None) -> C.CDLL:
-    """Load the library (or a generated one at `path`) and attach the C-ABI signatures."""
+    """Load the library and attach the C-ABI signatures.  A generated library (`path` given) carries the GroupGEMM entry
+    points only; the default library must export everything the header declares."""
     p = Path(path) if path is not None else LIB_PATH
     key = str(p)
     if key in _cached:
@@ -50,6 +55,8 @@ def load(path: str | Path | None = None) -> C.CDLL:
         )
     lib = C.CDLL(str(p))
     for name, (res, args) in SIGNATURES.items():
+        if path is not None and name not in GEMM_ONLY and not hasattr(lib, name):
+            continue
         fn = getattr(lib, name)
         fn.restype = res
         fn.argtypes = args

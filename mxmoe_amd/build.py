@@ -25,14 +25,32 @@ HIPCC_FLAGS = [
 ]
 
 
-def hipcc_build(sources, out: Path, extra=(), verbose: bool = False) -> Path:
-    cmd = ["hipcc", *HIPCC_FLAGS, *extra, f"-I{CSRC / 'include'}", f"-I{PKG.parent / 'include'}", *map(str, sources), "-o", str(out)]
-    res = subprocess.run(cmd, capture_output=True, text=True)
-    err = "\n".join(l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l)
-    if res.returncode != 0:
-        raise RuntimeError(f"hipcc failed ({res.returncode}):\n{' '.join(cmd)}\n{err}")
-    if verbose and err.strip():
-        print(err, file=sys.stderr)
+def hipcc_build(sources, out: Path, extra=(), verbose: bool = False, jobs: int = 8) -> Path:
+    """Compile each source to an object (in parallel) and link them into the shared library `out`."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    sources = [Path(s) for s in sources]
+    out = Path(out)
+    objdir = out.parent / f".obj_{out.stem}"
+    objdir.mkdir(parents=True, exist_ok=True)
+    inc = [f"-I{CSRC / 'include'}", f"-I{PKG.parent / 'include'}"]
+    compile_flags = [f for f in HIPCC_FLAGS if f != "-shared"]
+
+    def run(cmd):
+        res = subprocess.run(cmd, capture_output=True, text=True)
+        err = "\n".join(l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l)
+        if res.returncode != 0:
+            raise RuntimeError(f"hipcc failed ({res.returncode}):\n{' '.join(map(str, cmd))}\n{err}")
+        if verbose and err.strip():
+            print(err, file=sys.stderr)
+
+    objs = [objdir / (s.stem + ".o") for s in sources]
+    with ThreadPoolExecutor(max_workers=max(1, jobs)) as ex:
+        list(ex.map(run, [["hipcc", *compile_flags, *extra, *inc, "-c", str(s), "-o", str(o)] for s, o in zip(sources, objs)]))
+    run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", *map(str, objs), "-o", str(out)])
+    for o in objs:
+        o.unlink()
+    objdir.rmdir()
     return out
 
 

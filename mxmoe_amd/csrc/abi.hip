@@ -1,9 +1,5 @@
 // C-ABI entry points of libmxmoe_amd.so and the default set of fused kernels.
-#include "../../include/mxmoe_amd.h"
-
-#include "include/mxmoe_launch.hpp"
-
-using namespace mxmoe;
+#include "include/mxmoe_abi_impl.hpp"
 
 namespace {
 
@@ -23,72 +19,3 @@ DefaultKernels g_default_kernels;
 
 }  // namespace
 
-extern "C" {
-
-const char* mxmoe_last_error(void) { return last_error().c_str(); }
-
-int mxmoe_num_kernels(void) { return (int)registry().size(); }
-
-const char* mxmoe_kernel_name(int kernel_id) {
-  if (kernel_id < 0 || kernel_id >= (int)registry().size()) return "";
-  return registry()[kernel_id].name.c_str();
-}
-
-int mxmoe_find_kernel(const char* name) {
-  const std::string n(name ? name : "");
-  for (int i = 0; i < (int)registry().size(); ++i) {
-    const std::string& k = registry()[i].name;
-    if (k == n || (k.size() >= n.size() && !n.empty() && k.compare(k.size() - n.size(), n.size(), n) == 0)) return i;
-  }
-  return -1;
-}
-
-int mxmoe_kernel_num_branches(int kernel_id) {
-  if (kernel_id < 0 || kernel_id >= (int)registry().size()) return -1;
-  return (int)registry()[kernel_id].branches.size();
-}
-
-int mxmoe_kernel_branch(int kernel_id, int branch, int32_t out[8]) {
-  if (kernel_id < 0 || kernel_id >= (int)registry().size()) { last_error() = "kernel id out of range"; return 2; }
-  const auto& k = registry()[kernel_id];
-  if (branch < 0 || branch >= (int)k.branches.size()) { last_error() = "branch out of range"; return 2; }
-  const BranchInfo& b = k.branches[branch];
-  out[0] = (int)b.fmt; out[1] = b.BM; out[2] = b.BN; out[3] = b.BK; out[4] = b.WGM; out[5] = b.WGN; out[6] = b.lds_bytes; out[7] = b.k_multiple;
-  return 0;
-}
-
-int mxmoe_group_gemm(int kernel_id, const void* const* As, const void* const* Bs, const void* const* scale_a, const void* const* scale_b,
-                     void* const* Cs, void* const* Ds, const int64_t* lda, const int64_t* ldb, const int64_t* ldc, const int64_t* ldd,
-                     const mxmoe_dim3* d_sizes, const mxmoe_dim3* h_sizes, const mxmoe_qparams* d_q, const mxmoe_qparams* h_q, int problem_count,
-                     int32_t* const* acc_dump, void* stream) {
-  (void)Ds; (void)lda; (void)ldb; (void)ldc; (void)ldd; (void)d_q;
-  if (problem_count < 0 || (problem_count > 0 && (!As || !Bs || !Cs || !d_sizes || !h_sizes || !h_q))) {
-    last_error() = "null argument";
-    return 5;
-  }
-  return group_gemm(kernel_id, As, Bs, scale_a, scale_b, Cs, acc_dump, d_sizes, h_sizes, h_q, problem_count, (hipStream_t)stream);
-}
-
-int mxmoe_group_gemm_plan(int kernel_id, const mxmoe_dim3* h_sizes, const mxmoe_qparams* h_q, int problem_count, int32_t* branch_out, int32_t* tiles_out) {
-  auto& reg = registry();
-  if (kernel_id < 0) {
-    for (int i = 0; i < (int)reg.size() && kernel_id < 0; ++i)
-      if (kernel_covers(reg[i], h_q, problem_count)) kernel_id = i;
-    if (kernel_id < 0) { last_error() = "quant type not supported"; return 1; }
-  }
-  if (kernel_id >= (int)reg.size()) { last_error() = "kernel id out of range"; return 2; }
-  const FusedKernel& k = reg[kernel_id];
-  int total = 0;
-  for (int i = 0; i < problem_count; ++i) {
-    const Fmt f = classify(h_q[i]);
-    const int b = f == Fmt::UNSUPPORTED ? -1 : pick_branch(k, f, (int)h_sizes[i].x);
-    if (b < 0) { last_error() = "quant type not supported"; return 1; }
-    if (branch_out) branch_out[i] = b;
-    const BranchInfo& bi = k.branches[b];
-    total += (int)((h_sizes[i].x + bi.BM - 1) / bi.BM) * (int)((h_sizes[i].y + bi.BN - 1) / bi.BN);
-  }
-  if (tiles_out) *tiles_out = total;
-  return kernel_id + 1000;  // plan succeeded: 1000 + the kernel that would run
-}
-
-}  // extern "C"

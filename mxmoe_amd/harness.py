@@ -1,0 +1,186 @@
+"""Bench / check harness over workload JSON files: the Python port of the reference's C++ `test` program
+(mxmoe/kernels/src/test.cu: parse_json_input :652-674, QInput::from_fp16 :218-413, bench_one_case :693-868,
+bench_input_file :870-946; timing protocol mxmoe/kernels/src/test_utils.h:97-191; check tolerance :70-95).
+
+Per (layer, "gate_up" | "down") problem list: fp16 operands ~ U(-1, 1) (seed 42), operands quantised + packed per problem,
+every registered fused kernel that covers the formats is timed (<= 30 warm-up, <= 50 timed launches, HIP events, median)
+and reported as `kernel_name, avg_time (ms), TFLOPS, speedup` against the best fp16 grouped GEMM of the same shapes (the
+reference's CUTLASS baseline; here the fp16 MFMA kernel), written to `<output>-<layer>-<gate_up|down>.csv`.
+Sequential and multi-stream launches (one launch per contiguous run of equal-format problems, on one stream or one
+stream per run — the reference's ablation launchers, kernel_sketch.py:148-406) are timed next to the fused launch.
+"""
+from __future__ import annotations
+
+import json
+import time
+
+import torch
+
+from . import _lib, pack
+from .group_gemm import GroupGemmLaunch
+from .quant import quant_minmax
+from .weights import quantize_and_pack
+
+
+def parse_input_file(path: str) -> dict:
+    """{layer name: {"gate_up": [...], "down": [...]}} with entries {"shape": [M, N, K], "w_bits", "a_bits", "gsize", "sym"}."""
+    with open(path) as f:
+        data = json.load(f)
+    return {k: v for k, v in data.items() if k.startswith("layer-")}
+
+
+def bench_func(fn, warmup: int = 20, iters: int = 50, max_warm_s: float = 10.0) -> dict:
+    """test_utils.h:97-191: warm-up (bounded by count and time), then `iters` launches timed one by one with device events;
+    returns min / max / trimmed mean / median in milliseconds (the reference reports the median)."""
+    t0 = time.time()
+    for _ in range(warmup):
+        fn()
+        if time.time() - t0 > max_warm_s:
+            break
+    torch.cuda.synchronize()
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+    for a, b in ev:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    ts = sorted(a.elapsed_time(b) for a, b in ev)
+    trim = ts[len(ts) // 10: len(ts) - len(ts) // 10] or ts
+    return {"min": ts[0], "max": ts[-1], "mean": sum(trim) / len(trim), "median": ts[len(ts) // 2]}
+
+
+def make_problem(entry: dict, gen: torch.Generator, device="cuda", keep_ref: bool = False) -> dict:
+    """Random fp16 operands for one workload entry, quantised and packed for its format (QInput::from_fp16)."""
+    m, n, k = entry["shape"]
+    qp = (entry["a_bits"], entry["w_bits"], entry["gsize"], bool(entry["sym"]))
+    a = (torch.rand(m, k, generator=gen, dtype=torch.float32) * 2 - 1).to(torch.float16).to(device)
+    b = (torch.rand(n, k, generator=gen, dtype=torch.float32) * 2 - 1).to(torch.float16).to(device)
+    pw = quantize_and_pack(b, qp)
+    prob = {"size": (m, n, k), "q": qp, "B": pw.data, "sb": pw.scale, "C": torch.zeros(m, n, dtype=torch.float16, device=device)}
+    if qp[0] < 16:
+        qa, sa, _ = quant_minmax(a, qp[0], -1, True) if m else (a, a[:, :1], None)
+        qi = qa.to(torch.int8)
+        prob["A"] = qi.contiguous() if qp[0] == 8 else pack.pack_int4_k(qi)
+        prob["sa"] = sa.reshape(-1).contiguous()
+    else:
+        prob["A"], prob["sa"] = a, None
+    if keep_ref:
+        prob["a16"], prob["b16"] = a, b
+    return prob
+
+
+def _launch_of(probs, lib, kernel_id=-1) -> GroupGemmLaunch:
+    return GroupGemmLaunch([p["A"] for p in probs], [p["B"] for p in probs], [p["sa"] for p in probs], [p["sb"] for p in probs],
+                           [p["C"] for p in probs], [p["size"] for p in probs], [p["q"] for p in probs], kernel_id=kernel_id, lib=lib)
+
+
+def _runs_of_equal_format(probs):
+    runs, cur = [], []
+    for p in probs:
+        if cur and p["q"] != cur[-1]["q"]:
+            runs.append(cur)
+            cur = []
+        cur.append(p)
+    if cur:
+        runs.append(cur)
+    return runs
+
+
+def tflops(probs, ms: float) -> float:
+    return sum(2 * m * n * k for (m, n, k) in (p["size"] for p in probs)) / (ms * 1e-3) / 1e12
+
+
+def bench_one_case(entries, lib=None, mode: str = "bench", filters=(), out_file: str | None = None, verbose: bool = False) -> dict:
+    """Time (or check) every registered kernel on one problem list; returns {impl: (avg_time_ms, TFLOPS, kernel_name)}."""
+    lib = lib or _lib.load()
+    default_lib = _lib.load()
+    gen = torch.Generator(device="cpu")
+    gen.manual_seed(42)
+    probs = [make_problem(e, gen, keep_ref=(mode == "check")) for e in entries]
+    probs = [p for p in probs if p["size"][0] > 0]
+
+    # fp16 baseline on the same shapes (role of the CUTLASS grouped GEMM, test.cu:774-781)
+    gen2 = torch.Generator(device="cpu")
+    gen2.manual_seed(42)
+    base_probs = [make_problem({**e, "a_bits": 16, "w_bits": 16, "gsize": -1, "sym": True}, gen2) for e in entries if e["shape"][0] > 0]
+    base = _launch_of(base_probs, default_lib)
+    base_ms = bench_func(base.run)["median"]
+    results = {"fp16-baseline": (base_ms, tflops(base_probs, base_ms), default_lib.mxmoe_kernel_name(base.plan()[0]).decode())}
+
+    rows = []
+    for kid in range(lib.mxmoe_num_kernels()):
+        name = lib.mxmoe_kernel_name(kid).decode()
+        if filters and not any(f in name for f in filters):
+            continue
+        g = _launch_of(probs, lib, kid)
+        try:
+            g.plan()
+        except RuntimeError:
+            continue  # this kernel has no tile for one of the formats
+        if mode == "check":
+            g.run()
+            torch.cuda.synchronize()
+            for p in probs:
+                ref = (p["a16"].float() @ p["b16"].float().T)
+                err = (p["C"].float() - ref).abs().max().item() if p["size"][0] else 0.0
+                tol = 1.0 if p["q"][1] >= 16 else float("inf")  # test_utils.h:71 — meaningful for fp16 only, as in the reference
+                print(f"{name}: problem {p['size']} {p['q']} max abs err vs fp16 reference {err:.4f}{' FAIL' if err > tol else ''}")
+            continue
+        ms = bench_func(g.run)["median"]
+        rows.append((ms, tflops(probs, ms), name))
+        if verbose:
+            print(f"{name}\navg_time: {ms:<8.4f}, TFLOPS: {tflops(probs, ms):<9.4f}")
+        time.sleep(0.05)
+    if mode == "check":
+        return results
+
+    if rows:
+        results["mxmoe-hz"] = min(rows)
+    # ablation launch policies with the best kernel library-wide: one launch per contiguous run of equal-format problems
+    runs = [_launch_of(r, lib) for r in _runs_of_equal_format(probs)]
+    try:
+        for r in runs:
+            r.plan()
+
+        def seq():
+            for r in runs:
+                r.run()
+
+        ms = bench_func(seq)["median"]
+        results["mxmoe-seq"] = (ms, tflops(probs, ms), f"seq_launch x{len(runs)}")
+        streams = [torch.cuda.Stream() for _ in runs]
+
+        def multi():
+            cur = torch.cuda.current_stream()
+            for s, r in zip(streams, runs):
+                s.wait_stream(cur)
+                r.run(stream=s.cuda_stream)
+            for s in streams:
+                cur.wait_stream(s)
+
+        ms = bench_func(multi)["median"]
+        results["mxmoe-ms"] = (ms, tflops(probs, ms), f"ms_launch x{len(runs)}")
+    except RuntimeError:
+        pass
+
+    base_tf = results["fp16-baseline"][1]
+    for impl, (ms, tf, name) in results.items():
+        print(f"{impl}: {name}\navg_time: {ms:<8.4f}, TFLOPS: {tf:<9.4f}, speedup: {tf / base_tf:<.3f}")
+    if out_file:
+        with open(out_file, "w") as f:
+            f.write("kernel_name,avg_time,TFLOPS,speedup\n")
+            for ms, tf, name in rows:
+                f.write(f"\"{name}\",{ms:.4f},{tf:.4f},{tf / base_tf:.3f}\n")
+    return results
+
+
+def bench_input_file(input_path: str, output_prefix: str | None = None, lib=None, mode: str = "bench", filters=(), verbose: bool = False) -> dict:
+    """test.cu:870-946: every layer of the workload file, gate_up then down; CSV per (layer, GEMM)."""
+    out = {}
+    for layer, shapes in parse_input_file(input_path).items():
+        idx = layer.split("-")[1]
+        for which in ("gate_up", "down"):
+            csv = f"{output_prefix}-{idx}-{which}.csv" if output_prefix else None
+            print(f"== {layer} {which}: {len(shapes[which])} problems")
+            out[(layer, which)] = bench_one_case(shapes[which], lib=lib, mode=mode, filters=filters, out_file=csv, verbose=verbose)
+    return out

@@ -1,0 +1,266 @@
+"""Tile descriptors of the gfx950 kernels, with the reference's class and field names.
+
+`TileConfig` / `QConfig` / `NO_QUANT` keep the fields (and therefore the dataclass `repr`, which is the key of the
+kernel-profile table) of mxmoe/kernels/tile_config.py:122-286.  What changes is the meaning the hardware gives them:
+WM x WN x WK counts 64-lane wavefronts (always 4 per workgroup here), MMA names an MFMA instruction, STAGE is the number of
+LDS buffers of the register-prefetched pipeline, and the candidate lists are those compiled for gfx950.
+"""
+from __future__ import annotations
+
+import dataclasses
+import re
+
+
+def get_gpu_info() -> dict:
+    """Replaces the pycuda / pynvml probe (tile_config.py:3-30): arch, compute-unit count, LDS per CU, clock."""
+    import torch
+
+    if not torch.cuda.is_available():
+        return {"cc": "gfx950", "sm_count": 256, "frequency": (2400, 2400), "max_shared_memory_per_mp": 160 * 1024}
+    p = torch.cuda.get_device_properties(0)
+    arch = getattr(p, "gcnArchName", "gfx950").split(":")[0]
+    clk = int(getattr(p, "clock_rate", 2400000) // 1000)
+    return {"cc": arch, "sm_count": p.multi_processor_count, "frequency": (clk, clk), "max_shared_memory_per_mp": 160 * 1024}
+
+
+TYPE_TO_BITS = {
+    **dict.fromkeys(["half", "bfloat16"], 16),
+    **dict.fromkeys(["float", "int32_t"], 32),
+    **dict.fromkeys(["int8_t", "uint8_t"], 8),
+    **dict.fromkeys(["int4_t", "uint4_t"], 4),
+    **dict.fromkeys(["int3_t", "uint3_t"], 3),
+}
+
+SUPPORTED_QCFG = [
+    "fp16",
+    "w8a8_g-1_sym",
+    "w4a4_g-1_sym",
+    *[f"w{w}a16_g128_{s}" for w in (4, 3) for s in ("sym", "asym")],
+]
+
+# (M, N, K) of one MFMA instruction
+MMA_SHAPE = {
+    "MFMA_F32_32x32x16_F16": (32, 32, 16),
+    "MFMA_I32_32x32x32_I8": (32, 32, 32),
+    "MFMA_I32_32x32x32_I8_FROM_I4": (32, 32, 32),  # int4 operands widened to int8 (16*v) in registers
+    "MFMA_F32_16x16x32_F16": (16, 16, 32),
+}
+MMA_TO_ACC_TYPE = {"MFMA_F32_32x32x16_F16": "float", "MFMA_I32_32x32x32_I8": "int32_t", "MFMA_I32_32x32x32_I8_FROM_I4": "int32_t", "MFMA_F32_16x16x32_F16": "float"}
+MMA_TO_INP_TYPE = {"MFMA_F32_32x32x16_F16": "half", "MFMA_I32_32x32x32_I8": "int8_t", "MFMA_I32_32x32x32_I8_FROM_I4": "int4_t", "MFMA_F32_16x16x32_F16": "half"}
+
+QCFG_TO_MMA = {
+    "fp16": "MFMA_F32_32x32x16_F16",
+    "w8a8_g-1_sym": "MFMA_I32_32x32x32_I8",
+    "w4a4_g-1_sym": "MFMA_I32_32x32x32_I8_FROM_I4",
+    **{f"w{w}a16_g128_{s}": "MFMA_F32_16x16x32_F16" for w in (4, 3) for s in ("sym", "asym")},
+}
+
+
+@dataclasses.dataclass
+class QConfigBase:
+    T_PACK: str = "half"
+    QBITS: int = 16
+    GSIZE: int = -1
+    SYM: bool = True
+    PACK_DIM: str = "PackDim::K"
+    USE_FP: bool = False
+    T_SCALE: str = "half"
+
+    def bytes_per_scale_zp(self):
+        raise NotImplementedError
+
+    def pack_num(self):
+        return 16 // self.QBITS
+
+    def qtype(self):
+        if self.QBITS >= 16:
+            return None
+        return f"{'int' if self.SYM else 'uint'}{self.QBITS}_t"
+
+
+@dataclasses.dataclass
+class NO_QUANT(QConfigBase):
+    def to_str(self):
+        return "NO_QUANT"
+
+    def bytes_per_scale_zp(self):
+        return 0
+
+
+@dataclasses.dataclass
+class QConfig(QConfigBase):
+    def to_str(self):
+        return f"QConfig<{self.T_PACK}, {'true' if self.SYM else 'false'}, {self.QBITS}, {self.GSIZE}, {self.PACK_DIM}, {'true' if self.USE_FP else 'false'}, {self.T_SCALE}>"
+
+    def bytes_per_scale_zp(self):
+        return TYPE_TO_BITS[self.T_SCALE] // 8 * (1 if self.SYM else 2)
+
+
+QCFG_W8A8 = QConfig(QBITS=8, GSIZE=-1, SYM=True, PACK_DIM="PackDim::K")
+QCFG_W4A4 = QConfig(QBITS=4, GSIZE=-1, SYM=True, PACK_DIM="PackDim::K")
+
+CFG_TEMPLATE = "TileConfig<{BM},{BN},{BK},{WM},{WN},{WK},{STAGE},{SPLITK},{MMA},{QCFGA},{QCFGB}>"
+
+
+@dataclasses.dataclass
+class TileConfig:
+    BM: int = 64
+    BN: int = 64
+    BK: int = 64
+    WM: int = 2
+    WN: int = 2
+    WK: int = 1
+    STAGE: int = 2
+    SPLITK: int = -1
+    MMA: str = "MFMA_F32_32x32x16_F16"
+    QCFGA: QConfigBase = dataclasses.field(default_factory=NO_QUANT)
+    QCFGB: QConfigBase = dataclasses.field(default_factory=NO_QUANT)
+
+    def to_str(self):
+        return CFG_TEMPLATE.format(BM=self.BM, BN=self.BN, BK=self.BK, WM=self.WM, WN=self.WN, WK=self.WK, STAGE=self.STAGE, SPLITK=self.SPLITK,
+                                   MMA=self.MMA, QCFGA=self.QCFGA.to_str(), QCFGB=self.QCFGB.to_str())
+
+    def __hash__(self):
+        return hash(self.to_str())
+
+    def __eq__(self, other):
+        return isinstance(other, TileConfig) and dataclasses.asdict(self) == dataclasses.asdict(other)
+
+    @property
+    def num_warps(self):
+        """Wavefronts per workgroup (the reference's warps per CTA); fused branches must agree (compose_kernel.py:69-71)."""
+        return self.WM * self.WN * self.WK
+
+    def warp_tile_mnk(self):
+        return self.BM // self.WM, self.BN // self.WN, self.BK // self.WK
+
+    def w_bits(self):
+        return self.QCFGB.QBITS
+
+    def a_bits(self):
+        return self.QCFGA.QBITS
+
+    def acc_type(self):
+        return MMA_TO_ACC_TYPE[self.MMA]
+
+    def is_a_quant(self):
+        return not isinstance(self.QCFGA, NO_QUANT)
+
+    def is_b_quant(self):
+        return not isinstance(self.QCFGB, NO_QUANT)
+
+    def set_qcfg(self, qcfg: "TileConfig") -> "TileConfig":
+        self.QCFGA, self.QCFGB = qcfg.QCFGA, qcfg.QCFGB
+        return self
+
+    def is_skinny(self) -> bool:
+        return self.MMA == "MFMA_F32_16x16x32_F16"
+
+    def smem_bytes_scale(self):
+        return 0  # scales are read straight from global memory in the epilogue / per group
+
+    def smem_bytes_tile(self):
+        """LDS bytes of the tile as compiled (csrc/include/mxmoe_tiles.hpp, mxmoe_wo_tiles.hpp)."""
+        if self.is_skinny():
+            return 16 * (1024 * 2 + 16)
+        return self.STAGE * (self.BM + self.BN) * 64
+
+    def cpp_type(self) -> str:
+        """The C++ tile type this descriptor instantiates."""
+        if self.is_skinny():
+            return f"SkinnyWoTile<{self.QCFGB.QBITS}, {self.BN}>"
+        op = {"MFMA_F32_32x32x16_F16": "Op::F16", "MFMA_I32_32x32x32_I8": "Op::I8", "MFMA_I32_32x32x32_I8_FROM_I4": "Op::I4"}[self.MMA]
+        return f"MfmaTile<{op}, {self.BM}, {self.BN}, {self.WM}, {self.WN}>"
+
+    def validate(self) -> None:
+        if self.num_warps != 4:
+            raise ValueError(f"{self!r}: gfx950 tiles use 4 wavefronts per workgroup")
+        if self.is_skinny():
+            if self.BM != 16 or self.BN % 64 or self.BK != 128:
+                raise ValueError(f"{self!r}: skinny weight-only tiles are 16 x (64k) x 128")
+            return
+        k_elems = {"MFMA_F32_32x32x16_F16": 32, "MFMA_I32_32x32x32_I8": 64, "MFMA_I32_32x32x32_I8_FROM_I4": 128}[self.MMA]
+        if self.BK != k_elems or self.STAGE != 2 or self.WK != 1 or (self.BM // self.WM) % 32 or (self.BN // self.WN) % 32:
+            raise ValueError(f"{self!r}: unsupported shape for {self.MMA} (BK must be {k_elems}, STAGE 2, wave tile a multiple of 32x32)")
+
+
+def get_info_from_qcfg_str(qcfg: str):
+    """'w4a4_g-1_sym' -> (w_bits, a_bits, gsize, sym)   (tile_config.py:288-294)."""
+    if qcfg.startswith("fp16"):
+        return 16, 16, -1, True
+    s = qcfg.split("_")
+    wbits = int(s[0].split("a")[0].split("w")[1])
+    abits = int(s[0].split("a")[1])
+    return wbits, abits, int(s[1].split("g")[1]), s[2] == "sym"
+
+
+def build_qcfgb_from_str(qcfg: str) -> QConfig:
+    w, _a, g, sym = get_info_from_qcfg_str(qcfg)
+    return QConfig(QBITS=w, GSIZE=g, SYM=sym, PACK_DIM="PackDim::MN")
+
+
+QCFG_MAP = {
+    "fp16": TileConfig(),
+    "w8a8_g-1_sym": TileConfig(QCFGA=QCFG_W8A8, QCFGB=QCFG_W8A8),
+    "w4a4_g-1_sym": TileConfig(QCFGA=QCFG_W4A4, QCFGB=QCFG_W4A4),
+    **{k: TileConfig(QCFGB=build_qcfgb_from_str(k)) for k in [f"w{w}a16_g128_{s}" for w in (4, 3) for s in ("sym", "asym")]},
+}
+
+
+def _with_q(t: TileConfig, qcfg: str) -> TileConfig:
+    return dataclasses.replace(t, QCFGA=QCFG_MAP[qcfg].QCFGA, QCFGB=QCFG_MAP[qcfg].QCFGB)
+
+
+def get_possible_tile_list(arch: str, qcfg: str) -> list:
+    """Candidate tiles per qcfg (hand-curated like tile_config.py:330-610, for gfx950)."""
+    if not str(arch).startswith("gfx95"):
+        raise ValueError(f"no tile list for arch {arch!r}: this library targets gfx950")
+    mma = QCFG_TO_MMA[qcfg]
+    if mma == "MFMA_F32_16x16x32_F16":
+        return [_with_q(TileConfig(BM=16, BN=bn, BK=128, WM=1, WN=4, WK=1, STAGE=2, MMA=mma), qcfg) for bn in (128, 64, 256)]
+    bk = {"MFMA_F32_32x32x16_F16": 32, "MFMA_I32_32x32x32_I8": 64, "MFMA_I32_32x32x32_I8_FROM_I4": 128}[mma]
+    shapes = [(128, 256, 2, 2), (64, 256, 1, 4), (32, 256, 1, 4), (128, 128, 2, 2), (256, 128, 2, 2)]
+    return [_with_q(TileConfig(BM=bm, BN=bn, BK=bk, WM=wm, WN=wn, WK=1, STAGE=2, MMA=mma), qcfg) for bm, bn, wm, wn in shapes]
+
+
+_FIELD = re.compile(r"(BM|BN|BK|WM|WN|WK|STAGE|SPLITK)=(-?\d+)")
+
+
+def parse_tile_repr(text: str, qcfg: str | None = None) -> list:
+    """Parse TileConfig reprs (the form `bits_solver.export_qconfig` writes: `{layer: repr(tuple_of_TileConfig)}`,
+    bits_solver.py:30,67-69) back into TileConfig objects."""
+    out = []
+    for chunk in text.split("TileConfig(")[1:]:
+        vals = {k: int(v) for k, v in _FIELD.findall(chunk.split("QCFGA")[0])}
+        mma = re.search(r"MMA='([^']+)'", chunk)
+        t = TileConfig(MMA=mma.group(1) if mma else TileConfig().MMA, **vals)
+        out.append(_with_q(t, qcfg) if qcfg else t)
+    return out
+
+
+def tile_from_dict(d: dict, qcfg: str) -> TileConfig:
+    """`{BM, BN, BK, WM, WN, WK, STAGE, SPLITK, MMA}` -> TileConfig carrying the qcfg's QCFGA / QCFGB."""
+    keys = ("BM", "BN", "BK", "WM", "WN", "WK", "STAGE", "SPLITK", "MMA")
+    t = TileConfig(**{k: d[k] for k in keys if k in d})
+    if "MMA" not in d:
+        t.MMA = QCFG_TO_MMA[qcfg]
+    return _with_q(t, qcfg)
+
+
+def load_tile_configs(obj: dict, qcfgs) -> dict:
+    """Accept both tile_config JSON forms: `{qcfg: [tile dicts or repr strings]}` (what run_mxmoe_gg.py:101-106 expects)
+    and `{layer: repr(tuple_of_TileConfig)}` (what the ILP writes); returns `{qcfg: [TileConfig]}`."""
+    qcfgs = sorted(qcfgs)
+    out = {}
+    if all(k in QCFG_MAP for k in obj):
+        for q, items in obj.items():
+            tiles = []
+            for it in items if isinstance(items, list) else [items]:
+                tiles += [tile_from_dict(it, q)] if isinstance(it, dict) else parse_tile_repr(it, q)
+            out[q] = tiles
+        return out
+    for _layer, text in obj.items():  # repr form: one tile per qcfg in sorted-qcfg order
+        tiles = parse_tile_repr(text)
+        for q, t in zip(qcfgs, tiles):
+            out.setdefault(q, []).append(_with_q(t, q))
+    return out

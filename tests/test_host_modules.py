@@ -1,0 +1,116 @@
+"""Host logic mirrored from the reference's Python side: qconfig schema, tile descriptors, workload generation, the
+kernel generator and the run_mxmoe_gg helpers.  No GPU."""
+import json
+import re
+from pathlib import Path
+
+import pytest
+
+from mxmoe_amd import synth
+from mxmoe_amd.kernels import gen_workload, qconfig, tile_config
+from mxmoe_amd.kernels.compose_kernel import KernelType, TemplateGenerator
+
+REF_TABLE = Path("/root/reference/perf/performance_table.json")
+
+
+def test_qconfig_schema_roundtrip(tmp_path):
+    d = synth.qconfig_dict(synth.get_config("c3"))
+    d["LT"] = {"note": "popped by readers"}                                # run_mxmoe_gg.py:14, qconfig.py:70
+    p = tmp_path / "q-wbits5.00.json"
+    p.write_text(json.dumps(d))
+    m = qconfig.build_qmodel_cfg_from_json(str(p))
+    assert set(m.layers) == {"0"} and len(m.layers["0"].experts) == 60
+    e0 = m.layers["0"].experts["0"]
+    assert e0.gate == e0.up                                                # gate and up share a format
+    assert str(e0.gate) in ("W4A4_g-1_sym", "W8A8_g-1_sym")
+    assert e0.gate.qparams() in (synth.W4A4, synth.W8A8)
+    assert qconfig.QLinearConfig.from_dict(e0.gate.to_dict()) == e0.gate
+    assert set(map(tuple, qconfig.get_all_wbits(m))) == {(4, -1, True), (8, -1, True)}
+    uni = qconfig.build_uni_qmodel_cfg(qconfig.QLinearConfig(w_bits=4, a_bits=4, w_sym=True), 2, 3)
+    assert len(uni.layers) == 2 and len(uni.layers["1"].experts) == 3
+
+
+def test_tile_config_repr_is_the_profile_table_key_shape():
+    t = tile_config.get_possible_tile_list("gfx950", "w4a4_g-1_sym")[0]
+    r = repr(t)
+    assert r.startswith("TileConfig(BM=128, BN=256, BK=128, WM=2, WN=2, WK=1, STAGE=2, SPLITK=-1, MMA='MFMA_I32_32x32x32_I8_FROM_I4', QCFGA=QConfig(T_PACK='half', QBITS=4")
+    if REF_TABLE.exists():                                                 # same field order as the keys of the reference's table
+        ref_key = next(iter(json.loads(REF_TABLE.read_text())["w4a4_g-1_sym"]["3"]))
+        assert re.findall(r"(\w+)=", ref_key) == re.findall(r"(\w+)=", r)
+    assert t.num_warps == 4 and t.smem_bytes_tile() == 2 * (128 + 256) * 64
+    assert tile_config.get_info_from_qcfg_str("w3a16_g128_asym") == (3, 16, 128, False)
+    with pytest.raises(ValueError):
+        tile_config.TileConfig(BM=128, BN=256, BK=64, WM=2, WN=4, MMA="MFMA_I32_32x32x32_I8").validate()   # 8 waves
+    with pytest.raises(ValueError):
+        tile_config.get_possible_tile_list("89", "fp16")
+
+
+def test_tile_config_json_both_forms():
+    qs = ["w4a4_g-1_sym", "w8a8_g-1_sym"]
+    a = tile_config.load_tile_configs({"w4a4_g-1_sym": [{"BM": 64, "BN": 256, "BK": 128, "WM": 1, "WN": 4}], "w8a8_g-1_sym": [{"BM": 128, "BN": 256, "BK": 64}]}, qs)
+    assert a["w4a4_g-1_sym"][0].cpp_type() == "MfmaTile<Op::I4, 64, 256, 1, 4>"
+    assert a["w8a8_g-1_sym"][0].QCFGA.QBITS == 8
+    pair = (tile_config.get_possible_tile_list("gfx950", qs[0])[1], tile_config.get_possible_tile_list("gfx950", qs[1])[0])
+    b = tile_config.load_tile_configs({"11": repr(pair)}, qs)              # the form bits_solver.export_qconfig writes
+    assert b[qs[0]][0] == pair[0] and b[qs[1]][0] == pair[1]
+
+
+def test_gen_workload_follows_the_reference_rules(tmp_path):
+    cfg = synth.get_config("c4")
+    trace, qcfg = tmp_path / "moe-gate.json", tmp_path / "q-wbits4.json"
+    trace.write_text(json.dumps(synth.trace_dict(cfg)))
+    qcfg.write_text(json.dumps(synth.qconfig_dict(cfg)))
+    w = gen_workload.generate_workload_from_gate_trace(str(trace), cfg.tokens, 0, str(tmp_path / "out" / "w.json"), str(qcfg))
+    assert json.loads((tmp_path / "out" / "w.json").read_text()) == w
+    gu, dn = w["layer-0"]["gate_up"], w["layer-0"]["down"]
+    assert w["num_tokens"] == 32 and len(gu) == 65 and len(dn) == 65
+    freq = json.loads(trace.read_text())["layer-0"]["access_freq"]
+    for e in range(64):
+        m = int(freq[e] / sum(freq) * 32 * 6)                              # gen_workload.py:88-89 floors
+        assert gu[e]["shape"] == [m, 2816, 2048] and dn[e]["shape"] == [m, 2048, 1408]
+    assert gu[64]["shape"] == [32, 2 * 1408 * 2, 2048] and dn[64]["shape"] == [32, 2048, 1408 * 2]
+    q = json.loads(qcfg.read_text())["0"]["experts"]["64"]["gate"]
+    assert dn[64]["w_bits"] == q["w_bits"]                                 # shared `down` takes the "gate" block's qcfg (:94)
+    w2 = gen_workload.generate_workload_from_gate_trace(str(trace), 64, 0, None, None, "w4a4_g-1_sym")
+    assert w2["layer-0"]["gate_up"][0]["a_bits"] == 4 and w2["layer-0"]["gate_up"][0]["sym"] is True
+    w3 = gen_workload.generate_workload_from_gate_trace(str(trace), 64, 0, None)
+    assert w3["layer-0"]["down"][3]["w_bits"] == 16
+
+
+def test_template_generator_product_and_sources(tmp_path):
+    tiles = {q: tile_config.get_possible_tile_list("gfx950", q)[:n] for q, n in (("w4a4_g-1_sym", 3), ("w8a8_g-1_sym", 2))}
+    g = TemplateGenerator("gfx950", ["w8a8_g-1_sym", "w4a4_g-1_sym"], KernelType.Fused, tiles, out_dir=tmp_path)
+    assert g.qcfgs == ["w4a4_g-1_sym", "w8a8_g-1_sym"]                     # sorted, as compose_kernel.py:82
+    files = g.generate_source_code()
+    assert len(g.combos) == 6 and len(files) == 7                          # 3 x 2 combinations + the ABI unit
+    src = (tmp_path / "hz_fused_4.hip").read_text()
+    assert 'register_fused<MfmaTile<Op::I4, 32, 256, 1, 4>, MfmaTile<Op::I8, 128, 256, 2, 2>>("groupgemm_hz_fused_4")' in src
+    assert "(a_bits == 4 && w_bits == 4 && gsize == -1 && sym == true)" in src
+    assert "groupgemm_hz_fused_5" in (tmp_path / "hz_fused_decl.hpp").read_text()
+    seq = TemplateGenerator("gfx950", ["w8a8_g-1_sym", "w4a4_g-1_sym"], KernelType.Sequential, tiles, out_dir=tmp_path / "seq")
+    assert len(seq.get_tile_configs()) == 5                                # one single-format kernel per (qcfg, tile)
+    with pytest.raises(ValueError, match="Unsupported qcfg"):
+        TemplateGenerator("gfx950", ["w2a16_g-1_sym"])
+
+
+def test_run_mxmoe_gg_helpers(tmp_path):
+    import run_mxmoe_gg as r
+
+    p = tmp_path / "q-wbits5.0.json"
+    p.write_text(json.dumps({**synth.qconfig_dict(synth.get_config("c5")), "LT": 1}))
+    assert r.get_qcfg_list(str(p), -1) == {"w4a4_g-1_sym", "w8a8_g-1_sym", "w4a16_g128_asym"}
+    assert r.get_qcfg_list(str(p), 7) == set()
+    assert str(p).split("wbits")[1].split(".json")[0] == "5.0"            # workload suffix rule, run_mxmoe_gg.py:54
+
+
+def test_synthetic_configs_match_the_baseline_shapes():
+    c3 = synth.get_config("c3")
+    ids, w = synth.make_routing(c3)
+    assert ids.shape == (8192, 4) and bool((ids.sort(dim=1).values.diff(dim=1) != 0).all())   # distinct experts per token
+    assert abs(float(w.sum(1).mean()) - 1) < 1e-5
+    f = synth.draw_formats(c3)
+    assert len(f) == 60 and {q for pair in f for q in pair} == {synth.W4A4, synth.W8A8}
+    c4 = synth.get_config("c4")
+    assert len(synth.draw_formats(c4)) == 65
+    w13, w2 = synth.expert_weights(c4, 64)
+    assert w13.shape == (2 * 2816, 2048) and w2.shape == (2048, 2816)
