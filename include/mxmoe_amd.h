@@ -51,7 +51,7 @@ int mxmoe_kernel_branch(int kernel_id, int branch, int32_t out[8]);
  * acc_dump (optional, may be NULL) is a DEVICE array of per-problem int32 [M,N] buffers (entries may be NULL) that
  * receive the raw accumulators (int32 for w8a8 / w4a4, fp32 bit patterns otherwise); used by the parity tests.
  * Errors: 1 "quant type not supported" (same text as the reference launcher, compose_kernel.py:433), 2 bad kernel id,
- * 3 unsupported shape (K not a multiple of the tile's K step, N not a multiple of 4), 4 launch failure. */
+ * 3 unsupported shape (K not a multiple of the tile's K step, N not a multiple of 8), 4 launch failure. */
 int mxmoe_group_gemm(int kernel_id, const void* const* As, const void* const* Bs, const void* const* scale_a, const void* const* scale_b,
                      void* const* Cs, void* const* Ds, const int64_t* lda, const int64_t* ldb, const int64_t* ldc, const int64_t* ldd,
                      const mxmoe_dim3* d_sizes, const mxmoe_dim3* h_sizes, const mxmoe_qparams* d_q, const mxmoe_qparams* h_q, int problem_count,

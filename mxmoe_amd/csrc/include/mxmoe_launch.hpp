@@ -65,8 +65,13 @@ struct Dispatch<I, T, Rest...> {
   }
 };
 
+// Waves per SIMD the register allocator should aim for: 2 (two co-resident workgroups per CU, 256 registers per lane) unless a
+// tile keeps more than 128 accumulator registers per lane, which needs the full 512-register budget of a lone wave.
 template <class... Tiles>
-__global__ void __launch_bounds__(kThreads, 2) fused_group_gemm_kernel(const FusedArgs args) {
+constexpr int kWavesPerSimd = ((Tiles::kAccRegs > 128) || ...) ? 1 : 2;
+
+template <class... Tiles>
+__global__ void __launch_bounds__(kThreads, kWavesPerSimd<Tiles...>) fused_group_gemm_kernel(const FusedArgs args) {
   extern __shared__ __align__(16) uint8_t smem[];
   const int wg = blockIdx.x;
   const int tile = (wg % kNumXcd) * args.chunk + wg / kNumXcd;
@@ -166,6 +171,17 @@ inline std::string& last_error() {
 
 template <class... Tiles>
 hipError_t launch_fused(const FusedArgs& a, int grid, int lds, hipStream_t s) {
+  // more than 64 KB of dynamic LDS must be opted into, once per device (kept out of library load time: no HIP call before first use)
+  static bool lds_opted_in[64] = {};
+  if (lds > 64 * 1024) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return hipGetLastError();
+    if (dev >= 0 && dev < 64 && !lds_opted_in[dev]) {
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&fused_group_gemm_kernel<Tiles...>), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+      if (e != hipSuccess) return e;
+      lds_opted_in[dev] = true;
+    }
+  }
   hipLaunchKernelGGL((fused_group_gemm_kernel<Tiles...>), dim3(grid), dim3(kThreads), lds, s, a);
   return hipGetLastError();
 }
@@ -184,9 +200,6 @@ int register_fused(const char* fn_name) {
   }
   k.name = n + fn_name;
   k.launch = &launch_fused<Tiles...>;
-  if (k.lds_bytes > 64 * 1024) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&fused_group_gemm_kernel<Tiles...>), hipFuncAttributeMaxDynamicSharedMemorySize, k.lds_bytes);
-  }
   registry().push_back(k);
   return (int)registry().size() - 1;
 }
@@ -260,9 +273,9 @@ inline int group_gemm(int kernel_id, const void* const* As, const void* const* B
         return 1;
       }
       const BranchInfo& bi = k.branches[b];
-      if (sz.z == 0 || sz.z % bi.k_multiple != 0 || sz.y % 4 != 0 || (bi.fmt != Fmt::FP16 && bi.fmt != Fmt::W8A8 && bi.fmt != Fmt::W4A4 && sz.y % 16 != 0)) {
+      if (sz.z == 0 || sz.z % bi.k_multiple != 0 || sz.y % 8 != 0 || (bi.fmt != Fmt::FP16 && bi.fmt != Fmt::W8A8 && bi.fmt != Fmt::W4A4 && sz.y % 16 != 0)) {
         char buf[200];
-        snprintf(buf, sizeof buf, "problem %d: shape [%u,%u,%u] not supported by tile %s (K %% %d, N %% 4)", base + i, sz.x, sz.y, sz.z, fmt_name(bi.fmt, true), bi.k_multiple);
+        snprintf(buf, sizeof buf, "problem %d: shape [%u,%u,%u] not supported by tile %s (K %% %d, N %% 8)", base + i, sz.x, sz.y, sz.z, fmt_name(bi.fmt, true), bi.k_multiple);
         last_error() = buf;
         return 3;
       }

@@ -18,6 +18,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "mxmoe_types.h"
 
 namespace mxmoe {
@@ -52,8 +54,43 @@ struct TileArgs {
 // fp16" into one v_fma_mixlo_f16, which rounds the exact product once; the reference arithmetic (and its CPU restatement) rounds
 // to fp32 first and to fp16 second, and the two differ on ties.
 __device__ __forceinline__ float keep_f32(float v) {
-  asm volatile("" : "+v"(v));
+  asm("" : "+v"(v));  // not volatile: it may be scheduled freely, it just cannot be looked through
   return v;
+}
+
+// Loads / stores through pointers known to be global memory.  Pointers fetched from the per-problem pointer arrays are
+// generic to the compiler, which would emit flat_* instructions; those also count on the LDS counter, so every wait for an
+// LDS read would wait for the global prefetch as well.
+#define MXMOE_GLOBAL __attribute__((address_space(1)))
+template <class T>
+__device__ __forceinline__ T gload(const void* p) {
+  return *(const MXMOE_GLOBAL T*)(p);
+}
+template <class T>
+__device__ __forceinline__ void gstore(void* p, const T& v) {
+  *(MXMOE_GLOBAL T*)(p) = v;
+}
+
+// Raw buffer resource over `bytes` bytes at `p` (stride 0: offsets are plain byte offsets, loads past the end return zero).
+__device__ __forceinline__ v4i make_rsrc(const void* p, unsigned bytes) {
+  const uint64_t a = (uint64_t)p;
+  v4i r;
+  r[0] = (int)(uint32_t)a;
+  r[1] = (int)((uint32_t)(a >> 32) & 0xFFFFu);
+  r[2] = (int)bytes;
+  r[3] = 0x00020000;
+  return r;
+}
+
+// One wave-wide 16-byte-per-lane load from a buffer straight into LDS (no register staging): lane l's 16 bytes land at
+// lds_addr + 16*l.  Issued as inline assembly so that the compiler does not serialise later LDS reads behind it; completion is
+// tracked by hand with vm_wait<N>() (loads retire in order).
+__device__ __forceinline__ void dma16_to_lds(const v4i& rsrc, int lds_addr, int voffset, int soffset) {
+  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds" : : "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset) : "memory", "m0");
+}
+template <int N>
+__device__ __forceinline__ void vm_wait() {
+  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
 }
 
 // LDS byte offset of 16-byte chunk `c` (0..3) of tile row `r`.  Rows are 64 bytes; the chunk index is XORed with
@@ -91,12 +128,18 @@ struct MfmaTile {
   static constexpr int kBits = OpTraits<OP>::kBitsPerElem;
   static constexpr int BK = kRowBytes * 8 / kBits;  // K elements per pipeline stage: 64 (int8), 128 (int4), 32 (fp16)
   static constexpr int kStageBytes = (BM + BN) * kRowBytes;
-  static constexpr int kLdsBytes = 2 * kStageBytes;
+  static constexpr int kStages = 3;
+  static constexpr int kLdsBytes = kStages * kStageBytes;
+  static constexpr int kAccRegs = FM * FN * 16;
   static constexpr int A_CHUNKS = BM * 4, B_CHUNKS = BN * 4;
   static constexpr int A_IT = (A_CHUNKS + kThreads - 1) / kThreads, B_IT = (B_CHUNKS + kThreads - 1) / kThreads;
   using Acc = typename OpTraits<OP>::Acc;
 
   __device__ static __forceinline__ void run(const TileArgs& t, uint8_t* __restrict__ smem) {
+#ifdef MXMOE_EXP_TIMING
+    long long ts[8];
+    ts[0] = __builtin_readcyclecounter();
+#endif
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
@@ -106,44 +149,31 @@ struct MfmaTile {
     const int KT = (int)(row_bytes / kRowBytes);
     const int m0 = t.tile_m * BM, n0 = t.tile_n * BN;
 
-    // ---- global -> register -> LDS staging plan: thread owns 16-byte chunk (row = idx/4, chunk = idx%4) ----
-    const uint8_t* ga[A_IT];
-    const uint8_t* gb[B_IT];
-    int la[A_IT], lb[B_IT];
+    // ---- global -> LDS staging plan.  A K slice of the tile is (BM + BN) rows of 64 bytes = (BM + BN) / 16 wave-wide loads of
+    // 1 KB, dealt round-robin to the 4 waves.  Each load writes 16 consecutive LDS rows; lane l fills 16-byte slot (row l/4, slot
+    // l%4) and therefore fetches the chunk the swizzle maps there.  The buffer resources cover exactly the valid rows of the
+    // tile, so rows past M (or N) arrive as zeros.
+    const int a_rows = min(BM, M - m0), b_rows = min(BN, N - n0);
+    const v4i rs_a = make_rsrc(t.A + (long)m0 * row_bytes, (unsigned)(a_rows * row_bytes));
+    const v4i rs_b = make_rsrc(t.B + (long)n0 * row_bytes, (unsigned)(b_rows * row_bytes));
+    constexpr int kDmaTotal = (BM + BN) / 16, kDmaA = BM / 16;
+    constexpr int kDma = (kDmaTotal + kWaves - 1) / kWaves;  // loads per wave per slice
+    const int uwave = __builtin_amdgcn_readfirstlane(wave);
+    const int lds_base = (int)(uintptr_t)smem;
+    int dma_voff[kDma];
 #pragma unroll
-    for (int i = 0; i < A_IT; ++i) {
-      const int idx = tid + i * kThreads;
-      const int r = idx >> 2, c = idx & 3;
-      const int gr = min(m0 + r, M - 1);  // tail rows re-read the last valid row; their results are never stored
-      ga[i] = t.A + (long)gr * row_bytes + c * 16;
-      la[i] = lds_chunk_off(r, c);
+    for (int i = 0; i < kDma; ++i) {
+      const int ii = uwave + kWaves * i;
+      const int r = (ii < kDmaA ? ii : ii - kDmaA) * 16 + (lane >> 2);
+      dma_voff[i] = r * (int)row_bytes + (((lane & 3) ^ ((r >> 1) & 3)) << 4);
     }
+    auto dma_slice = [&](int kt, int stage) {
+      const int koff = kt * kRowBytes;
 #pragma unroll
-    for (int i = 0; i < B_IT; ++i) {
-      const int idx = tid + i * kThreads;
-      const int r = idx >> 2, c = idx & 3;
-      const int gr = min(n0 + r, N - 1);
-      gb[i] = t.B + (long)gr * row_bytes + c * 16;
-      lb[i] = BM * kRowBytes + lds_chunk_off(r, c);
-    }
-    v4i ra[A_IT], rb[B_IT];
-
-    auto g_load = [&](int kt) {
-#pragma unroll
-      for (int i = 0; i < A_IT; ++i)
-        if (A_CHUNKS % kThreads == 0 || tid + i * kThreads < A_CHUNKS) ra[i] = *reinterpret_cast<const v4i*>(ga[i] + (long)kt * kRowBytes);
-#pragma unroll
-      for (int i = 0; i < B_IT; ++i)
-        if (B_CHUNKS % kThreads == 0 || tid + i * kThreads < B_CHUNKS) rb[i] = *reinterpret_cast<const v4i*>(gb[i] + (long)kt * kRowBytes);
-    };
-    auto s_store = [&](int stage) {
-      uint8_t* s = smem + stage * kStageBytes;
-#pragma unroll
-      for (int i = 0; i < A_IT; ++i)
-        if (A_CHUNKS % kThreads == 0 || tid + i * kThreads < A_CHUNKS) *reinterpret_cast<v4i*>(s + la[i]) = ra[i];
-#pragma unroll
-      for (int i = 0; i < B_IT; ++i)
-        if (B_CHUNKS % kThreads == 0 || tid + i * kThreads < B_CHUNKS) *reinterpret_cast<v4i*>(s + lb[i]) = rb[i];
+      for (int i = 0; i < kDma; ++i) {
+        const int ii = uwave + kWaves * i;
+        if (kDmaTotal % kWaves == 0 || ii < kDmaTotal) dma16_to_lds(ii < kDmaA ? rs_a : rs_b, lds_base + stage * kStageBytes + ii * 1024, dma_voff[i], koff);
+      }
     };
 
     // ---- LDS -> MFMA fragment plan: lane reads row (lane & 31) of a 32-row block, chunk 2*ks + (lane >> 5) ----
@@ -161,78 +191,155 @@ struct MfmaTile {
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
-    g_load(0);
-    s_store(0);
-    __syncthreads();
-
-    for (int kt = 0; kt < KT; ++kt) {
-      const bool more = kt + 1 < KT;
-      if (more) g_load(kt + 1);
-      const uint8_t* s = smem + (kt & 1) * kStageBytes;
-#pragma unroll
-      for (int ks = 0; ks < 2; ++ks) {
-        v4i af[FM], bf[FN];
-#pragma unroll
-        for (int i = 0; i < FM; ++i) af[i] = *reinterpret_cast<const v4i*>(s + ((fa + i * 32 * kRowBytes) ^ (ks << 5)));
-#pragma unroll
-        for (int j = 0; j < FN; ++j) bf[j] = *reinterpret_cast<const v4i*>(s + ((fb + j * 32 * kRowBytes) ^ (ks << 5)));
-        if constexpr (OP == Op::I8) {
-#pragma unroll
-          for (int i = 0; i < FM; ++i)
-#pragma unroll
-            for (int j = 0; j < FN; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[j], af[i], acc[i][j], 0, 0, 0);
-        } else if constexpr (OP == Op::I4) {
-          // nibble n of a byte -> int8 holding 16 * signed(n): even elements via (x << 4), odd via x, both masked to the high nibbles
-          v4i alo[FM], ahi[FM], blo[FN], bhi[FN];
-#pragma unroll
-          for (int i = 0; i < FM; ++i) {
-            alo[i] = (af[i] << 4) & (int)0xF0F0F0F0;
-            ahi[i] = af[i] & (int)0xF0F0F0F0;
-          }
-#pragma unroll
-          for (int j = 0; j < FN; ++j) {
-            blo[j] = (bf[j] << 4) & (int)0xF0F0F0F0;
-            bhi[j] = bf[j] & (int)0xF0F0F0F0;
-          }
-#pragma unroll
-          for (int i = 0; i < FM; ++i)
-#pragma unroll
-            for (int j = 0; j < FN; ++j) {
-              acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(blo[j], alo[i], acc[i][j], 0, 0, 0);
-              acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bhi[j], ahi[i], acc[i][j], 0, 0, 0);
-            }
-        } else {
-#pragma unroll
-          for (int i = 0; i < FM; ++i)
-#pragma unroll
-            for (int j = 0; j < FN; ++j)
-              acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, bf[j]), __builtin_bit_cast(v8h, af[i]), acc[i][j], 0, 0, 0);
-        }
+    // The main loop is software-pipelined by hand at the granularity of one "unit" = one k-step of one 32-channel block
+    // (FM or 2*FM MFMAs).  While the MFMAs of unit u run, the packed fragment of unit u+2 is read from LDS and the fragment of
+    // unit u+1 is widened to MFMA operands (int4 only), so LDS latency and the unpack VALU work hide under the matrix pipe.
+    // Three LDS stages let the read-ahead run into the next K slice without waiting for this iteration's barrier:
+    //   iteration kt:  start the loads of slice kt+2 into stage (kt+2)%3, units 0..U-3 on stage kt%3, wait for this wave's
+    //   loads of slice kt+1, barrier, units U-2, U-1 (whose read-ahead touches stage (kt+1)%3).
+    constexpr int U = 2 * FN;  // units per K slice
+    auto lds_a = [&](const uint8_t* st, int step, int i) { return *reinterpret_cast<const v4i*>(st + ((fa + i * 32 * kRowBytes) ^ (step << 5))); };
+    auto lds_b = [&](const uint8_t* st, int step, int j) { return *reinterpret_cast<const v4i*>(st + ((fb + j * 32 * kRowBytes) ^ (step << 5))); };
+    auto widen = [&](const v4i& p, v4i& lo, v4i& hi) {
+      if constexpr (OP == Op::I4) {
+        // nibble n of a byte -> int8 holding 16 * signed(n): even elements via (x << 4), odd via x, both masked to the high nibbles
+        lo = (p << 4) & (int)0xF0F0F0F0;
+        hi = p & (int)0xF0F0F0F0;
+      } else {
+        lo = p;
       }
-      if (more) s_store((kt + 1) & 1);
-      __syncthreads();
+    };
+    auto mma = [&](Acc& c, const v4i& alo, const v4i& ahi, const v4i& blo, const v4i& bhi) {
+      if constexpr (OP == Op::I8) {
+        c = __builtin_amdgcn_mfma_i32_32x32x32_i8(blo, alo, c, 0, 0, 0);
+      } else if constexpr (OP == Op::I4) {
+        c = __builtin_amdgcn_mfma_i32_32x32x32_i8(blo, alo, c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_i32_32x32x32_i8(bhi, ahi, c, 0, 0, 0);
+      } else {
+        c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, blo), __builtin_bit_cast(v8h, alo), c, 0, 0, 0);
+      }
+    };
+
+    v4i alo[FM], ahi[FM];        // operands of the A fragments of the current k-step
+    v4i pa[FM];                  // packed A fragments of the next k-step
+    v4i pb[2];                   // packed B fragments: slot u&1 is free once unit u is widened, and receives unit u+2
+    v4i blo[2], bhi[2];          // operands of the B fragments of units u, u+1
+
+#ifdef MXMOE_EXP_TIMING
+    ts[1] = __builtin_amdgcn_s_memrealtime();
+#endif
+    dma_slice(0, 0);
+    dma_slice(1, 1);  // past the end of K this reads zeros or a neighbouring row; such a slice is never consumed
+    if (kDmaTotal % kWaves == 0 || uwave + kWaves * (kDma - 1) < kDmaTotal) vm_wait<kDma>(); else vm_wait<kDma - 1>();  // slice 0 has landed
+    __syncthreads();
+#ifdef MXMOE_EXP_TIMING
+    ts[2] = __builtin_readcyclecounter();
+#endif
+    {
+      const uint8_t* st = smem;
+#pragma unroll
+      for (int i = 0; i < FM; ++i) {
+        pa[i] = lds_a(st, 0, i);
+        widen(pa[i], alo[i], ahi[i]);
+      }
+      pb[0] = lds_b(st, 0, 0);
+      pb[1] = lds_b(st, 0, 1);
+      widen(pb[0], blo[0], bhi[0]);
     }
 
-    // ---- epilogue.  Lane holds token m = lane & 31 and channels 8*(r/4) + 4*(lane >> 5) + (r & 3) of each 32x32 block ----
+    // Every iteration has the same shape, including the last two: their extra prefetch lands in LDS stages nobody consumes
+    // (buffer loads past the tile read zeros), which keeps the loop body one straight-line block.
+#ifdef MXMOE_EXP_TIMING
+    ts[3] = __builtin_readcyclecounter();
+#endif
+    int sidx = 0;
+#pragma unroll 1
+    for (int kt = 0; kt < KT; ++kt) {
+      const uint8_t* sc = smem + sidx * kStageBytes;
+      const int nidx = sidx == 2 ? 0 : sidx + 1;
+      const uint8_t* sn = smem + nidx * kStageBytes;
+#ifndef MXMOE_EXP_NODMA
+      dma_slice(kt + 2, nidx == 2 ? 0 : nidx + 1);  // its stage was last read before the previous barrier
+#endif
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int step = u / FN, j = u % FN;
+        if (u == U - 2) {
+#ifndef MXMOE_EXP_NODMA
+          // this wave's part of slice kt+1 is in LDS (loads retire in order; only its loads of slice kt+2 may be in flight);
+          // after the barrier everybody's part is
+          if (kDmaTotal % kWaves == 0 || uwave + kWaves * (kDma - 1) < kDmaTotal) vm_wait<kDma>(); else vm_wait<kDma - 1>();
+#endif
+#ifndef MXMOE_EXP_NOBAR
+          __syncthreads();
+#endif
+        }
+        // read ahead: packed B fragment of unit u+2, packed A fragments of the next k-step
+        if (u + 2 < U) {
+          pb[u & 1] = lds_b(sc, (u + 2) / FN, (u + 2) % FN);
+        } else {
+          pb[u & 1] = lds_b(sn, 0, u + 2 - U);
+        }
+        if (j == FN - 2) {
+#pragma unroll
+          for (int i = 0; i < FM; ++i) pa[i] = step == 0 ? lds_a(sc, 1, i) : lds_a(sn, 0, i);
+        }
+        // operands of unit u+1; on the last unit of a k-step each A operand is refreshed right after its last use
+        widen(pb[(u + 1) & 1], blo[(u + 1) & 1], bhi[(u + 1) & 1]);
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+          mma(acc[i][j], alo[i], ahi[i], blo[u & 1], bhi[u & 1]);
+          if (j == FN - 1) widen(pa[i], alo[i], ahi[i]);
+        }
+        __builtin_amdgcn_sched_barrier(0);  // keep the units in program order: the pipeline above is the schedule
+      }
+      sidx = nidx;
+    }
+
+    // ---- epilogue.  Lane holds token m = lane & 31 and channels 8*(r/4) + 4*(lane >> 5) + (r & 3) of each 32x32 block.
+    // The scaled fp16 results go through a per-wave LDS patch laid out [token][channel] so that the global stores are 16 bytes
+    // per lane along a row (TN*2 contiguous bytes per token) instead of 8-byte pieces scattered over 32 rows.
+#ifdef MXMOE_EXP_TIMING
+    ts[4] = __builtin_readcyclecounter();
+#endif
+    __syncthreads();  // every wave is done reading the pipeline stages: LDS can be reused
+    constexpr int kPitch = TN * 2 + 8;  // bytes per token row of the patch; the odd multiple of 8 spreads rows over banks
+    static_assert(kWaves * TM * kPitch <= kLdsBytes, "epilogue patch must fit the pipeline's LDS");
+    uint8_t* patch = smem + wave * (TM * kPitch);
     const int nq = (lane >> 5) * 4;
+    // all scales of this lane are fetched up front, in one batch of independent loads
+    _Float16 s_a[FM];
+    v4h s_b[FN][4];
+    if constexpr (OP != Op::F16) {
+#pragma unroll
+      for (int i = 0; i < FM; ++i) {
+        const int m = m0 + wm * TM + i * 32 + lrow;
+        s_a[i] = m < M ? gload<_Float16>(t.sa + m) : (_Float16)0.0f;
+      }
+#pragma unroll
+      for (int j = 0; j < FN; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int n = n0 + wn * TN + j * 32 + q * 8 + nq;
+          s_b[j][q] = v4h{(_Float16)0.0f, (_Float16)0.0f, (_Float16)0.0f, (_Float16)0.0f};
+          if (n < N) s_b[j][q] = gload<v4h>(t.sb + n);  // N is a multiple of 8, so a quad is all-in or all-out
+        }
+    }
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
-      const int m = m0 + wm * TM + i * 32 + lrow;
-      if (m >= M) continue;
-      _Float16 s_a = (_Float16)1.0f;
-      if constexpr (OP != Op::F16) s_a = t.sa[m];
+      const int ml = i * 32 + lrow;
+      const int m = m0 + wm * TM + ml;
 #pragma unroll
       for (int j = 0; j < FN; ++j) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const int n = n0 + wn * TN + j * 32 + q * 8 + nq;
-          if (n >= N) continue;  // N is a multiple of 4, so a quad is all-in or all-out
+          const int nl = j * 32 + q * 8 + nq;
+          const int n = n0 + wn * TN + nl;
           v4h o;
           if constexpr (OP == Op::F16) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) o[e] = (_Float16)acc[i][j][q * 4 + e];
           } else {
-            const v4h s_b = *reinterpret_cast<const v4h*>(t.sb + n);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
               int a = acc[i][j][q * 4 + e];
@@ -240,21 +347,47 @@ struct MfmaTile {
               // float(acc) * (sa * sb) rounded to half, as the reference epilogue (mm_tile.cuh:490-493, 642-646) except that the
               // scale product stays in fp32, where it is exact: the reference rounds it to fp16 first, which turns subnormal
               // (a few significant bits) for typical int8 scales and breaks the 1e-2 agreement with the fake-quant path.
-              const float s = (float)s_a * (float)s_b[e];
-              o[e] = (_Float16)keep_f32((float)a * s);
-              if (t.acc_dump) t.acc_dump[(long)m * N + n + e] = a;
+              const float sc = (float)s_a[i] * (float)s_b[j][q][e];
+              o[e] = (_Float16)keep_f32((float)a * sc);
+              if (t.acc_dump && m < M && n < N) gstore<int>(t.acc_dump + (long)m * N + n + e, a);
             }
           }
           if constexpr (OP == Op::F16) {
-            if (t.acc_dump) {
+            if (t.acc_dump && m < M && n < N) {
 #pragma unroll
-              for (int e = 0; e < 4; ++e) t.acc_dump[(long)m * N + n + e] = __builtin_bit_cast(int, acc[i][j][q * 4 + e]);
+              for (int e = 0; e < 4; ++e) gstore<int>(t.acc_dump + (long)m * N + n + e, __builtin_bit_cast(int, acc[i][j][q * 4 + e]));
             }
           }
-          *reinterpret_cast<v4h*>(t.C + (long)m * N + n) = o;
+          *reinterpret_cast<v4h*>(patch + ml * kPitch + nl * 2) = o;
         }
       }
     }
+    // same-wave LDS traffic is ordered, so no barrier is needed between the patch writes above and the reads below
+    constexpr int kLanesPerRow = TN / 8;           // 16-byte pieces per token row
+    constexpr int kRowsPerPass = 64 / kLanesPerRow;
+    const int pr = lane / kLanesPerRow, pc = lane % kLanesPerRow;
+#pragma unroll
+    for (int r0 = 0; r0 < TM; r0 += kRowsPerPass) {
+      const int ml = r0 + pr;
+      const int m = m0 + wm * TM + ml;
+      const int n = n0 + wn * TN + pc * 8;
+      const v4i v = *reinterpret_cast<const v4i*>(patch + ml * kPitch + pc * 16);
+#ifdef MXMOE_EXP_NOSTORE
+      if (m < M && n < N && v[0] == 0x12345678) gstore<v4i>(t.C + (long)m * N + n, v);
+#else
+      if (m < M && n < N) gstore<v4i>(t.C + (long)m * N + n, v);
+#endif
+    }
+#ifdef MXMOE_EXP_TIMING
+    ts[6] = __builtin_readcyclecounter();
+    ts[2] = __builtin_amdgcn_s_memrealtime();
+    __syncthreads();
+    if (tid == 0) {
+      long long* dst = reinterpret_cast<long long*>(t.C + (long)m0 * N + n0);
+      for (int i = 0; i < 7; ++i) dst[i] = ts[i];
+      dst[7] = ((long long)__builtin_amdgcn_s_getreg(63508) << 32) | (unsigned)__builtin_amdgcn_s_getreg(63492);
+    }
+#endif
   }
 };
 

@@ -34,6 +34,7 @@ struct SkinnyWoTile {
   static constexpr int R = BN / 64;                  // 16-row blocks per wave
   static constexpr int kXStride = KC * 2 + 16;       // bytes per activation row in LDS (+16 so 8 rows cover 8 bank groups)
   static constexpr int kLdsBytes = 16 * kXStride;
+  static constexpr int kAccRegs = R * 4;
   static constexpr int kLaneBytes = WBITS * 4;       // packed bytes per lane per (row block, k block)
   static constexpr int kBlockBytes = 64 * kLaneBytes;
 
@@ -44,12 +45,11 @@ struct SkinnyWoTile {
   __device__ static __forceinline__ WReg load_w(const uint8_t* p) {
     WReg w;
     if constexpr (WBITS == 4) {
-      const v4i v = *reinterpret_cast<const v4i*>(p);
+      const v4i v = gload<v4i>(p);
       w.d[0] = v[0]; w.d[1] = v[1]; w.d[2] = v[2]; w.d[3] = v[3];
     } else {
       // three dword loads (4-byte aligned); a 16-byte vector load would read past the end of the last block
-      const int* q = reinterpret_cast<const int*>(p);
-      w.d[0] = q[0]; w.d[1] = q[1]; w.d[2] = q[2];
+      w.d[0] = gload<int>(p); w.d[1] = gload<int>(p + 4); w.d[2] = gload<int>(p + 8);
     }
     return w;
   }
@@ -120,7 +120,7 @@ struct SkinnyWoTile {
         const int row = idx / (KC / 8), ch = idx % (KC / 8);
         if (ch * 8 < kcur) {
           v4i v = {0, 0, 0, 0};
-          if (m0 + row < M) v = *reinterpret_cast<const v4i*>(X + (long)(m0 + row) * K + kc0 + ch * 8);
+          if (m0 + row < M) v = gload<v4i>(X + (long)(m0 + row) * K + kc0 + ch * 8);
           *reinterpret_cast<v4i*>(smem + row * kXStride + ch * 16) = v;
         }
       }
@@ -132,7 +132,7 @@ struct SkinnyWoTile {
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         wq[r] = load_w(wp[r] + (long)kb0 * kBlockBytes);
-        sz[r] = *reinterpret_cast<const v4i*>(sp[r] + (long)kb0 * 64);
+        sz[r] = gload<v4i>(sp[r] + (long)kb0 * 64);
       }
       for (int kb = 0; kb < nkb; ++kb) {
         WReg wn[R];
@@ -141,7 +141,7 @@ struct SkinnyWoTile {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
           wn[r] = load_w(wp[r] + (long)kbn * kBlockBytes);
-          szn[r] = *reinterpret_cast<const v4i*>(sp[r] + (long)kbn * 64);
+          szn[r] = gload<v4i>(sp[r] + (long)kbn * 64);
         }
         v8h xf[4];
         const uint8_t* xs = smem + lm * kXStride + (kb * 128 + lg * 32) * 2;
@@ -175,10 +175,10 @@ struct SkinnyWoTile {
         v4h o;
 #pragma unroll
         for (int e = 0; e < 4; ++e) o[e] = (_Float16)acc[r][e];
-        *reinterpret_cast<v4h*>(t.C + (long)m * N + n) = o;
+        gstore<v4h>(t.C + (long)m * N + n, o);
         if (t.acc_dump) {
 #pragma unroll
-          for (int e = 0; e < 4; ++e) t.acc_dump[(long)m * N + n + e] = __builtin_bit_cast(int, acc[r][e]);
+          for (int e = 0; e < 4; ++e) gstore<int>(t.acc_dump + (long)m * N + n + e, __builtin_bit_cast(int, acc[r][e]));
         }
       }
     }
