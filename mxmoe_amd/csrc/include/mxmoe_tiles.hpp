@@ -136,10 +136,6 @@ struct MfmaTile {
   using Acc = typename OpTraits<OP>::Acc;
 
   __device__ static __forceinline__ void run(const TileArgs& t, uint8_t* __restrict__ smem) {
-#ifdef MXMOE_EXP_TIMING
-    long long ts[8];
-    ts[0] = __builtin_readcyclecounter();
-#endif
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
@@ -225,16 +221,10 @@ struct MfmaTile {
     v4i pb[2];                   // packed B fragments: slot u&1 is free once unit u is widened, and receives unit u+2
     v4i blo[2], bhi[2];          // operands of the B fragments of units u, u+1
 
-#ifdef MXMOE_EXP_TIMING
-    ts[1] = __builtin_amdgcn_s_memrealtime();
-#endif
     dma_slice(0, 0);
     dma_slice(1, 1);  // past the end of K this reads zeros or a neighbouring row; such a slice is never consumed
     if (kDmaTotal % kWaves == 0 || uwave + kWaves * (kDma - 1) < kDmaTotal) vm_wait<kDma>(); else vm_wait<kDma - 1>();  // slice 0 has landed
     __syncthreads();
-#ifdef MXMOE_EXP_TIMING
-    ts[2] = __builtin_readcyclecounter();
-#endif
     {
       const uint8_t* st = smem;
 #pragma unroll
@@ -249,30 +239,21 @@ struct MfmaTile {
 
     // Every iteration has the same shape, including the last two: their extra prefetch lands in LDS stages nobody consumes
     // (buffer loads past the tile read zeros), which keeps the loop body one straight-line block.
-#ifdef MXMOE_EXP_TIMING
-    ts[3] = __builtin_readcyclecounter();
-#endif
     int sidx = 0;
 #pragma unroll 1
     for (int kt = 0; kt < KT; ++kt) {
       const uint8_t* sc = smem + sidx * kStageBytes;
       const int nidx = sidx == 2 ? 0 : sidx + 1;
       const uint8_t* sn = smem + nidx * kStageBytes;
-#ifndef MXMOE_EXP_NODMA
       dma_slice(kt + 2, nidx == 2 ? 0 : nidx + 1);  // its stage was last read before the previous barrier
-#endif
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const int step = u / FN, j = u % FN;
         if (u == U - 2) {
-#ifndef MXMOE_EXP_NODMA
           // this wave's part of slice kt+1 is in LDS (loads retire in order; only its loads of slice kt+2 may be in flight);
           // after the barrier everybody's part is
           if (kDmaTotal % kWaves == 0 || uwave + kWaves * (kDma - 1) < kDmaTotal) vm_wait<kDma>(); else vm_wait<kDma - 1>();
-#endif
-#ifndef MXMOE_EXP_NOBAR
           __syncthreads();
-#endif
         }
         // read ahead: packed B fragment of unit u+2, packed A fragments of the next k-step
         if (u + 2 < U) {
@@ -299,22 +280,19 @@ struct MfmaTile {
     // ---- epilogue.  Lane holds token m = lane & 31 and channels 8*(r/4) + 4*(lane >> 5) + (r & 3) of each 32x32 block.
     // The scaled fp16 results go through a per-wave LDS patch laid out [token][channel] so that the global stores are 16 bytes
     // per lane along a row (TN*2 contiguous bytes per token) instead of 8-byte pieces scattered over 32 rows.
-#ifdef MXMOE_EXP_TIMING
-    ts[4] = __builtin_readcyclecounter();
-#endif
-    __syncthreads();  // every wave is done reading the pipeline stages: LDS can be reused
-    constexpr int kPitch = TN * 2 + 8;  // bytes per token row of the patch; the odd multiple of 8 spreads rows over banks
-    static_assert(kWaves * TM * kPitch <= kLdsBytes, "epilogue patch must fit the pipeline's LDS");
-    uint8_t* patch = smem + wave * (TM * kPitch);
     const int nq = (lane >> 5) * 4;
-    // all scales of this lane are fetched up front, in one batch of independent loads
-    _Float16 s_a[FM];
+    // all scales of this lane are fetched in one batch of independent loads, issued before the barrier so that their latency
+    // overlaps the wait for the slowest wave
+    float s_a[FM];
     v4h s_b[FN][4];
     if constexpr (OP != Op::F16) {
 #pragma unroll
       for (int i = 0; i < FM; ++i) {
         const int m = m0 + wm * TM + i * 32 + lrow;
-        s_a[i] = m < M ? gload<_Float16>(t.sa + m) : (_Float16)0.0f;
+        s_a[i] = m < M ? (float)gload<_Float16>(t.sa + m) : 0.0f;
+        // the int4 accumulator holds 256 * sum; 2^-8 folded into the (exact) scale product gives bit-identical results to
+        // shifting first: float(256 * x) == 256 * float(x), and scaling by a power of two commutes with rounding
+        if constexpr (OP == Op::I4) s_a[i] *= 0.00390625f;
       }
 #pragma unroll
       for (int j = 0; j < FN; ++j)
@@ -325,6 +303,10 @@ struct MfmaTile {
           if (n < N) s_b[j][q] = gload<v4h>(t.sb + n);  // N is a multiple of 8, so a quad is all-in or all-out
         }
     }
+    __syncthreads();  // every wave is done reading the pipeline stages: LDS can be reused
+    constexpr int kPitch = TN * 2 + 8;  // bytes per token row of the patch; the odd multiple of 8 spreads rows over banks
+    static_assert(kWaves * TM * kPitch <= kLdsBytes, "epilogue patch must fit the pipeline's LDS");
+    uint8_t* patch = smem + wave * (TM * kPitch);
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
       const int ml = i * 32 + lrow;
@@ -342,20 +324,21 @@ struct MfmaTile {
           } else {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-              int a = acc[i][j][q * 4 + e];
-              if constexpr (OP == Op::I4) a >>= 8;  // exact: the accumulator is 256 * sum
               // float(acc) * (sa * sb) rounded to half, as the reference epilogue (mm_tile.cuh:490-493, 642-646) except that the
               // scale product stays in fp32, where it is exact: the reference rounds it to fp16 first, which turns subnormal
               // (a few significant bits) for typical int8 scales and breaks the 1e-2 agreement with the fake-quant path.
-              const float sc = (float)s_a[i] * (float)s_b[j][q][e];
-              o[e] = (_Float16)keep_f32((float)a * sc);
-              if (t.acc_dump && m < M && n < N) gstore<int>(t.acc_dump + (long)m * N + n + e, a);
+              const float sc = s_a[i] * (float)s_b[j][q][e];
+              o[e] = (_Float16)keep_f32((float)acc[i][j][q * 4 + e] * sc);
             }
           }
-          if constexpr (OP == Op::F16) {
-            if (t.acc_dump && m < M && n < N) {
+          if (t.acc_dump && m < M && n < N) {
 #pragma unroll
-              for (int e = 0; e < 4; ++e) gstore<int>(t.acc_dump + (long)m * N + n + e, __builtin_bit_cast(int, acc[i][j][q * 4 + e]));
+            for (int e = 0; e < 4; ++e) {
+              const auto v = acc[i][j][q * 4 + e];
+              int a;
+              if constexpr (OP == Op::F16) a = __builtin_bit_cast(int, (float)v); else a = (int)v;
+              if constexpr (OP == Op::I4) a >>= 8;  // exact
+              gstore<int>(t.acc_dump + (long)m * N + n + e, a);
             }
           }
           *reinterpret_cast<v4h*>(patch + ml * kPitch + nl * 2) = o;
@@ -372,22 +355,8 @@ struct MfmaTile {
       const int m = m0 + wm * TM + ml;
       const int n = n0 + wn * TN + pc * 8;
       const v4i v = *reinterpret_cast<const v4i*>(patch + ml * kPitch + pc * 16);
-#ifdef MXMOE_EXP_NOSTORE
-      if (m < M && n < N && v[0] == 0x12345678) gstore<v4i>(t.C + (long)m * N + n, v);
-#else
       if (m < M && n < N) gstore<v4i>(t.C + (long)m * N + n, v);
-#endif
     }
-#ifdef MXMOE_EXP_TIMING
-    ts[6] = __builtin_readcyclecounter();
-    ts[2] = __builtin_amdgcn_s_memrealtime();
-    __syncthreads();
-    if (tid == 0) {
-      long long* dst = reinterpret_cast<long long*>(t.C + (long)m0 * N + n0);
-      for (int i = 0; i < 7; ++i) dst[i] = ts[i];
-      dst[7] = ((long long)__builtin_amdgcn_s_getreg(63508) << 32) | (unsigned)__builtin_amdgcn_s_getreg(63492);
-    }
-#endif
   }
 };
 
