@@ -57,8 +57,10 @@ int mxmoe_group_gemm(int kernel_id, const void* const* As, const void* const* Bs
                      const mxmoe_dim3* d_sizes, const mxmoe_dim3* h_sizes, const mxmoe_qparams* d_q, const mxmoe_qparams* h_q, int problem_count,
                      int32_t* const* acc_dump, void* stream);
 
-/* Tile count and branch choice the launcher would make, without launching: fills branch_out[p] and returns the total
- * number of tiles through *tiles_out.  Host-only; used by the scheduler tests and the kernel-profile table. */
+/* Tile count and branch choice the launcher would make, without launching.  The launcher runs the rows of a problem as at
+ * most two segments (whole tiles of the largest shape, then the remainder with the cheapest shape that covers it):
+ * branch_out[p] receives the branch of the first segment and *tiles_out the total number of tiles over all segments.
+ * Host-only; used by the scheduler tests and the kernel-profile table.  Returns 1000 + kernel id on success. */
 int mxmoe_group_gemm_plan(int kernel_id, const mxmoe_dim3* h_sizes, const mxmoe_qparams* h_q, int problem_count, int32_t* branch_out, int32_t* tiles_out);
 
 /* ---- token permutation: replaces gg_permute_inp and the sort / bincount prologue of quant_inp_act

@@ -64,11 +64,14 @@ int mxmoe_group_gemm_plan(int kernel_id, const mxmoe_dim3* h_sizes, const mxmoe_
   int total = 0;
   for (int i = 0; i < problem_count; ++i) {
     const Fmt f = classify(h_q[i]);
-    const int b = f == Fmt::UNSUPPORTED ? -1 : pick_branch(k, f, (int)h_sizes[i].x);
-    if (b < 0) { last_error() = "quant type not supported"; return 1; }
-    if (branch_out) branch_out[i] = b;
-    const BranchInfo& bi = k.branches[b];
-    total += (int)((h_sizes[i].x + bi.BM - 1) / bi.BM) * (int)((h_sizes[i].y + bi.BN - 1) / bi.BN);
+    Segment sg[2];
+    const int ns = f == Fmt::UNSUPPORTED ? -1 : plan_segments(k, f, (int)h_sizes[i].x, sg);
+    if (ns < 0) { last_error() = "quant type not supported"; return 1; }
+    if (branch_out) branch_out[i] = ns ? sg[0].branch : pick_branch(k, f, 1);
+    for (int j = 0; j < ns; ++j) {
+      const BranchInfo& bi = k.branches[sg[j].branch];
+      total += ((sg[j].rows + bi.BM - 1) / bi.BM) * (int)((h_sizes[i].y + bi.BN - 1) / bi.BN);
+    }
   }
   if (tiles_out) *tiles_out = total;
   return kernel_id + 1000;  // plan succeeded: 1000 + the kernel that would run

@@ -25,7 +25,8 @@
 
 namespace mxmoe {
 
-constexpr int kMaxProblems = 256;  // per launch; longer problem lists are split into several launches
+constexpr int kMaxProblems = 128;  // per launch; longer problem lists are split into several launches
+constexpr int kMaxEntries = 2 * kMaxProblems;  // a problem is run as at most two row segments, each with its own tile shape
 constexpr int kNumXcd = 8;
 
 struct FusedArgs {
@@ -37,11 +38,14 @@ struct FusedArgs {
   int32_t* const* acc;  // optional accumulator dumps (null, or per-problem pointers which may themselves be null)
   const mxmoe_dim3* sizes;
   int problem_offset;   // first problem of this launch inside the arrays above
-  int num_problems;
+  int num_entries;
   int total_tiles;
   int chunk;                      // tiles per XCD = ceil(total_tiles / 8)
-  int prefix[kMaxProblems];       // inclusive prefix sum of tiles per problem
-  uint8_t branch[kMaxProblems];   // which tile type runs each problem
+  int prefix[kMaxEntries];        // inclusive prefix sum of tiles per entry
+  int row0[kMaxEntries];          // first row of the entry's segment inside its problem
+  int rows[kMaxEntries];          // rows of the segment
+  uint16_t problem[kMaxEntries];  // problem (relative to problem_offset) the entry belongs to
+  uint8_t branch[kMaxEntries];    // which tile type runs the entry
 };
 
 template <int I, class... Tiles>
@@ -77,14 +81,14 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd<Tiles...>) fused_group
   const int tile = (wg % kNumXcd) * args.chunk + wg / kNumXcd;
   if (tile >= args.total_tiles) return;
   // tile_scheduler.cuh:25-37 — first problem whose inclusive prefix exceeds the tile index (binary search here)
-  int lo = 0, hi = args.num_problems - 1;
+  int lo = 0, hi = args.num_entries - 1;
   while (lo < hi) {
     const int mid = (lo + hi) >> 1;
     if (tile < args.prefix[mid]) hi = mid; else lo = mid + 1;
   }
-  const int p = lo;
-  const int local = tile - (p ? args.prefix[p - 1] : 0);
-  const int gp = args.problem_offset + p;
+  const int en = lo;
+  const int local = tile - (en ? args.prefix[en - 1] : 0);
+  const int gp = args.problem_offset + args.problem[en];
   const mxmoe_dim3 sz = args.sizes[gp];
   TileArgs t;
   t.A = args.As[gp];
@@ -93,11 +97,12 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd<Tiles...>) fused_group
   t.sb = args.sb ? args.sb[gp] : nullptr;
   t.C = args.Cs[gp];
   t.acc_dump = args.acc ? args.acc[gp] : nullptr;
-  t.M = (int)sz.x;
+  t.row0 = args.row0[en];
+  t.M = t.row0 + args.rows[en];  // rows past the segment are treated like rows past the problem
   t.N = (int)sz.y;
   t.K = (int)sz.z;
   t.tile_m = t.tile_n = 0;
-  Dispatch<0, Tiles...>::go(args.branch[p], t, local, smem);
+  Dispatch<0, Tiles...>::go(args.branch[en], t, local, smem);
 }
 
 // ------------------------------------------------------------------ host side ------------------------------------------------------------------
@@ -204,29 +209,66 @@ int register_fused(const char* fn_name) {
   return (int)registry().size() - 1;
 }
 
-// Pick the branch of `k` that runs a problem: same format, then fewest padded rows, then the larger tile.
-inline int pick_branch(const FusedKernel& k, Fmt f, int M) {
+// Relative cost of one tile of BM rows (same BN, same K), measured on MI355X: a 64-row tile costs ~0.62 and a 32-row tile ~0.41
+// of a 128-row tile (fixed prologue / epilogue and a less efficient wave tile).
+inline double tile_cost(int BM) { return 0.22 + 0.78 * BM / 128.0; }
+
+// Cheapest branch of format `f` for a block of `rows` rows run with one tile shape: cost = ceil(rows / BM) * tile_cost(BM).
+inline int pick_branch(const FusedKernel& k, Fmt f, int rows) {
   int best = -1;
-  long best_pad = 0;
+  double best_cost = 0;
   static const int force_bm = getenv("MXMOE_FORCE_BM") ? atoi(getenv("MXMOE_FORCE_BM")) : 0;
   for (int i = 0; i < (int)k.branches.size(); ++i) {
     const auto& b = k.branches[i];
     if (b.fmt != f) continue;
     if (force_bm && b.BM != force_bm) continue;
-    const long pad = (long)((M + b.BM - 1) / b.BM) * b.BM;
-    if (best < 0 || pad < best_pad || (pad == best_pad && b.BM > k.branches[best].BM)) {
+    const double c = (double)((rows + b.BM - 1) / b.BM) * tile_cost(b.BM);
+    if (best < 0 || c < best_cost - 1e-9 || (c < best_cost + 1e-9 && b.BM > k.branches[best].BM)) {
       best = i;
-      best_pad = pad;
+      best_cost = c;
     }
   }
   return best;
+}
+
+struct Segment {
+  int row0, rows, branch;
+};
+
+// Split the M rows of a problem into at most two segments: whole tiles of the largest shape, then the remainder with the shape
+// that covers it most cheaply.  Returns the number of segments (0 for M == 0), or -1 when the kernel has no tile for `f`.
+inline int plan_segments(const FusedKernel& k, Fmt f, int M, Segment out[2]) {
+  int big = -1;
+  for (int i = 0; i < (int)k.branches.size(); ++i)
+    if (k.branches[i].fmt == f && (big < 0 || k.branches[i].BM > k.branches[big].BM)) big = i;
+  if (big < 0) return -1;
+  if (M <= 0) return 0;
+  static const bool no_split = getenv("MXMOE_NO_SPLIT") != nullptr;
+  const int bm = k.branches[big].BM;
+  const int full = (M / bm) * bm, rem = M - full;
+  const int whole = pick_branch(k, f, M);
+  if (rem == 0 || full == 0 || no_split) {
+    out[0] = Segment{0, M, whole};
+    return 1;
+  }
+  const int rb = pick_branch(k, f, rem);
+  const double split_cost = (full / bm) * tile_cost(bm) + (double)((rem + k.branches[rb].BM - 1) / k.branches[rb].BM) * tile_cost(k.branches[rb].BM);
+  const double whole_cost = (double)((M + k.branches[whole].BM - 1) / k.branches[whole].BM) * tile_cost(k.branches[whole].BM);
+  if (whole_cost <= split_cost + 1e-9 || rb == big) {
+    out[0] = Segment{0, M, rb == big ? big : whole};
+    return 1;
+  }
+  out[0] = Segment{0, full, big};
+  out[1] = Segment{full, rem, rb};
+  return 2;
 }
 
 // A kernel can run a problem list when it has a branch for every format in it.
 inline bool kernel_covers(const FusedKernel& k, const mxmoe_qparams* q, int count) {
   for (int i = 0; i < count; ++i) {
     const Fmt f = classify(q[i]);
-    if (f == Fmt::UNSUPPORTED || pick_branch(k, f, 1) < 0) return false;
+    Segment sg[2];
+    if (f == Fmt::UNSUPPORTED || plan_segments(k, f, 1, sg) < 0) return false;
   }
   return true;
 }
@@ -262,27 +304,34 @@ inline int group_gemm(int kernel_id, const void* const* As, const void* const* B
     a.acc = acc;
     a.sizes = d_sizes;
     a.problem_offset = base;
-    a.num_problems = n;
-    int total = 0;
+    int total = 0, ne = 0;
     for (int i = 0; i < n; ++i) {
       const mxmoe_dim3& sz = h_sizes[base + i];
       const Fmt f = classify(h_q[base + i]);
-      const int b = f == Fmt::UNSUPPORTED ? -1 : pick_branch(k, f, (int)sz.x);
-      if (b < 0) {
+      Segment sg[2];
+      const int ns = f == Fmt::UNSUPPORTED ? -1 : plan_segments(k, f, (int)sz.x, sg);
+      if (ns < 0) {
         last_error() = "quant type not supported";
         return 1;
       }
-      const BranchInfo& bi = k.branches[b];
-      if (sz.z == 0 || sz.z % bi.k_multiple != 0 || sz.y % 8 != 0 || (bi.fmt != Fmt::FP16 && bi.fmt != Fmt::W8A8 && bi.fmt != Fmt::W4A4 && sz.y % 16 != 0)) {
-        char buf[200];
-        snprintf(buf, sizeof buf, "problem %d: shape [%u,%u,%u] not supported by tile %s (K %% %d, N %% 8)", base + i, sz.x, sz.y, sz.z, fmt_name(bi.fmt, true), bi.k_multiple);
-        last_error() = buf;
-        return 3;
+      for (int j = 0; j < ns; ++j) {
+        const BranchInfo& bi = k.branches[sg[j].branch];
+        if (sz.z == 0 || sz.z % bi.k_multiple != 0 || sz.y % 8 != 0 || (bi.fmt != Fmt::FP16 && bi.fmt != Fmt::W8A8 && bi.fmt != Fmt::W4A4 && sz.y % 16 != 0)) {
+          char buf[200];
+          snprintf(buf, sizeof buf, "problem %d: shape [%u,%u,%u] not supported by tile %s (K %% %d, N %% 8)", base + i, sz.x, sz.y, sz.z, fmt_name(bi.fmt, true), bi.k_multiple);
+          last_error() = buf;
+          return 3;
+        }
+        total += ((sg[j].rows + bi.BM - 1) / bi.BM) * (int)((sz.y + bi.BN - 1) / bi.BN);
+        a.prefix[ne] = total;
+        a.row0[ne] = sg[j].row0;
+        a.rows[ne] = sg[j].rows;
+        a.problem[ne] = (uint16_t)i;
+        a.branch[ne] = (uint8_t)sg[j].branch;
+        ++ne;
       }
-      total += (int)((sz.x + bi.BM - 1) / bi.BM) * (int)((sz.y + bi.BN - 1) / bi.BN);  // M == 0 contributes no tiles
-      a.prefix[i] = total;
-      a.branch[i] = (uint8_t)b;
     }
+    a.num_entries = ne;
     if (total == 0) continue;
     a.total_tiles = total;
     a.chunk = (total + kNumXcd - 1) / kNumXcd;

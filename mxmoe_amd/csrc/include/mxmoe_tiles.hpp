@@ -46,7 +46,8 @@ struct TileArgs {
   const _Float16* sb;    // per-channel scales [N]   (w-a formats) or group scale/zero table (weight-only)
   _Float16* C;           // output [M, N] fp16 row-major
   int32_t* acc_dump;     // optional [M, N] int32 / fp32-bits accumulator dump (tests), may be null
-  int M, N, K;
+  int M, N, K;           // M = end row of the segment this tile belongs to (rows at or past M are not computed)
+  int row0;              // first row of the segment: tile_m counts BM-row tiles from here
   int tile_m, tile_n;
 };
 
@@ -143,7 +144,7 @@ struct MfmaTile {
     const int M = t.M, N = t.N;
     const long row_bytes = (long)t.K * kBits / 8;
     const int KT = (int)(row_bytes / kRowBytes);
-    const int m0 = t.tile_m * BM, n0 = t.tile_n * BN;
+    const int m0 = t.row0 + t.tile_m * BM, n0 = t.tile_n * BN;
 
     // ---- global -> LDS staging plan.  A K slice of the tile is (BM + BN) rows of 64 bytes = (BM + BN) / 16 wave-wide loads of
     // 1 KB, dealt round-robin to the 4 waves.  Each load writes 16 consecutive LDS rows; lane l fills 16-byte slot (row l/4, slot

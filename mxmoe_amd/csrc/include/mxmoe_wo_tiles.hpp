@@ -88,7 +88,7 @@ struct SkinnyWoTile {
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int M = t.M, N = t.N, K = t.K;
-    const int m0 = t.tile_m * BM, n0 = t.tile_n * BN;
+    const int m0 = t.row0 + t.tile_m * BM, n0 = t.tile_n * BN;
     const int KB = K / 128;  // k blocks (= quantisation groups) per row
     const int lm = lane & 15, lg = lane >> 4;
 
