@@ -189,11 +189,11 @@ struct MfmaTile {
         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
     // The main loop is software-pipelined by hand at the granularity of one "unit" = one k-step of one 32-channel block
-    // (FM or 2*FM MFMAs).  While the MFMAs of unit u run, the packed fragment of unit u+2 is read from LDS and the fragment of
+    // (FM or 2*FM MFMAs).  While the MFMAs of unit u run, the packed fragment of unit u+3 is read from LDS and the fragment of
     // unit u+1 is widened to MFMA operands (int4 only), so LDS latency and the unpack VALU work hide under the matrix pipe.
     // Three LDS stages let the read-ahead run into the next K slice without waiting for this iteration's barrier:
-    //   iteration kt:  start the loads of slice kt+2 into stage (kt+2)%3, units 0..U-3 on stage kt%3, wait for this wave's
-    //   loads of slice kt+1, barrier, units U-2, U-1 (whose read-ahead touches stage (kt+1)%3).
+    //   iteration kt:  start the loads of slice kt+2 into stage (kt+2)%3, units 0..U-4 on stage kt%3, wait for this wave's
+    //   loads of slice kt+1, barrier, units U-3 .. U-1 (whose read-ahead touches stage (kt+1)%3).
     constexpr int U = 2 * FN;  // units per K slice
     auto lds_a = [&](const uint8_t* st, int step, int i) { return *reinterpret_cast<const v4i*>(st + ((fa + i * 32 * kRowBytes) ^ (step << 5))); };
     auto lds_b = [&](const uint8_t* st, int step, int j) { return *reinterpret_cast<const v4i*>(st + ((fb + j * 32 * kRowBytes) ^ (step << 5))); };
@@ -219,12 +219,22 @@ struct MfmaTile {
 
     v4i alo[FM], ahi[FM];        // operands of the A fragments of the current k-step
     v4i pa[FM];                  // packed A fragments of the next k-step
-    v4i pb[2];                   // packed B fragments: slot u&1 is free once unit u is widened, and receives unit u+2
+    v4i pb[4];                   // packed B fragments of units u+1 .. u+3 (slot = unit & 3; U is a multiple of 4 or equals 4)
     v4i blo[2], bhi[2];          // operands of the B fragments of units u, u+1
 
+    // wait until at most the loads of the `newer` most recent slices of this wave are still in flight (loads retire in order)
+    auto wait_slices = [&](int newer) {
+      if (newer <= 0) {
+        vm_wait<0>();
+      } else if (kDmaTotal % kWaves == 0 || uwave + kWaves * (kDma - 1) < kDmaTotal) {
+        vm_wait<kDma>();
+      } else {
+        vm_wait<kDma - 1>();
+      }
+    };
     dma_slice(0, 0);
-    dma_slice(1, 1);  // past the end of K this reads zeros or a neighbouring row; such a slice is never consumed
-    if (kDmaTotal % kWaves == 0 || uwave + kWaves * (kDma - 1) < kDmaTotal) vm_wait<kDma>(); else vm_wait<kDma - 1>();  // slice 0 has landed
+    if (KT > 1) dma_slice(1, 1);
+    wait_slices(KT > 1 ? 1 : 0);  // slice 0 has landed
     __syncthreads();
     {
       const uint8_t* st = smem;
@@ -235,39 +245,42 @@ struct MfmaTile {
       }
       pb[0] = lds_b(st, 0, 0);
       pb[1] = lds_b(st, 0, 1);
+      pb[2] = lds_b(st, 2 / FN, 2 % FN);
       widen(pb[0], blo[0], bhi[0]);
     }
 
-    // Every iteration has the same shape, including the last two: their extra prefetch lands in LDS stages nobody consumes
-    // (buffer loads past the tile read zeros), which keeps the loop body one straight-line block.
+    // Every iteration has the same shape, including the last two, whose read-ahead touches a stage nobody filled (the
+    // fragments read there are never used); only the issue of new loads and the wait count depend on the position.
     int sidx = 0;
 #pragma unroll 1
     for (int kt = 0; kt < KT; ++kt) {
       const uint8_t* sc = smem + sidx * kStageBytes;
       const int nidx = sidx == 2 ? 0 : sidx + 1;
       const uint8_t* sn = smem + nidx * kStageBytes;
-      dma_slice(kt + 2, nidx == 2 ? 0 : nidx + 1);  // its stage was last read before the previous barrier
+      const bool more2 = kt + 2 < KT;  // no load is ever issued past the end of K: nothing may land in LDS during the epilogue
+      if (more2) dma_slice(kt + 2, nidx == 2 ? 0 : nidx + 1);  // its stage was last read before the previous barrier
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const int step = u / FN, j = u % FN;
-        if (u == U - 2) {
+        if (u == U - 3) {
           // this wave's part of slice kt+1 is in LDS (loads retire in order; only its loads of slice kt+2 may be in flight);
           // after the barrier everybody's part is
-          if (kDmaTotal % kWaves == 0 || uwave + kWaves * (kDma - 1) < kDmaTotal) vm_wait<kDma>(); else vm_wait<kDma - 1>();
+          wait_slices(more2 ? 1 : 0);
           __syncthreads();
         }
-        // read ahead: packed B fragment of unit u+2, packed A fragments of the next k-step
-        if (u + 2 < U) {
-          pb[u & 1] = lds_b(sc, (u + 2) / FN, (u + 2) % FN);
+        // read ahead (LDS latency is longer than one unit of MFMAs): packed B fragment of unit u+3, packed A fragments of the
+        // next k-step two units before they are widened
+        if (u + 3 < U) {
+          pb[(u + 3) & 3] = lds_b(sc, (u + 3) / FN, (u + 3) % FN);
         } else {
-          pb[u & 1] = lds_b(sn, 0, u + 2 - U);
+          pb[(u + 3) & 3] = lds_b(sn, (u + 3 - U) / FN, (u + 3 - U) % FN);
         }
-        if (j == FN - 2) {
+        if (j == (FN >= 3 ? FN - 3 : 0)) {
 #pragma unroll
           for (int i = 0; i < FM; ++i) pa[i] = step == 0 ? lds_a(sc, 1, i) : lds_a(sn, 0, i);
         }
         // operands of unit u+1; on the last unit of a k-step each A operand is refreshed right after its last use
-        widen(pb[(u + 1) & 1], blo[(u + 1) & 1], bhi[(u + 1) & 1]);
+        widen(pb[(u + 1) & 3], blo[(u + 1) & 1], bhi[(u + 1) & 1]);
 #pragma unroll
         for (int i = 0; i < FM; ++i) {
           mma(acc[i][j], alo[i], ahi[i], blo[u & 1], bhi[u & 1]);
