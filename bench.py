@@ -19,6 +19,10 @@ import time
 
 PEAK = {"int8": 5000.0, "fp16": 2500.0, "hbm": 8000.0}  # MI355X: TOP/s dense int8 MFMA, TFLOP/s dense fp16 MFMA, GB/s HBM3E
 
+# HBM bytes per launch of the dominant (gate_up) kernel, from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE runs scaled by the
+# same counters on a plain 256 MiB copy (summaries: profiles/fused_group_gemm_<workload>.txt, profiles/counter_calibration_copy_256MiB.txt)
+TRAFFIC = {"c2": 484864913, "c3": 792419903, "c4": 194396740}
+
 
 def build_layer(name: str, tokens: int | None):
     import torch
@@ -64,22 +68,46 @@ def time_layer(layer, steps: int, warmup: int):
     return wall / steps, up, dn
 
 
+def launch_duration(plan, n: int = 20) -> float:
+    """Average duration (ms) of one launch: n back-to-back launches between two HIP events on the launch stream (no event
+    between launches, so dispatch gaps of a few microseconds do not count as kernel time)."""
+    import torch
+
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    plan.run()
+    torch.cuda.synchronize()
+    a.record()
+    for _ in range(n):
+        plan.run()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / n
+
+
+def _default_tokens(name: str) -> int:
+    from mxmoe_amd import synth
+
+    return synth.CONFIGS[name].tokens if name in synth.CONFIGS else -1
+
+
 def roofline_of(cfg, layer, up_ms: float, dn_ms: float):
     """Roofline entry of the dominant launch.  Compute-bound layers (w-a formats at thousands of tokens): ops of the
     gate_up launch against the int8 (or fp16) MFMA peak.  Skinny weight-only layers: algorithmic bytes against HBM."""
     st = layer.state
     by = layer.algorithmic_bytes()
-    name, ms, plan = ("gate_up", up_ms, st["gg1"]) if up_ms >= dn_ms else ("down", dn_ms, st["gg2"])
+    name, plan = ("gate_up", st["gg1"]) if up_ms >= dn_ms else ("down", st["gg2"])
+    ms = launch_duration(plan)
+    traffic = TRAFFIC.get(cfg.name) if name == "gate_up" and cfg.tokens == _default_tokens(cfg.name) else None
     fmts = {q[:2] for q in plan.qparams}
     compute_bound = cfg.tokens * cfg.topk / cfg.num_experts >= 128
     if compute_bound:
         peak = PEAK["fp16"] if all(a >= 16 for a, _ in fmts) else PEAK["int8"]
         ach = plan.ops / (ms * 1e-3) / 1e12
         return {"kernel": f"fused_group_gemm[{name}]", "bound": "mfma", "achieved": round(ach, 2), "peak": peak, "unit": "TFLOP/s",
-                "frac": round(ach / peak, 4), "traffic": None, "launch_us": round(ms * 1e3, 2), "algorithmic_bytes": by[name]["total"]}
+                "frac": round(ach / peak, 4), "traffic": traffic, "launch_us": round(ms * 1e3, 2), "algorithmic_bytes": by[name]["total"]}
     ach = by[name]["total"] / (ms * 1e-3) / 1e9
     return {"kernel": f"fused_group_gemm[{name}]", "bound": "hbm", "achieved": round(ach, 1), "peak": PEAK["hbm"], "unit": "GB/s",
-            "frac": round(ach / PEAK["hbm"], 4), "traffic": None, "launch_us": round(ms * 1e3, 2), "algorithmic_bytes": by[name]["total"]}
+            "frac": round(ach / PEAK["hbm"], 4), "traffic": traffic, "launch_us": round(ms * 1e3, 2), "algorithmic_bytes": by[name]["total"]}
 
 
 def cpu_baseline(cfg, budget_s: float = 20.0):
@@ -146,6 +174,8 @@ def main() -> int:
     ap.add_argument("--also", default="c3,c4", help="comma-separated extra workloads reported under 'also' (empty to skip)")
     ap.add_argument("--tokens", type=int, default=None)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", type=int, default=0, metavar="BYTES",
+                    help="instead of the benchmark, run a plain device copy of BYTES bytes 5 times (reference point for the FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (the layer would shard by expert; see DESIGN.md). Use --gpus 1.", file=sys.stderr)
@@ -156,6 +186,15 @@ def main() -> int:
     if not torch.cuda.is_available():
         print("bench.py needs a GPU (no CPU fallback exists for the HIP kernels)", file=sys.stderr)
         return 2
+    if args.copy_calibration:
+        src = torch.empty(args.copy_calibration, dtype=torch.uint8, device="cuda").fill_(1)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_bytes": args.copy_calibration, "copies": 5}))
+        return 0
     from mxmoe_amd import synth
 
     cfg, layer, main_res = run_workload(args.workload, args.steps, args.warmup, args.tokens)
