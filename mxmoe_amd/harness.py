@@ -53,8 +53,12 @@ def make_problem(entry: dict, gen: torch.Generator, device="cuda", keep_ref: boo
     """Random fp16 operands for one workload entry, quantised and packed for its format (QInput::from_fp16)."""
     m, n, k = entry["shape"]
     qp = (entry["a_bits"], entry["w_bits"], entry["gsize"], bool(entry["sym"]))
-    a = (torch.rand(m, k, generator=gen, dtype=torch.float32) * 2 - 1).to(torch.float16).to(device)
-    b = (torch.rand(n, k, generator=gen, dtype=torch.float32) * 2 - 1).to(torch.float16).to(device)
+    if gen is None:  # values drawn on the device (timing-only problems)
+        a = torch.rand(m, k, dtype=torch.float16, device=device) * 2 - 1
+        b = torch.rand(n, k, dtype=torch.float16, device=device) * 2 - 1
+    else:
+        a = (torch.rand(m, k, generator=gen, dtype=torch.float32) * 2 - 1).to(torch.float16).to(device)
+        b = (torch.rand(n, k, generator=gen, dtype=torch.float32) * 2 - 1).to(torch.float16).to(device)
     pw = quantize_and_pack(b, qp)
     prob = {"size": (m, n, k), "q": qp, "B": pw.data, "sb": pw.scale, "C": torch.zeros(m, n, dtype=torch.float16, device=device)}
     if qp[0] < 16:

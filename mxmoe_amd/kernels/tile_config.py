@@ -3,7 +3,7 @@
 `TileConfig` / `QConfig` / `NO_QUANT` keep the fields (and therefore the dataclass `repr`, which is the key of the
 kernel-profile table) of mxmoe/kernels/tile_config.py:122-286.  What changes is the meaning the hardware gives them:
 WM x WN x WK counts 64-lane wavefronts (always 4 per workgroup here), MMA names an MFMA instruction, STAGE is the number of
-LDS buffers of the register-prefetched pipeline, and the candidate lists are those compiled for gfx950.
+LDS ring slots of the DMA pipeline (3 for the MFMA tiles; 2 = the register double buffer of the skinny tiles), and the candidate lists are those compiled for gfx950.
 """
 from __future__ import annotations
 
@@ -180,8 +180,8 @@ class TileConfig:
                 raise ValueError(f"{self!r}: skinny weight-only tiles are 16 x (64k) x 128")
             return
         k_elems = {"MFMA_F32_32x32x16_F16": 32, "MFMA_I32_32x32x32_I8": 64, "MFMA_I32_32x32x32_I8_FROM_I4": 128}[self.MMA]
-        if self.BK != k_elems or self.STAGE != 2 or self.WK != 1 or (self.BM // self.WM) % 32 or (self.BN // self.WN) % 32:
-            raise ValueError(f"{self!r}: unsupported shape for {self.MMA} (BK must be {k_elems}, STAGE 2, wave tile a multiple of 32x32)")
+        if self.BK != k_elems or self.STAGE != 3 or self.WK != 1 or (self.BM // self.WM) % 32 or (self.BN // self.WN) % 32:
+            raise ValueError(f"{self!r}: unsupported shape for {self.MMA} (BK must be {k_elems}, STAGE 3, wave tile a multiple of 32x32)")
 
 
 def get_info_from_qcfg_str(qcfg: str):
@@ -220,7 +220,7 @@ def get_possible_tile_list(arch: str, qcfg: str) -> list:
         return [_with_q(TileConfig(BM=16, BN=bn, BK=128, WM=1, WN=4, WK=1, STAGE=2, MMA=mma), qcfg) for bn in (128, 64, 256)]
     bk = {"MFMA_F32_32x32x16_F16": 32, "MFMA_I32_32x32x32_I8": 64, "MFMA_I32_32x32x32_I8_FROM_I4": 128}[mma]
     shapes = [(128, 256, 2, 2), (64, 256, 1, 4), (32, 256, 1, 4), (128, 128, 2, 2), (256, 128, 2, 2)]
-    return [_with_q(TileConfig(BM=bm, BN=bn, BK=bk, WM=wm, WN=wn, WK=1, STAGE=2, MMA=mma), qcfg) for bm, bn, wm, wn in shapes]
+    return [_with_q(TileConfig(BM=bm, BN=bn, BK=bk, WM=wm, WN=wn, WK=1, STAGE=3, MMA=mma), qcfg) for bm, bn, wm, wn in shapes]
 
 
 _FIELD = re.compile(r"(BM|BN|BK|WM|WN|WK|STAGE|SPLITK)=(-?\d+)")

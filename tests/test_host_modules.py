@@ -33,11 +33,11 @@ def test_qconfig_schema_roundtrip(tmp_path):
 def test_tile_config_repr_is_the_profile_table_key_shape():
     t = tile_config.get_possible_tile_list("gfx950", "w4a4_g-1_sym")[0]
     r = repr(t)
-    assert r.startswith("TileConfig(BM=128, BN=256, BK=128, WM=2, WN=2, WK=1, STAGE=2, SPLITK=-1, MMA='MFMA_I32_32x32x32_I8_FROM_I4', QCFGA=QConfig(T_PACK='half', QBITS=4")
+    assert r.startswith("TileConfig(BM=128, BN=256, BK=128, WM=2, WN=2, WK=1, STAGE=3, SPLITK=-1, MMA='MFMA_I32_32x32x32_I8_FROM_I4', QCFGA=QConfig(T_PACK='half', QBITS=4")
     if REF_TABLE.exists():                                                 # same field order as the keys of the reference's table
         ref_key = next(iter(json.loads(REF_TABLE.read_text())["w4a4_g-1_sym"]["3"]))
         assert re.findall(r"(\w+)=", ref_key) == re.findall(r"(\w+)=", r)
-    assert t.num_warps == 4 and t.smem_bytes_tile() == 2 * (128 + 256) * 64
+    assert t.num_warps == 4 and t.smem_bytes_tile() == 3 * (128 + 256) * 64
     assert tile_config.get_info_from_qcfg_str("w3a16_g128_asym") == (3, 16, 128, False)
     with pytest.raises(ValueError):
         tile_config.TileConfig(BM=128, BN=256, BK=64, WM=2, WN=4, MMA="MFMA_I32_32x32x32_I8").validate()   # 8 waves
@@ -114,3 +114,91 @@ def test_synthetic_configs_match_the_baseline_shapes():
     assert len(synth.draw_formats(c4)) == 65
     w13, w2 = synth.expert_weights(c4, 64)
     assert w13.shape == (2 * 2816, 2048) and w2.shape == (2048, 2816)
+
+
+# ---- kernel-profile table: consumer on the reference's schema, producer pieces ----
+
+def _ref_table():
+    import json
+    from pathlib import Path
+
+    fx = json.loads((Path(__file__).parent / "golden" / "perf_table_sm89_excerpt.json").read_text())
+    return fx, fx["entries"]
+
+
+def test_perf_table_reference_schema():
+    fx, table = _ref_table()
+    assert len(fx["qcfgs"]) == 19
+    assert fx["slots"]["w8a8_g-1_sym"] == ["1", "2", "3", "4"] and fx["slots"]["w4a16_g128_asym"] == ["1"]
+    for q, slots in table.items():
+        for s, tiles in slots.items():
+            for key, rec in tiles.items():
+                assert key.startswith("TileConfig(BM=") and set(rec) == {"first_iter_cost", "inc", "stderr"}
+
+
+def test_perf_table_keys_round_trip_through_tile_config():
+    """repr(TileConfig) is the table key: a key parsed back into a TileConfig must print as the same key."""
+    from mxmoe_amd.kernels.tile_config import parse_tile_repr
+
+    _, table = _ref_table()
+    for q, slot in (("w8a8_g-1_sym", "3"), ("w4a4_g-1_sym", "3")):
+        for key in table[q][slot]:
+            (t,) = parse_tile_repr(key, q)
+            assert repr(t) == key
+
+
+def test_get_runtime_cost_known_answers():
+    from mxmoe_amd.kernels.tile_config import parse_tile_repr
+    from mxmoe_amd.perf_table import ProblemShape, get_runtime_cost, slot_of, table_key
+
+    _, table = _ref_table()
+    assert slot_of("w4a16_g128_asym") == "1" and slot_of("w8a8_g-1_sym") == "3"
+    assert table_key("w2a16_g128_asym") == "w2a16_g128_asym_accfp16" and table_key("w4a4_g-1_sym") == "w4a4_g-1_sym"
+    strategies = ["w4a4_g-1_sym", "w8a8_g-1_sym"]
+    keys = {q: list(table[q]["3"])[:2] for q in strategies}
+    tiles = {q: [parse_tile_repr(k, q)[0] for k in keys[q]] for q in strategies}
+    work = [[ProblemShape(546, 2816, 2048), ProblemShape(546, 2048, 1408)], [ProblemShape(1, 2816, 2048), ProblemShape(1, 2048, 1408)]]
+    combos, cost = get_runtime_cost(work, strategies, table, tile_cfgs=tiles)
+    assert len(combos) == 4 and len(cost) == 2 and len(cost[0]) == 2 and len(cost[0][0]) == 2 and len(cost[0][0][0]) == 4
+    # all four tiles are 128 x 128: ceil(546/128) * (2816/128) = 5 * 22 = 110 tiles; (2048/128) = 16 -> 80; one row -> 22 and 16
+    inc = {q: [table[q]["3"][k]["inc"] for k in keys[q]] for q in strategies}
+    for ci, (t4, t8) in enumerate(combos):
+        i4, i8 = tiles["w4a4_g-1_sym"].index(t4), tiles["w8a8_g-1_sym"].index(t8)
+        assert cost[0][0][0][ci] == inc["w4a4_g-1_sym"][i4] * 110
+        assert cost[0][1][1][ci] == inc["w8a8_g-1_sym"][i8] * 80
+        assert cost[1][0][1][ci] == inc["w8a8_g-1_sym"][i8] * 22
+        assert cost[1][1][0][ci] == inc["w4a4_g-1_sym"][i4] * 16
+    assert inc["w4a4_g-1_sym"][0] == 0.004520000000000001  # value of the reference's table itself
+
+
+def test_perf_table_alias_and_weight_only_slot():
+    from mxmoe_amd.perf_table import ProblemShape, get_runtime_cost
+
+    _, table = _ref_table()
+
+    class Tile:
+        def __init__(self, key, bm, bn):
+            self.key, self.BM, self.BN, self.num_warps = key, bm, bn, 4
+
+        def __repr__(self):
+            return self.key
+
+    key = list(table["w2a16_g128_asym_accfp16"]["1"])[3]  # BM=64, BN=128
+    _, cost = get_runtime_cost([[ProblemShape(100, 256, 4096)]], ["w2a16_g128_asym"], table, tile_cfgs={"w2a16_g128_asym": [Tile(key, 64, 128)]})
+    assert cost == [[[[0.013920000000000002 * 4]]]]
+
+
+def test_perf_table_fit_and_sweep_shapes():
+    from mxmoe_amd.kernels.tile_config import get_possible_tile_list
+    from mxmoe_amd.perf_table import ProblemShape, linear_fit, sweep_entry
+
+    icpt, slope, err = linear_fit([1, 2, 3, 4], [3.0, 5.0, 7.0, 9.0])
+    assert abs(icpt - 1.0) < 1e-12 and abs(slope - 2.0) < 1e-12 and err < 1e-12
+    _, slope, err = linear_fit([0, 1, 2], [0.0, 1.0, 0.0])
+    assert abs(slope) < 1e-12 and abs(err - (2.0 / 3 / 1 / 2) ** 0.5) < 1e-12  # rss = 2/3, n-2 = 1, sxx = 2
+    for q in ("w4a4_g-1_sym", "w4a16_g128_asym"):
+        for t in get_possible_tile_list("gfx950", q):
+            for w in (1, 3):
+                e = sweep_entry(t, q, 2048, w, cus=256)
+                m, n, k = e["shape"]
+                assert ProblemShape(m, n, k).num_tiles(t) == 256 * w and k == 2048
