@@ -18,6 +18,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <utility>
+
 #include <type_traits>
 
 #include "mxmoe_types.h"
@@ -94,10 +96,32 @@ __device__ __forceinline__ void vm_wait() {
   asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
 }
 
-// LDS byte offset of 16-byte chunk `c` (0..3) of tile row `r`.  Rows are 64 bytes; the chunk index is XORed with
-// bits 1..2 of the row so rows r, r+1 (which share a 128-byte bank line) and the next three row pairs all land
-// on different 16-byte groups.
-__device__ __forceinline__ int lds_chunk_off(int r, int c) { return r * kRowBytes + ((c ^ ((r >> 1) & 3)) << 4); }
+// Swizzle of the four 16-byte chunks of a 64-byte LDS row.  A wave-wide 16-byte read is served 16 lanes (256 bytes, all 64
+// banks) per cycle; lanes 0..15 read the same chunk of 16 consecutive rows, so rows r, r+4, r+8, r+12 (same position inside
+// a 256-byte bank line) must store that chunk at four different places.  XORing the chunk index with row bits 1..2 separates
+// every second row, bit 3 on top separates the two halves of the 16 rows; the same map is conflict-free if the hardware
+// serves 8 lanes (128 bytes) per cycle.
+__device__ __forceinline__ int lds_swizzle(int r) { return ((r >> 1) & 3) ^ ((r >> 3) & 1); }
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>): a loop whose index is a compile-time constant in the body
+template <int... Is, class F>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, Is...>, F&& f) {
+  (f(std::integral_constant<int, Is>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(std::make_integer_sequence<int, N>{}, f);
+}
+
+// Scheduling pattern of one pipeline unit: KMF times (one MFMA, then an even share of the unit's NV VALU instructions).
+template <int NV, int KMF, int M>
+__device__ __forceinline__ void sched_mfma_valu() {
+  if constexpr (M < KMF) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    if constexpr (NV > 0) __builtin_amdgcn_sched_group_barrier(0x002, (NV + KMF - 1 - M) / KMF, 0);
+    sched_mfma_valu<NV, KMF, M + 1>();
+  }
+}
 
 template <Op OP>
 struct OpTraits;
@@ -162,20 +186,24 @@ struct MfmaTile {
     for (int i = 0; i < kDma; ++i) {
       const int ii = uwave + kWaves * i;
       const int r = (ii < kDmaA ? ii : ii - kDmaA) * 16 + (lane >> 2);
-      dma_voff[i] = r * (int)row_bytes + (((lane & 3) ^ ((r >> 1) & 3)) << 4);
+      dma_voff[i] = r * (int)row_bytes + (((lane & 3) ^ lds_swizzle(r)) << 4);
     }
-    auto dma_slice = [&](int kt, int stage) {
-      const int koff = kt * kRowBytes;
-#pragma unroll
-      for (int i = 0; i < kDma; ++i) {
-        const int ii = uwave + kWaves * i;
-        if (kDmaTotal % kWaves == 0 || ii < kDmaTotal) dma16_to_lds(ii < kDmaA ? rs_a : rs_b, lds_base + stage * kStageBytes + ii * 1024, dma_voff[i], koff);
+    // load i of this wave (i < kDma) of the slice at byte offset koff, into stage `stage`; `live` = false turns it into a load of
+    // zero bytes (nothing is fetched, nothing lands in LDS, the load still counts for s_waitcnt like any other)
+    auto dma_one = [&](int i, int koff, int stage, bool live) {
+      const int ii = uwave + kWaves * i;
+      if (kDmaTotal % kWaves == 0 || ii < kDmaTotal) {
+        v4i rs = ii < kDmaA ? rs_a : rs_b;
+        if (!live) rs[2] = 0;
+        dma16_to_lds(rs, lds_base + stage * kStageBytes + ii * 1024, dma_voff[i], koff);
       }
     };
+    // whether this wave has a load number kDma-1 (the 1 KB pieces of a slice do not always divide evenly among the waves)
+    const bool has_last = kDmaTotal % kWaves == 0 || uwave + kWaves * (kDma - 1) < kDmaTotal;
 
     // ---- LDS -> MFMA fragment plan: lane reads row (lane & 31) of a 32-row block, chunk 2*ks + (lane >> 5) ----
     const int lrow = lane & 31;
-    const int swz = (lrow >> 1) & 3;
+    const int swz = lds_swizzle(lrow);
     const int c0 = (((lane >> 5) ^ swz) << 4);  // k-step 0; k-step 1 is c0 ^ 32
     const int fa = (wm * TM + lrow) * kRowBytes + c0;
     const int fb = BM * kRowBytes + (wn * TN + lrow) * kRowBytes + c0;
@@ -189,107 +217,129 @@ struct MfmaTile {
         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
     // The main loop is software-pipelined by hand at the granularity of one "unit" = one k-step of one 32-channel block
-    // (FM or 2*FM MFMAs).  While the MFMAs of unit u run, the packed fragment of unit u+3 is read from LDS and the fragment of
-    // unit u+1 is widened to MFMA operands (int4 only), so LDS latency and the unpack VALU work hide under the matrix pipe.
-    // Three LDS stages let the read-ahead run into the next K slice without waiting for this iteration's barrier:
-    //   iteration kt:  start the loads of slice kt+2 into stage (kt+2)%3, units 0..U-4 on stage kt%3, wait for this wave's
-    //   loads of slice kt+1, barrier, units U-3 .. U-1 (whose read-ahead touches stage (kt+1)%3).
+    // (FM or 2*FM MFMAs).  While the MFMAs of unit u run, the packed fragment of unit u+LA is read from LDS and the fragment of
+    // unit u+1 is widened to MFMA operands (int4 only); the activation-side operands of the next k-step are read at the first
+    // unit of a k-step and widened, a few registers per unit, into a second operand buffer during its last units.  So LDS
+    // latency (which grows well beyond its idle value while direct-to-LDS loads are landing) and the unpack VALU work hide
+    // under the matrix pipe, and the VALU work is spread evenly between the MFMAs.
+    // Three LDS stages let the read-ahead run into the next K slice:
+    //   iteration kt:  the loads of slice kt+2 into stage (kt+2)%3 are issued one or two per unit (a burst of them delays the
+    //   LDS reads of every wave on the CU); units 0..UB-1 touch stage kt%3 only; at unit UB the wave waits for its loads of
+    //   slice kt+1 and passes the barrier; the remaining units also read stage (kt+1)%3.
+    // The loop body is branch-free: past the end of K the loads are zero-length (they fetch nothing) and the read-ahead touches
+    // a stage whose contents are never used.
     constexpr int U = 2 * FN;  // units per K slice
+    static_assert(FN == 2 || FN == 4, "the fragment ring below assumes 4 or 8 units per K slice");
+    constexpr int LA = U == 8 ? 5 : 3;               // units of read-ahead of the packed B fragments
+    constexpr int RB = LA > 3 ? 8 : 4;               // ring slots for them (slot = unit % RB)
+    constexpr int UB = (U - LA < FN) ? U - LA : FN;  // unit that holds the barrier
+    constexpr int NW = FN >= 4 ? 2 : 1;              // units over which the next k-step's A operands are widened
+    constexpr int kAPiece = FM * 4 / NW;             // dwords of packed A widened per such unit
+    constexpr int kOps = OP == Op::I4 ? 2 : 1;       // operand registers per fragment (low / high nibbles)
+    // load i of a slice is issued at the top of unit i * U / kDma; at the barrier unit the loads of the current iteration issued
+    // so far are the only ones that may still be in flight
+    constexpr int kIssuedAtBarrier = ((UB + 1) * kDma + U - 1) / U;
+    constexpr bool kLastBeforeBarrier = (kDma - 1) * U / kDma <= UB;
     auto lds_a = [&](const uint8_t* st, int step, int i) { return *reinterpret_cast<const v4i*>(st + ((fa + i * 32 * kRowBytes) ^ (step << 5))); };
     auto lds_b = [&](const uint8_t* st, int step, int j) { return *reinterpret_cast<const v4i*>(st + ((fb + j * 32 * kRowBytes) ^ (step << 5))); };
-    auto widen = [&](const v4i& p, v4i& lo, v4i& hi) {
+    // nibble n of a byte -> int8 holding 16 * signed(n): even elements via (x << 4), odd via x, both masked to the high nibbles
+    auto widen = [&](const v4i& p, v4i* o) {
       if constexpr (OP == Op::I4) {
-        // nibble n of a byte -> int8 holding 16 * signed(n): even elements via (x << 4), odd via x, both masked to the high nibbles
-        lo = (p << 4) & (int)0xF0F0F0F0;
-        hi = p & (int)0xF0F0F0F0;
+        o[0] = (p << 4) & (int)0xF0F0F0F0;
+        o[1] = p & (int)0xF0F0F0F0;
       } else {
-        lo = p;
+        o[0] = p;
       }
     };
-    auto mma = [&](Acc& c, const v4i& alo, const v4i& ahi, const v4i& blo, const v4i& bhi) {
+    auto mma = [&](Acc& c, const v4i* a, const v4i* b) {
       if constexpr (OP == Op::I8) {
-        c = __builtin_amdgcn_mfma_i32_32x32x32_i8(blo, alo, c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_i32_32x32x32_i8(b[0], a[0], c, 0, 0, 0);
       } else if constexpr (OP == Op::I4) {
-        c = __builtin_amdgcn_mfma_i32_32x32x32_i8(blo, alo, c, 0, 0, 0);
-        c = __builtin_amdgcn_mfma_i32_32x32x32_i8(bhi, ahi, c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_i32_32x32x32_i8(b[0], a[0], c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_i32_32x32x32_i8(b[1], a[1], c, 0, 0, 0);
       } else {
-        c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, blo), __builtin_bit_cast(v8h, alo), c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, b[0]), __builtin_bit_cast(v8h, a[0]), c, 0, 0, 0);
       }
     };
 
-    v4i alo[FM], ahi[FM];        // operands of the A fragments of the current k-step
-    v4i pa[FM];                  // packed A fragments of the next k-step
-    v4i pb[4];                   // packed B fragments of units u+1 .. u+3 (slot = unit & 3; U is a multiple of 4 or equals 4)
-    v4i blo[2], bhi[2];          // operands of the B fragments of units u, u+1
+    v4i aop[2][FM][kOps];  // A operands of the current k-step (buffer = k-step parity) and of the next one
+    v4i pa[FM];            // packed A fragments of the next k-step (int4 only)
+    v4i pb[RB];            // packed B fragments of units u+1 .. u+LA
+    v4i bop[2][kOps];      // B operands of units u, u+1
 
-    // wait until at most the loads of the `newer` most recent slices of this wave are still in flight (loads retire in order)
-    auto wait_slices = [&](int newer) {
-      if (newer <= 0) {
-        vm_wait<0>();
-      } else if (kDmaTotal % kWaves == 0 || uwave + kWaves * (kDma - 1) < kDmaTotal) {
-        vm_wait<kDma>();
-      } else {
-        vm_wait<kDma - 1>();
-      }
-    };
-    dma_slice(0, 0);
-    if (KT > 1) dma_slice(1, 1);
-    wait_slices(KT > 1 ? 1 : 0);  // slice 0 has landed
-    __syncthreads();
-    {
-      const uint8_t* st = smem;
+    // prologue: slices 0 and 1 in flight, wait for slice 0 (loads retire in order), prime the fragment pipeline
 #pragma unroll
-      for (int i = 0; i < FM; ++i) {
-        pa[i] = lds_a(st, 0, i);
-        widen(pa[i], alo[i], ahi[i]);
-      }
-      pb[0] = lds_b(st, 0, 0);
-      pb[1] = lds_b(st, 0, 1);
-      pb[2] = lds_b(st, 2 / FN, 2 % FN);
-      widen(pb[0], blo[0], bhi[0]);
-    }
+    for (int i = 0; i < kDma; ++i) dma_one(i, 0, 0, true);
+#pragma unroll
+    for (int i = 0; i < kDma; ++i) dma_one(i, kRowBytes, 1, KT > 1);
+    if (has_last) vm_wait<kDma>(); else vm_wait<kDma - 1>();
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < FM; ++i) widen(lds_a(smem, 0, i), aop[0][i]);
+#pragma unroll
+    for (int u = 1; u < LA; ++u) pb[u] = lds_b(smem, u / FN, u % FN);
+    widen(lds_b(smem, 0, 0), bop[0]);
 
-    // Every iteration has the same shape, including the last two, whose read-ahead touches a stage nobody filled (the
-    // fragments read there are never used); only the issue of new loads and the wait count depend on the position.
     int sidx = 0;
 #pragma unroll 1
     for (int kt = 0; kt < KT; ++kt) {
       const uint8_t* sc = smem + sidx * kStageBytes;
       const int nidx = sidx == 2 ? 0 : sidx + 1;
       const uint8_t* sn = smem + nidx * kStageBytes;
-      const bool more2 = kt + 2 < KT;  // no load is ever issued past the end of K: nothing may land in LDS during the epilogue
-      if (more2) dma_slice(kt + 2, nidx == 2 ? 0 : nidx + 1);  // its stage was last read before the previous barrier
+      // slice kt+2 goes into the stage that was last read before the previous iteration's barrier
+      const int nstage = nidx == 2 ? 0 : nidx + 1;
+      const int nkoff = __builtin_amdgcn_readfirstlane((kt + 2) * kRowBytes);
+      const bool nlive = kt + 2 < KT;
+      static_for<U>([&](auto uc) {
+        constexpr int u = decltype(uc)::value;
+        constexpr int step = u / FN, j = u % FN;
+        static_for<kDma>([&](auto ic) {
+          constexpr int i = decltype(ic)::value;
+          if constexpr (i * U / kDma == u) dma_one(i, nkoff, nstage, nlive);
+        });
+        // reads of this slice's stage: packed B fragment of unit u+LA, A fragments of k-step 1
+        if (u + LA < U) pb[(u + LA) % RB] = lds_b(sc, (u + LA) / FN, (u + LA) % FN);
+        if (u == 0) {
 #pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const int step = u / FN, j = u % FN;
-        if (u == U - 3) {
-          // this wave's part of slice kt+1 is in LDS (loads retire in order; only its loads of slice kt+2 may be in flight);
-          // after the barrier everybody's part is
-          wait_slices(more2 ? 1 : 0);
+          for (int i = 0; i < FM; ++i) {
+            if constexpr (OP == Op::I4) pa[i] = lds_a(sc, 1, i); else aop[1][i][0] = lds_a(sc, 1, i);
+          }
+        }
+        if (u == UB) {
+          // this wave's part of slice kt+1 is in LDS (only its loads of slice kt+2 may be in flight); after the barrier
+          // everybody's part is, and everybody is done reading the stage that the next iteration's loads overwrite
+          if (!kLastBeforeBarrier || has_last) vm_wait<kIssuedAtBarrier>(); else vm_wait<kIssuedAtBarrier - 1>();
           __syncthreads();
         }
-        // read ahead (LDS latency is longer than one unit of MFMAs): packed B fragment of unit u+3, packed A fragments of the
-        // next k-step two units before they are widened
-        if (u + 3 < U) {
-          pb[(u + 3) & 3] = lds_b(sc, (u + 3) / FN, (u + 3) % FN);
-        } else {
-          pb[(u + 3) & 3] = lds_b(sn, (u + 3 - U) / FN, (u + 3 - U) % FN);
-        }
-        if (j == (FN >= 3 ? FN - 3 : 0)) {
+        // reads of the next slice's stage
+        if (u + LA >= U) pb[(u + LA) % RB] = lds_b(sn, (u + LA - U) / FN, (u + LA - U) % FN);
+        if (u == FN) {
 #pragma unroll
-          for (int i = 0; i < FM; ++i) pa[i] = step == 0 ? lds_a(sc, 1, i) : lds_a(sn, 0, i);
+          for (int i = 0; i < FM; ++i) {
+            if constexpr (OP == Op::I4) pa[i] = lds_a(sn, 0, i); else aop[0][i][0] = lds_a(sn, 0, i);
+          }
         }
-        // operands of unit u+1; on the last unit of a k-step each A operand is refreshed right after its last use
-        widen(pb[(u + 1) & 3], blo[(u + 1) & 1], bhi[(u + 1) & 1]);
+        // operands of unit u+1, and this unit's share of the next k-step's A operands
+        widen(pb[(u + 1) % RB], bop[(u + 1) & 1]);
+        if constexpr (OP == Op::I4) {
+          if (j >= FN - NW) {
 #pragma unroll
-        for (int i = 0; i < FM; ++i) {
-          mma(acc[i][j], alo[i], ahi[i], blo[u & 1], bhi[u & 1]);
-          if (j == FN - 1) widen(pa[i], alo[i], ahi[i]);
+            for (int d = (j - (FN - NW)) * kAPiece; d < (j - (FN - NW) + 1) * kAPiece; ++d) {
+              aop[step ^ 1][d / 4][0][d % 4] = (pa[d / 4][d % 4] << 4) & (int)0xF0F0F0F0;
+              aop[step ^ 1][d / 4][1][d % 4] = pa[d / 4][d % 4] & (int)0xF0F0F0F0;
+            }
+          }
         }
+#pragma unroll
+        for (int i = 0; i < FM; ++i) mma(acc[i][j], aop[step][i], bop[u & 1]);
+        // issue order inside the unit: LDS reads first, then the VALU work dealt evenly between the MFMAs
+        __builtin_amdgcn_sched_group_barrier(0x100, 1 + FM, 0);
+        sched_mfma_valu<(OP == Op::I4 ? 12 + (j >= FN - NW ? 3 * kAPiece : 0) : 0), kOps * FM, 0>();
         __builtin_amdgcn_sched_barrier(0);  // keep the units in program order: the pipeline above is the schedule
-      }
+      });
       sidx = nidx;
     }
+    vm_wait<0>();  // nothing may still land in LDS once the epilogue reuses it
 
     // ---- epilogue.  Lane holds token m = lane & 31 and channels 8*(r/4) + 4*(lane >> 5) + (r & 3) of each 32x32 block.
     // The scaled fp16 results go through a per-wave LDS patch laid out [token][channel] so that the global stores are 16 bytes
