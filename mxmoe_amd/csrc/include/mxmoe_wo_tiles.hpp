@@ -1,7 +1,9 @@
 // Skinny weight-only tiles (w4a16 / w3a16, group 128) for experts that receive a handful of tokens.
 //
 // These problems are HBM-bound: every packed weight is read exactly once and the work is arranged around that
-// stream.  Counterpart of the reference's cta_gemm_wxa16g128 with BM = 16 tiles
+// stream.  A workgroup owns 16 tokens x BN channels; its 4 waves split K into contiguous quarters, keep their quarter of the
+// activations in registers and stream the packed weights through a deep register ring (no LDS and no barrier in the loop);
+// the four partial sums meet in LDS at the end and are added in a fixed order.  Counterpart of the reference's cta_gemm_wxa16g128 with BM = 16 tiles
 // (mxmoe/kernels/src/include/cta_gemm.cuh:292-421, dequant mxmoe/kernels/src/include/quantize.cuh:134-214).
 //
 // Packed weight layout (own format, produced by mxmoe_amd.pack): [N/16][K/128][64 lanes][WBITS dwords].
@@ -26,17 +28,20 @@
 
 namespace mxmoe {
 
-template <int WBITS_, int BN_, int KC_ = 1024>
+template <int WBITS_, int BN_>
 struct SkinnyWoTile {
-  static constexpr int WBITS = WBITS_, BM = 16, BN = BN_, KC = KC_;
+  static constexpr int WBITS = WBITS_, BM = 16, BN = BN_;
   static_assert(WBITS == 4 || WBITS == 3, "w4 / w3 only");
-  static_assert(BN % 64 == 0, "BN rows are dealt to 4 waves in 16-row blocks");
-  static constexpr int R = BN / 64;                  // 16-row blocks per wave
-  static constexpr int kXStride = KC * 2 + 16;       // bytes per activation row in LDS (+16 so 8 rows cover 8 bank groups)
-  static constexpr int kLdsBytes = 16 * kXStride;
-  static constexpr int kAccRegs = R * 4;
-  static constexpr int kLaneBytes = WBITS * 4;       // packed bytes per lane per (row block, k block)
+  static_assert(BN % 64 == 0, "the final reduction deals 16-channel blocks to 4 waves");
+  static constexpr int NB = BN / 16;                 // 16-channel blocks per tile
+  static constexpr int KP = 4;                       // k blocks (128 wide) per pass of a wave: their activations live in registers
+  static constexpr int kRedBytes = kWaves * NB * 64 * 16;  // per-wave partial sums for the final reduction
+  static constexpr int kScaleBytes = NB * KP * 64;         // per-wave patch of (scale, zero) pairs of one pass
+  static constexpr int kLdsBytes = kRedBytes + kWaves * kScaleBytes;
+  static constexpr int kAccRegs = NB * 4;
+  static constexpr int kLaneBytes = WBITS * 4;       // packed bytes per lane per (channel block, k block)
   static constexpr int kBlockBytes = 64 * kLaneBytes;
+  static constexpr int kRing = 12;                   // packed blocks in flight per wave
 
   struct WReg {
     int d[WBITS];
@@ -48,26 +53,25 @@ struct SkinnyWoTile {
       const v4i v = gload<v4i>(p);
       w.d[0] = v[0]; w.d[1] = v[1]; w.d[2] = v[2]; w.d[3] = v[3];
     } else {
-      // three dword loads (4-byte aligned); a 16-byte vector load would read past the end of the last block
-      w.d[0] = gload<int>(p); w.d[1] = gload<int>(p + 4); w.d[2] = gload<int>(p + 8);
+      typedef int v3i __attribute__((ext_vector_type(3)));
+      const v3i v = gload<v3i>(p);  // 12 bytes: a 16-byte load would read past the end of the last block
+      w.d[0] = v[0]; w.d[1] = v[1]; w.d[2] = v[2];
     }
     return w;
   }
 
-  // 8 packed values of one dword -> 8 fp16 integers in k order.
+  // 8 packed values of one dword -> 8 fp16 numbers in k order, each still carrying the bias of its magic constant:
+  // 0x6400 | q is the fp16 number 1024 + q (elements 0, 1, 4, 5), 0x5400 | (q << 4) is 64 + q (elements 2, 3, 6, 7).
+  // The biases are taken out of the 128-wide partial sum instead of out of every weight (see pass()).
   template <int MASK_LO, int MASK_HI>
   __device__ static __forceinline__ v8h cvt8(int d) {
-    const v2h k1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
-    const v2h k64 = {(_Float16)64.0f, (_Float16)64.0f};
     const int d8 = (int)((unsigned)d >> 8);
-    const v2h h0 = __builtin_bit_cast(v2h, (d & MASK_LO) | 0x64006400) - k1024;
-    const v2h h1 = __builtin_bit_cast(v2h, (d & MASK_HI) | 0x54005400) - k64;
-    const v2h h2 = __builtin_bit_cast(v2h, (d8 & MASK_LO) | 0x64006400) - k1024;
-    const v2h h3 = __builtin_bit_cast(v2h, (d8 & MASK_HI) | 0x54005400) - k64;
-    v8h o;
-    o[0] = h0[0]; o[1] = h0[1]; o[2] = h1[0]; o[3] = h1[1];
-    o[4] = h2[0]; o[5] = h2[1]; o[6] = h3[0]; o[7] = h3[1];
-    return o;
+    v4i o;
+    o[0] = (d & MASK_LO) | 0x64006400;
+    o[1] = (d & MASK_HI) | 0x54005400;
+    o[2] = (d8 & MASK_LO) | 0x64006400;
+    o[3] = (d8 & MASK_HI) | 0x54005400;
+    return __builtin_bit_cast(v8h, o);
   }
 
   // The four 8-value MFMA operands (k sub-blocks j = 0..3) of one lane's 32 weights.
@@ -83,102 +87,125 @@ struct SkinnyWoTile {
     }
   }
 
+  // One pass of a wave: NKB (<= KP) consecutive k blocks starting at kb0, against all NB channel blocks of the tile.
+  // The wave's activations of these k blocks are loaded once into registers and its (scale, zero) pairs into a private LDS
+  // patch; the packed weight blocks then stream through a ring of kRing register buffers with no barrier in the loop, so
+  // kRing KB per wave are always in flight.  Per 128-wide group g and channel n the pass adds
+  //   s * (sum_k x[k] * (q[k] + bias[k])  -  sum_k x[k] * bias[k])  +  z * sum_k x[k]
+  // where the first sum comes from 4 MFMAs on the biased weights and the other two from MFMAs of x against constant operands.
+  template <int NKB>
+  __device__ static __forceinline__ void pass(const TileArgs& t, int kb0, int m0, int n0, int nbv, int lane, uint8_t* __restrict__ spatch, v4f (&acc)[NB]) {
+    const int K = t.K, KB = K / 128;
+    const int lm = lane & 15, lg = lane >> 4;
+    const v8h ones = {(_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f};
+    const v8h bias = {(_Float16)1024.0f, (_Float16)1024.0f, (_Float16)64.0f, (_Float16)64.0f, (_Float16)1024.0f, (_Float16)1024.0f, (_Float16)64.0f, (_Float16)64.0f};
+    constexpr int Q = NB * NKB;  // blocks of this pass, channel block major
+
+    // (scale, zero) pairs of the pass: 64 bytes per block, NKB consecutive blocks per channel block -> LDS [nb][s][64 B]
+    const uint8_t* sb = reinterpret_cast<const uint8_t*>(t.sb) + ((long)(n0 / 16) * KB + kb0) * 64;
+#pragma unroll
+    for (int c = lane; c < Q * 4; c += 64) {  // 16-byte pieces
+      const int nb = c / (NKB * 4), rest = c % (NKB * 4);
+      const v4i v = gload<v4i>(sb + ((long)(nb < nbv ? nb : 0) * KB) * 64 + rest * 16);
+      *reinterpret_cast<v4i*>(spatch + c * 16) = v;
+    }
+    // activations: lane holds row lm, k = 128*(kb0 + s) + 32*lg + 8*j + 0..7
+    v8h xf[NKB][4];
+    {
+      const int m = m0 + lm;
+      const _Float16* xr = reinterpret_cast<const _Float16*>(t.A) + (long)(m < t.M ? m : 0) * K + kb0 * 128 + lg * 32;
+#pragma unroll
+      for (int s = 0; s < NKB; ++s)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const v4i v = gload<v4i>(xr + s * 128 + j * 8);
+          xf[s][j] = m < t.M ? __builtin_bit_cast(v8h, v) : v8h{};
+        }
+    }
+    const uint8_t* wb = t.B + ((long)(n0 / 16) * KB + kb0) * kBlockBytes + lane * kLaneBytes;
+    auto w_of = [&](int q) { const int nb = q / NKB < nbv ? q / NKB : 0; return load_w(wb + ((long)nb * KB + q % NKB) * kBlockBytes); };
+    WReg wr[kRing];
+#pragma unroll
+    for (int q = 0; q < kRing && q < Q; ++q) wr[q] = w_of(q);
+    __builtin_amdgcn_sched_barrier(0);
+
+    v4f sx[NKB], sxb[NKB];  // per k block: sum of x, sum of x * bias  (row = any channel, column = token)
+#pragma unroll
+    for (int s = 0; s < NKB; ++s) {
+      sx[s] = sxb[s] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        sx[s] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, xf[s][j], sx[s], 0, 0, 0);
+        sxb[s] = __builtin_amdgcn_mfma_f32_16x16x32_f16(bias, xf[s][j], sxb[s], 0, 0, 0);
+      }
+    }
+    static_for<Q>([&](auto qc) {
+      constexpr int q = decltype(qc)::value;
+      constexpr int nb = q / NKB, s = q % NKB;
+      v8h wf[4];
+      unpack(wr[q % kRing], wf);
+      if constexpr (q + kRing < Q) wr[q % kRing] = w_of(q + kRing);
+      const v8h s8 = __builtin_bit_cast(v8h, *reinterpret_cast<const v4i*>(spatch + q * 64 + lg * 16));  // (scale, zero) of channels 4*lg .. 4*lg+3
+      __builtin_amdgcn_sched_barrier(0);  // the refill is issued here, kRing blocks ahead of its use, not where the scheduler likes it
+      v4f part = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) part = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf[j], xf[s][j], part, 0, 0, 0);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[nb][e] = __builtin_fmaf(part[e] - sxb[s][e], (float)s8[2 * e], __builtin_fmaf(sx[s][e], (float)s8[2 * e + 1], acc[nb][e]));
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  }
+
   __device__ static __forceinline__ void run(const TileArgs& t, uint8_t* __restrict__ smem) {
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int M = t.M, N = t.N, K = t.K;
     const int m0 = t.row0 + t.tile_m * BM, n0 = t.tile_n * BN;
     const int KB = K / 128;  // k blocks (= quantisation groups) per row
     const int lm = lane & 15, lg = lane >> 4;
+    const int nbv = min(NB, (N - n0) / 16);  // channel blocks of this tile that exist
 
-    const _Float16* X = reinterpret_cast<const _Float16*>(t.A);
-    const v8h ones = {(_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f};
-
-    // row blocks of this wave: nb = n0/16 + wave + 4*r
-    const uint8_t* wp[R];
-    const uint8_t* sp[R];
-    bool live[R];
+    // the K range is dealt to the 4 waves in contiguous quarters; each wave sums its quarter for every channel of the tile
+    const int KW = (KB + kWaves - 1) / kWaves;
+    const int kb_lo = min(KB, wave * KW), kb_hi = min(KB, kb_lo + KW);
+    uint8_t* spatch = smem + kRedBytes + wave * kScaleBytes;
+    v4f acc[NB];
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      const int nb = n0 / 16 + wave + 4 * r;
-      live[r] = nb * 16 < N;
-      const int nbc = live[r] ? nb : 0;
-      wp[r] = t.B + ((long)nbc * KB) * kBlockBytes + lane * kLaneBytes;
-      sp[r] = reinterpret_cast<const uint8_t*>(t.sb) + ((long)nbc * KB) * 64 + lg * 16;  // 16 channels * (scale, zero) * 2 B per block
+    for (int nb = 0; nb < NB; ++nb) acc[nb] = v4f{0.f, 0.f, 0.f, 0.f};
+    for (int kb = kb_lo; kb < kb_hi; kb += KP) {
+      const int nk = min(KP, kb_hi - kb);
+      if (nk == 4) pass<4>(t, kb, m0, n0, nbv, lane, spatch, acc);
+      else if (nk == 3) pass<3>(t, kb, m0, n0, nbv, lane, spatch, acc);
+      else if (nk == 2) pass<2>(t, kb, m0, n0, nbv, lane, spatch, acc);
+      else pass<1>(t, kb, m0, n0, nbv, lane, spatch, acc);
     }
 
-    v4f acc[R];
+    // reduction over the 4 waves in a fixed order (wave 0 + 1 + 2 + 3), 16-channel blocks dealt round-robin to the waves
+    v4f* red = reinterpret_cast<v4f*>(smem);
 #pragma unroll
-    for (int r = 0; r < R; ++r) acc[r] = v4f{0.f, 0.f, 0.f, 0.f};
-
-    for (int kc0 = 0; kc0 < K; kc0 += KC) {
-      const int kcur = min(KC, K - kc0);
-      if (kc0) __syncthreads();  // previous chunk fully consumed before it is overwritten
-      // stage activation rows m0..m0+15, columns kc0..kc0+kcur, zero-filling rows past M
-      for (int idx = tid; idx < 16 * (KC / 8); idx += kThreads) {
-        const int row = idx / (KC / 8), ch = idx % (KC / 8);
-        if (ch * 8 < kcur) {
-          v4i v = {0, 0, 0, 0};
-          if (m0 + row < M) v = gload<v4i>(X + (long)(m0 + row) * K + kc0 + ch * 8);
-          *reinterpret_cast<v4i*>(smem + row * kXStride + ch * 16) = v;
-        }
-      }
-      __syncthreads();
-
-      const int kb0 = kc0 / 128, nkb = kcur / 128;
-      WReg wq[R];
-      v4i sz[R];
-#pragma unroll
-      for (int r = 0; r < R; ++r) {
-        wq[r] = load_w(wp[r] + (long)kb0 * kBlockBytes);
-        sz[r] = gload<v4i>(sp[r] + (long)kb0 * 64);
-      }
-      for (int kb = 0; kb < nkb; ++kb) {
-        WReg wn[R];
-        v4i szn[R];
-        const int kbn = kb0 + min(kb + 1, nkb - 1);  // last iteration re-loads its own block (harmless, keeps the loop branch-free)
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-          wn[r] = load_w(wp[r] + (long)kbn * kBlockBytes);
-          szn[r] = gload<v4i>(sp[r] + (long)kbn * 64);
-        }
-        v8h xf[4];
-        const uint8_t* xs = smem + lm * kXStride + (kb * 128 + lg * 32) * 2;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) xf[j] = *reinterpret_cast<const v8h*>(xs + j * 16);
-        v4f sx = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int j = 0; j < 4; ++j) sx = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, xf[j], sx, 0, 0, 0);
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-          v8h wf[4];
-          unpack(wq[r], wf);
-          v4f part = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-          for (int j = 0; j < 4; ++j) part = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf[j], xf[j], part, 0, 0, 0);
-          const v8h s8 = __builtin_bit_cast(v8h, sz[r]);  // (scale, zero) of channels 4*lg .. 4*lg+3
-#pragma unroll
-          for (int e = 0; e < 4; ++e) acc[r][e] += part[e] * (float)s8[2 * e] + sx[e] * (float)s8[2 * e + 1];
-          wq[r] = wn[r];
-          sz[r] = szn[r];
-        }
-      }
-    }
-
+    for (int nb = 0; nb < NB; ++nb) red[(wave * NB + nb) * 64 + lane] = acc[nb];
+    __syncthreads();
     const int m = m0 + lm;
-    if (m < M) {
 #pragma unroll
-      for (int r = 0; r < R; ++r) {
-        if (!live[r]) continue;
-        const int n = n0 + (wave + 4 * r) * 16 + lg * 4;
+    for (int r = 0; r < NB / kWaves; ++r) {
+      const int nb = wave + kWaves * r;
+      v4f sum = red[nb * 64 + lane];
+#pragma unroll
+      for (int w = 1; w < kWaves; ++w) {
+        const v4f p = red[(w * NB + nb) * 64 + lane];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sum[e] += p[e];
+      }
+      if (m < M && nb < nbv) {
+        const int n = n0 + nb * 16 + lg * 4;
         v4h o;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) o[e] = (_Float16)acc[r][e];
+        for (int e = 0; e < 4; ++e) o[e] = (_Float16)sum[e];
         gstore<v4h>(t.C + (long)m * N + n, o);
         if (t.acc_dump) {
 #pragma unroll
-          for (int e = 0; e < 4; ++e) gstore<int>(t.acc_dump + (long)m * N + n + e, __builtin_bit_cast(int, acc[r][e]));
+          for (int e = 0; e < 4; ++e) gstore<int>(t.acc_dump + (long)m * N + n + e, __builtin_bit_cast(int, sum[e]));
         }
       }
     }

@@ -162,7 +162,7 @@ class TileConfig:
     def smem_bytes_tile(self):
         """LDS bytes of the tile as compiled (csrc/include/mxmoe_tiles.hpp, mxmoe_wo_tiles.hpp)."""
         if self.is_skinny():
-            return 16 * (1024 * 2 + 16)
+            return 4 * (self.BN // 16) * (64 * 16 + 4 * 64)  # per-wave partial sums of the final reduction + (scale, zero) patches
         return self.STAGE * (self.BM + self.BN) * 64
 
     def cpp_type(self) -> str:
