@@ -174,6 +174,14 @@ inline std::string& last_error() {
   return e;
 }
 
+template <int WBITS, int BM, int BN>
+struct BranchOf<WoMfmaTile<WBITS, BM, BN>> {
+  static BranchInfo get() {
+    using T = WoMfmaTile<WBITS, BM, BN>;
+    return BranchInfo{WBITS == 4 ? Fmt::W4A16 : Fmt::W3A16, BM, BN, 128, 2, 2, T::kLdsBytes, 128, 0};
+  }
+};
+
 template <class... Tiles>
 hipError_t launch_fused(const FusedArgs& a, int grid, int lds, hipStream_t s) {
   // more than 64 KB of dynamic LDS must be opted into, once per device (kept out of library load time: no HIP call before first use)

@@ -212,4 +212,163 @@ struct SkinnyWoTile {
   }
 };
 
+// Weight-only tile for experts with many tokens (w4a16 / w3a16, group 128): 128 tokens x 128 channels per workgroup, 64 x 64 per
+// wave.  Counterpart of the reference's cta_gemm_multistage_qb_v2 with its larger tiles
+// (mxmoe/kernels/src/include/cta_gemm.cuh:113-286) and of Converter::dequant_frag (quantize.cuh:134-214): every packed weight
+// becomes fp16 as fma(q, scale, zero) in fp16, one rounding, exactly like the reference's __hfma2, and the products are summed in
+// fp32 by the fp16 MFMA over the whole of K.
+// Same packed weight and (scale, zero) layouts as the skinny tile: a wave streams its 4 channel blocks of each 128-wide k block
+// straight from global memory through a register ring and reuses each dequantised block for 4 token blocks x 4 MFMAs, so the
+// unpack work is a fraction of the matrix work.  Activations go global -> LDS (direct loads, two stages of 128 rows x 256 B,
+// 16-byte chunks XOR-swizzled with the row so that the 16 rows a read touches hit 16 different bank groups).
+template <int WBITS_, int BM_ = 128, int BN_ = 128>
+struct WoMfmaTile {
+  static constexpr int WBITS = WBITS_, BM = BM_, BN = BN_;
+  static_assert(BM == 128 && BN == 128, "2 x 2 waves of 64 tokens x 64 channels");
+  using Sk = SkinnyWoTile<WBITS, 128>;
+  static constexpr int kStageBytes = BM * 256;
+  static constexpr int kLdsBytes = 2 * kStageBytes;
+  static constexpr int kAccRegs = 64;
+  static constexpr int kLaneBytes = Sk::kLaneBytes, kBlockBytes = Sk::kBlockBytes;
+  static constexpr int kDma = kStageBytes / 1024 / kWaves;  // direct-to-LDS loads per wave per stage
+
+  __device__ static __forceinline__ void run(const TileArgs& t, uint8_t* __restrict__ smem) {
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int M = t.M, N = t.N, K = t.K;
+    const int m0 = t.row0 + t.tile_m * BM, n0 = t.tile_n * BN;
+    const int KB = K / 128;
+    const int lm = lane & 15, lg = lane >> 4;
+    // channel blocks of this wave that exist; a wave whose 64 channels all lie past N runs on the tile's first blocks instead
+    // (every wave must take part in the barriers) and stores nothing
+    const int nbv = max(0, min(4, (N - n0) / 16 - wn * 4));
+    const int nb0 = n0 / 16 + (nbv > 0 ? wn * 4 : 0);
+
+    // activations: buffer resource over the valid rows of the tile (rows past M read as zeros)
+    const int a_rows = min(BM, M - m0);
+    const v4i rs_x = make_rsrc(t.A + (long)m0 * K * 2, (unsigned)((long)a_rows * K * 2));
+    const int lds_base = (int)(uintptr_t)smem;
+    int dma_voff[kDma], dma_lds[kDma];
+#pragma unroll
+    for (int i = 0; i < kDma; ++i) {
+      const int ii = wave * kDma + i;             // 1 KB piece = 4 rows
+      const int row = 4 * ii + (lane >> 4);
+      dma_voff[i] = row * K * 2 + (((lane & 15) ^ (row & 15)) << 4);
+      dma_lds[i] = ii * 1024;
+    }
+    auto dma_x = [&](int kb, int stage) {
+      const int koff = __builtin_amdgcn_readfirstlane(kb * 256);
+#pragma unroll
+      for (int i = 0; i < kDma; ++i) dma16_to_lds(rs_x, __builtin_amdgcn_readfirstlane(lds_base + stage * kStageBytes + dma_lds[i]), dma_voff[i], koff);
+    };
+    // fragment reads: token row wm*64 + mb*16 + lm, chunk lg*4 + j
+    const int xrow = wm * 64 + lm;
+    auto lds_x = [&](int stage, int mb, int j) {
+      const int row = xrow + mb * 16;
+      return *reinterpret_cast<const v4i*>(smem + stage * kStageBytes + row * 256 + (((lg * 4 + j) ^ (row & 15)) << 4));
+    };
+
+    // weights: blocks (n0/16 + wn*4 + nb, kb); ring of 8 = two k blocks ahead.  Loads past the end of K re-read the last k block
+    // (never used) so that every iteration issues the same number of loads, which the wait for the activation stage relies on.
+    const uint8_t* wb = t.B + ((long)nb0 * KB) * kBlockBytes + lane * kLaneBytes;
+    const uint8_t* sb = reinterpret_cast<const uint8_t*>(t.sb) + ((long)nb0 * KB) * 64 + lm * 4;
+    auto w_of = [&](int nb, int kb) { return Sk::load_w(wb + ((long)(nb < nbv ? nb : 0) * KB + min(kb, KB - 1)) * kBlockBytes); };
+    auto s_of = [&](int nb, int kb) { return gload<int>(sb + ((long)(nb < nbv ? nb : 0) * KB + min(kb, KB - 1)) * 64); };
+    typename Sk::WReg wr[8];
+    int sr[8];
+
+    v4f acc[4][4];  // [channel block][token block]
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb) acc[nb][mb] = v4f{0.f, 0.f, 0.f, 0.f};
+
+    {
+      // prologue: exactly 8 ring loads are younger than the loads of the first activation stage, as in every later iteration
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        wr[q] = w_of(q, 0);
+        sr[q] = s_of(q, 0);
+      }
+      asm volatile("" ::: "memory");
+      dma_x(0, 0);
+#pragma unroll
+      for (int q = 4; q < 8; ++q) {
+        wr[q] = w_of(q - 4, 1);
+        sr[q] = s_of(q - 4, 1);
+      }
+      asm volatile("" ::: "memory");
+      const v8h bias = {(_Float16)1024.0f, (_Float16)1024.0f, (_Float16)64.0f, (_Float16)64.0f, (_Float16)1024.0f, (_Float16)1024.0f, (_Float16)64.0f, (_Float16)64.0f};
+      // one k block; PAR = parity of kb, a compile-time constant so that the ring slots are fixed registers
+      auto step = [&](auto parc, int kb) {
+        constexpr int st = decltype(parc)::value;
+        // the activation stage of this k block has landed: the only younger loads are the 8 ring refills of the last iteration
+        // (or the 8 ring loads of the prologue)
+        vm_wait<8>();
+        __syncthreads();  // ... for every wave; and every wave holds the previous stage's fragments in registers by now
+        if (kb + 1 < KB) dma_x(kb + 1, st ^ 1);
+        v8h xf[4][4];
+#pragma unroll
+        for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) xf[mb][j] = __builtin_bit_cast(v8h, lds_x(st, mb, j));
+#pragma unroll
+        for (int nb = 0; nb < 4; ++nb) {
+          constexpr int base = st * 4;
+          v8h wf[4];
+          Sk::unpack(wr[base + nb], wf);
+          const v2h sz = __builtin_bit_cast(v2h, sr[base + nb]);
+          wr[base + nb] = w_of(nb, kb + 2);
+          sr[base + nb] = s_of(nb, kb + 2);
+          const v8h s8 = {sz[0], sz[0], sz[0], sz[0], sz[0], sz[0], sz[0], sz[0]};
+          const v8h z8 = {sz[1], sz[1], sz[1], sz[1], sz[1], sz[1], sz[1], sz[1]};
+#pragma unroll
+          for (int j = 0; j < 4; ++j) wf[j] = __builtin_elementwise_fma(wf[j] - bias, s8, z8);  // exact q, then fma(q, scale, zero) in fp16
+#pragma unroll
+          for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[nb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf[j], xf[mb][j], acc[nb][mb], 0, 0, 0);
+        }
+      };
+#pragma unroll 1
+      for (int kb = 0; kb < KB; kb += 2) {
+        step(std::integral_constant<int, 0>{}, kb);
+        if (kb + 1 < KB) step(std::integral_constant<int, 1>{}, kb + 1);
+      }
+    }
+    vm_wait<0>();
+    __syncthreads();  // LDS is reused for the output patch
+
+    // epilogue: [token][channel] fp16 patch per wave (64 x 64, row pitch 136 B), then 16-byte row-contiguous stores
+    constexpr int kPitch = 64 * 2 + 8;
+    uint8_t* patch = smem + wave * (64 * kPitch);
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb) {
+        v4h o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = (_Float16)acc[nb][mb][e];
+        *reinterpret_cast<v4h*>(patch + (mb * 16 + lm) * kPitch + (nb * 16 + lg * 4) * 2) = o;
+        if (t.acc_dump) {
+          const int m = m0 + wm * 64 + mb * 16 + lm, n = n0 + wn * 64 + nb * 16 + lg * 4;
+          if (m < M && n < N) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) gstore<int>(t.acc_dump + (long)m * N + n + e, __builtin_bit_cast(int, acc[nb][mb][e]));
+          }
+        }
+      }
+    const int pr = lane >> 3, pc = lane & 7;  // 8 lanes x 16 B per 64-channel row, 8 rows per pass
+#pragma unroll
+    for (int r0 = 0; r0 < 64; r0 += 8) {
+      const int ml = r0 + pr;
+      const int m = m0 + wm * 64 + ml, n = n0 + wn * 64 + pc * 8;
+      const v4i v = *reinterpret_cast<const v4i*>(patch + ml * kPitch + pc * 16);
+      if (m < M && n < N) gstore<v4i>(t.C + (long)m * N + n, v);
+    }
+  }
+};
+
 }  // namespace mxmoe

@@ -153,8 +153,11 @@ class TileConfig:
         self.QCFGA, self.QCFGB = qcfg.QCFGA, qcfg.QCFGB
         return self
 
-    def is_skinny(self) -> bool:
+    def is_weight_only(self) -> bool:
         return self.MMA == "MFMA_F32_16x16x32_F16"
+
+    def is_skinny(self) -> bool:
+        return self.is_weight_only() and self.BM == 16
 
     def smem_bytes_scale(self):
         return 0  # scales are read straight from global memory in the epilogue / per group
@@ -163,21 +166,25 @@ class TileConfig:
         """LDS bytes of the tile as compiled (csrc/include/mxmoe_tiles.hpp, mxmoe_wo_tiles.hpp)."""
         if self.is_skinny():
             return 4 * (self.BN // 16) * (64 * 16 + 4 * 64)  # per-wave partial sums of the final reduction + (scale, zero) patches
+        if self.is_weight_only():
+            return 2 * self.BM * 256  # two stages of BM activation rows x one 128-wide k block
         return self.STAGE * (self.BM + self.BN) * 64
 
     def cpp_type(self) -> str:
         """The C++ tile type this descriptor instantiates."""
         if self.is_skinny():
             return f"SkinnyWoTile<{self.QCFGB.QBITS}, {self.BN}>"
+        if self.is_weight_only():
+            return f"WoMfmaTile<{self.QCFGB.QBITS}, {self.BM}, {self.BN}>"
         op = {"MFMA_F32_32x32x16_F16": "Op::F16", "MFMA_I32_32x32x32_I8": "Op::I8", "MFMA_I32_32x32x32_I8_FROM_I4": "Op::I4"}[self.MMA]
         return f"MfmaTile<{op}, {self.BM}, {self.BN}, {self.WM}, {self.WN}>"
 
     def validate(self) -> None:
         if self.num_warps != 4:
             raise ValueError(f"{self!r}: gfx950 tiles use 4 wavefronts per workgroup")
-        if self.is_skinny():
-            if self.BM != 16 or self.BN % 64 or self.BK != 128:
-                raise ValueError(f"{self!r}: skinny weight-only tiles are 16 x (64k) x 128")
+        if self.is_weight_only():
+            if self.BK != 128 or not ((self.BM == 16 and self.BN % 64 == 0 and (self.WM, self.WN) == (1, 4)) or (self.BM, self.BN, self.WM, self.WN) == (128, 128, 2, 2)):
+                raise ValueError(f"{self!r}: weight-only tiles are 16 x (64k) x 128 (1 x 4 waves) or 128 x 128 x 128 (2 x 2 waves)")
             return
         k_elems = {"MFMA_F32_32x32x16_F16": 32, "MFMA_I32_32x32x32_I8": 64, "MFMA_I32_32x32x32_I8_FROM_I4": 128}[self.MMA]
         if self.BK != k_elems or self.STAGE != 3 or self.WK != 1 or (self.BM // self.WM) % 32 or (self.BN // self.WN) % 32:
@@ -217,7 +224,8 @@ def get_possible_tile_list(arch: str, qcfg: str) -> list:
         raise ValueError(f"no tile list for arch {arch!r}: this library targets gfx950")
     mma = QCFG_TO_MMA[qcfg]
     if mma == "MFMA_F32_16x16x32_F16":
-        return [_with_q(TileConfig(BM=16, BN=bn, BK=128, WM=1, WN=4, WK=1, STAGE=2, MMA=mma), qcfg) for bn in (128, 64, 256)]
+        skinny = [_with_q(TileConfig(BM=16, BN=bn, BK=128, WM=1, WN=4, WK=1, STAGE=2, MMA=mma), qcfg) for bn in (128, 64)]
+        return skinny + [_with_q(TileConfig(BM=128, BN=128, BK=128, WM=2, WN=2, WK=1, STAGE=2, MMA=mma), qcfg)]
     bk = {"MFMA_F32_32x32x16_F16": 32, "MFMA_I32_32x32x32_I8": 64, "MFMA_I32_32x32x32_I8_FROM_I4": 128}[mma]
     shapes = [(128, 256, 2, 2), (64, 256, 1, 4), (32, 256, 1, 4), (128, 128, 2, 2), (256, 128, 2, 2)]
     return [_with_q(TileConfig(BM=bm, BN=bn, BK=bk, WM=wm, WN=wn, WK=1, STAGE=3, MMA=mma), qcfg) for bm, bn, wm, wn in shapes]

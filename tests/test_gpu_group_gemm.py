@@ -102,6 +102,37 @@ def test_weight_only_skinny():
         assert _rel(out, p["ref"]) <= 1e-2, (p["size"], p["q"], _rel(out, p["ref"]))
 
 
+def test_weight_only_many_tokens():
+    """Experts with many tokens run the 128 x 128 dequantise-to-fp16 MFMA tile (and the remainder rows the skinny one)."""
+    import ctypes as C
+
+    from mxmoe_amd import _lib
+    from mxmoe_amd.weights import quantize_and_pack
+
+    rng = np.random.default_rng(5)
+    probs = []
+    for (m, n, k, bits, sym) in [(200, 256, 512, 4, False), (129, 384, 1408, 3, False), (64, 128, 128, 4, True), (300, 2816, 256, 3, True),
+                                 (128, 192, 256, 4, False), (7, 256, 256, 4, False)]:
+        x = rng.standard_normal((m, k)).astype(F16)
+        w = (rng.standard_normal((n, k)) * 0.02).astype(F16)
+        pw = quantize_and_pack(torch.from_numpy(w), (16, bits, 128, sym))
+        q, s, z = O.quant_minmax(w, bits, 128, sym)
+        ref = O.gemm_fakequant(x, O.dequant(q, s, z, 128))
+        probs.append(dict(A=torch.from_numpy(x).to(DEV), B=pw.data.to(DEV), sb=pw.scale.to(DEV), ref=ref, size=(m, n, k), q=(16, bits, 128, sym)))
+    g, outs, _ = _launch(probs, dump=False)
+    kid, branches, _ = g.plan()
+    lib = _lib.load()
+    info = (C.c_int32 * 8)()
+    bms = []
+    for b in branches:
+        assert lib.mxmoe_kernel_branch(kid, b, info) == 0
+        bms.append(info[1])
+    assert bms[:5] == [128] * 5 and bms[5] == 16, bms
+    for p, out in zip(probs, outs):
+        assert np.isfinite(out).all()
+        assert _rel(out, p["ref"]) <= 1e-2, (p["size"], p["q"], _rel(out, p["ref"]))
+
+
 def test_unsupported_format_raises_reference_message():
     rng = np.random.default_rng(4)
     p = _wxax_problem(rng, 4, 256, 128, 8)
