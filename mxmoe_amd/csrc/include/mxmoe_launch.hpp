@@ -28,6 +28,7 @@ namespace mxmoe {
 constexpr int kMaxProblems = 128;  // per launch; longer problem lists are split into several launches
 constexpr int kMaxEntries = 2 * kMaxProblems;  // a problem is run as at most two row segments, each with its own tile shape
 constexpr int kNumXcd = 8;
+constexpr int kMaxPhases = 8;
 
 struct FusedArgs {
   const uint8_t* const* As;
@@ -40,7 +41,13 @@ struct FusedArgs {
   int problem_offset;   // first problem of this launch inside the arrays above
   int num_entries;
   int total_tiles;
-  int chunk;                      // tiles per XCD = ceil(total_tiles / 8)
+  // Phases: the entries are sorted so that the most expensive tile shapes come first (workgroups are dispatched in index order,
+  // so the cheap tiles fill the tail of the launch).  Phase p covers tiles [phase_tile0[p], phase_tile0[p+1]) and workgroups
+  // [phase_wg0[p], phase_wg0[p+1]); inside a phase, workgroup v maps to tile (v % 8) * chunk + v / 8 so that each XCD (one L2)
+  // works on a contiguous run of tiles.
+  int num_phases;
+  int phase_tile0[kMaxPhases + 1];
+  int phase_wg0[kMaxPhases + 1];
   int prefix[kMaxEntries];        // inclusive prefix sum of tiles per entry
   int row0[kMaxEntries];          // first row of the entry's segment inside its problem
   int rows[kMaxEntries];          // rows of the segment
@@ -78,8 +85,14 @@ template <class... Tiles>
 __global__ void __launch_bounds__(kThreads, kWavesPerSimd<Tiles...>) fused_group_gemm_kernel(const FusedArgs args) {
   extern __shared__ __align__(16) uint8_t smem[];
   const int wg = blockIdx.x;
-  const int tile = (wg % kNumXcd) * args.chunk + wg / kNumXcd;
-  if (tile >= args.total_tiles) return;
+  int ph = 0;
+  while (ph + 1 < args.num_phases && wg >= args.phase_wg0[ph + 1]) ++ph;
+  const int v = wg - args.phase_wg0[ph];
+  const int ntiles = args.phase_tile0[ph + 1] - args.phase_tile0[ph];
+  const int chunk = (ntiles + kNumXcd - 1) / kNumXcd;
+  const int pt = (v % kNumXcd) * chunk + v / kNumXcd;
+  if (pt >= ntiles) return;
+  const int tile = args.phase_tile0[ph] + pt;
   // tile_scheduler.cuh:25-37 — first problem whose inclusive prefix exceeds the tile index (binary search here)
   int lo = 0, hi = args.num_entries - 1;
   while (lo < hi) {
@@ -217,20 +230,38 @@ int register_fused(const char* fn_name) {
   return (int)registry().size() - 1;
 }
 
-// Relative cost of one tile of BM rows (same BN, same K), measured on MI355X: a 64-row tile costs ~0.62 and a 32-row tile ~0.41
-// of a 128-row tile (fixed prologue / epilogue and a less efficient wave tile).
-inline double tile_cost(int BM) { return 0.22 + 0.78 * BM / 128.0; }
+// Run time of one tile of a branch relative to the 128 x 256 tile of the same format (same K), from the kernel-profile table
+// measured on MI355X (ms per 256 tiles at K = 2048).  Small tiles pay a fixed prologue / epilogue and use the matrix pipe less
+// well; the weight-only entries compare the skinny streaming tile with the 128 x 128 dequantise-to-fp16 tile.
+inline double tile_cost(const BranchInfo& b) {
+  struct Row { Fmt f; int bm, bn; double c; };
+  static const Row table[] = {
+      {Fmt::W4A4, 128, 256, 1.00}, {Fmt::W4A4, 64, 256, 0.58}, {Fmt::W4A4, 32, 256, 0.48}, {Fmt::W4A4, 128, 128, 0.50}, {Fmt::W4A4, 256, 128, 0.95},
+      {Fmt::W8A8, 128, 256, 1.00}, {Fmt::W8A8, 64, 256, 0.74}, {Fmt::W8A8, 32, 256, 0.56}, {Fmt::W8A8, 128, 128, 0.56}, {Fmt::W8A8, 256, 128, 1.01},
+      {Fmt::FP16, 128, 256, 1.00}, {Fmt::FP16, 64, 256, 0.69}, {Fmt::FP16, 32, 256, 0.53}, {Fmt::FP16, 128, 128, 0.57}, {Fmt::FP16, 256, 128, 1.09},
+      {Fmt::W4A16, 16, 128, 0.37}, {Fmt::W4A16, 16, 64, 0.20}, {Fmt::W4A16, 128, 128, 1.00},
+      {Fmt::W3A16, 16, 128, 0.31}, {Fmt::W3A16, 16, 64, 0.20}, {Fmt::W3A16, 128, 128, 1.00},
+  };
+  for (const Row& r : table)
+    if (r.f == b.fmt && r.bm == b.BM && r.bn == b.BN) return r.c;
+  return (0.22 + 0.78 * b.BM / 128.0) * b.BN / 256.0;  // shapes without a measurement
+}
 
-// Cheapest branch of format `f` for a block of `rows` rows run with one tile shape: cost = ceil(rows / BM) * tile_cost(BM).
-inline int pick_branch(const FusedKernel& k, Fmt f, int rows) {
+// Rough run time of one tile across formats, used only to order the tile list (expensive shapes first): the matrix pipe runs
+// fp16 at half the int8 rate, and int4 operands are widened to int8.
+inline double branch_cost(const BranchInfo& b) {
+  const double per_k = b.fmt == Fmt::FP16 ? 2.0 : (b.fmt == Fmt::W4A16 || b.fmt == Fmt::W3A16) ? 1.2 : (b.fmt == Fmt::W8A8 ? 1.25 : 1.0);
+  return tile_cost(b) * per_k;
+}
+
+// Cheapest branch of format `f` for a block of `rows` x `N` run with one tile shape: cost = row tiles * column tiles * tile_cost.
+inline int pick_branch(const FusedKernel& k, Fmt f, int rows, int N) {
   int best = -1;
   double best_cost = 0;
-  static const int force_bm = getenv("MXMOE_FORCE_BM") ? atoi(getenv("MXMOE_FORCE_BM")) : 0;
   for (int i = 0; i < (int)k.branches.size(); ++i) {
     const auto& b = k.branches[i];
     if (b.fmt != f) continue;
-    if (force_bm && b.BM != force_bm) continue;
-    const double c = (double)((rows + b.BM - 1) / b.BM) * tile_cost(b.BM);
+    const double c = (double)((rows + b.BM - 1) / b.BM) * ((N + b.BN - 1) / b.BN) * tile_cost(b);
     if (best < 0 || c < best_cost - 1e-9 || (c < best_cost + 1e-9 && b.BM > k.branches[best].BM)) {
       best = i;
       best_cost = c;
@@ -243,26 +274,36 @@ struct Segment {
   int row0, rows, branch;
 };
 
-// Split the M rows of a problem into at most two segments: whole tiles of the largest shape, then the remainder with the shape
-// that covers it most cheaply.  Returns the number of segments (0 for M == 0), or -1 when the kernel has no tile for `f`.
-inline int plan_segments(const FusedKernel& k, Fmt f, int M, Segment out[2]) {
+// Split the M rows of an M x N problem into at most two segments: whole tiles of the shape that is cheapest per output element,
+// then the remainder with the shape that covers it most cheaply.  Returns the number of segments (0 for M == 0), or -1 when
+// the kernel has no tile for `f`.
+inline int plan_segments(const FusedKernel& k, Fmt f, int M, int N, Segment out[2]) {
   int big = -1;
-  for (int i = 0; i < (int)k.branches.size(); ++i)
-    if (k.branches[i].fmt == f && (big < 0 || k.branches[i].BM > k.branches[big].BM)) big = i;
+  double big_unit = 0;
+  for (int i = 0; i < (int)k.branches.size(); ++i) {
+    const auto& b = k.branches[i];
+    if (b.fmt != f) continue;
+    const double unit = tile_cost(b) * ((N + b.BN - 1) / b.BN) / b.BM;  // cost per row of the problem
+    if (big < 0 || unit < big_unit - 1e-12 || (unit < big_unit + 1e-12 && b.BM > k.branches[big].BM)) {
+      big = i;
+      big_unit = unit;
+    }
+  }
   if (big < 0) return -1;
   if (M <= 0) return 0;
-  static const bool no_split = getenv("MXMOE_NO_SPLIT") != nullptr;
+  auto cost_of = [&](int branch, int rows) {
+    const auto& b = k.branches[branch];
+    return (double)((rows + b.BM - 1) / b.BM) * ((N + b.BN - 1) / b.BN) * tile_cost(b);
+  };
   const int bm = k.branches[big].BM;
   const int full = (M / bm) * bm, rem = M - full;
-  const int whole = pick_branch(k, f, M);
-  if (rem == 0 || full == 0 || no_split) {
+  const int whole = pick_branch(k, f, M, N);
+  if (rem == 0 || full == 0) {
     out[0] = Segment{0, M, whole};
     return 1;
   }
-  const int rb = pick_branch(k, f, rem);
-  const double split_cost = (full / bm) * tile_cost(bm) + (double)((rem + k.branches[rb].BM - 1) / k.branches[rb].BM) * tile_cost(k.branches[rb].BM);
-  const double whole_cost = (double)((M + k.branches[whole].BM - 1) / k.branches[whole].BM) * tile_cost(k.branches[whole].BM);
-  if (whole_cost <= split_cost + 1e-9 || rb == big) {
+  const int rb = pick_branch(k, f, rem, N);
+  if (cost_of(whole, M) <= cost_of(big, full) + cost_of(rb, rem) + 1e-9 || rb == big) {
     out[0] = Segment{0, M, rb == big ? big : whole};
     return 1;
   }
@@ -276,7 +317,7 @@ inline bool kernel_covers(const FusedKernel& k, const mxmoe_qparams* q, int coun
   for (int i = 0; i < count; ++i) {
     const Fmt f = classify(q[i]);
     Segment sg[2];
-    if (f == Fmt::UNSUPPORTED || plan_segments(k, f, 1, sg) < 0) return false;
+    if (f == Fmt::UNSUPPORTED || plan_segments(k, f, 1, 256, sg) < 0) return false;
   }
   return true;
 }
@@ -312,12 +353,16 @@ inline int group_gemm(int kernel_id, const void* const* As, const void* const* B
     a.acc = acc;
     a.sizes = d_sizes;
     a.problem_offset = base;
-    int total = 0, ne = 0;
+    struct Entry {
+      int row0, rows, problem, branch, tiles;
+    };
+    Entry entries[kMaxEntries];
+    int nent = 0;
     for (int i = 0; i < n; ++i) {
       const mxmoe_dim3& sz = h_sizes[base + i];
       const Fmt f = classify(h_q[base + i]);
       Segment sg[2];
-      const int ns = f == Fmt::UNSUPPORTED ? -1 : plan_segments(k, f, (int)sz.x, sg);
+      const int ns = f == Fmt::UNSUPPORTED ? -1 : plan_segments(k, f, (int)sz.x, (int)sz.y, sg);
       if (ns < 0) {
         last_error() = "quant type not supported";
         return 1;
@@ -330,20 +375,47 @@ inline int group_gemm(int kernel_id, const void* const* As, const void* const* B
           last_error() = buf;
           return 3;
         }
-        total += ((sg[j].rows + bi.BM - 1) / bi.BM) * (int)((sz.y + bi.BN - 1) / bi.BN);
+        entries[nent++] = Entry{sg[j].row0, sg[j].rows, i, sg[j].branch, ((sg[j].rows + bi.BM - 1) / bi.BM) * (int)((sz.y + bi.BN - 1) / bi.BN)};
+      }
+    }
+    // most expensive tile shape first; problems keep their order inside a shape (neighbouring tiles share operands)
+    constexpr int kMaxBranches = 32;
+    int order[kMaxBranches];
+    const int nb = std::min((int)k.branches.size(), kMaxBranches);
+    for (int b = 0; b < nb; ++b) order[b] = b;
+    std::stable_sort(order, order + nb, [&](int x, int y) { return branch_cost(k.branches[x]) > branch_cost(k.branches[y]); });
+    int total = 0, ne = 0, wg = 0, np = 0;
+    for (int oi = 0; oi < nb; ++oi) {
+      const int b = order[oi];
+      const int tile0 = total;
+      for (int ei = 0; ei < nent; ++ei) {
+        const Entry& en = entries[ei];
+        if (en.branch != b || en.tiles == 0) continue;
+        total += en.tiles;
         a.prefix[ne] = total;
-        a.row0[ne] = sg[j].row0;
-        a.rows[ne] = sg[j].rows;
-        a.problem[ne] = (uint16_t)i;
-        a.branch[ne] = (uint8_t)sg[j].branch;
+        a.row0[ne] = en.row0;
+        a.rows[ne] = en.rows;
+        a.problem[ne] = (uint16_t)en.problem;
+        a.branch[ne] = (uint8_t)en.branch;
         ++ne;
       }
+      if (total == tile0) continue;
+      // shapes beyond the phase table share the last phase (their relative order is kept)
+      if (np < kMaxPhases) {
+        a.phase_tile0[np] = tile0;
+        a.phase_wg0[np] = wg;
+        ++np;
+      }
+      const int p0 = a.phase_tile0[np - 1];
+      wg = a.phase_wg0[np - 1] + (total - p0 + kNumXcd - 1) / kNumXcd * kNumXcd;
     }
     a.num_entries = ne;
     if (total == 0) continue;
     a.total_tiles = total;
-    a.chunk = (total + kNumXcd - 1) / kNumXcd;
-    const hipError_t e = k.launch(a, a.chunk * kNumXcd, k.lds_bytes, stream);
+    a.num_phases = np;
+    a.phase_tile0[np] = total;
+    a.phase_wg0[np] = wg;
+    const hipError_t e = k.launch(a, wg, k.lds_bytes, stream);
     if (e != hipSuccess) {
       last_error() = std::string("kernel launch failed: ") + hipGetErrorString(e);
       return 4;

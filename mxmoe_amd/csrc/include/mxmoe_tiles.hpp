@@ -345,15 +345,16 @@ struct MfmaTile {
     // The scaled fp16 results go through a per-wave LDS patch laid out [token][channel] so that the global stores are 16 bytes
     // per lane along a row (TN*2 contiguous bytes per token) instead of 8-byte pieces scattered over 32 rows.
     const int nq = (lane >> 5) * 4;
-    // all scales of this lane are fetched in one batch of independent loads, issued before the barrier so that their latency
-    // overlaps the wait for the slowest wave
+    // all scales of this lane are fetched in one batch of independent, unconditional loads (indices clamped into the tensor;
+    // rows / channels past the edge are never stored), issued before the barrier so that their latency overlaps the wait for
+    // the slowest wave
     float s_a[FM];
     v4h s_b[FN][4];
     if constexpr (OP != Op::F16) {
 #pragma unroll
       for (int i = 0; i < FM; ++i) {
-        const int m = m0 + wm * TM + i * 32 + lrow;
-        s_a[i] = m < M ? (float)gload<_Float16>(t.sa + m) : 0.0f;
+        const int m = min(m0 + wm * TM + i * 32 + lrow, M - 1);
+        s_a[i] = (float)gload<_Float16>(t.sa + m);
         // the int4 accumulator holds 256 * sum; 2^-8 folded into the (exact) scale product gives bit-identical results to
         // shifting first: float(256 * x) == 256 * float(x), and scaling by a power of two commutes with rounding
         if constexpr (OP == Op::I4) s_a[i] *= 0.00390625f;
@@ -362,64 +363,73 @@ struct MfmaTile {
       for (int j = 0; j < FN; ++j)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const int n = n0 + wn * TN + j * 32 + q * 8 + nq;
-          s_b[j][q] = v4h{(_Float16)0.0f, (_Float16)0.0f, (_Float16)0.0f, (_Float16)0.0f};
-          if (n < N) s_b[j][q] = gload<v4h>(t.sb + n);  // N is a multiple of 8, so a quad is all-in or all-out
+          const int n = min(n0 + wn * TN + j * 32 + q * 8 + nq, N - 4);  // N is a multiple of 8, so a quad is all-in or all-out
+          s_b[j][q] = gload<v4h>(t.sb + n);
         }
+    }
+    if (t.acc_dump) {  // parity tests only
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int m = m0 + wm * TM + i * 32 + lrow, n = n0 + wn * TN + j * 32 + (r / 4) * 8 + nq + (r & 3);
+            const auto v = acc[i][j][r];
+            int a;
+            if constexpr (OP == Op::F16) a = __builtin_bit_cast(int, (float)v); else a = (int)v;
+            if constexpr (OP == Op::I4) a >>= 8;  // exact
+            if (m < M && n < N) gstore<int>(t.acc_dump + (long)m * N + n, a);
+          }
     }
     __syncthreads();  // every wave is done reading the pipeline stages: LDS can be reused
     constexpr int kPitch = TN * 2 + 8;  // bytes per token row of the patch; the odd multiple of 8 spreads rows over banks
-    static_assert(kWaves * TM * kPitch <= kLdsBytes, "epilogue patch must fit the pipeline's LDS");
-    uint8_t* patch = smem + wave * (TM * kPitch);
-#pragma unroll
-    for (int i = 0; i < FM; ++i) {
-      const int ml = i * 32 + lrow;
-      const int m = m0 + wm * TM + ml;
-#pragma unroll
-      for (int j = 0; j < FN; ++j) {
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int nl = j * 32 + q * 8 + nq;
-          const int n = n0 + wn * TN + nl;
-          v4h o;
-          if constexpr (OP == Op::F16) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) o[e] = (_Float16)acc[i][j][q * 4 + e];
-          } else {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              // float(acc) * (sa * sb) rounded to half, as the reference epilogue (mm_tile.cuh:490-493, 642-646) except that the
-              // scale product stays in fp32, where it is exact: the reference rounds it to fp16 first, which turns subnormal
-              // (a few significant bits) for typical int8 scales and breaks the 1e-2 agreement with the fake-quant path.
-              const float sc = s_a[i] * (float)s_b[j][q][e];
-              o[e] = (_Float16)keep_f32((float)acc[i][j][q * 4 + e] * sc);
-            }
-          }
-          if (t.acc_dump && m < M && n < N) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const auto v = acc[i][j][q * 4 + e];
-              int a;
-              if constexpr (OP == Op::F16) a = __builtin_bit_cast(int, (float)v); else a = (int)v;
-              if constexpr (OP == Op::I4) a >>= 8;  // exact
-              gstore<int>(t.acc_dump + (long)m * N + n + e, a);
-            }
-          }
-          *reinterpret_cast<v4h*>(patch + ml * kPitch + nl * 2) = o;
-        }
-      }
-    }
-    // same-wave LDS traffic is ordered, so no barrier is needed between the patch writes above and the reads below
+    // the patch holds FI of the wave's FM 32-row blocks at a time (all of them when the pipeline's LDS is large enough)
+    constexpr int FI = kWaves * TM * kPitch <= kLdsBytes ? FM : (kWaves * (TM / 2) * kPitch <= kLdsBytes ? FM / 2 : 1);
+    static_assert(kWaves * FI * 32 * kPitch <= kLdsBytes && FM % FI == 0, "epilogue patch must fit the pipeline's LDS");
+    uint8_t* patch = smem + wave * (FI * 32 * kPitch);
     constexpr int kLanesPerRow = TN / 8;           // 16-byte pieces per token row
     constexpr int kRowsPerPass = 64 / kLanesPerRow;
     const int pr = lane / kLanesPerRow, pc = lane % kLanesPerRow;
 #pragma unroll
-    for (int r0 = 0; r0 < TM; r0 += kRowsPerPass) {
-      const int ml = r0 + pr;
-      const int m = m0 + wm * TM + ml;
-      const int n = n0 + wn * TN + pc * 8;
-      const v4i v = *reinterpret_cast<const v4i*>(patch + ml * kPitch + pc * 16);
-      if (m < M && n < N) gstore<v4i>(t.C + (long)m * N + n, v);
+    for (int i0 = 0; i0 < FM; i0 += FI) {
+#pragma unroll
+      for (int ii = 0; ii < FI; ++ii) {
+        const int i = i0 + ii;
+        const int ml = ii * 32 + lrow;
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int nl = j * 32 + q * 8 + nq;
+            v4h o;
+            if constexpr (OP == Op::F16) {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) o[e] = (_Float16)acc[i][j][q * 4 + e];
+            } else {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                // float(acc) * (sa * sb) rounded to half, as the reference epilogue (mm_tile.cuh:490-493, 642-646) except that the
+                // scale product stays in fp32, where it is exact: the reference rounds it to fp16 first, which turns subnormal
+                // (a few significant bits) for typical int8 scales and breaks the 1e-2 agreement with the fake-quant path.
+                const float sc = s_a[i] * (float)s_b[j][q][e];
+                o[e] = (_Float16)keep_f32((float)acc[i][j][q * 4 + e] * sc);
+              }
+            }
+            *reinterpret_cast<v4h*>(patch + ml * kPitch + nl * 2) = o;
+          }
+        }
+      }
+      // same-wave LDS traffic is ordered, so no barrier is needed between the patch writes above and the reads below, nor before
+      // the next round of writes
+#pragma unroll
+      for (int r0 = 0; r0 < FI * 32; r0 += kRowsPerPass) {
+        const int ml = r0 + pr;
+        const int m = m0 + wm * TM + i0 * 32 + ml;
+        const int n = n0 + wn * TN + pc * 8;
+        const v4i v = *reinterpret_cast<const v4i*>(patch + ml * kPitch + pc * 16);
+        if (m < M && n < N) gstore<v4i>(t.C + (long)m * N + n, v);
+      }
     }
   }
 };
