@@ -94,6 +94,18 @@ int mxmoe_silu_mul_quant(const void* gate_up, const void* gate_up_shared, void* 
                          int N, int N_shared, int rows_routed, int num_tokens, int num_experts, int has_shared, int rotate, int had_k, int had_f,
                          const float* had_signs, void* stream);
 
+/* ---- un-permute + top-k weighted combine: the step after the down launch.  The reference declares it as an empty stub
+ *      (gg_unpermute_out, mxmoe/kernels/src/ref_bind.cu:66); the contract here is the one its callers need ----
+ *
+ * out[t, :] = half( sum_{k ascending} topk_weights[t, k] * float(down_out[row(t, k), :])  + float(shared_out[t, :]) ), accumulated in fp32
+ * (each product rounded, then each sum), where row(t, k) is the sorted row whose src_slot equals t * topk + k; slots whose
+ * expert id was dropped contribute nothing.  down_out [rows, K] fp16 are the rows of the down launch in sorted order,
+ * shared_out [num_tokens, K] fp16 or NULL, topk_weights [num_tokens, topk] fp32, src_slot [rows] int64 as written by
+ * mxmoe_build_permutation, out [num_tokens, K] fp16, all DEVICE pointers.  workspace: mxmoe_combine_workspace_bytes() bytes. */
+size_t mxmoe_combine_workspace_bytes(int num_tokens, int topk);
+int mxmoe_unpermute_combine(const void* down_out, const void* shared_out, const float* topk_weights, const int64_t* src_slot, int rows, int num_tokens, int topk,
+                            int K, void* out, void* workspace, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -32,6 +32,8 @@ SIGNATURES = {
     "mxmoe_quant_act": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P]),
     "mxmoe_silu_mul_quant": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P]),
     "mxmoe_group_gemm_plan": (_I, [_I, C.POINTER(Dim3), C.POINTER(QParams), _I, C.POINTER(C.c_int32), C.POINTER(C.c_int32)]),
+    "mxmoe_combine_workspace_bytes": (C.c_size_t, [_I, _I]),
+    "mxmoe_unpermute_combine": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P]),
 }
 
 _cached = {}

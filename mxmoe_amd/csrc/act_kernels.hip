@@ -426,6 +426,50 @@ static int launch_rows(const RowArgs& a, int lds_bytes, hipStream_t s) {
 
 using namespace mxmoe;
 
+// ---- un-permute + top-k weighted combine: the step after the down launch (the reference leaves it as the empty stub
+// gg_unpermute_out, mxmoe/kernels/src/ref_bind.cu:66) ----
+//
+// row_of_slot[t * topk + k] = sorted row that holds (token t, slot k), or -1 when that slot's expert id was dropped.
+__global__ void combine_fill_kernel(int32_t* __restrict__ row_of_slot, int slots) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < slots) row_of_slot[i] = -1;
+}
+__global__ void combine_invert_kernel(const int64_t* __restrict__ src_slot, int rows, int slots, int32_t* __restrict__ row_of_slot) {
+  const int r = blockIdx.x * blockDim.x + threadIdx.x;
+  if (r < rows) {
+    const int64_t sl = src_slot[r];
+    if (sl >= 0 && sl < slots) row_of_slot[sl] = r;
+  }
+}
+// One workgroup per token: out[t] = half( sum_k w[t,k] * float(down[row(t,k)])  (k ascending, fp32: product rounded, then the
+// sum rounded)  + float(shared[t]) ).  Pure streaming: every down row is read once, 16 bytes per lane.
+__global__ void __launch_bounds__(256) combine_kernel(const _Float16* __restrict__ down, const _Float16* __restrict__ shared, const float* __restrict__ weights,
+                                                      const int32_t* __restrict__ row_of_slot, int topk, int K, _Float16* __restrict__ out) {
+  const int t = blockIdx.x;
+  for (int c = threadIdx.x * 8; c < K; c += 256 * 8) {
+    float acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = 0.0f;
+    for (int k = 0; k < topk; ++k) {
+      const int r = row_of_slot[t * topk + k];
+      if (r < 0) continue;
+      const float w = weights[t * topk + k];
+      const v8h v = *reinterpret_cast<const v8h*>(down + (size_t)r * K + c);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] = acc[e] + w * (float)v[e];
+    }
+    v8h o;
+    if (shared) {
+      const v8h v = *reinterpret_cast<const v8h*>(shared + (size_t)t * K + c);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] = acc[e] + (float)v[e];
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = (_Float16)keep_f32(acc[e]);
+    *reinterpret_cast<v8h*>(out + (size_t)t * K + c) = o;
+  }
+}
+
 extern "C" {
 
 size_t mxmoe_permute_workspace_bytes(int total, int num_experts) {
@@ -520,6 +564,33 @@ int mxmoe_silu_mul_quant(const void* gate_up, const void* gate_up_shared, void* 
   const int nmax = N > a.plan_shared.n ? N : a.plan_shared.n;
   const int lds = (nmax + a.plan.kb * a.plan.kb + 8) * (int)sizeof(float);
   return launch_rows<true>(a, lds, (hipStream_t)stream);
+}
+
+size_t mxmoe_combine_workspace_bytes(int num_tokens, int topk) { return (size_t)num_tokens * topk * sizeof(int32_t); }
+
+int mxmoe_unpermute_combine(const void* down_out, const void* shared_out, const float* topk_weights, const int64_t* src_slot, int rows, int num_tokens, int topk,
+                            int K, void* out, void* workspace, void* stream) {
+  if (num_tokens <= 0 || topk <= 0 || K <= 0 || K % 8 || rows < 0 || rows > num_tokens * topk) {
+    last_error() = "bad combine size (K must be a multiple of 8, rows <= tokens * topk)";
+    return 3;
+  }
+  if (!down_out || !topk_weights || !src_slot || !out || !workspace) {
+    last_error() = "null pointer";
+    return 5;
+  }
+  hipStream_t s = (hipStream_t)stream;
+  const int slots = num_tokens * topk;
+  int32_t* row_of_slot = reinterpret_cast<int32_t*>(workspace);
+  hipLaunchKernelGGL(combine_fill_kernel, dim3((slots + 255) / 256), dim3(256), 0, s, row_of_slot, slots);
+  if (rows > 0) hipLaunchKernelGGL(combine_invert_kernel, dim3((rows + 255) / 256), dim3(256), 0, s, src_slot, rows, slots, row_of_slot);
+  hipLaunchKernelGGL(combine_kernel, dim3(num_tokens), dim3(256), 0, s, reinterpret_cast<const _Float16*>(down_out), reinterpret_cast<const _Float16*>(shared_out),
+                     topk_weights, row_of_slot, topk, K, reinterpret_cast<_Float16*>(out));
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    last_error() = std::string("kernel launch failed: ") + hipGetErrorString(e);
+    return 4;
+  }
+  return 0;
 }
 
 }  // extern "C"

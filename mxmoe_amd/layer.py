@@ -68,6 +68,12 @@ class MxMoELayer:
     def down(self):
         self.state["gg2"].run()
 
+    def combine(self, topk_weights: torch.Tensor) -> torch.Tensor:
+        """Un-permute and mix the down outputs back into token order: [T, K] fp16."""
+        cfg, st = self.cfg, self.state
+        st["final"] = ops.gg_unpermute_out(st["out_store"], st["topk_ids"], topk_weights.to(self.device), cfg.num_experts, cfg.hidden, cfg.num_shared)
+        return st["final"]
+
     def forward(self, hidden, topk_ids, dump_acc: bool = False):
         """Full layer up to the per-problem down-projection outputs (list of [M_p, K] fp16, sorted-by-expert rows)."""
         self.prepare(hidden, topk_ids, dump_acc)

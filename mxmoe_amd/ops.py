@@ -167,6 +167,31 @@ def silu_mul_then_quant(inp, num_problems: int, num_experts: int, K: int, N: int
     return inp_list, scale_list, out_list, inp_store, scale_store, out_store
 
 
+def gg_unpermute_out(out_store: torch.Tensor, topk_ids: torch.Tensor, topk_weights: torch.Tensor, num_experts: int, K: int, num_shared_experts: int = 0,
+                     output: torch.Tensor | None = None) -> torch.Tensor:
+    """The step after the down launch, which the reference leaves as an empty stub (`gg_unpermute_out`, ref_bind.cu:66):
+    output[t] = sum_k topk_weights[t, k] * down(row of (t, k)) (+ the shared expert's row t), fp32 accumulation in slot order,
+    rounded once to fp16.  `out_store` is the flat down-projection store returned by `silu_mul_then_quant` (routed rows in sorted
+    order, then the shared expert's rows)."""
+    lib = _lib.load()
+    ids = topk_ids.to(torch.int32).contiguous()
+    t, k = ids.shape
+    w = topk_weights.to(torch.float32).contiguous()
+    assert w.shape == (t, k) and w.is_cuda and out_store.is_cuda and out_store.dtype == torch.float16
+    _dst, _perm, slot, recv = build_permutation(ids, num_experts)  # stable, so the same order the rows were produced in
+    rows = int(recv.sum().item())
+    flat = out_store.reshape(-1)
+    need = (rows + (t if num_shared_experts else 0)) * K
+    if flat.numel() < need:
+        raise RuntimeError(f"out_store holds {flat.numel()} elements, the layer produced {need}")
+    out = output if output is not None else torch.empty((t, K), dtype=torch.float16, device=flat.device)
+    assert out.shape == (t, K) and out.dtype == torch.float16 and out.is_contiguous()
+    ws = torch.empty(lib.mxmoe_combine_workspace_bytes(t, k), dtype=torch.uint8, device=flat.device)
+    shared_ptr = flat.data_ptr() + rows * K * 2 if num_shared_experts else None
+    _lib.check(lib, lib.mxmoe_unpermute_combine(flat.data_ptr(), shared_ptr, w.data_ptr(), slot.data_ptr(), rows, t, k, K, out.data_ptr(), ws.data_ptr(), _stream()))
+    return out
+
+
 def _problem_lists(num_experts: int, experts, recv_cpu, num_tokens: int):
     has_shared = len(experts) > num_experts
     for e in range(num_experts + (1 if has_shared else 0)):

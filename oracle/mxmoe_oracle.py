@@ -428,3 +428,28 @@ def linear_block(x: np.ndarray, w: np.ndarray, qp, rotate: bool):
     wq = fake_quant(w, w_bits, g, sym) if w_bits < 16 else w
     out = gemm_fakequant(x, wq)
     return out, out, None
+
+
+def unpermute_combine(down_rows, src_slot, topk_weights, shared=None):
+    """The step after the down projection: out[t] = sum_k w[t, k] * down(row of (t, k)) + shared[t].
+
+    The reference only has an empty stub for it (`gg_unpermute_out`, mxmoe/kernels/src/ref_bind.cu:66); the arithmetic fixed here is
+    fp32, slots in ascending k, every product and every sum rounded to fp32, one final rounding to fp16.  `src_slot[r]` is the
+    flattened (token, slot) index of sorted row r (rows of dropped expert ids simply do not appear).
+    Pinned by: one-hot weights return the routed row itself, a dense float64 evaluation to fp16 tolerance, invariance under the
+    order of the sorted rows (tests/test_oracle_host.py)."""
+    w = np.asarray(topk_weights, dtype=np.float32)
+    t, k = w.shape
+    rows = np.asarray(down_rows, dtype=np.float16)
+    row_of = np.full(t * k, -1, dtype=np.int64)
+    row_of[np.asarray(src_slot, dtype=np.int64)] = np.arange(len(src_slot))
+    acc = np.zeros((t, rows.shape[1]), dtype=np.float32)
+    for j in range(k):
+        r = row_of.reshape(t, k)[:, j]
+        ok = r >= 0
+        prod = (w[ok, j][:, None] * rows[r[ok]].astype(np.float32)).astype(np.float32)
+        acc[ok] = (acc[ok] + prod).astype(np.float32)
+    if shared is not None:
+        acc = (acc + np.asarray(shared, dtype=np.float16).astype(np.float32)).astype(np.float32)
+    return acc.astype(np.float16)
+

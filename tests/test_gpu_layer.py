@@ -78,3 +78,42 @@ def test_mixed_layer_with_shared_expert_within_tolerance():
         assert _rel(r["g_mid"], r["mid"]) <= 1e-2, f"gate_up, expert {r['e']}"
         # the down input differs in the last fp16 bit from the oracle's, so compare the end result at the stated tolerance
         assert _rel(r["g_out"], r["out"]) <= 1e-2, f"down, expert {r['e']}"
+
+
+def test_unpermute_combine_bit_exact():
+    """The step after the down launch against the oracle: routed only, with a shared expert, and with dropped expert ids."""
+    from mxmoe_amd import ops
+
+    rng = np.random.default_rng(11)
+    for (t, k, e, n, shared, drop) in [(50, 4, 8, 256, False, False), (33, 6, 16, 1408, True, False), (17, 2, 4, 2048, True, True), (1, 1, 1, 8, False, False)]:
+        ids = np.stack([rng.permutation(e)[:k] for _ in range(t)]).astype(np.int32)
+        if drop:
+            ids[::3, 0] = e + 5                  # ids outside [0, E) are dropped by the permutation
+        _, _, slot, recv = O.permute_by_expert(np.where(ids < e, ids, e), e + 1)
+        rows_n = int(recv[:e].sum())
+        slot = slot[:rows_n]
+        rows = rng.standard_normal((rows_n, n)).astype(F16)
+        sh = rng.standard_normal((t, n)).astype(F16) if shared else None
+        w = rng.random((t, k)).astype(np.float32)
+        store = np.concatenate([rows.reshape(-1)] + ([sh.reshape(-1)] if shared else []))
+        out = ops.gg_unpermute_out(torch.from_numpy(store).cuda(), torch.from_numpy(ids).cuda(), torch.from_numpy(w).cuda(), e, n, 2 if shared else 0)
+        ref = O.unpermute_combine(rows, slot, w, sh)
+        assert np.array_equal(out.cpu().numpy().view(np.uint16), ref.view(np.uint16)), (t, k, e, n, shared, drop)
+
+
+def test_layer_combine_end_to_end():
+    from mxmoe_amd import synth
+    from mxmoe_amd.layer import MxMoELayer
+
+    cfg = synth.MoEConfig("t", "test", 6, 2, 256, 1408, 48, num_shared=2, rotate=1, formats=(synth.W4A4, synth.W8A8), format_probs=(0.5, 0.5))
+    hidden = synth.make_hidden(cfg)
+    ids, w = synth.make_routing(cfg)
+    layer = MxMoELayer(cfg)
+    outs = layer.forward(hidden, ids)
+    final = layer.combine(w)
+    torch.cuda.synchronize()
+    _, _, slot, recv = O.permute_by_expert(ids.numpy(), cfg.num_experts)
+    rows = np.concatenate([o.cpu().numpy() for o in outs[:-1]])
+    ref = O.unpermute_combine(rows, slot, w.numpy(), outs[-1].cpu().numpy())
+    assert final.shape == (cfg.tokens, cfg.hidden)
+    assert np.array_equal(final.cpu().numpy().view(np.uint16), ref.view(np.uint16))

@@ -63,3 +63,58 @@ def test_tile_scheduler_visits_every_tile_once():
             seen.add((pi, tm, tn))
         assert len(seen) == sum(-(-m // bm) * -(-n // bn) for (m, n), (bm, bn) in zip(mn, tiles))
         assert O.tile_to_problem(prefix[-1], prefix, mn, tiles)[0] == -1
+
+
+# ---- un-permute + top-k weighted combine ----
+
+def _combine_case(seed, t=7, k=3, e=5, n=16, drop=False):
+    rng = np.random.default_rng(seed)
+    ids = np.stack([rng.permutation(e)[:k] for _ in range(t)]).astype(np.int32)
+    _, _, slot, recv = O.permute_by_expert(ids, e)
+    rows = rng.standard_normal((int(recv.sum()), n)).astype(np.float16)
+    w = rng.random((t, k)).astype(np.float32)
+    w /= w.sum(1, keepdims=True)
+    return ids, slot, rows, w
+
+
+def test_combine_one_hot_weights_return_the_routed_row():
+    ids, slot, rows, w = _combine_case(0)
+    t, k = w.shape
+    for j in range(k):
+        onehot = np.zeros_like(w)
+        onehot[:, j] = 1.0
+        out = O.unpermute_combine(rows, slot, onehot)
+        for tok in range(t):
+            r = int(np.where(slot == tok * k + j)[0][0])
+            assert np.array_equal(out[tok].view(np.uint16), rows[r].view(np.uint16))
+
+
+def test_combine_matches_dense_float64_and_adds_shared():
+    ids, slot, rows, w = _combine_case(1, t=33, k=4, e=9, n=64)
+    t, k = w.shape
+    shared = np.random.default_rng(2).standard_normal((t, 64)).astype(np.float16)
+    dense = np.zeros((t, 64))
+    for r, s in enumerate(slot):
+        dense[s // k] += float(w[s // k, s % k]) * rows[r].astype(np.float64)
+    out = O.unpermute_combine(rows, slot, w)
+    assert np.abs(out.astype(np.float64) - dense).max() <= 2e-3 * np.abs(dense).max()
+    out_s = O.unpermute_combine(rows, slot, w, shared)
+    assert np.abs(out_s.astype(np.float64) - (dense + shared.astype(np.float64))).max() <= 2e-3 * np.abs(dense + shared).max()
+    # a wrong sign, a dropped shared term or a transposed weight matrix would fail the two checks above; slot order is fixed:
+    flipped = O.unpermute_combine(rows, slot, w[:, ::-1].copy())
+    assert not np.array_equal(flipped, out)
+
+
+def test_combine_does_not_depend_on_the_order_of_the_sorted_rows():
+    ids, slot, rows, w = _combine_case(3, t=12, k=2, e=4, n=8)
+    p = np.random.default_rng(4).permutation(len(slot))
+    assert np.array_equal(O.unpermute_combine(rows, slot, w), O.unpermute_combine(rows[p], slot[p], w))
+
+
+def test_combine_skips_dropped_slots():
+    ids, slot, rows, w = _combine_case(5, t=6, k=2, e=3, n=8)
+    keep = slot % 2 == 0                         # pretend every second slot's expert id was out of range
+    out = O.unpermute_combine(rows[keep], slot[keep], w)
+    w0 = w.copy()
+    w0[:, 1] = 0.0
+    assert np.array_equal(out, O.unpermute_combine(rows, slot, w0))
