@@ -152,6 +152,33 @@ def cpu_baseline(cfg, budget_s: float = 20.0):
                       f"activation fake-quant + fp32 matmuls + SiLU timed, {spent:.1f} s"}
 
 
+def time_whole_layer(cfg, layer, reps: int = 5) -> dict:
+    """Wall time of the whole layer forward as a caller of the ops sees it (permute + rotate + quantise, gate_up launch, SiLU*up +
+    rotate + quantise, down launch, un-permute + combine), including the host work of the ops (offset tables, allocations).
+    Reported next to the GroupGEMM figure, never as `value`."""
+    import torch
+
+    from mxmoe_amd import synth
+
+    hidden = synth.make_hidden(cfg).cuda()
+    ids, w = synth.make_routing(cfg)
+    ids, w = ids.cuda(), w.cuda()
+    parts = {"prologue": 0.0, "gate_up": 0.0, "act": 0.0, "down": 0.0, "combine": 0.0}
+    for rep in range(reps + 1):
+        torch.cuda.synchronize()
+        marks = [time.perf_counter()]
+        for fn in (lambda: layer.prepare(hidden, ids), layer.gate_up, layer.act, layer.down, lambda: layer.combine(w)):
+            fn()
+            torch.cuda.synchronize()
+            marks.append(time.perf_counter())
+        if rep:  # first repetition warms allocations up
+            for k, a, b in zip(parts, marks, marks[1:]):
+                parts[k] += (b - a) * 1e3 / reps
+    out = {f"{k}_ms": round(v, 4) for k, v in parts.items()}
+    out["layer_ms"] = round(sum(parts.values()), 4)
+    return out
+
+
 def run_workload(name: str, steps: int, warmup: int, tokens=None):
     cfg, layer = build_layer(name, tokens)
     ms, up, dn = time_layer(layer, steps, warmup)
@@ -161,7 +188,7 @@ def run_workload(name: str, steps: int, warmup: int, tokens=None):
         "workload": name, "tops": round(ops / (ms * 1e-3) / 1e12, 2), "ms_per_step": round(ms, 4),
         "gate_up_us": round(up * 1e3, 2), "down_us": round(dn * 1e3, 2),
         "gate_up_tops": round(st["gg1"].ops / (up * 1e-3) / 1e12, 2), "down_tops": round(st["gg2"].ops / (dn * 1e-3) / 1e12, 2),
-        "ops": ops, "roofline": roofline_of(cfg, layer, up, dn),
+        "ops": ops, "roofline": roofline_of(cfg, layer, up, dn), "whole_layer": time_whole_layer(cfg, layer),
     }
 
 
@@ -224,7 +251,7 @@ def main() -> int:
         "config": {"workload": f"{args.workload}: {cfg.description}", "experts": cfg.num_experts, "topk": cfg.topk, "hidden": cfg.hidden,
                    "intermediate": cfg.inter, "tokens": cfg.tokens, "formats": fm, "step": "gate_up GroupGEMM launch + down GroupGEMM launch"},
         "roofline": main_res["roofline"],
-        "detail": {k: main_res[k] for k in ("gate_up_us", "down_us", "gate_up_tops", "down_tops", "ops")},
+        "detail": {k: main_res[k] for k in ("gate_up_us", "down_us", "gate_up_tops", "down_tops", "ops", "whole_layer")},
         "also": also,
     }
     if not args.no_cpu_baseline:

@@ -163,25 +163,69 @@ __global__ void __launch_bounds__(256) row_quant_kernel(const RowArgs a) {
     for (int i = tid; i < a.plan.kb * a.plan.kb; i += 256) sg[i] = a.signs[i];
   }
 
+  // Row bookkeeping (expert, tag, offsets, source pointer) and the row's data are fetched one row ahead: each is a chain of
+  // dependent global loads, several microseconds long, that must not sit in front of every row's arithmetic.
+  struct RowMeta {
+    int e, tag;
+    long start_row, inp_off, scale_off;
+    const _Float16* srow;
+    bool shared_row;
+  };
+  auto load_meta = [&](int row) {
+    RowMeta m;
+    m.shared_row = row >= a.R;
+    m.e = m.shared_row ? a.E : a.dst_exp[row];
+    m.tag = (int)a.table[m.e];
+    m.start_row = a.table[a.Et + m.e];
+    m.inp_off = a.table[2 * a.Et + m.e];
+    m.scale_off = a.table[3 * a.Et + m.e];
+    const int n = (m.shared_row ? a.plan_shared : a.plan).n;
+    if (SILU) {
+      m.srow = m.shared_row ? a.src_shared + (long)(row - a.R) * 2 * n : a.src + (long)row * 2 * n;
+    } else {
+      m.srow = a.src + (m.shared_row ? (long)(row - a.R) : (long)a.perm[row]) * n;
+    }
+    return m;
+  };
+  auto load_data = [&](const RowMeta& m, v8h (&g)[MAXC], v8h (&u)[MAXC]) {
+    const int n = (m.shared_row ? a.plan_shared : a.plan).n;
+#pragma unroll
+    for (int i = 0; i < MAXC; ++i) {
+      const int c = tid + i * 256;
+      if (c < (n >> 3)) {
+        g[i] = *reinterpret_cast<const v8h*>(m.srow + c * 8);
+        if (SILU) u[i] = *reinterpret_cast<const v8h*>(m.srow + n + c * 8);
+      }
+    }
+  };
+  RowMeta next_meta;
+  v8h next_g[MAXC], next_u[MAXC];
+  if ((int)blockIdx.x < a.rows) {
+    next_meta = load_meta(blockIdx.x);
+    load_data(next_meta, next_g, next_u);
+  }
+
   for (int row = blockIdx.x; row < a.rows; row += gridDim.x) {
-    const bool shared_row = row >= a.R;
-    const int e = shared_row ? a.E : a.dst_exp[row];
+    const RowMeta cur = next_meta;
+    v8h cur_g[MAXC], cur_u[MAXC];
+#pragma unroll
+    for (int i = 0; i < MAXC; ++i) {
+      cur_g[i] = next_g[i];
+      if (SILU) cur_u[i] = next_u[i];
+    }
+    if (row + (int)gridDim.x < a.rows) {
+      next_meta = load_meta(row + gridDim.x);
+      load_data(next_meta, next_g, next_u);
+    }
+    const bool shared_row = cur.shared_row;
     const RotPlan pl = shared_row ? a.plan_shared : a.plan;
     const int n = pl.n;
     const int nchunks = n >> 3;
-    const int tag = (int)a.table[e];
-    const long start_row = a.table[a.Et + e];
-    const long inp_off = a.table[2 * a.Et + e];
-    const long scale_off = a.table[3 * a.Et + e];
-    const long lrow = row - start_row;
+    const int tag = cur.tag;
+    const long inp_off = cur.inp_off;
+    const long scale_off = cur.scale_off;
+    const long lrow = row - cur.start_row;
     const bool rot = a.rotate == 2 || (a.rotate == 1 && tag != 0);
-
-    const _Float16* srow;
-    if (SILU) {
-      srow = shared_row ? a.src_shared + (long)(row - a.R) * 2 * n : a.src + (long)row * 2 * n;
-    } else {
-      srow = a.src + (shared_row ? (long)(row - a.R) : (long)a.perm[row]) * n;
-    }
 
     float v[MAXC][8];
     __syncthreads();  // previous row fully consumed (and the sign table staged)
@@ -189,9 +233,9 @@ __global__ void __launch_bounds__(256) row_quant_kernel(const RowArgs a) {
     for (int i = 0; i < MAXC; ++i) {
       const int c = tid + i * 256;
       if (c < nchunks) {
-        const v8h g = *reinterpret_cast<const v8h*>(srow + c * 8);
+        const v8h g = cur_g[i];
         if (SILU) {
-          const v8h u = *reinterpret_cast<const v8h*>(srow + n + c * 8);
+          const v8h u = cur_u[i];
 #pragma unroll
           for (int j = 0; j < 8; ++j) {
             const float gf = (float)g[j];
@@ -378,6 +422,135 @@ __global__ void __launch_bounds__(256) row_quant_kernel(const RowArgs a) {
   }
 }
 
+// One row per WAVE, for rows whose rotation is a pure Sylvester transform (n = 512 * NI, NI a power of two): lane l holds the NI
+// 8-element chunks l + 64*i.  The butterfly strides map to three levels, taken in the same ascending order as everywhere else:
+// 1, 2, 4 inside a chunk (registers), 8 .. 256 across the lanes (cross-lane exchange, no LDS staging, no barrier),
+// 512 .. n/2 between a lane's own chunks (registers).  Four independent rows per workgroup, nothing shared between them.
+template <int NI, bool SILU>
+__global__ void __launch_bounds__(256) row_quant_wave_kernel(const RowArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int n = a.plan.n;  // == a.plan_shared.n == 512 * NI
+  const int stride_rows = gridDim.x * 4;
+  for (int row = blockIdx.x * 4 + wave; row < a.rows; row += stride_rows) {
+    const bool shared_row = row >= a.R;
+    const int e = shared_row ? a.E : a.dst_exp[row];
+    const int tag = (int)a.table[e];
+    const long lrow = row - a.table[a.Et + e];
+    const long inp_off = a.table[2 * a.Et + e];
+    const long scale_off = a.table[3 * a.Et + e];
+    const bool rot = a.rotate == 2 || (a.rotate == 1 && tag != 0);
+    const _Float16* srow;
+    if (SILU) {
+      srow = shared_row ? a.src_shared + (long)(row - a.R) * 2 * n : a.src + (long)row * 2 * n;
+    } else {
+      srow = a.src + (shared_row ? (long)(row - a.R) : (long)a.perm[row]) * n;
+    }
+    float v[NI][8];
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int c = lane + 64 * i;
+      const v8h g = *reinterpret_cast<const v8h*>(srow + c * 8);
+      if (SILU) {
+        const v8h u = *reinterpret_cast<const v8h*>(srow + n + c * 8);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float gf = (float)g[j];
+          const float s = gf / (1.0f + exp_fixed(-gf));
+          v[i][j] = round_h(keep_f32(s * (float)u[j]));
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[i][j] = (float)g[j];
+      }
+    }
+    if (rot) {
+#pragma unroll
+      for (int i = 0; i < NI; ++i)
+#pragma unroll
+        for (int h = 1; h < 8; h <<= 1)
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            if (!(j & h)) {
+              const float p = v[i][j], q = v[i][j + h];
+              v[i][j] = p + q;
+              v[i][j + h] = p - q;
+            }
+#pragma unroll
+      for (int m = 1; m < 64; m <<= 1) {
+        const bool upper = lane & m;
+#pragma unroll
+        for (int i = 0; i < NI; ++i)
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const float o = __shfl_xor(v[i][j], m);
+            v[i][j] = upper ? o - v[i][j] : v[i][j] + o;
+          }
+      }
+#pragma unroll
+      for (int hi = 1; hi < NI; hi <<= 1)
+#pragma unroll
+        for (int i = 0; i < NI; ++i)
+          if (!(i & hi)) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+              const float p = v[i][j], q = v[i + hi][j];
+              v[i][j] = p + q;
+              v[i + hi][j] = p - q;
+            }
+          }
+#pragma unroll
+      for (int i = 0; i < NI; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[i][j] = round_h(keep_f32(v[i][j] * a.plan.scale));
+    }
+    if (tag == 0) {
+      _Float16* out = reinterpret_cast<_Float16*>(a.inp_store) + inp_off + lrow * n;
+#pragma unroll
+      for (int i = 0; i < NI; ++i) {
+        v8h o;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) o[j] = (_Float16)v[i][j];
+        *reinterpret_cast<v8h*>(out + (lane + 64 * i) * 8) = o;
+      }
+      continue;
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[i][j]));
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
+    const float upper = tag == 1 ? 127.0f : 7.0f;
+    float scale = round_h(amax / upper);   // fp16 division: fp32 quotient of two fp16 values, rounded to fp16
+    if (scale == 0.0f) scale = 1.0f;       // quantize.cuh:258
+    if (lane == 0) a.scale_store[scale_off + lrow] = (_Float16)scale;
+    uint8_t* out = a.inp_store + 2 * (inp_off + lrow * (tag == 1 ? n / 2 : n / 4));
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int c = lane + 64 * i;
+      int q[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float r = round_h(v[i][j] / scale);
+        q[j] = (int)rintf(fminf(fmaxf(r, -upper), upper));
+      }
+      if (tag == 1) {
+        uint2 w;
+        w.x = (q[0] & 0xFF) | ((q[1] & 0xFF) << 8) | ((q[2] & 0xFF) << 16) | ((unsigned)(q[3] & 0xFF) << 24);
+        w.y = (q[4] & 0xFF) | ((q[5] & 0xFF) << 8) | ((q[6] & 0xFF) << 16) | ((unsigned)(q[7] & 0xFF) << 24);
+        *reinterpret_cast<uint2*>(out + c * 8) = w;
+      } else {
+        unsigned w = 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) w |= (unsigned)(q[j] & 0xF) << (4 * j);
+        *reinterpret_cast<unsigned*>(out + c * 4) = w;
+      }
+    }
+  }
+}
+
 static int make_plan(int n, int had_k, int had_f, bool rotate, RotPlan* p) {
   p->n = n;
   p->scale = 1.0f / sqrtf((float)n);
@@ -405,6 +578,23 @@ static int launch_rows(const RowArgs& a, int lds_bytes, hipStream_t s) {
   if (lds_bytes > 64 * 1024) {
     last_error() = "row too long for the activation kernels";
     return 3;
+  }
+  // pure power-of-two rows (no table-driven Hadamard factor): one row per wave
+  const int n = a.plan.n;
+  if (a.plan.kb == 1 && a.plan_shared.kb == 1 && a.plan_shared.n == n && n % 512 == 0 && n <= 4096 && (n & (n - 1)) == 0) {
+    const int wgrid = (a.rows + 3) / 4 < cus * 8 ? (a.rows + 3) / 4 : cus * 8;
+    switch (n / 512) {
+      case 1: hipLaunchKernelGGL((row_quant_wave_kernel<1, SILU>), dim3(wgrid), dim3(256), 0, s, a); break;
+      case 2: hipLaunchKernelGGL((row_quant_wave_kernel<2, SILU>), dim3(wgrid), dim3(256), 0, s, a); break;
+      case 4: hipLaunchKernelGGL((row_quant_wave_kernel<4, SILU>), dim3(wgrid), dim3(256), 0, s, a); break;
+      default: hipLaunchKernelGGL((row_quant_wave_kernel<8, SILU>), dim3(wgrid), dim3(256), 0, s, a); break;
+    }
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+      last_error() = std::string("kernel launch failed: ") + hipGetErrorString(e);
+      return 4;
+    }
+    return 0;
   }
   if (chunks <= 1) hipLaunchKernelGGL((row_quant_kernel<1, SILU>), dim3(grid), dim3(256), lds_bytes, s, a);
   else if (chunks <= 2) hipLaunchKernelGGL((row_quant_kernel<2, SILU>), dim3(grid), dim3(256), lds_bytes, s, a);

@@ -65,10 +65,12 @@ template <int I, class T, class... Rest>
 struct Dispatch<I, T, Rest...> {
   __device__ static __forceinline__ void go(int branch, TileArgs& t, int local, uint8_t* smem) {
     if (branch == I) {
-      // tile_scheduler.cuh:40-49: local index -> (row tile, column tile), column tile fastest
-      const int grid_n = (t.N + T::BN - 1) / T::BN;
-      t.tile_m = local / grid_n;
-      t.tile_n = local - t.tile_m * grid_n;
+      // local index -> (row tile, column tile) as tile_scheduler.cuh:40-49, but row tile fastest: neighbouring workgroups then share
+      // one block of weight rows (the large operand: it is fetched once per expert) and sweep the expert's activations, which
+      // are small enough to stay in L2
+      const int grid_m = (t.M - t.row0 + T::BM - 1) / T::BM;
+      t.tile_n = local / grid_m;
+      t.tile_m = local - t.tile_n * grid_m;
       T::run(t, smem);
     } else {
       Dispatch<I + 1, Rest...>::go(branch, t, local, smem);
