@@ -324,7 +324,7 @@ __global__ void __launch_bounds__(256) row_quant_kernel(const RowArgs a) {
               const float s = sr[bp];
               const float* vv = vb + (long)bp * mc * 8;
 #pragma unroll
-              for (int j = 0; j < 8; ++j) acc[j] = acc[j] + s * vv[j];
+              for (int j = 0; j < 8; ++j) acc[j] = __builtin_fmaf(s, vv[j], acc[j]);  // s = +-1: the product is exact, so this is acc + s*v
             }
 #pragma unroll
             for (int j = 0; j < 8; ++j) v[i][j] = acc[j];
