@@ -43,9 +43,13 @@ int mxmoe_kernel_branch(int kernel_id, int branch, int32_t out[8]);
  *
  *   format            As[p]                      Bs[p]                               scale_a[p]      scale_b[p]
  *   fp16              fp16 [M,K]                 fp16 [N,K]                          -               -
- *   w8a8_g-1_sym      int8 [M,K]                 int8 [N,K]                          fp16 [M]        fp16 [N]
- *   w4a4_g-1_sym      int4 [M,K/2] (even k low)  int4 [N,K/2]                        fp16 [M]        fp16 [N]
+ *   w8a8_g-1_sym      int8 [M,K]                 fragment blocks of int8 [N,K]  (*)  fp16 [M]        fp16 [N]
+ *   w4a4_g-1_sym      int4 [M,K/2] (even k low)  fragment blocks of int4 [N,K/2] (*) fp16 [M]        fp16 [N]
  *   w{4,3}a16_g128    fp16 [M,K]                 packed [N/16][K/128][64][w dwords]  -               fp16 [N/16][K/128][16][2]
+ *
+ * (*) weights of the integer formats are stored in MFMA fragment order: uint8 [ceil(N/32)][KB/64][2][64 lanes][16], KB = bytes per
+ *     row; lane l of block (nb, ks, step) holds bytes ks*64 + (2*step + (l >> 5))*16 .. +16 of channel nb*32 + (l & 31), channels past N
+ *     are zero (mxmoe_amd.pack.pack_wxax_fragments; the role of the reference's pack_wxax / permute_weight, quantize.cuh:318-381,424-475).
  *
  * kernel_id = -1 selects the first registered kernel that has a tile for every format in h_q.
  * acc_dump (optional, may be NULL) is a DEVICE array of per-problem int32 [M,N] buffers (entries may be NULL) that

@@ -6,12 +6,12 @@ namespace {
 // Default fused kernels.  Generated libraries (mxmoe_amd.kernels.compose_kernel) register their own sets.
 struct DefaultKernels {
   DefaultKernels() {
-    register_fused<MfmaTile<Op::I4, 256, 128, 2, 2>, MfmaTile<Op::I4, 128, 256, 2, 2>, MfmaTile<Op::I4, 64, 256, 1, 4>, MfmaTile<Op::I4, 32, 256, 1, 4>,
-                   MfmaTile<Op::I8, 128, 256, 2, 2>, MfmaTile<Op::I8, 64, 256, 1, 4>, MfmaTile<Op::I8, 32, 256, 1, 4>>("groupgemm_hz_fused_wxax");
+    register_fused<WxAxTile<Op::I4, 128, 256>, WxAxTile<Op::I4, 64, 256>, WxAxTile<Op::I4, 32, 256>,
+                   WxAxTile<Op::I8, 128, 256>, WxAxTile<Op::I8, 64, 256>, WxAxTile<Op::I8, 32, 256>>("groupgemm_hz_fused_wxax");
     register_fused<MfmaTile<Op::F16, 128, 256, 2, 2>, MfmaTile<Op::F16, 64, 256, 1, 4>, MfmaTile<Op::F16, 32, 256, 1, 4>>("groupgemm_hz_fused_fp16");
     register_fused<SkinnyWoTile<4, 128>, SkinnyWoTile<3, 128>, WoMfmaTile<4>, WoMfmaTile<3>>("groupgemm_hz_fused_wo");
     // every format in one launch (layers that mix weight-only, w-a and fp16 blocks)
-    register_fused<MfmaTile<Op::I4, 128, 256, 2, 2>, MfmaTile<Op::I4, 32, 256, 1, 4>, MfmaTile<Op::I8, 128, 256, 2, 2>, MfmaTile<Op::I8, 32, 256, 1, 4>,
+    register_fused<WxAxTile<Op::I4, 128, 256>, WxAxTile<Op::I4, 32, 256>, WxAxTile<Op::I8, 128, 256>, WxAxTile<Op::I8, 32, 256>,
                    MfmaTile<Op::F16, 128, 256, 2, 2>, MfmaTile<Op::F16, 32, 256, 1, 4>, SkinnyWoTile<4, 128>, SkinnyWoTile<3, 128>, WoMfmaTile<4>, WoMfmaTile<3>>("groupgemm_hz_fused_all");
   }
 };

@@ -162,6 +162,13 @@ struct BranchOf<MfmaTile<OP, BM, BN, WGM, WGN>> {
     return BranchInfo{f, BM, BN, T::BK, WGM, WGN, T::kLdsBytes, T::BK, 0};
   }
 };
+template <Op OP, int BM, int BN>
+struct BranchOf<WxAxTile<OP, BM, BN>> {
+  static BranchInfo get() {
+    using T = WxAxTile<OP, BM, BN>;
+    return BranchInfo{OP == Op::I8 ? Fmt::W8A8 : Fmt::W4A4, BM, BN, T::BK, 1, 4, T::kLdsBytes, T::BK, 0};
+  }
+};
 template <int WBITS, int BN>
 struct BranchOf<SkinnyWoTile<WBITS, BN>> {
   static BranchInfo get() {

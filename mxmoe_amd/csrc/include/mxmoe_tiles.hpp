@@ -434,4 +434,279 @@ struct MfmaTile {
   }
 };
 
+// ---------------------------------------------------------------------------------------------------------------------------------
+// WxAxTile: w4a4 / w8a8 tile whose WEIGHTS never touch LDS.
+//
+// Expert weights are static, so they are stored in HBM in MFMA fragment order (mxmoe_amd.pack.pack_wxax_fragments):
+//   [N/32 channel blocks][K slices of 64 B][2 k-steps][64 lanes][16 B],  lane l = 16-byte k-group (l >> 5) of channel (l & 31).
+// A wave's operand of one k-step of one 32-channel block is then a single coalesced 1 KB load straight into registers.  The 4
+// waves of a workgroup each own BN/4 = 64 channels (no weight is loaded twice) and all BM token rows; only the activations
+// (BM x 64 B per slice) go through LDS (direct-to-LDS loads, 3-stage ring, swizzled as in MfmaTile).  Compared with staging
+// both operands, LDS carries a third of the write traffic and two thirds of the read traffic of a w8a8 slice, and the reads
+// no longer queue behind landing weight data.
+//
+// Pipeline unit = one k-step of one 32-channel block (2*FM or FM MFMAs), 4 units per K slice.  At unit u the wave
+//   - issues this unit's share of the activation loads of slice kt+2 and re-loads the weight fragment used by unit u-1 for
+//     slice kt+kDepth (its registers are free again): kDepth * 4 KB of weights per wave are always in flight;
+//   - at the first unit of a k-step reads the activation fragments of the next k-step from LDS;
+//   - int4: widens the weight fragment of unit u+1, and on the last unit of a k-step the activation fragments of the next
+//     k-step, each right after its last use.
+// Waits: vmcnt counts the direct-to-LDS loads and the weight loads together, in issue order; the barrier unit (2) waits until
+// only the loads issued after this wave's activation loads of slice kt+1 are outstanding (a fixed count, see kYounger).
+template <Op OP, int BM_, int BN_>
+struct WxAxTile {
+  static_assert(OP == Op::I4 || OP == Op::I8, "integer formats only");
+  static constexpr Op kOp = OP;
+  static constexpr int BM = BM_, BN = BN_, WGM = 1, WGN = 4;
+  static constexpr int TM = BM, TN = BN / 4;
+  static constexpr int FM = TM / 32, FN = TN / 32;
+  static_assert(BM % 32 == 0 && FN == 2, "BM x 256 tiles: 4 waves x 64 channels");
+  static constexpr int kBits = OpTraits<OP>::kBitsPerElem;
+  static constexpr int BK = kRowBytes * 8 / kBits;
+  static constexpr int kStageBytes = BM * kRowBytes;
+  static constexpr int kStages = 3;
+  static constexpr int kPitch = TN * 2 + 8;                      // bytes per token row of the epilogue patch
+  static constexpr int FI = FM >= 2 ? 2 : 1;                     // 32-row blocks of the patch written per round
+  static constexpr int kPatchBytes = kWaves * FI * 32 * kPitch;
+  static constexpr int kLdsBytes = kStages * kStageBytes > kPatchBytes ? kStages * kStageBytes : kPatchBytes;
+  static constexpr int kAccRegs = FM * FN * 16;
+  static constexpr int kOps = OP == Op::I4 ? 2 : 1;
+  static constexpr int U = 4;                                    // units per K slice
+  static constexpr int kDmaTotal = BM / 16;                      // 1 KB pieces of one activation slice
+  static constexpr int kDma = (kDmaTotal + kWaves - 1) / kWaves;
+  static_assert(kDmaTotal % kWaves == 0 || kDma == 1, "a wave has either all kDma pieces or none");
+  static_assert(kDma <= U, "one activation load per unit");
+  // loads issued after a wave's last activation load of a slice and before the barrier unit of the next iteration
+  static constexpr int kYounger = (U - (kDma - 1)) + (kDma < 2 ? kDma : 2) + 2;
+  // K slices of weight fragments in flight per wave: int8 slices are half as long in time, so they are fetched further ahead
+  static constexpr int kDepth = OP == Op::I4 ? 2 : 4;
+  using Acc = v16i;
+
+  __device__ static __forceinline__ void widen(const v4i& p, v4i* o) {
+    if constexpr (OP == Op::I4) {
+      o[0] = (p << 4) & (int)0xF0F0F0F0;
+      o[1] = p & (int)0xF0F0F0F0;
+    } else {
+      o[0] = p;
+    }
+  }
+
+  __device__ static __forceinline__ void run(const TileArgs& t, uint8_t* __restrict__ smem) {
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int M = t.M, N = t.N;
+    const long row_bytes = (long)t.K * kBits / 8;
+    const int KT = (int)(row_bytes / kRowBytes);
+    const int m0 = t.row0 + t.tile_m * BM, n0 = t.tile_n * BN;
+
+    // activations: global -> LDS
+    const int a_rows = min(BM, M - m0);
+    const v4i rs_a = make_rsrc(t.A + (long)m0 * row_bytes, (unsigned)(a_rows * row_bytes));
+    const int lds_base = (int)(uintptr_t)smem;
+    int dma_voff[kDma];
+#pragma unroll
+    for (int i = 0; i < kDma; ++i) {
+      const int r = (wave + kWaves * i) * 16 + (lane >> 2);
+      dma_voff[i] = r * (int)row_bytes + (((lane & 3) ^ lds_swizzle(r)) << 4);
+    }
+    auto dma_a = [&](int i, int kt, int stage) {
+      const int ii = wave + kWaves * i;
+      if (kDmaTotal % kWaves == 0 || ii < kDmaTotal) {
+        v4i rs = rs_a;
+        if (kt >= KT) rs[2] = 0;  // past the end of K: a load of zero bytes, still counted by vmcnt
+        dma16_to_lds(rs, lds_base + stage * kStageBytes + ii * 1024, dma_voff[i], __builtin_amdgcn_readfirstlane(kt * kRowBytes));
+      }
+    };
+    const int lrow = lane & 31;
+    const int fa = lrow * kRowBytes + (((lane >> 5) ^ lds_swizzle(lrow)) << 4);
+    auto lds_a = [&](const uint8_t* st, int step, int i) { return *reinterpret_cast<const v4i*>(st + ((fa + i * 32 * kRowBytes) ^ (step << 5))); };
+
+    // weights: global -> registers, fragment (j, step) of slice kt at ((nb * KT + kt) * 2 + step) * 1 KB
+    const int nblk = (N + 31) / 32;
+    const uint8_t* bptr[FN];
+#pragma unroll
+    for (int j = 0; j < FN; ++j) {
+      const int nb = min(n0 / 32 + wave * FN + j, nblk - 1);  // blocks past N re-read the last one; their results are never stored
+      bptr[j] = t.B + (long)nb * KT * 2048 + lane * 16;
+    }
+    auto load_b = [&](int j, int step, int kt) { return gload<v4i>(bptr[j] + ((long)min(kt, KT - 1) * 2 + step) * 1024); };
+
+    Acc acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+      for (int j = 0; j < FN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+
+    v4i pbq[kDepth][FN][2];  // packed weight fragments [slice % kDepth][block][k-step]
+    v4i bop[2][kOps];        // int4: widened weight operands of units u, u+1
+    v4i aop[2][FM][kOps];    // activation operands; int8 double-buffers them by k-step parity, int4 widens in place (buffer 0)
+    v4i pa[FM];              // int4: packed activation fragments of the next k-step
+
+    auto mma = [&](Acc& c, const v4i* a, const v4i* b) {
+      c = __builtin_amdgcn_mfma_i32_32x32x32_i8(b[0], a[0], c, 0, 0, 0);
+      if constexpr (OP == Op::I4) c = __builtin_amdgcn_mfma_i32_32x32x32_i8(b[1], a[1], c, 0, 0, 0);
+    };
+
+    // ---- prologue: slices 0 .. kDepth-2 complete, then the load pattern of one (virtual) iteration for slice kDepth-1, so that
+    // the counts below hold from kt = 0
+#pragma unroll
+    for (int i = 0; i < kDma; ++i) dma_a(i, 0, 0);
+#pragma unroll
+    for (int d = 0; d < kDepth - 1; ++d)
+#pragma unroll
+      for (int j = 0; j < FN; ++j)
+#pragma unroll
+        for (int s = 0; s < 2; ++s) pbq[d][j][s] = load_b(j, s, d);
+    vm_wait<0>();
+    __syncthreads();
+    static_for<U>([&](auto uc) {
+      constexpr int u = decltype(uc)::value;
+      if constexpr (u < kDma) dma_a(u, 1, 1);
+      asm volatile("" ::: "memory");
+      if constexpr (u == 0) pbq[kDepth - 2][1][1] = load_b(1, 1, kDepth - 2);  // in place of "fragment of the previous iteration's last unit"
+      else pbq[kDepth - 1][(u - 1) % FN][(u - 1) / FN] = load_b((u - 1) % FN, (u - 1) / FN, kDepth - 1);
+      asm volatile("" ::: "memory");
+    });
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+      if constexpr (OP == Op::I4) {
+        const v4i p = lds_a(smem, 0, i);
+        widen(p, aop[0][i]);
+      } else {
+        aop[0][i][0] = lds_a(smem, 0, i);
+      }
+    }
+    if constexpr (OP == Op::I4) widen(pbq[0][0][0], bop[0]);
+
+    // ---- one K slice; P = kt % kDepth (compile-time, so the ring slots are fixed registers)
+    auto slice = [&](auto parc, int kt, const uint8_t* sc, const uint8_t* sn, int nstage) {
+      constexpr int P = decltype(parc)::value;
+      constexpr int Pprev = (P + kDepth - 1) % kDepth, Pnext = (P + 1) % kDepth;
+      static_for<U>([&](auto uc) {
+        constexpr int u = decltype(uc)::value;
+        constexpr int step = u / FN, j = u % FN;
+        if (u == 2) {
+          // this wave's activation loads of slice kt+1 have landed; after the barrier everybody's have, and everybody is done
+          // reading the stage that the loads of the next iteration overwrite
+          vm_wait<kYounger>();
+          __syncthreads();
+        }
+        if constexpr (u < kDma) dma_a(u, kt + 2, nstage);
+        asm volatile("" ::: "memory");
+        // re-load the fragment that unit u-1 used, kDepth slices ahead
+        if constexpr (u == 0) pbq[Pprev][1][1] = load_b(1, 1, kt - 1 + kDepth);
+        else pbq[P][(u - 1) % FN][(u - 1) / FN] = load_b((u - 1) % FN, (u - 1) / FN, kt + kDepth);
+        asm volatile("" ::: "memory");
+        // activation fragments of the next k-step
+        if (j == 0) {
+#pragma unroll
+          for (int i = 0; i < FM; ++i) {
+            const v4i p = step == 0 ? lds_a(sc, 1, i) : lds_a(sn, 0, i);
+            if constexpr (OP == Op::I4) pa[i] = p; else aop[step ^ 1][i][0] = p;
+          }
+        }
+        if constexpr (OP == Op::I4) {
+          // weight operands of unit u+1
+          if constexpr (u + 1 < U) widen(pbq[P][(u + 1) % FN][(u + 1) / FN], bop[(u + 1) & 1]);
+          else widen(pbq[Pnext][0][0], bop[0]);
+#pragma unroll
+          for (int i = 0; i < FM; ++i) {
+            mma(acc[i][j], aop[0][i], bop[u & 1]);
+            if (j == FN - 1) widen(pa[i], aop[0][i]);  // next k-step's operand, right after the last use of this one
+          }
+          __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, FM, 0);
+          sched_mfma_valu<12 + (j == FN - 1 ? 12 * FM : 0), 2 * FM, 0>();
+        } else {
+#pragma unroll
+          for (int i = 0; i < FM; ++i) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(pbq[P][j][step], aop[step][i][0], acc[i][j], 0, 0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      });
+    };
+
+    int sidx = 0;
+#pragma unroll 1
+    for (int kt0 = 0; kt0 < KT; kt0 += kDepth) {
+      static_for<kDepth>([&](auto dc) {
+        constexpr int d = decltype(dc)::value;
+        if (kt0 + d < KT) {
+          const int nidx = sidx == 2 ? 0 : sidx + 1;
+          const int nn = nidx == 2 ? 0 : nidx + 1;
+          slice(dc, kt0 + d, smem + sidx * kStageBytes, smem + nidx * kStageBytes, nn);
+          sidx = nidx;
+        }
+      });
+    }
+    vm_wait<0>();  // nothing may still land in LDS once the epilogue reuses it
+
+    // ---- epilogue (as MfmaTile): lane holds token lane & 31 and channels 8*(r/4) + 4*(lane >> 5) + (r & 3) of each 32x32 block
+    const int nq = (lane >> 5) * 4;
+    float s_a[FM];
+    v4h s_b[FN][4];
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+      const int m = min(m0 + i * 32 + lrow, M - 1);
+      s_a[i] = (float)gload<_Float16>(t.sa + m);
+      if constexpr (OP == Op::I4) s_a[i] *= 0.00390625f;  // the int4 accumulator holds 256 * sum (exact power of two)
+    }
+#pragma unroll
+    for (int j = 0; j < FN; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int n = min(n0 + wave * TN + j * 32 + q * 8 + nq, N - 4);
+        s_b[j][q] = gload<v4h>(t.sb + n);
+      }
+    if (t.acc_dump) {  // parity tests only
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int m = m0 + i * 32 + lrow, n = n0 + wave * TN + j * 32 + (r / 4) * 8 + nq + (r & 3);
+            int a = (int)acc[i][j][r];
+            if constexpr (OP == Op::I4) a >>= 8;  // exact
+            if (m < M && n < N) gstore<int>(t.acc_dump + (long)m * N + n, a);
+          }
+    }
+    __syncthreads();  // every wave is done reading the activation stages: LDS can be reused
+    uint8_t* patch = smem + wave * (FI * 32 * kPitch);
+    constexpr int kLanesPerRow = TN / 8, kRowsPerPass = 64 / kLanesPerRow;
+    const int pr = lane / kLanesPerRow, pc = lane % kLanesPerRow;
+#pragma unroll
+    for (int i0 = 0; i0 < FM; i0 += FI) {
+#pragma unroll
+      for (int ii = 0; ii < FI; ++ii) {
+        const int i = i0 + ii;
+        const int ml = ii * 32 + lrow;
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            v4h o;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              // float(acc) * (sa * sb) rounded once to half; the scale product stays in fp32 (see MfmaTile)
+              const float sc = s_a[i] * (float)s_b[j][q][e];
+              o[e] = (_Float16)keep_f32((float)acc[i][j][q * 4 + e] * sc);
+            }
+            *reinterpret_cast<v4h*>(patch + ml * kPitch + (j * 32 + q * 8 + nq) * 2) = o;
+          }
+      }
+#pragma unroll
+      for (int r0 = 0; r0 < FI * 32; r0 += kRowsPerPass) {
+        const int ml = r0 + pr;
+        const int m = m0 + i0 * 32 + ml;
+        const int n = n0 + wave * TN + pc * 8;
+        const v4i v = *reinterpret_cast<const v4i*>(patch + ml * kPitch + pc * 16);
+        if (m < M && n < N) gstore<v4i>(t.C + (long)m * N + n, v);
+      }
+    }
+  }
+};
+
 }  // namespace mxmoe

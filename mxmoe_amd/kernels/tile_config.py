@@ -168,6 +168,8 @@ class TileConfig:
             return 4 * (self.BN // 16) * (64 * 16 + 4 * 64)  # per-wave partial sums of the final reduction + (scale, zero) patches
         if self.is_weight_only():
             return 2 * self.BM * 256  # two stages of BM activation rows x one 128-wide k block
+        if self.MMA != "MFMA_F32_32x32x16_F16":  # activations only: 3 stages of BM x 64 B, or the epilogue patch if larger
+            return max(self.STAGE * self.BM * 64, 4 * min(self.BM, 64) * (64 * 2 + 8))
         return self.STAGE * (self.BM + self.BN) * 64
 
     def cpp_type(self) -> str:
@@ -177,6 +179,8 @@ class TileConfig:
         if self.is_weight_only():
             return f"WoMfmaTile<{self.QCFGB.QBITS}, {self.BM}, {self.BN}>"
         op = {"MFMA_F32_32x32x16_F16": "Op::F16", "MFMA_I32_32x32x32_I8": "Op::I8", "MFMA_I32_32x32x32_I8_FROM_I4": "Op::I4"}[self.MMA]
+        if op != "Op::F16":
+            return f"WxAxTile<{op}, {self.BM}, {self.BN}>"
         return f"MfmaTile<{op}, {self.BM}, {self.BN}, {self.WM}, {self.WN}>"
 
     def validate(self) -> None:
@@ -189,6 +193,8 @@ class TileConfig:
         k_elems = {"MFMA_F32_32x32x16_F16": 32, "MFMA_I32_32x32x32_I8": 64, "MFMA_I32_32x32x32_I8_FROM_I4": 128}[self.MMA]
         if self.BK != k_elems or self.STAGE != 3 or self.WK != 1 or (self.BM // self.WM) % 32 or (self.BN // self.WN) % 32:
             raise ValueError(f"{self!r}: unsupported shape for {self.MMA} (BK must be {k_elems}, STAGE 3, wave tile a multiple of 32x32)")
+        if self.MMA != "MFMA_F32_32x32x16_F16" and ((self.WM, self.WN) != (1, 4) or self.BN != 256 or self.BM not in (32, 64, 128)):
+            raise ValueError(f"{self!r}: integer tiles are BM x 256 with 1 x 4 waves (each wave streams its own 64 weight channels), BM in 32 / 64 / 128")
 
 
 def get_info_from_qcfg_str(qcfg: str):
@@ -227,7 +233,10 @@ def get_possible_tile_list(arch: str, qcfg: str) -> list:
         skinny = [_with_q(TileConfig(BM=16, BN=bn, BK=128, WM=1, WN=4, WK=1, STAGE=2, MMA=mma), qcfg) for bn in (128, 64)]
         return skinny + [_with_q(TileConfig(BM=128, BN=128, BK=128, WM=2, WN=2, WK=1, STAGE=2, MMA=mma), qcfg)]
     bk = {"MFMA_F32_32x32x16_F16": 32, "MFMA_I32_32x32x32_I8": 64, "MFMA_I32_32x32x32_I8_FROM_I4": 128}[mma]
-    shapes = [(128, 256, 2, 2), (64, 256, 1, 4), (32, 256, 1, 4), (128, 128, 2, 2), (256, 128, 2, 2)]
+    if mma == "MFMA_F32_32x32x16_F16":
+        shapes = [(128, 256, 2, 2), (64, 256, 1, 4), (32, 256, 1, 4), (128, 128, 2, 2), (256, 128, 2, 2)]
+    else:
+        shapes = [(128, 256, 1, 4), (64, 256, 1, 4), (32, 256, 1, 4)]
     return [_with_q(TileConfig(BM=bm, BN=bn, BK=bk, WM=wm, WN=wn, WK=1, STAGE=3, MMA=mma), qcfg) for bm, bn, wm, wn in shapes]
 
 

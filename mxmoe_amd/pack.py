@@ -32,6 +32,28 @@ def unpack_int4_k(p: torch.Tensor) -> torch.Tensor:
     return torch.where(v >= 8, v - 16, v).to(torch.int8)
 
 
+def pack_wxax_fragments(rows: torch.Tensor) -> torch.Tensor:
+    """Row-major packed weight bytes [N, KB] (int8 codes, or int4 pairs from `pack_int4_k`; KB a multiple of 64) -> the MFMA
+    fragment order the w4a4 / w8a8 tiles load straight into registers: uint8 [ceil(N/32), KB/64, 2, 64, 16] (flattened).
+
+    Block (nb, ks, step) is one 1 KB wave-wide load: lane l = 16-byte k-group (l >> 5) of channel nb*32 + (l & 31), bytes
+    ks*64 + (2*step + (l >> 5))*16 .. +16 of that channel's row.  Channels past N are zero rows.
+    (The reference's `pack_wxax` / `permute_weight`, quantize.cuh:318-381,424-475, play the same role for ldmatrix.)"""
+    r = rows.contiguous().view(torch.uint8)
+    n, kb = r.shape
+    assert kb % 64 == 0, "K must fill whole 64-byte slices"
+    n32 = (n + 31) // 32
+    if n32 * 32 != n:
+        r = torch.cat([r, torch.zeros((n32 * 32 - n, kb), dtype=torch.uint8, device=r.device)])
+    return r.view(n32, 32, kb // 64, 2, 2, 16).permute(0, 2, 3, 4, 1, 5).contiguous().reshape(-1)
+
+
+def unpack_wxax_fragments(frag: torch.Tensor, n: int, kb: int) -> torch.Tensor:
+    """Inverse of `pack_wxax_fragments` -> uint8 [n, kb]."""
+    n32 = (n + 31) // 32
+    return frag.view(n32, kb // 64, 2, 2, 32, 16).permute(0, 4, 1, 2, 3, 5).reshape(n32 * 32, kb)[:n].contiguous()
+
+
 def pack_weight_only(q: torch.Tensor, bits: int) -> torch.Tensor:
     """Unsigned weight codes [N, K] (0 .. 2^bits - 1) -> int32 [N/16, K/128, 64, bits] (flattened to 1-D).
 

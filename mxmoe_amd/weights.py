@@ -26,7 +26,8 @@ class PackedWeight:
 def quantize_and_pack(w: torch.Tensor, qparams, keep_codes: bool = False) -> PackedWeight:
     """RTN-quantise `w` [N, K] fp16 for `(a_bits, w_bits, gsize, sym)` and pack it.
 
-    fp16: kept as is.  w8a8 / w4a4: per-channel symmetric codes, int8 [N, K] / packed nibbles [N, K/2], fp16 scale [N].
+    fp16: kept as is.  w8a8 / w4a4: per-channel symmetric codes (int8 / packed nibbles, K contiguous) re-ordered into MFMA
+    fragment blocks (`pack.pack_wxax_fragments`), fp16 scale [N].
     w4a16 / w3a16 group-128: unsigned codes in the wave-interleaved layout with a (scale, zero) table; symmetric
     variants are stored offset-binary with zero = -2^(b-1) * scale (exact).
     """
@@ -38,7 +39,7 @@ def quantize_and_pack(w: torch.Tensor, qparams, keep_codes: bool = False) -> Pac
     if a_bits < 16:
         assert gsize == -1 and sym, "w-a formats are per-channel symmetric"
         qi = q.to(torch.int8)
-        data = qi.contiguous() if w_bits == 8 else pack.pack_int4_k(qi)
+        data = pack.pack_wxax_fragments(qi if w_bits == 8 else pack.pack_int4_k(qi))
         return PackedWeight(data, scale.reshape(n).contiguous(), tuple(qparams), n, k, qi if keep_codes else None)
     assert gsize == 128, "weight-only kernels implement group size 128"
     g = k // gsize

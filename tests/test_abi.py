@@ -57,10 +57,10 @@ def test_plan_counts_tiles_like_the_reference_launcher(lib):
     rc, br, tiles = _plan(lib, -1, probs)
     assert rc == 1000                                                     # first registered kernel covers w4a4 + w8a8
     out = (C.c_int32 * 8)()
-    # 546 rows of w4a4 run as two segments: 2 whole 256 x 128 tiles rows, then the 34 remaining rows with one 64 x 256 tile row
+    # 546 rows of w4a4 run as two segments: 4 whole 128 x 256 tile rows, then the 34 remaining rows with one 64 x 256 tile row
     lib.mxmoe_kernel_branch(0, br[0], out)
-    assert (out[1], out[2]) == (256, 128)
-    exp = 2 * (2816 // 128) + 1 * (2816 // 256) + 0 + 1 * (2048 // 256)
+    assert (out[1], out[2]) == (128, 256)
+    exp = 4 * (2816 // 256) + 1 * (2816 // 256) + 0 + 1 * (2048 // 256)
     assert tiles == exp
     lib.mxmoe_kernel_branch(0, br[2], out)
     assert out[0] == 1 and out[1] == 32                                  # 20 rows of w8a8 -> the 32-row w8a8 tile

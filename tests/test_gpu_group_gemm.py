@@ -27,6 +27,7 @@ def _wxax_problem(rng, m, n, k, bits, rotate=False):
     if bits == 4:
         ta, tb = pack.pack_int4_k(ta), pack.pack_int4_k(tb)
     acc = O.int_gemm(qa, qb)
+    tb = pack.pack_wxax_fragments(tb)                      # weights travel in MFMA fragment order
     return dict(A=ta.to(DEV), B=tb.to(DEV), sa=torch.from_numpy(sa.reshape(-1)).to(DEV), sb=torch.from_numpy(sb.reshape(-1)).to(DEV),
                 acc=acc, out=O.epilogue_wxax(acc, sa.reshape(-1), sb.reshape(-1)),
                 fq=O.gemm_fakequant(O.dequant(qa, sa, 0 * sa, -1), O.dequant(qb, sb, 0 * sb, -1)),

@@ -33,11 +33,11 @@ def test_qconfig_schema_roundtrip(tmp_path):
 def test_tile_config_repr_is_the_profile_table_key_shape():
     t = tile_config.get_possible_tile_list("gfx950", "w4a4_g-1_sym")[0]
     r = repr(t)
-    assert r.startswith("TileConfig(BM=128, BN=256, BK=128, WM=2, WN=2, WK=1, STAGE=3, SPLITK=-1, MMA='MFMA_I32_32x32x32_I8_FROM_I4', QCFGA=QConfig(T_PACK='half', QBITS=4")
+    assert r.startswith("TileConfig(BM=128, BN=256, BK=128, WM=1, WN=4, WK=1, STAGE=3, SPLITK=-1, MMA='MFMA_I32_32x32x32_I8_FROM_I4', QCFGA=QConfig(T_PACK='half', QBITS=4")
     if REF_TABLE.exists():                                                 # same field order as the keys of the reference's table
         ref_key = next(iter(json.loads(REF_TABLE.read_text())["w4a4_g-1_sym"]["3"]))
         assert re.findall(r"(\w+)=", ref_key) == re.findall(r"(\w+)=", r)
-    assert t.num_warps == 4 and t.smem_bytes_tile() == 3 * (128 + 256) * 64
+    assert t.num_warps == 4 and t.smem_bytes_tile() == 4 * 64 * (64 * 2 + 8)   # activations only (3 x 8 KB) < epilogue patch
     assert tile_config.get_info_from_qcfg_str("w3a16_g128_asym") == (3, 16, 128, False)
     with pytest.raises(ValueError):
         tile_config.TileConfig(BM=128, BN=256, BK=64, WM=2, WN=4, MMA="MFMA_I32_32x32x32_I8").validate()   # 8 waves
@@ -48,7 +48,7 @@ def test_tile_config_repr_is_the_profile_table_key_shape():
 def test_tile_config_json_both_forms():
     qs = ["w4a4_g-1_sym", "w8a8_g-1_sym"]
     a = tile_config.load_tile_configs({"w4a4_g-1_sym": [{"BM": 64, "BN": 256, "BK": 128, "WM": 1, "WN": 4}], "w8a8_g-1_sym": [{"BM": 128, "BN": 256, "BK": 64}]}, qs)
-    assert a["w4a4_g-1_sym"][0].cpp_type() == "MfmaTile<Op::I4, 64, 256, 1, 4>"
+    assert a["w4a4_g-1_sym"][0].cpp_type() == "WxAxTile<Op::I4, 64, 256>"
     assert a["w8a8_g-1_sym"][0].QCFGA.QBITS == 8
     pair = (tile_config.get_possible_tile_list("gfx950", qs[0])[1], tile_config.get_possible_tile_list("gfx950", qs[1])[0])
     b = tile_config.load_tile_configs({"11": repr(pair)}, qs)              # the form bits_solver.export_qconfig writes
@@ -84,7 +84,7 @@ def test_template_generator_product_and_sources(tmp_path):
     files = g.generate_source_code()
     assert len(g.combos) == 6 and len(files) == 7                          # 3 x 2 combinations + the ABI unit
     src = (tmp_path / "hz_fused_4.hip").read_text()
-    assert 'register_fused<MfmaTile<Op::I4, 32, 256, 1, 4>, MfmaTile<Op::I8, 128, 256, 2, 2>>("groupgemm_hz_fused_4")' in src
+    assert 'register_fused<WxAxTile<Op::I4, 32, 256>, WxAxTile<Op::I8, 128, 256>>("groupgemm_hz_fused_4")' in src
     assert "(a_bits == 4 && w_bits == 4 && gsize == -1 && sym == true)" in src
     assert "groupgemm_hz_fused_5" in (tmp_path / "hz_fused_decl.hpp").read_text()
     seq = TemplateGenerator("gfx950", ["w8a8_g-1_sym", "w4a4_g-1_sym"], KernelType.Sequential, tiles, out_dir=tmp_path / "seq")

@@ -64,3 +64,18 @@ def test_weight_only_scale_table_layout():
     z = -s
     t = pack.pack_weight_only_scales(s, z).reshape(n // 16, g, 16, 2)
     assert t[1, 2, 5, 0] == s[16 + 5, 2] and t[1, 2, 5, 1] == z[16 + 5, 2]
+
+
+def test_wxax_fragment_order_round_trip_and_lane_map():
+    """Weights of the w4a4 / w8a8 tiles: block (nb, ks, step) is one 1 KB wave load, lane l = k-group l >> 5 of channel l & 31."""
+    torch.manual_seed(0)
+    n, kb = 70, 192                                               # 70 channels (padded to 96), 3 slices of 64 bytes
+    rows = torch.randint(0, 256, (n, kb), dtype=torch.uint8)
+    frag = pack.pack_wxax_fragments(rows)
+    assert frag.numel() == 96 * kb
+    assert torch.equal(pack.unpack_wxax_fragments(frag, n, kb), rows)
+    f = frag.view(3, 3, 2, 64, 16)
+    for (nb, ks, step, lane) in [(0, 0, 0, 0), (1, 2, 1, 37), (2, 1, 0, 63), (2, 0, 1, 5)]:
+        ch, kg = nb * 32 + (lane & 31), lane >> 5
+        want = rows[ch, ks * 64 + (2 * step + kg) * 16: ks * 64 + (2 * step + kg) * 16 + 16] if ch < n else torch.zeros(16, dtype=torch.uint8)
+        assert torch.equal(f[nb, ks, step, lane], want)
