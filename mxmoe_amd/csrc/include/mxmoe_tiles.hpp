@@ -91,6 +91,19 @@ __device__ __forceinline__ v4i make_rsrc(const void* p, unsigned bytes) {
 __device__ __forceinline__ void dma16_to_lds(const v4i& rsrc, int lds_addr, int voffset, int soffset) {
   asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds" : : "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset) : "memory", "m0");
 }
+// 16-byte-per-lane global load whose completion the caller tracks itself (the compiler's own bookkeeping knows nothing of the
+// direct-to-LDS loads that share the counter and would drain the queue far too early).  The value may only be used after
+// vm_wait_for<N>(v) with N = number of vector-memory loads issued after this one; a value that is never used must still be
+// passed to vm_wait_for before its register may die (the load writes the register whenever it completes).
+__device__ __forceinline__ v4i gload16_untracked(const uint8_t* p) {
+  v4i v;
+  asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(p) : "memory");
+  return v;
+}
+template <int N>
+__device__ __forceinline__ void vm_wait_for(v4i& v) {
+  asm volatile("s_waitcnt vmcnt(%1)" : "+v"(v) : "n"(N) : "memory");
+}
 template <int N>
 __device__ __forceinline__ void vm_wait() {
   asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
@@ -482,6 +495,22 @@ struct WxAxTile {
   static constexpr int kDepth = OP == Op::I4 ? 2 : 4;
   using Acc = v16i;
 
+  // Vector-memory loads a wave issues in units a..b of one iteration: one weight fragment per unit, plus one activation load in
+  // each of the first nd units (before the fragment).
+  static constexpr int ops_in(int a, int b, int nd) {
+    int n = 0;
+    for (int u = a; u <= b; ++u) n += 1 + (u < nd ? 1 : 0);
+    return n;
+  }
+  // Loads issued after the load of fragment `uf` (= k-step * FN + block) of a slice, up to and including the unit that first
+  // uses it: the fragment of unit uf is (re)loaded at unit uf+1 kDepth slices earlier and first used at unit uf-1 (int4: widened
+  // one unit ahead) or uf (int8).
+  static constexpr int younger_than_fragment(int uf, int nd) {
+    const int ul = (uf + 1) % U, kl = -kDepth + (uf == U - 1 ? 1 : 0);
+    const int uc = OP == Op::I4 ? (uf + U - 1) % U : uf, kc = OP == Op::I4 && uf == 0 ? -1 : 0;
+    return ops_in(ul + 1, U - 1, nd) + ops_in(0, U - 1, nd) * (kc - kl - 1) + ops_in(0, uc, nd);
+  }
+
   __device__ static __forceinline__ void widen(const v4i& p, v4i* o) {
     if constexpr (OP == Op::I4) {
       o[0] = (p << 4) & (int)0xF0F0F0F0;
@@ -518,6 +547,12 @@ struct WxAxTile {
         dma16_to_lds(rs, lds_base + stage * kStageBytes + ii * 1024, dma_voff[i], __builtin_amdgcn_readfirstlane(kt * kRowBytes));
       }
     };
+    const bool has_dma = kDmaTotal % kWaves == 0 || wave < kDmaTotal;  // whether this wave issues activation loads at all
+    // wait until the weight fragment `uf` of the current slice has arrived (see younger_than_fragment), then hand it out
+    auto ready = [&](auto ufc, v4i& frag) {
+      constexpr int uf = decltype(ufc)::value;
+      if (has_dma) vm_wait_for<younger_than_fragment(uf, kDma)>(frag); else vm_wait_for<younger_than_fragment(uf, 0)>(frag);
+    };
     const int lrow = lane & 31;
     const int fa = lrow * kRowBytes + (((lane >> 5) ^ lds_swizzle(lrow)) << 4);
     auto lds_a = [&](const uint8_t* st, int step, int i) { return *reinterpret_cast<const v4i*>(st + ((fa + i * 32 * kRowBytes) ^ (step << 5))); };
@@ -530,7 +565,7 @@ struct WxAxTile {
       const int nb = min(n0 / 32 + wave * FN + j, nblk - 1);  // blocks past N re-read the last one; their results are never stored
       bptr[j] = t.B + (long)nb * KT * 2048 + lane * 16;
     }
-    auto load_b = [&](int j, int step, int kt) { return gload<v4i>(bptr[j] + ((long)min(kt, KT - 1) * 2 + step) * 1024); };
+    auto load_b = [&](int j, int step, int kt) { return gload16_untracked(bptr[j] + ((long)min(kt, KT - 1) * 2 + step) * 1024); };
 
     Acc acc[FM][FN];
 #pragma unroll
@@ -560,7 +595,12 @@ struct WxAxTile {
       for (int j = 0; j < FN; ++j)
 #pragma unroll
         for (int s = 0; s < 2; ++s) pbq[d][j][s] = load_b(j, s, d);
-    vm_wait<0>();
+#pragma unroll
+    for (int d = 0; d < kDepth - 1; ++d)
+#pragma unroll
+      for (int j = 0; j < FN; ++j)
+#pragma unroll
+        for (int s = 0; s < 2; ++s) vm_wait_for<0>(pbq[d][j][s]);
     __syncthreads();
     static_for<U>([&](auto uc) {
       constexpr int u = decltype(uc)::value;
@@ -610,8 +650,13 @@ struct WxAxTile {
         }
         if constexpr (OP == Op::I4) {
           // weight operands of unit u+1
-          if constexpr (u + 1 < U) widen(pbq[P][(u + 1) % FN][(u + 1) / FN], bop[(u + 1) & 1]);
-          else widen(pbq[Pnext][0][0], bop[0]);
+          if constexpr (u + 1 < U) {
+            ready(std::integral_constant<int, u + 1>{}, pbq[P][(u + 1) % FN][(u + 1) / FN]);
+            widen(pbq[P][(u + 1) % FN][(u + 1) / FN], bop[(u + 1) & 1]);
+          } else {
+            ready(std::integral_constant<int, 0>{}, pbq[Pnext][0][0]);
+            widen(pbq[Pnext][0][0], bop[0]);
+          }
 #pragma unroll
           for (int i = 0; i < FM; ++i) {
             mma(acc[i][j], aop[0][i], bop[u & 1]);
@@ -621,6 +666,7 @@ struct WxAxTile {
           __builtin_amdgcn_sched_group_barrier(0x100, FM, 0);
           sched_mfma_valu<12 + (j == FN - 1 ? 12 * FM : 0), 2 * FM, 0>();
         } else {
+          ready(uc, pbq[P][j][step]);
 #pragma unroll
           for (int i = 0; i < FM; ++i) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(pbq[P][j][step], aop[step][i][0], acc[i][j], 0, 0, 0);
         }
@@ -641,7 +687,15 @@ struct WxAxTile {
         }
       });
     }
-    vm_wait<0>();  // nothing may still land in LDS once the epilogue reuses it
+    // Nothing may still land in LDS once the epilogue reuses it, and nothing in registers either: the fragments fetched past the
+    // end of K are never used, so without this tie the compiler would hand their registers to the epilogue while the loads are
+    // still in flight.
+#pragma unroll
+    for (int d = 0; d < kDepth; ++d)
+#pragma unroll
+      for (int j = 0; j < FN; ++j)
+#pragma unroll
+        for (int s = 0; s < 2; ++s) vm_wait_for<0>(pbq[d][j][s]);
 
     // ---- epilogue (as MfmaTile): lane holds token lane & 31 and channels 8*(r/4) + 4*(lane >> 5) + (r & 3) of each 32x32 block
     const int nq = (lane >> 5) * 4;
