@@ -151,8 +151,9 @@ __device__ __forceinline__ float exp_fixed(float t) {
 
 __device__ __forceinline__ float round_h(float v) { return (float)(_Float16)v; }
 
-template <int MAXC, bool SILU>
-__global__ void __launch_bounds__(256) row_quant_kernel(const RowArgs a) {
+// NT threads per workgroup (256, or 192 when that wastes fewer lanes: a 1408-element row is 176 chunks of 8).
+template <int MAXC, bool SILU, int NT>
+__global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
   extern __shared__ __align__(16) float lds[];
   const int tid = threadIdx.x;
   const int nmax = max(a.plan.n, a.plan_shared.n);
@@ -160,7 +161,7 @@ __global__ void __launch_bounds__(256) row_quant_kernel(const RowArgs a) {
   float* sg = lds + nmax;          // [kb*kb]
   float* red = sg + a.plan.kb * a.plan.kb;  // [8]
   if (a.signs) {
-    for (int i = tid; i < a.plan.kb * a.plan.kb; i += 256) sg[i] = a.signs[i];
+    for (int i = tid; i < a.plan.kb * a.plan.kb; i += NT) sg[i] = a.signs[i];
   }
 
   // Row bookkeeping (expert, tag, offsets, source pointer) and the row's data are fetched one row ahead: each is a chain of
@@ -191,7 +192,7 @@ __global__ void __launch_bounds__(256) row_quant_kernel(const RowArgs a) {
     const int n = (m.shared_row ? a.plan_shared : a.plan).n;
 #pragma unroll
     for (int i = 0; i < MAXC; ++i) {
-      const int c = tid + i * 256;
+      const int c = tid + i * NT;
       if (c < (n >> 3)) {
         g[i] = *reinterpret_cast<const v8h*>(m.srow + c * 8);
         if (SILU) u[i] = *reinterpret_cast<const v8h*>(m.srow + n + c * 8);
@@ -231,7 +232,7 @@ __global__ void __launch_bounds__(256) row_quant_kernel(const RowArgs a) {
     __syncthreads();  // previous row fully consumed (and the sign table staged)
 #pragma unroll
     for (int i = 0; i < MAXC; ++i) {
-      const int c = tid + i * 256;
+      const int c = tid + i * NT;
       if (c < nchunks) {
         const v8h g = cur_g[i];
         if (SILU) {
@@ -272,7 +273,7 @@ __global__ void __launch_bounds__(256) row_quant_kernel(const RowArgs a) {
         __syncthreads();
 #pragma unroll
         for (int i = 0; i < MAXC; ++i) {
-          const int c = tid + i * 256;
+          const int c = tid + i * NT;
           if (c < nchunks) {
             const float* o = x + (c ^ hc) * 8;
             const bool upper = c & hc;
@@ -283,7 +284,7 @@ __global__ void __launch_bounds__(256) row_quant_kernel(const RowArgs a) {
         __syncthreads();
 #pragma unroll
         for (int i = 0; i < MAXC; ++i) {
-          const int c = tid + i * 256;
+          const int c = tid + i * NT;
           if (c < nchunks) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) x[c * 8 + j] = v[i][j];
@@ -301,7 +302,7 @@ __global__ void __launch_bounds__(256) row_quant_kernel(const RowArgs a) {
         __syncthreads();
 #pragma unroll
         for (int i = 0; i < MAXC; ++i) {
-          const int c = tid + i * 256;
+          const int c = tid + i * NT;
           if (c < nchunks) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) x[c * 8 + j] = v[i][j];
@@ -311,7 +312,7 @@ __global__ void __launch_bounds__(256) row_quant_kernel(const RowArgs a) {
         // dense B stage: t[b] = sum_{b'} B[b][b'] v[b'], b' ascending, starting from 0
 #pragma unroll
         for (int i = 0; i < MAXC; ++i) {
-          const int c = tid + i * 256;
+          const int c = tid + i * NT;
           if (c < nchunks) {
             const int k = c / mc, jc = c - k * mc;
             const int blk = k / pl.kb, b = k - blk * pl.kb;
@@ -336,7 +337,7 @@ __global__ void __launch_bounds__(256) row_quant_kernel(const RowArgs a) {
           __syncthreads();
 #pragma unroll
           for (int i = 0; i < MAXC; ++i) {
-            const int c = tid + i * 256;
+            const int c = tid + i * NT;
             if (c < nchunks) {
 #pragma unroll
               for (int j = 0; j < 8; ++j) x[c * 8 + j] = v[i][j];
@@ -345,7 +346,7 @@ __global__ void __launch_bounds__(256) row_quant_kernel(const RowArgs a) {
           __syncthreads();
 #pragma unroll
           for (int i = 0; i < MAXC; ++i) {
-            const int c = tid + i * 256;
+            const int c = tid + i * NT;
             if (c < nchunks) {
               const bool upper = ((c / (pl.kb * mc)) & hh) != 0;
               const float* o = x + (long)(upper ? c - hc : c + hc) * 8;
@@ -366,7 +367,7 @@ __global__ void __launch_bounds__(256) row_quant_kernel(const RowArgs a) {
       _Float16* out = reinterpret_cast<_Float16*>(a.inp_store) + inp_off + lrow * n;
 #pragma unroll
       for (int i = 0; i < MAXC; ++i) {
-        const int c = tid + i * 256;
+        const int c = tid + i * NT;
         if (c < nchunks) {
           v8h o;
 #pragma unroll
@@ -379,7 +380,7 @@ __global__ void __launch_bounds__(256) row_quant_kernel(const RowArgs a) {
     float amax = 0.0f;
 #pragma unroll
     for (int i = 0; i < MAXC; ++i) {
-      const int c = tid + i * 256;
+      const int c = tid + i * NT;
       if (c < nchunks) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[i][j]));
@@ -390,7 +391,9 @@ __global__ void __launch_bounds__(256) row_quant_kernel(const RowArgs a) {
     __syncthreads();
     if ((tid & 63) == 0) red[tid >> 6] = amax;
     __syncthreads();
-    amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    amax = red[0];
+#pragma unroll
+    for (int w = 1; w < NT / 64; ++w) amax = fmaxf(amax, red[w]);
     const float upper = tag == 1 ? 127.0f : 7.0f;
     float scale = round_h(amax / upper);   // fp16 division: fp32 quotient of two fp16 values, rounded to fp16
     if (scale == 0.0f) scale = 1.0f;       // quantize.cuh:258
@@ -398,7 +401,7 @@ __global__ void __launch_bounds__(256) row_quant_kernel(const RowArgs a) {
     uint8_t* out = a.inp_store + 2 * (inp_off + lrow * (tag == 1 ? n / 2 : n / 4));
 #pragma unroll
     for (int i = 0; i < MAXC; ++i) {
-      const int c = tid + i * 256;
+      const int c = tid + i * NT;
       if (c < nchunks) {
         int q[8];
 #pragma unroll
@@ -570,7 +573,6 @@ static int make_plan(int n, int had_k, int had_f, bool rotate, RotPlan* p) {
 template <bool SILU>
 static int launch_rows(const RowArgs& a, int lds_bytes, hipStream_t s) {
   const int nmax = a.plan.n > a.plan_shared.n ? a.plan.n : a.plan_shared.n;
-  const int chunks = (nmax / 8 + 255) / 256;
   int dev = 0, cus = 256;
   (void)hipGetDevice(&dev);
   (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
@@ -596,13 +598,23 @@ static int launch_rows(const RowArgs& a, int lds_bytes, hipStream_t s) {
     }
     return 0;
   }
-  if (chunks <= 1) hipLaunchKernelGGL((row_quant_kernel<1, SILU>), dim3(grid), dim3(256), lds_bytes, s, a);
-  else if (chunks <= 2) hipLaunchKernelGGL((row_quant_kernel<2, SILU>), dim3(grid), dim3(256), lds_bytes, s, a);
-  else if (chunks <= 3) hipLaunchKernelGGL((row_quant_kernel<3, SILU>), dim3(grid), dim3(256), lds_bytes, s, a);
-  else if (chunks <= 7) hipLaunchKernelGGL((row_quant_kernel<7, SILU>), dim3(grid), dim3(256), lds_bytes, s, a);
-  else {
-    last_error() = "row too long for the activation kernels";
-    return 3;
+  // workgroup size and chunks per thread with the fewest idle lanes
+  const int nchunks = nmax / 8;
+  static const int kShapes[][2] = {{192, 1}, {256, 1}, {192, 2}, {256, 2}, {192, 3}, {256, 3}, {256, 7}};
+  int pick = -1;
+  for (int i = 0; i < 7 && pick < 0; ++i)
+    if (kShapes[i][0] * kShapes[i][1] >= nchunks) pick = i;
+  switch (pick) {
+    case 0: hipLaunchKernelGGL((row_quant_kernel<1, SILU, 192>), dim3(grid), dim3(192), lds_bytes, s, a); break;
+    case 1: hipLaunchKernelGGL((row_quant_kernel<1, SILU, 256>), dim3(grid), dim3(256), lds_bytes, s, a); break;
+    case 2: hipLaunchKernelGGL((row_quant_kernel<2, SILU, 192>), dim3(grid), dim3(192), lds_bytes, s, a); break;
+    case 3: hipLaunchKernelGGL((row_quant_kernel<2, SILU, 256>), dim3(grid), dim3(256), lds_bytes, s, a); break;
+    case 4: hipLaunchKernelGGL((row_quant_kernel<3, SILU, 192>), dim3(grid), dim3(192), lds_bytes, s, a); break;
+    case 5: hipLaunchKernelGGL((row_quant_kernel<3, SILU, 256>), dim3(grid), dim3(256), lds_bytes, s, a); break;
+    case 6: hipLaunchKernelGGL((row_quant_kernel<7, SILU, 256>), dim3(grid), dim3(256), lds_bytes, s, a); break;
+    default:
+      last_error() = "row too long for the activation kernels";
+      return 3;
   }
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
