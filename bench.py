@@ -21,7 +21,7 @@ PEAK = {"int8": 5000.0, "fp16": 2500.0, "hbm": 8000.0}  # MI355X: TOP/s dense in
 
 # HBM bytes per launch of the dominant (gate_up) kernel, from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE runs scaled by the
 # same counters on a plain 256 MiB copy (summaries: profiles/fused_group_gemm_<workload>.txt, profiles/counter_calibration_copy_256MiB.txt)
-TRAFFIC = {"c2": 567901535, "c3": 768704711, "c4": 190233177}
+TRAFFIC = {"c2": 573772163, "c3": 789348508, "c4": 190252525}
 
 
 def build_layer(name: str, tokens: int | None):
@@ -152,9 +152,10 @@ def cpu_baseline(cfg, budget_s: float = 20.0):
                       f"activation fake-quant + fp32 matmuls + SiLU timed, {spent:.1f} s"}
 
 
-def time_whole_layer(cfg, layer, reps: int = 5) -> dict:
+def time_whole_layer(cfg, layer, reps: int = 7) -> dict:
     """Wall time of the whole layer forward as a caller of the ops sees it (permute + rotate + quantise, gate_up launch, SiLU*up +
-    rotate + quantise, down launch, un-permute + combine), including the host work of the ops (offset tables, allocations).
+    rotate + quantise, down launch, un-permute + combine), including the host work of the ops (offset tables, allocations); median of
+    `reps` repetitions.
     Reported next to the GroupGEMM figure, never as `value`."""
     import torch
 
@@ -163,17 +164,19 @@ def time_whole_layer(cfg, layer, reps: int = 5) -> dict:
     hidden = synth.make_hidden(cfg).cuda()
     ids, w = synth.make_routing(cfg)
     ids, w = ids.cuda(), w.cuda()
-    parts = {"prologue": 0.0, "gate_up": 0.0, "act": 0.0, "down": 0.0, "combine": 0.0}
-    for rep in range(reps + 1):
+    names = ("prologue", "gate_up", "act", "down", "combine")
+    samples = {k: [] for k in names}
+    for rep in range(reps + 2):
         torch.cuda.synchronize()
         marks = [time.perf_counter()]
         for fn in (lambda: layer.prepare(hidden, ids), layer.gate_up, layer.act, layer.down, lambda: layer.combine(w)):
             fn()
             torch.cuda.synchronize()
             marks.append(time.perf_counter())
-        if rep:  # first repetition warms allocations up
-            for k, a, b in zip(parts, marks, marks[1:]):
-                parts[k] += (b - a) * 1e3 / reps
+        if rep >= 2:  # the first repetitions settle the allocator
+            for k, a, b in zip(names, marks, marks[1:]):
+                samples[k].append((b - a) * 1e3)
+    parts = {k: sorted(v)[len(v) // 2] for k, v in samples.items()}
     out = {f"{k}_ms": round(v, 4) for k, v in parts.items()}
     out["layer_ms"] = round(sum(parts.values()), 4)
     return out

@@ -6,6 +6,7 @@ contraction is off: the quantiser and the Hadamard rotation must round exactly l
 """
 from __future__ import annotations
 
+import re
 import subprocess
 import sys
 from pathlib import Path
@@ -26,6 +27,24 @@ HIPCC_FLAGS = [
 ]
 
 
+def check_no_spills(remarks: str) -> None:
+    """Refuse a build in which a WxAxTile kernel spills vector registers.
+
+    Those tiles load weight fragments with loads the compiler does not track (the waits are placed by hand): a fragment register
+    that the compiler spills or re-uses while its load is in flight is overwritten when the load lands, and when that register
+    holds an address the next access faults.  `remarks` is hipcc's -Rpass-analysis=kernel-resource-usage output."""
+    name = None
+    for line in remarks.splitlines():
+        m = re.search(r"remark: Function Name: (\S+)", line)
+        if m:
+            name = m.group(1)
+            continue
+        m = re.search(r"remark:\s+VGPRs Spill: (\d+)", line)
+        if m and name and "WxAxTile" in name and int(m.group(1)) > 0:
+            raise RuntimeError(f"{name}: {m.group(1)} vector registers spilled in a kernel with hand-tracked loads; shrink the tile's "
+                               f"register ring or lower its waves per SIMD")
+
+
 def hipcc_build(sources, out: Path, extra=(), verbose: bool = False, jobs: int = 8) -> Path:
     """Compile each source to an object (in parallel) and link them into the shared library `out`."""
     from concurrent.futures import ThreadPoolExecutor
@@ -42,12 +61,14 @@ def hipcc_build(sources, out: Path, extra=(), verbose: bool = False, jobs: int =
         err = "\n".join(l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l)
         if res.returncode != 0:
             raise RuntimeError(f"hipcc failed ({res.returncode}):\n{' '.join(map(str, cmd))}\n{err}")
+        check_no_spills(err)
+        err = "\n".join(l for l in err.splitlines() if "kernel-resource-usage" not in l and not re.match(r"\s*(\d+\s*)?\||In file included", l))
         if verbose and err.strip():
             print(err, file=sys.stderr)
 
     objs = [objdir / (s.stem + ".o") for s in sources]
     with ThreadPoolExecutor(max_workers=max(1, jobs)) as ex:
-        list(ex.map(run, [["hipcc", *compile_flags, *extra, *inc, "-c", str(s), "-o", str(o)] for s, o in zip(sources, objs)]))
+        list(ex.map(run, [["hipcc", *compile_flags, *extra, *inc, "-Rpass-analysis=kernel-resource-usage", "-c", str(s), "-o", str(o)] for s, o in zip(sources, objs)]))
     run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", *map(str, objs), "-o", str(out)])
     for o in objs:
         o.unlink()

@@ -202,3 +202,14 @@ def test_perf_table_fit_and_sweep_shapes():
                 e = sweep_entry(t, q, 2048, w, cus=256)
                 m, n, k = e["shape"]
                 assert ProblemShape(m, n, k).num_tiles(t) == 256 * w and k == 2048
+
+
+def test_build_refuses_spilling_wxax_kernels():
+    """A WxAxTile kernel that spills vector registers must not be built (its hand-tracked loads would land in re-used registers)."""
+    from mxmoe_amd.build import check_no_spills
+
+    fmt = "t.hpp:1:1: remark: Function Name: {} [-Rpass-analysis=kernel-resource-usage]\nt.hpp:1:1: remark:     VGPRs Spill: {} [-Rpass-analysis=kernel-resource-usage]\n"
+    check_no_spills(fmt.format("_ZN5mxmoe8WxAxTileILi1EEE", 0))
+    check_no_spills(fmt.format("_ZN5mxmoe12SkinnyWoTileILi4EEE", 3))        # compiler-tracked loads: spills are only slow
+    with pytest.raises(RuntimeError, match="spilled"):
+        check_no_spills(fmt.format("_ZN5mxmoe8WxAxTileILi1EEE", 45))
