@@ -160,6 +160,19 @@ __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
   float* x = lds;                  // [nmax]
   float* sg = lds + nmax;          // [kb*kb]
   float* red = sg + a.plan.kb * a.plan.kb;  // [8]
+  // A chunk of 8 values lives in two planes of 16 bytes (values 0-3, values 4-7): consecutive lanes then touch consecutive 16-byte
+  // words and a wave's 128-bit accesses spread over all banks (32-byte lane strides would hit every bank twice).
+  float4* xlo = reinterpret_cast<float4*>(x);
+  float4* xhi = xlo + (nmax >> 3);
+  auto put = [&](int c, const float (&w)[8]) {
+    xlo[c] = make_float4(w[0], w[1], w[2], w[3]);
+    xhi[c] = make_float4(w[4], w[5], w[6], w[7]);
+  };
+  auto get = [&](int c, float (&w)[8]) {
+    const float4 l = xlo[c], h = xhi[c];
+    w[0] = l.x; w[1] = l.y; w[2] = l.z; w[3] = l.w;
+    w[4] = h.x; w[5] = h.y; w[6] = h.z; w[7] = h.w;
+  };
   if (a.signs) {
     for (int i = tid; i < a.plan.kb * a.plan.kb; i += NT) sg[i] = a.signs[i];
   }
@@ -260,8 +273,7 @@ __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
               }
             }
           }
-#pragma unroll
-          for (int j = 0; j < 8; ++j) x[c * 8 + j] = v[i][j];
+          put(c, v[i]);
         }
       }
     }
@@ -275,7 +287,8 @@ __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
         for (int i = 0; i < MAXC; ++i) {
           const int c = tid + i * NT;
           if (c < nchunks) {
-            const float* o = x + (c ^ hc) * 8;
+            float o[8];
+            get(c ^ hc, o);
             const bool upper = c & hc;
 #pragma unroll
             for (int j = 0; j < 8; ++j) v[i][j] = upper ? o[j] - v[i][j] : v[i][j] + o[j];
@@ -286,8 +299,7 @@ __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
         for (int i = 0; i < MAXC; ++i) {
           const int c = tid + i * NT;
           if (c < nchunks) {
-#pragma unroll
-            for (int j = 0; j < 8; ++j) x[c * 8 + j] = v[i][j];
+            put(c, v[i]);
           }
         }
       }
@@ -304,8 +316,7 @@ __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
         for (int i = 0; i < MAXC; ++i) {
           const int c = tid + i * NT;
           if (c < nchunks) {
-#pragma unroll
-            for (int j = 0; j < 8; ++j) x[c * 8 + j] = v[i][j];
+            put(c, v[i]);
           }
         }
         __syncthreads();
@@ -316,14 +327,15 @@ __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
           if (c < nchunks) {
             const int k = c / mc, jc = c - k * mc;
             const int blk = k / pl.kb, b = k - blk * pl.kb;
-            const float* vb = x + ((long)blk * pl.kb * mc + jc) * 8;
+            const int vb = blk * pl.kb * mc + jc;
             const float* sr = sg + b * pl.kb;
             float acc[8];
 #pragma unroll
             for (int j = 0; j < 8; ++j) acc[j] = 0.0f;
             for (int bp = 0; bp < pl.kb; ++bp) {
               const float s = sr[bp];
-              const float* vv = vb + (long)bp * mc * 8;
+              float vv[8];
+              get(vb + bp * mc, vv);
 #pragma unroll
               for (int j = 0; j < 8; ++j) acc[j] = __builtin_fmaf(s, vv[j], acc[j]);  // s = +-1: the product is exact, so this is acc + s*v
             }
@@ -339,8 +351,7 @@ __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
           for (int i = 0; i < MAXC; ++i) {
             const int c = tid + i * NT;
             if (c < nchunks) {
-#pragma unroll
-              for (int j = 0; j < 8; ++j) x[c * 8 + j] = v[i][j];
+              put(c, v[i]);
             }
           }
           __syncthreads();
@@ -349,7 +360,8 @@ __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
             const int c = tid + i * NT;
             if (c < nchunks) {
               const bool upper = ((c / (pl.kb * mc)) & hh) != 0;
-              const float* o = x + (long)(upper ? c - hc : c + hc) * 8;
+              float o[8];
+              get(upper ? c - hc : c + hc, o);
 #pragma unroll
               for (int j = 0; j < 8; ++j) v[i][j] = upper ? o[j] - v[i][j] : v[i][j] + o[j];
             }
