@@ -75,7 +75,8 @@ def main(argv=None) -> int:
     trace = args.trace
     exact = False
     if args.synthetic:
-        cfg, trace, args.qconfig = materialise_synthetic(args.synthetic, None if "--bs" not in (argv or sys.argv) else bs)
+        cfg, trace, synthetic_qcfg = materialise_synthetic(args.synthetic, None if "--bs" not in (argv or sys.argv) else bs)
+        args.qconfig = args.qconfig or synthetic_qcfg  # e.g. a qconfig the allocator (mxmoe_amd.bits_solver) wrote for this workload
         model_id, dataset, bs, layer, exact = cfg.model, "synthetic", cfg.tokens, 0, True
 
     if args.qconfig is not None:
