@@ -13,13 +13,23 @@ from .weights import quantize_and_pack
 
 
 class MxMoELayer:
-    def __init__(self, cfg: MoEConfig, device="cuda", formats=None, weights=None, keep_codes: bool = False):
+    def __init__(self, cfg: MoEConfig, device="cuda", formats=None, weights=None, keep_codes: bool = False, packed=None):
+        """weights: [(W13, W2)] fp16 per expert (default: the configuration's seeded synthetic weights); packed: ([PackedWeight] for
+        gate_up, [PackedWeight] for down) already quantised and packed, e.g. from `checkpoint.load_layer` (formats are taken from them)."""
         self.cfg = cfg
         self.device = torch.device(device)
-        self.formats = formats or draw_formats(cfg)
         self.n_exp_total = cfg.num_experts + (1 if cfg.num_shared else 0)
-        self.w13, self.w2 = [], []
-        for e in range(self.n_exp_total):
+        if packed is not None:
+            self.w13, self.w2 = list(packed[0]), list(packed[1])
+            assert len(self.w13) == len(self.w2) == self.n_exp_total, "one packed gate_up and down block per expert (shared expert last)"
+            for w in self.w13 + self.w2:
+                w.data = w.data.to(self.device)
+                w.scale = None if w.scale is None else w.scale.to(self.device)
+            self.formats = [(tuple(a.qparams), tuple(b.qparams)) for a, b in zip(self.w13, self.w2)]
+        else:
+            self.formats = formats or draw_formats(cfg)
+            self.w13, self.w2 = [], []
+        for e in range(self.n_exp_total if packed is None else 0):
             w13, w2 = weights[e] if weights is not None else expert_weights(cfg, e)
             gu, dn = self.formats[e]
             self.w13.append(quantize_and_pack(w13.to(self.device), gu, keep_codes))

@@ -117,3 +117,40 @@ def test_layer_combine_end_to_end():
     ref = O.unpermute_combine(rows, slot, w.numpy(), outs[-1].cpu().numpy())
     assert final.shape == (cfg.tokens, cfg.hidden)
     assert np.array_equal(final.cpu().numpy().view(np.uint16), ref.view(np.uint16))
+
+
+def test_layer_from_checkpoint_file_keeps_the_function(tmp_path):
+    """fp16 weights -> rotate + quantise + pack -> file -> layer: identical to packing in place, and (the weight rotation cancelling
+    the online rotation of the activations) still the function of the fp16 MLP up to w8a8 quantisation noise."""
+    from mxmoe_amd import checkpoint as C
+    from mxmoe_amd import synth
+    from mxmoe_amd.layer import MxMoELayer
+
+    cfg = synth.MoEConfig("t", "qwen2_moe", 4, 2, 256, 1408, 64, rotate=1, formats=(synth.W8A8,), format_probs=(1.0,))
+    formats = [(synth.W8A8, synth.W8A8)] * cfg.num_experts
+    experts = [synth.expert_weights(cfg, e) for e in range(cfg.num_experts)]
+    tensors, meta = C.pack_layer(experts, formats, rotate=1, model="qwen2_moe")
+    path = str(tmp_path / "layer.safetensors")
+    C.save_layer(path, tensors, meta)
+    w13, w2, _ = C.load_layer(path, device="cuda")
+    hidden = synth.make_hidden(cfg)
+    ids, w = synth.make_routing(cfg)
+
+    from_file = MxMoELayer(cfg, packed=(w13, w2))
+    from_file.forward(hidden, ids)
+    a = from_file.combine(w).cpu()
+    in_place = MxMoELayer(cfg, formats=formats, weights=[(C.rotate_input_weights(w13_), C.rotate_input_weights(w2_)) for w13_, w2_ in experts])
+    in_place.forward(hidden, ids)
+    b = in_place.combine(w).cpu()
+    assert torch.equal(a, b)
+
+    # the fp16 MLP with the ORIGINAL weights, fp32 arithmetic
+    x = hidden.float()
+    ref = torch.zeros(cfg.tokens, cfg.hidden)
+    for t in range(cfg.tokens):
+        for j in range(cfg.topk):
+            w13_, w2_ = experts[int(ids[t, j])]
+            h = w13_.float() @ x[t]
+            g, u = h[:cfg.inter], h[cfg.inter:]
+            ref[t] += float(w[t, j]) * (w2_.float() @ (g * torch.sigmoid(g) * u))
+    assert _rel(a.float().numpy(), ref.numpy()) <= 5e-2
