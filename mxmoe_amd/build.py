@@ -45,6 +45,62 @@ def check_no_spills(remarks: str) -> None:
                                f"register ring or lower its waves per SIMD")
 
 
+def check_untracked_load_copies(asm: str) -> None:
+    """Refuse device code in which a register is moved by the compiler while a hand-tracked load into it is in flight.
+
+    The weight fragments of the WxAxTile kernels are loaded by inline-assembly `global_load_dwordx4` whose completion only the
+    hand-placed `s_waitcnt vmcnt(N) ; landed v[a:b]` knows about.  A register-to-register copy (or a spill) of such a register,
+    which the register allocator is free to insert wherever the value is live across a branch or a loop edge, copies whatever the
+    register holds at that moment.  `asm` is hipcc's -S output for the device.  Every kernel is walked in layout order with the set
+    of registers in flight (added by an inline-assembly load, removed by the wait that names them); loop bodies are walked twice,
+    so that loads issued at the bottom of an iteration are in flight at its top."""
+    lines = asm.splitlines()
+    starts = [i for i, l in enumerate(lines) if re.match(r"^_Z\w+:", l)]
+
+    def regs_of(text):
+        out = set()
+        for a, b in re.findall(r"\bv\[(\d+):(\d+)\]", text):
+            out.update(range(int(a), int(b) + 1))
+        out.update(int(a) for a in re.findall(r"\bv(\d+)\b", text))
+        return out
+
+    for si, start in enumerate(starts):
+        end = starts[si + 1] if si + 1 < len(starts) else len(lines)
+        kernel = lines[start].split(":")[0]
+        # loop regions: header line .. end of the last block that names the header
+        label_lines = [i for i in range(start, end) if re.match(r"^\.LBB\d+_\d+:", lines[i])]
+        regions = []
+        for h in (i for i in range(start, end) if "Loop Header" in lines[i]):
+            name = lines[h].split(":")[0].strip().lstrip(".L")
+            members = [i for i in range(start, end) if re.search(rf"Header={name}\b", lines[i])]
+            last = max([h] + members)
+            nxt = next((i for i in label_lines if i > last), end)
+            regions.append((min([h] + members), nxt))
+        order, pos = [], start
+        for lo, hi in sorted(regions):
+            if lo < pos:
+                continue
+            order += list(range(pos, lo)) + list(range(lo, hi)) * 2
+            pos = hi
+        order += list(range(pos, end))
+        inflight, in_asm = set(), False
+        for i in order:
+            t = lines[i].strip()
+            if t.startswith(";;#ASMSTART"):
+                in_asm = True
+            elif t.startswith(";;#ASMEND"):
+                in_asm = False
+            elif in_asm and t.startswith("global_load"):
+                inflight |= regs_of(t.split(",")[0])
+            elif in_asm and t.startswith("s_waitcnt") and "; landed" in t:
+                inflight -= regs_of(t.split("; landed")[1])
+            elif not in_asm and inflight and re.match(r"(v_mov_b|v_accvgpr_|scratch_|v_swap_)", t) and regs_of(t) & inflight:
+                raise RuntimeError(f"{kernel}: line {i + 1} `{t}` moves a register while a hand-tracked load into it is in flight; "
+                                   f"restructure the tile so that no fragment register is live across a branch")
+        if inflight:
+            raise RuntimeError(f"{kernel}: hand-tracked loads into v{sorted(inflight)} are never waited for")
+
+
 def hipcc_build(sources, out: Path, extra=(), verbose: bool = False, jobs: int = 8) -> Path:
     """Compile each source to an object (in parallel) and link them into the shared library `out`."""
     from concurrent.futures import ThreadPoolExecutor
@@ -67,8 +123,21 @@ def hipcc_build(sources, out: Path, extra=(), verbose: bool = False, jobs: int =
             print(err, file=sys.stderr)
 
     objs = [objdir / (s.stem + ".o") for s in sources]
+
+    def scan(src):
+        # device assembly of the same translation unit, only to be checked
+        out_s = objdir / (src.stem + ".s")
+        run(["hipcc", *[f for f in compile_flags if f != "-fPIC"], *extra, *inc, "-S", "--cuda-device-only", str(src), "-o", str(out_s)])
+        try:
+            check_untracked_load_copies(out_s.read_text())
+        finally:
+            out_s.unlink()
+
     with ThreadPoolExecutor(max_workers=max(1, jobs)) as ex:
-        list(ex.map(run, [["hipcc", *compile_flags, *extra, *inc, "-Rpass-analysis=kernel-resource-usage", "-c", str(s), "-o", str(o)] for s, o in zip(sources, objs)]))
+        jobs_ = [ex.submit(run, ["hipcc", *compile_flags, *extra, *inc, "-Rpass-analysis=kernel-resource-usage", "-c", str(s), "-o", str(o)]) for s, o in zip(sources, objs)]
+        jobs_ += [ex.submit(scan, s) for s in sources]
+        for j in jobs_:
+            j.result()
     run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", *map(str, objs), "-o", str(out)])
     for o in objs:
         o.unlink()

@@ -122,7 +122,7 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd<Tiles...>) fused_group
 
 // ------------------------------------------------------------------ host side ------------------------------------------------------------------
 
-enum class Fmt { FP16, W8A8, W4A4, W4A16, W3A16, UNSUPPORTED };
+enum class Fmt { FP16, W8A8, W4A4, W4A16, W3A16, W2A16, UNSUPPORTED };
 
 inline Fmt classify(const mxmoe_qparams& q) {
   if (q.a_bits >= 16 && q.w_bits >= 16) return Fmt::FP16;
@@ -130,6 +130,7 @@ inline Fmt classify(const mxmoe_qparams& q) {
   if (q.a_bits == 4 && q.w_bits == 4 && q.gsize == -1 && q.sym) return Fmt::W4A4;
   if (q.a_bits >= 16 && q.w_bits == 4 && q.gsize == 128) return Fmt::W4A16;
   if (q.a_bits >= 16 && q.w_bits == 3 && q.gsize == 128) return Fmt::W3A16;
+  if (q.a_bits >= 16 && q.w_bits == 2 && q.gsize == 128) return Fmt::W2A16;
   return Fmt::UNSUPPORTED;
 }
 
@@ -140,6 +141,7 @@ inline const char* fmt_name(Fmt f, bool sym) {
     case Fmt::W4A4: return "w4a4_g-1_sym";
     case Fmt::W4A16: return sym ? "w4a16_g128_sym" : "w4a16_g128_asym";
     case Fmt::W3A16: return sym ? "w3a16_g128_sym" : "w3a16_g128_asym";
+    case Fmt::W2A16: return sym ? "w2a16_g128_sym" : "w2a16_g128_asym";
     default: return "unsupported";
   }
 }
@@ -173,7 +175,7 @@ template <int WBITS, int BN>
 struct BranchOf<SkinnyWoTile<WBITS, BN>> {
   static BranchInfo get() {
     using T = SkinnyWoTile<WBITS, BN>;
-    return BranchInfo{WBITS == 4 ? Fmt::W4A16 : Fmt::W3A16, T::BM, BN, 128, 1, 4, T::kLdsBytes, 128, 0};
+    return BranchInfo{WBITS == 4 ? Fmt::W4A16 : WBITS == 3 ? Fmt::W3A16 : Fmt::W2A16, T::BM, BN, 128, 1, 4, T::kLdsBytes, 128, 0};
   }
 };
 
@@ -200,7 +202,7 @@ template <int WBITS, int BM, int BN>
 struct BranchOf<WoMfmaTile<WBITS, BM, BN>> {
   static BranchInfo get() {
     using T = WoMfmaTile<WBITS, BM, BN>;
-    return BranchInfo{WBITS == 4 ? Fmt::W4A16 : Fmt::W3A16, BM, BN, 128, 2, 2, T::kLdsBytes, 128, 0};
+    return BranchInfo{WBITS == 4 ? Fmt::W4A16 : WBITS == 3 ? Fmt::W3A16 : Fmt::W2A16, BM, BN, 128, 2, 2, T::kLdsBytes, 128, 0};
   }
 };
 
@@ -252,6 +254,7 @@ inline double tile_cost(const BranchInfo& b) {
       {Fmt::FP16, 128, 256, 1.00}, {Fmt::FP16, 64, 256, 0.69}, {Fmt::FP16, 32, 256, 0.53}, {Fmt::FP16, 128, 128, 0.57}, {Fmt::FP16, 256, 128, 1.09},
       {Fmt::W4A16, 16, 128, 0.37}, {Fmt::W4A16, 16, 64, 0.20}, {Fmt::W4A16, 128, 128, 1.00},
       {Fmt::W3A16, 16, 128, 0.31}, {Fmt::W3A16, 16, 64, 0.20}, {Fmt::W3A16, 128, 128, 1.00},
+      {Fmt::W2A16, 16, 128, 0.25}, {Fmt::W2A16, 16, 64, 0.20}, {Fmt::W2A16, 128, 128, 1.00},
   };
   for (const Row& r : table)
     if (r.f == b.fmt && r.bm == b.BM && r.bn == b.BN) return r.c;
@@ -261,7 +264,7 @@ inline double tile_cost(const BranchInfo& b) {
 // Rough run time of one tile across formats, used only to order the tile list (expensive shapes first): the matrix pipe runs
 // fp16 at half the int8 rate, and int4 operands are widened to int8.
 inline double branch_cost(const BranchInfo& b) {
-  const double per_k = b.fmt == Fmt::FP16 ? 2.0 : (b.fmt == Fmt::W4A16 || b.fmt == Fmt::W3A16) ? 1.2 : (b.fmt == Fmt::W8A8 ? 1.25 : 1.0);
+  const double per_k = b.fmt == Fmt::FP16 ? 2.0 : (b.fmt == Fmt::W4A16 || b.fmt == Fmt::W3A16 || b.fmt == Fmt::W2A16) ? 1.2 : (b.fmt == Fmt::W8A8 ? 1.25 : 1.0);
   return tile_cost(b) * per_k;
 }
 

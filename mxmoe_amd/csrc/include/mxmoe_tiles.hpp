@@ -102,7 +102,7 @@ __device__ __forceinline__ v4i gload16_untracked(const uint8_t* p) {
 }
 template <int N>
 __device__ __forceinline__ void vm_wait_for(v4i& v) {
-  asm volatile("s_waitcnt vmcnt(%1)" : "+v"(v) : "n"(N) : "memory");
+  asm volatile("s_waitcnt vmcnt(%1) ; landed %0" : "+v"(v) : "n"(N) : "memory");  // the comment names the register for the build's ISA check
 }
 template <int N>
 __device__ __forceinline__ void vm_wait() {
@@ -486,8 +486,12 @@ struct WxAxTile {
   static constexpr int kOps = OP == Op::I4 ? 2 : 1;
   static constexpr int U = 4;                                    // units per K slice
   static constexpr int kDmaTotal = BM / 16;                      // 1 KB pieces of one activation slice
+  // Activation loads per wave and slice.  Every wave issues the same number of loads, because the hand-placed waits count them: a
+  // tile with fewer pieces than waves (BM = 32) has the spare waves fetch a piece a second time (same bytes to the same LDS
+  // address) rather than branch on "does this wave load" around the waits - a value that is live across such a branch gets
+  // copied between registers, and a copy of a fragment register whose load is still in flight copies stale data.
   static constexpr int kDma = (kDmaTotal + kWaves - 1) / kWaves;
-  static_assert(kDmaTotal % kWaves == 0 || kDma == 1, "a wave has either all kDma pieces or none");
+  static_assert(kDmaTotal % kWaves == 0 || kDma == 1, "fewer pieces than waves: one (possibly repeated) piece per wave");
   static_assert(kDma <= U, "one activation load per unit");
   // loads issued after a wave's last activation load of a slice and before the barrier unit of the next iteration
   static constexpr int kYounger = (U - (kDma - 1)) + (kDma < 2 ? kDma : 2) + 2;
@@ -536,22 +540,19 @@ struct WxAxTile {
     int dma_voff[kDma];
 #pragma unroll
     for (int i = 0; i < kDma; ++i) {
-      const int r = (wave + kWaves * i) * 16 + (lane >> 2);
+      const int r = ((wave + kWaves * i) % kDmaTotal) * 16 + (lane >> 2);
       dma_voff[i] = r * (int)row_bytes + (((lane & 3) ^ lds_swizzle(r)) << 4);
     }
     auto dma_a = [&](int i, int kt, int stage) {
-      const int ii = wave + kWaves * i;
-      if (kDmaTotal % kWaves == 0 || ii < kDmaTotal) {
-        v4i rs = rs_a;
-        if (kt >= KT) rs[2] = 0;  // past the end of K: a load of zero bytes, still counted by vmcnt
-        dma16_to_lds(rs, lds_base + stage * kStageBytes + ii * 1024, dma_voff[i], __builtin_amdgcn_readfirstlane(kt * kRowBytes));
-      }
+      const int ii = (wave + kWaves * i) % kDmaTotal;
+      v4i rs = rs_a;
+      if (kt >= KT) rs[2] = 0;  // past the end of K: a load of zero bytes, still counted by vmcnt
+      dma16_to_lds(rs, lds_base + stage * kStageBytes + ii * 1024, dma_voff[i], __builtin_amdgcn_readfirstlane(kt * kRowBytes));
     };
-    const bool has_dma = kDmaTotal % kWaves == 0 || wave < kDmaTotal;  // whether this wave issues activation loads at all
     // wait until the weight fragment `uf` of the current slice has arrived (see younger_than_fragment), then hand it out
     auto ready = [&](auto ufc, v4i& frag) {
       constexpr int uf = decltype(ufc)::value;
-      if (has_dma) vm_wait_for<younger_than_fragment(uf, kDma)>(frag); else vm_wait_for<younger_than_fragment(uf, 0)>(frag);
+      vm_wait_for<younger_than_fragment(uf, kDma)>(frag);
     };
     const int lrow = lane & 31;
     const int fa = lrow * kRowBytes + (((lane >> 5) ^ lds_swizzle(lrow)) << 4);

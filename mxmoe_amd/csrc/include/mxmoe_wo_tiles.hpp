@@ -12,6 +12,7 @@
 // expert streams linearly.  Within a dword, element e of its 8 values sits in nibble (e >> 1) + 4*(e & 1), which
 // lets two masks and one shift produce four fp16 pairs in k order (magic-number conversion, no per-element shifts).
 // w3 stores 24 values in the low 3 bits of the 24 nibbles of three dwords; the 24 spare top bits hold values 24..31.
+// w2 stores values 16d..16d+7 in the low two bits of the nibbles of dword d and values 16d+8..16d+15 in the high two.
 //
 // The group scale is applied to the fp32 partial sum of each 128-wide group instead of to every weight:
 //   sum_k x[k]*(q[k]*s + z) = s * sum_k x[k]*q[k] + z * sum_k x[k]
@@ -31,7 +32,7 @@ namespace mxmoe {
 template <int WBITS_, int BN_>
 struct SkinnyWoTile {
   static constexpr int WBITS = WBITS_, BM = 16, BN = BN_;
-  static_assert(WBITS == 4 || WBITS == 3, "w4 / w3 only");
+  static_assert(WBITS == 4 || WBITS == 3 || WBITS == 2, "w4 / w3 / w2 only");
   static_assert(BN % 64 == 0, "the final reduction deals 16-channel blocks to 4 waves");
   static constexpr int NB = BN / 16;                 // 16-channel blocks per tile
   static constexpr int KP = 4;                       // k blocks (128 wide) per pass of a wave: their activations live in registers
@@ -52,10 +53,14 @@ struct SkinnyWoTile {
     if constexpr (WBITS == 4) {
       const v4i v = gload<v4i>(p);
       w.d[0] = v[0]; w.d[1] = v[1]; w.d[2] = v[2]; w.d[3] = v[3];
-    } else {
+    } else if constexpr (WBITS == 3) {
       typedef int v3i __attribute__((ext_vector_type(3)));
       const v3i v = gload<v3i>(p);  // 12 bytes: a 16-byte load would read past the end of the last block
       w.d[0] = v[0]; w.d[1] = v[1]; w.d[2] = v[2];
+    } else {
+      typedef int v2i __attribute__((ext_vector_type(2)));
+      const v2i v = gload<v2i>(p);
+      w.d[0] = v[0]; w.d[1] = v[1];
     }
     return w;
   }
@@ -79,11 +84,17 @@ struct SkinnyWoTile {
     if constexpr (WBITS == 4) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) out[j] = cvt8<0x000F000F, 0x00F000F0>(w.d[j]);
-    } else {
+    } else if constexpr (WBITS == 3) {
 #pragma unroll
       for (int j = 0; j < 3; ++j) out[j] = cvt8<0x00070007, 0x00700070>(w.d[j]);
       const int t = (int)(((unsigned)w.d[0] >> 3) & 0x11111111u) | (int)(((unsigned)w.d[1] >> 2) & 0x22222222u) | (int)(((unsigned)w.d[2] >> 1) & 0x44444444u);
       out[3] = cvt8<0x00070007, 0x00700070>(t);
+    } else {
+#pragma unroll
+      for (int d = 0; d < 2; ++d) {
+        out[2 * d] = cvt8<0x00030003, 0x00300030>(w.d[d]);
+        out[2 * d + 1] = cvt8<0x00030003, 0x00300030>((int)((unsigned)w.d[d] >> 2));
+      }
     }
   }
 

@@ -35,7 +35,7 @@ SUPPORTED_QCFG = [
     "fp16",
     "w8a8_g-1_sym",
     "w4a4_g-1_sym",
-    *[f"w{w}a16_g128_{s}" for w in (4, 3) for s in ("sym", "asym")],
+    *[f"w{w}a16_g128_{s}" for w in (4, 3, 2) for s in ("sym", "asym")],
 ]
 
 # (M, N, K) of one MFMA instruction
@@ -52,7 +52,7 @@ QCFG_TO_MMA = {
     "fp16": "MFMA_F32_32x32x16_F16",
     "w8a8_g-1_sym": "MFMA_I32_32x32x32_I8",
     "w4a4_g-1_sym": "MFMA_I32_32x32x32_I8_FROM_I4",
-    **{f"w{w}a16_g128_{s}": "MFMA_F32_16x16x32_F16" for w in (4, 3) for s in ("sym", "asym")},
+    **{f"w{w}a16_g128_{s}": "MFMA_F32_16x16x32_F16" for w in (4, 3, 2) for s in ("sym", "asym")},
 }
 
 
@@ -216,7 +216,7 @@ QCFG_MAP = {
     "fp16": TileConfig(),
     "w8a8_g-1_sym": TileConfig(QCFGA=QCFG_W8A8, QCFGB=QCFG_W8A8),
     "w4a4_g-1_sym": TileConfig(QCFGA=QCFG_W4A4, QCFGB=QCFG_W4A4),
-    **{k: TileConfig(QCFGB=build_qcfgb_from_str(k)) for k in [f"w{w}a16_g128_{s}" for w in (4, 3) for s in ("sym", "asym")]},
+    **{k: TileConfig(QCFGB=build_qcfgb_from_str(k)) for k in [f"w{w}a16_g128_{s}" for w in (4, 3, 2) for s in ("sym", "asym")]},
 }
 
 

@@ -61,13 +61,19 @@ def pack_weight_only(q: torch.Tensor, bits: int) -> torch.Tensor:
     bits == 4: dword j holds values 8j..8j+7, value e in nibble (e >> 1) + 4*(e & 1).
     bits == 3: dwords 0..2 hold values 0..23 in the low three bits of their nibbles; bit 3 of nibble p of
     dword d holds bit d of value 24 + e(p).
+    bits == 2: dword d holds values 16d..16d+7 in the low two bits of its nibbles and values 16d+8..16d+15 in the high two.
     """
-    assert bits in (3, 4)
+    assert bits in (2, 3, 4)
     n, k = q.shape
     assert n % 16 == 0 and k % 128 == 0
     v = q.to(torch.int64).reshape(n // 16, 16, k // 128, 4, 32)       # [nb, row, kb, g, e32]
     v = v.permute(0, 2, 3, 1, 4).reshape(n // 16, k // 128, 64, 32)    # lane = g*16 + row
     shifts = torch.tensor([4 * p for p in _NIBBLE_OF_ELEM], dtype=torch.int64, device=q.device)
+    if bits == 2:
+        pairs = v.reshape(*v.shape[:-1], 2, 2, 8)                      # [.., dword, low / high half of the nibbles, e]
+        dw = ((pairs[..., 0, :] | (pairs[..., 1, :] << 2)) << shifts).sum(dim=-1)
+        dw = torch.where(dw >= 2**31, dw - 2**32, dw).to(torch.int32)
+        return dw.reshape(-1).contiguous()
     ndw = 4 if bits == 4 else 3
     main = v[..., : ndw * 8].reshape(*v.shape[:-1], ndw, 8)
     dw = (main << shifts).sum(dim=-1)                                  # [nb, kb, 64, ndw]

@@ -213,3 +213,28 @@ def test_build_refuses_spilling_wxax_kernels():
     check_no_spills(fmt.format("_ZN5mxmoe12SkinnyWoTileILi4EEE", 3))        # compiler-tracked loads: spills are only slow
     with pytest.raises(RuntimeError, match="spilled"):
         check_no_spills(fmt.format("_ZN5mxmoe8WxAxTileILi1EEE", 45))
+
+
+def test_build_refuses_moves_of_registers_with_loads_in_flight():
+    """The build's ISA check: a register written by a hand-tracked (inline-assembly) load may not be moved before the wait that names it."""
+    from mxmoe_amd.build import check_untracked_load_copies as chk
+
+    def kernel(body):
+        return "_Z6kernelv:\n" + "\n".join(body) + "\n\ts_endpgm\n"
+
+    load = ["\t;;#ASMSTART", "\tglobal_load_dwordx4 v[10:13], v[2:3], off", "\t;;#ASMEND"]
+    wait = ["\t;;#ASMSTART", "\ts_waitcnt vmcnt(3) ; landed v[10:13]", "\t;;#ASMEND"]
+    move = ["\tv_mov_b64_e32 v[20:21], v[10:11]"]
+    chk(kernel(load + wait + move))                                  # copy of a landed value: fine
+    chk(kernel(load + ["\tv_mov_b32_e32 v30, v31"] + wait))          # unrelated registers: fine
+    with pytest.raises(RuntimeError, match="in flight"):
+        chk(kernel(load + move + wait))
+    with pytest.raises(RuntimeError, match="never waited"):
+        chk(kernel(load))
+    # loop: the load at the bottom of an iteration is in flight at the top of the next one
+    loop = [".LBB0_1:                                ; =>This Inner Loop Header: Depth=1"] + move + wait + ["\tv_and_b32_e32 v5, v10, v4"] + load + \
+           ["\ts_cbranch_scc1 .LBB0_1", ".LBB0_2:"] + wait
+    with pytest.raises(RuntimeError, match="in flight"):
+        chk(kernel(load + loop))
+    ok_loop = [".LBB0_1:                                ; =>This Inner Loop Header: Depth=1"] + wait + move + load + ["\ts_cbranch_scc1 .LBB0_1", ".LBB0_2:"] + wait
+    chk(kernel(load + ok_loop))

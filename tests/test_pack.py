@@ -24,6 +24,8 @@ def _unpack_model(dw, bits):
     dw = dw.astype(np.int64) & 0xFFFFFFFF
     if bits == 4:
         return np.concatenate([_cvt8(dw[..., j], 4) for j in range(4)], axis=-1)
+    if bits == 2:  # out[2d] = cvt8(d), out[2d + 1] = cvt8(d >> 2), two-bit masks
+        return np.concatenate([_cvt8(dw[..., d] >> sh, 2) for d in range(2) for sh in (0, 2)], axis=-1)
     t = ((dw[..., 0] >> 3) & 0x11111111) | ((dw[..., 1] >> 2) & 0x22222222) | ((dw[..., 2] >> 1) & 0x44444444)
     return np.concatenate([_cvt8(dw[..., j], 3) for j in range(3)] + [_cvt8(t, 3)], axis=-1)
 
@@ -44,7 +46,7 @@ def test_int4_k_pack_roundtrip_and_nibble_order():
 
 
 def test_weight_only_pack_matches_kernel_unpack_model():
-    for bits in (4, 3):
+    for bits in (4, 3, 2):
         n, k = 48, 384
         codes = torch.randint(0, 1 << bits, (n, k), dtype=torch.uint8)
         dw = pack.pack_weight_only(codes, bits).numpy().reshape(n // 16, k // 128, 64, bits)
