@@ -29,7 +29,7 @@ const char* mxmoe_kernel_name(int kernel_id);
 /* Index of the kernel whose name equals or ends with `name`, or -1. */
 int mxmoe_find_kernel(const char* name);
 /* Number of tile branches of a kernel, and the description of one:
- * out[0..7] = {format (0 fp16, 1 w8a8, 2 w4a4, 3 w4a16 g128, 4 w3a16 g128), BM, BN, BK, WGM, WGN, lds_bytes, k_multiple}. */
+ * out[0..7] = {format (0 fp16, 1 w8a8, 2 w4a4, 3 w4a16 g128, 4 w3a16 g128, 5 w2a16 g128), BM, BN, BK, WGM, WGN, lds_bytes, k_multiple}. */
 int mxmoe_kernel_num_branches(int kernel_id);
 int mxmoe_kernel_branch(int kernel_id, int branch, int32_t out[8]);
 
@@ -45,7 +45,7 @@ int mxmoe_kernel_branch(int kernel_id, int branch, int32_t out[8]);
  *   fp16              fp16 [M,K]                 fp16 [N,K]                          -               -
  *   w8a8_g-1_sym      int8 [M,K]                 fragment blocks of int8 [N,K]  (*)  fp16 [M]        fp16 [N]
  *   w4a4_g-1_sym      int4 [M,K/2] (even k low)  fragment blocks of int4 [N,K/2] (*) fp16 [M]        fp16 [N]
- *   w{4,3}a16_g128    fp16 [M,K]                 packed [N/16][K/128][64][w dwords]  -               fp16 [N/16][K/128][16][2]
+ *   w{4,3,2}a16_g128  fp16 [M,K]                 packed [N/16][K/128][64][w dwords]  -               fp16 [N/16][K/128][16][2]
  *
  * (*) weights of the integer formats are stored in MFMA fragment order: uint8 [ceil(N/32)][KB/64][2][64 lanes][16], KB = bytes per
  *     row; lane l of block (nb, ks, step) holds bytes ks*64 + (2*step + (l >> 5))*16 .. +16 of channel nb*32 + (l & 31), channels past N
