@@ -25,7 +25,7 @@
 
 namespace mxmoe {
 
-constexpr int kMaxProblems = 128;  // per launch; longer problem lists are split into several launches
+constexpr int kMaxProblems = 120;  // per launch (the tables ride in the 4 KB kernel argument block); longer problem lists are split into several launches
 constexpr int kMaxEntries = 2 * kMaxProblems;  // a problem is run as at most two row segments, each with its own tile shape
 constexpr int kNumXcd = 8;
 constexpr int kMaxPhases = 8;
@@ -48,12 +48,15 @@ struct FusedArgs {
   int num_phases;
   int phase_tile0[kMaxPhases + 1];
   int phase_wg0[kMaxPhases + 1];
-  int prefix[kMaxEntries];        // inclusive prefix sum of tiles per entry
-  int row0[kMaxEntries];          // first row of the entry's segment inside its problem
-  int rows[kMaxEntries];          // rows of the segment
-  uint16_t problem[kMaxEntries];  // problem (relative to problem_offset) the entry belongs to
-  uint8_t branch[kMaxEntries];    // which tile type runs the entry
+  // One entry per row segment of a problem, 16 bytes so that a workgroup fetches its entry with one scalar load: first tile of the
+  // entry (exclusive prefix sum of tiles), first row of the segment inside its problem, rows of the segment, and
+  // problem (relative to problem_offset) | tile type << 16.
+  struct Entry {
+    int first, row0, rows, problem_branch;
+  };
+  Entry entry[kMaxEntries];
 };
+static_assert(sizeof(FusedArgs) <= 4096, "kernel arguments are limited to 4 KB");
 
 template <int I, class... Tiles>
 struct Dispatch;
@@ -95,15 +98,16 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd<Tiles...>) fused_group
   const int pt = (v % kNumXcd) * chunk + v / kNumXcd;
   if (pt >= ntiles) return;
   const int tile = args.phase_tile0[ph] + pt;
-  // tile_scheduler.cuh:25-37 — first problem whose inclusive prefix exceeds the tile index (binary search here)
+  // tile_scheduler.cuh:25-37 — the entry that holds the tile: last entry whose first tile is <= tile (binary search here; all
+  // indices are wave-uniform, so these are scalar loads from the argument block)
   int lo = 0, hi = args.num_entries - 1;
   while (lo < hi) {
-    const int mid = (lo + hi) >> 1;
-    if (tile < args.prefix[mid]) hi = mid; else lo = mid + 1;
+    const int mid = (lo + hi + 1) >> 1;
+    if (args.entry[mid].first <= tile) lo = mid; else hi = mid - 1;
   }
-  const int en = lo;
-  const int local = tile - (en ? args.prefix[en - 1] : 0);
-  const int gp = args.problem_offset + args.problem[en];
+  const FusedArgs::Entry en = args.entry[lo];
+  const int local = tile - en.first;
+  const int gp = args.problem_offset + (en.problem_branch & 0xFFFF);
   const mxmoe_dim3 sz = args.sizes[gp];
   TileArgs t;
   t.A = args.As[gp];
@@ -112,12 +116,12 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd<Tiles...>) fused_group
   t.sb = args.sb ? args.sb[gp] : nullptr;
   t.C = args.Cs[gp];
   t.acc_dump = args.acc ? args.acc[gp] : nullptr;
-  t.row0 = args.row0[en];
-  t.M = t.row0 + args.rows[en];  // rows past the segment are treated like rows past the problem
+  t.row0 = en.row0;
+  t.M = t.row0 + en.rows;  // rows past the segment are treated like rows past the problem
   t.N = (int)sz.y;
   t.K = (int)sz.z;
   t.tile_m = t.tile_n = 0;
-  Dispatch<0, Tiles...>::go(args.branch[en], t, local, smem);
+  Dispatch<0, Tiles...>::go(en.problem_branch >> 16, t, local, smem);
 }
 
 // ------------------------------------------------------------------ host side ------------------------------------------------------------------
@@ -405,12 +409,8 @@ inline int group_gemm(int kernel_id, const void* const* As, const void* const* B
       for (int ei = 0; ei < nent; ++ei) {
         const Entry& en = entries[ei];
         if (en.branch != b || en.tiles == 0) continue;
+        a.entry[ne] = FusedArgs::Entry{total, en.row0, en.rows, en.problem | (en.branch << 16)};
         total += en.tiles;
-        a.prefix[ne] = total;
-        a.row0[ne] = en.row0;
-        a.rows[ne] = en.rows;
-        a.problem[ne] = (uint16_t)en.problem;
-        a.branch[ne] = (uint8_t)en.branch;
         ++ne;
       }
       if (total == tile0) continue;
