@@ -63,9 +63,9 @@ def _offsets(recv_cpu, num_tokens: int, num_experts: int, has_shared: bool, qpar
     et = num_experts + (1 if has_shared else 0)
     if len(qparams_per_exp) < et:
         raise RuntimeError(f"qparams_per_exp has {len(qparams_per_exp)} entries, need {et}")
-    rows = []
-    table = torch.zeros((4, et), dtype=torch.int64)
-    inp_sizes, scale_sizes, lds = [], [], []
+    rows, inp_sizes, scale_sizes, lds = [], [], [], []
+    cols = [[], [], [], []]                                  # tag, first row, input offset, scale offset per expert
+    recv_list = recv_cpu.tolist() if hasattr(recv_cpu, "tolist") else list(recv_cpu)
     acc = io = so = 0
     for e in range(et):
         a_bits, _w, g, _s = qparams_per_exp[e]
@@ -75,8 +75,9 @@ def _offsets(recv_cpu, num_tokens: int, num_experts: int, has_shared: bool, qpar
         width = ld_shared if e == num_experts else ld
         qld = width if tag == 0 else (width // 2 if tag == 1 else width // 4)
         sld = 0 if tag == 0 else 1
-        n = num_tokens if e == num_experts else int(recv_cpu[e])
-        table[0, e], table[1, e], table[2, e], table[3, e] = tag, acc, io, so
+        n = num_tokens if e == num_experts else int(recv_list[e])
+        for c, v in zip(cols, (tag, acc, io, so)):
+            c.append(v)
         rows.append(n)
         inp_sizes.append(qld * n)
         scale_sizes.append(sld * n)
@@ -84,17 +85,18 @@ def _offsets(recv_cpu, num_tokens: int, num_experts: int, has_shared: bool, qpar
         acc += n
         io += qld * n
         so += sld * n
-    return table, rows, inp_sizes, scale_sizes, lds, io, so
+    return torch.tensor(cols, dtype=torch.int64), rows, inp_sizes, scale_sizes, lds, io, so
 
 
 def _views(store, scale_store, table, rows, inp_sizes, scale_sizes, lds):
     inp_list, scale_list = [], []
+    inp_off, scale_off = table[2].tolist(), table[3].tolist()
     for e, n in enumerate(rows):
         if n == 0:
             continue
-        off = int(table[2, e])
+        off = inp_off[e]
         inp_list.append(store[off:off + inp_sizes[e]].view(n, lds[e]))
-        soff = int(table[3, e])
+        soff = scale_off[e]
         scale_list.append(scale_store[soff:soff + scale_sizes[e]])
     return inp_list, scale_list
 
@@ -194,8 +196,9 @@ def gg_unpermute_out(out_store: torch.Tensor, topk_ids: torch.Tensor, topk_weigh
 
 def _problem_lists(num_experts: int, experts, recv_cpu, num_tokens: int):
     has_shared = len(experts) > num_experts
+    recv_list = recv_cpu.tolist()
     for e in range(num_experts + (1 if has_shared else 0)):
-        n = num_tokens if e == num_experts else int(recv_cpu[e])
+        n = num_tokens if e == num_experts else int(recv_list[e])
         if n:
             yield e, n
 
