@@ -54,34 +54,44 @@ __global__ void __launch_bounds__(64) perm_hist_kernel(const int32_t* __restrict
   for (int e = threadIdx.x; e < E; e += 64) hist[blockIdx.x * E + e] = cnt[e];
 }
 
-// one workgroup: per expert, exclusive scan over blocks; expert offsets; counts as int64
-__global__ void __launch_bounds__(256) perm_scan_kernel(int32_t* __restrict__ hist, int blocks, int E, int64_t* __restrict__ recv, int32_t* __restrict__ expert_off) {
-  extern __shared__ int32_t tot[];
-  for (int e = threadIdx.x; e < E; e += 256) {
-    int run = 0;
-    for (int b = 0; b < blocks; ++b) {
-      const int v = hist[b * E + e];
-      hist[b * E + e] = run;
-      run += v;
-    }
-    tot[e] = run;
-    recv[e] = run;
+// inclusive scan of one value per lane across the wave
+__device__ __forceinline__ int wave_inclusive_scan(int v, int lane) {
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const int t = __shfl_up(v, o);
+    if (lane >= o) v += t;
   }
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    int run = 0;
-    for (int e = 0; e < E; ++e) {
-      expert_off[e] = run;
-      run += tot[e];
-    }
+  return v;
+}
+
+// one single-wave workgroup per expert: exclusive scan of the expert's per-block counts (64 blocks per step); total -> recv
+__global__ void __launch_bounds__(64) perm_scan_kernel(int32_t* __restrict__ hist, int blocks, int E, int64_t* __restrict__ recv) {
+  const int e = blockIdx.x, lane = threadIdx.x;
+  int carry = 0;
+  for (int b0 = 0; b0 < blocks; b0 += 64) {
+    const int b = b0 + lane;
+    const int v = b < blocks ? hist[b * E + e] : 0;
+    const int inc = wave_inclusive_scan(v, lane);
+    if (b < blocks) hist[b * E + e] = carry + inc - v;
+    carry += __shfl(inc, 63);
   }
+  if (lane == 0) recv[e] = carry;
 }
 
 __global__ void __launch_bounds__(64) perm_scatter_kernel(const int32_t* __restrict__ ids, int total, int E, int topk, int nbits, const int32_t* __restrict__ hist,
-                                                          const int32_t* __restrict__ expert_off, int32_t* __restrict__ dst_exp_sorted, int64_t* __restrict__ perm,
+                                                          const int64_t* __restrict__ recv, int32_t* __restrict__ dst_exp_sorted, int64_t* __restrict__ perm,
                                                           int64_t* __restrict__ src_slot) {
   extern __shared__ int32_t run[];  // next free rank per expert for this block
-  for (int e = threadIdx.x; e < E; e += 64) run[e] = expert_off[e] + hist[blockIdx.x * E + e];
+  {  // first row of every expert = exclusive scan of the per-expert totals, plus this block's offset inside the expert
+    int carry = 0;
+    for (int e0 = 0; e0 < E; e0 += 64) {
+      const int e = e0 + (int)threadIdx.x;
+      const int v = e < E ? (int)recv[e] : 0;
+      const int inc = wave_inclusive_scan(v, threadIdx.x);
+      if (e < E) run[e] = carry + inc - v + hist[blockIdx.x * E + e];
+      carry += __shfl(inc, 63);
+    }
+  }
   __syncthreads();
   const int lane = threadIdx.x;
   const int base = blockIdx.x * kPermChunk;
@@ -701,13 +711,12 @@ int mxmoe_build_permutation(const int32_t* topk_ids, int num_tokens, int topk, i
   hipStream_t s = (hipStream_t)stream;
   const int blocks = (total + kPermChunk - 1) / kPermChunk;
   int32_t* hist = reinterpret_cast<int32_t*>(workspace);
-  int32_t* expert_off = hist + (size_t)blocks * num_experts;
   int nbits = 1;
   while ((1 << nbits) <= num_experts) ++nbits;  // ids 0..E (E = parked lanes)
   const size_t lds = (size_t)num_experts * sizeof(int32_t);
   hipLaunchKernelGGL(perm_hist_kernel, dim3(blocks), dim3(64), lds, s, topk_ids, total, num_experts, hist);
-  hipLaunchKernelGGL(perm_scan_kernel, dim3(1), dim3(256), lds, s, hist, blocks, num_experts, recv_tokens_per_exp, expert_off);
-  hipLaunchKernelGGL(perm_scatter_kernel, dim3(blocks), dim3(64), lds, s, topk_ids, total, num_experts, topk, nbits, hist, expert_off, dst_exp_sorted, perm_indices,
+  hipLaunchKernelGGL(perm_scan_kernel, dim3(num_experts), dim3(64), 0, s, hist, blocks, num_experts, recv_tokens_per_exp);
+  hipLaunchKernelGGL(perm_scatter_kernel, dim3(blocks), dim3(64), lds, s, topk_ids, total, num_experts, topk, nbits, hist, recv_tokens_per_exp, dst_exp_sorted, perm_indices,
                      src_slot);
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
