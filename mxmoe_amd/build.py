@@ -83,6 +83,19 @@ def check_untracked_load_copies(asm: str) -> None:
             order += list(range(pos, lo)) + list(range(lo, hi)) * 2
             pos = hi
         order += list(range(pos, end))
+        # a loop that issues hand-tracked loads counts every vector-memory instruction: the compiler must not add its own there
+        for lo, hi in regions:
+            body = [lines[i].strip() for i in range(lo, hi)]
+            tracked, inside = False, False
+            for t in body:
+                inside = True if t.startswith(";;#ASMSTART") else False if t.startswith(";;#ASMEND") else inside
+                tracked |= inside and t.startswith("global_load")
+            inside = False
+            for k, t in enumerate(body):
+                inside = True if t.startswith(";;#ASMSTART") else False if t.startswith(";;#ASMEND") else inside
+                if tracked and not inside and re.match(r"(global_|buffer_|flat_|scratch_)(load|store|atomic)", t):
+                    raise RuntimeError(f"{kernel}: line {lo + k + 1} `{t}`: compiler-generated vector-memory instruction inside a loop whose "
+                                       f"loads are counted by hand")
         inflight, in_asm = set(), False
         for i in order:
             t = lines[i].strip()

@@ -238,3 +238,18 @@ def test_build_refuses_moves_of_registers_with_loads_in_flight():
         chk(kernel(load + loop))
     ok_loop = [".LBB0_1:                                ; =>This Inner Loop Header: Depth=1"] + wait + move + load + ["\ts_cbranch_scc1 .LBB0_1", ".LBB0_2:"] + wait
     chk(kernel(load + ok_loop))
+
+
+def test_build_refuses_compiler_memory_instructions_in_hand_counted_loops():
+    from mxmoe_amd.build import check_untracked_load_copies as chk
+
+    load = ["\t;;#ASMSTART", "\tglobal_load_dwordx4 v[10:13], v[2:3], off", "\t;;#ASMEND"]
+    wait = ["\t;;#ASMSTART", "\ts_waitcnt vmcnt(3) ; landed v[10:13]", "\t;;#ASMEND"]
+    head = [".LBB0_1:                                ; =>This Inner Loop Header: Depth=1"]
+    tail = ["\ts_cbranch_scc1 .LBB0_1", ".LBB0_2:"]
+    mk = lambda body: "_Z6kernelv:\n" + "\n".join(load + head + body + tail + wait) + "\n\ts_endpgm\n"
+    chk(mk(wait + load))
+    with pytest.raises(RuntimeError, match="counted by hand"):
+        chk(mk(wait + ["\tglobal_load_dword v40, v[2:3], off"] + load))
+    # loops without hand-tracked loads may hold any memory instruction
+    chk("_Z6kernelv:\n" + "\n".join(head + ["\tglobal_load_dword v40, v[2:3], off"] + tail) + "\n\ts_endpgm\n")
