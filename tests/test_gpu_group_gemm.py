@@ -90,6 +90,24 @@ def test_wxax_few_row_problems_every_wave_every_launch():
                 assert np.array_equal(out.view(np.uint16), p["out"].view(np.uint16))
 
 
+def test_more_problems_than_one_launch_holds():
+    """A problem list longer than one launch's table (120 problems) runs as several launches; empty problems in between are skipped."""
+    rng = np.random.default_rng(12)
+    probs = []
+    for i in range(150):
+        m = [0, 1, 5, 33, 64][i % 5]
+        b = 4 if i % 2 else 8
+        p = _wxax_problem(rng, max(m, 1), 256, 128, b)
+        if m == 0:
+            p.update(A=torch.zeros((0, 128 if b == 8 else 64), dtype=torch.int8, device=DEV), sa=torch.zeros(0, dtype=torch.float16, device=DEV),
+                     size=(0, 256, 128), acc=p["acc"][:0], out=p["out"][:0])
+        probs.append(p)
+    _, outs, accs = _launch(probs)
+    for i, (p, out, acc) in enumerate(zip(probs, outs, accs)):
+        assert np.array_equal(acc, p["acc"]), f"problem {i} {p['size']}"
+        assert np.array_equal(out.view(np.uint16), p["out"].view(np.uint16)), f"problem {i} {p['size']}"
+
+
 def test_fp16_group_gemm():
     rng = np.random.default_rng(2)
     probs = []
