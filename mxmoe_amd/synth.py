@@ -13,7 +13,7 @@ Seeds (torch.Generator on the CPU): weights 0, activations 1, router 2, format d
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, field, replace
+from dataclasses import dataclass, replace
 
 import torch
 
