@@ -92,6 +92,12 @@ class MxMoELayer:
         self.down()
         return self.state["out"]
 
+    def __call__(self, hidden: torch.Tensor, topk_ids: torch.Tensor, topk_weights: torch.Tensor) -> torch.Tensor:
+        """The whole MoE MLP, `(hidden [T, K] fp16, topk_ids [T, k] int32, topk_weights [T, k] fp32) -> [T, K] fp16`: what a serving
+        framework's fused-MoE operator computes after routing (permute, quantise, gate_up, SiLU * up, down, un-permute + combine)."""
+        self.forward(hidden, topk_ids)
+        return self.combine(topk_weights)
+
     # ---- accounting -----------------------------------------------------------------------------------------
     def gemm_ops(self) -> int:
         st = self.state

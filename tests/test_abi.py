@@ -78,3 +78,41 @@ def test_missing_library_fails_loudly(tmp_path):
 
     with pytest.raises(RuntimeError, match="no CPU fallback"):
         _lib.load(tmp_path / "libmissing.so")
+
+
+def test_plan_bounds_on_random_problem_lists(lib):
+    """Host planner on random problem lists (every format, empty problems, lists longer than one launch's table): it never fails, and
+    the tile count lies between what the largest and the smallest tile shapes of the chosen kernel would need."""
+    import random
+
+    rnd = random.Random(7)
+    fmts = [((4, 4, -1, True), 128), ((8, 8, -1, True), 64), ((16, 4, 128, False), 128), ((16, 3, 128, False), 128), ((16, 2, 128, True), 128),
+            ((16, 16, -1, True), 32)]
+    out = (C.c_int32 * 8)()
+    for trial in range(40):
+        nprob = rnd.choice([1, 3, 17, 60, 121, 260])
+        pick = rnd.sample(fmts, rnd.choice([1, 2, 3]))
+        probs = []
+        for _ in range(nprob):
+            q, kmul = rnd.choice(pick)
+            m = rnd.choice([0, 1, 7, 31, 32, 33, 100, 129, 546, 5000, 40000])
+            n = 16 * rnd.randint(1, 400)
+            k = kmul * rnd.randint(1, 40)
+            probs.append(((m, n, k), q))
+        rc, br, tiles = _plan(lib, -1, probs)
+        assert rc >= 1000, (lib.mxmoe_last_error(), probs[:3])
+        kid = rc - 1000
+        shapes = []
+        for b in range(lib.mxmoe_kernel_num_branches(kid)):
+            assert lib.mxmoe_kernel_branch(kid, b, out) == 0
+            shapes.append((out[0], out[1], out[2]))
+        lo = hi = 0
+        fmt_id = {(4, 4): 2, (8, 8): 1, (16, 4): 3, (16, 3): 4, (16, 2): 5, (16, 16): 0}
+        for (m, n, k), q in probs:
+            mine = [(bm, bn) for f, bm, bn in shapes if f == fmt_id[(q[0], q[1])]]
+            assert mine, "the chosen kernel has a tile for every format of the list"
+            if m == 0:
+                continue
+            lo += min(-(-m // bm) * -(-n // bn) for bm, bn in mine if bm == max(x for x, _ in mine))
+            hi += max(-(-m // bm) * -(-n // bn) for bm, bn in mine)
+        assert lo <= tiles <= hi, (trial, lo, tiles, hi)

@@ -112,6 +112,8 @@ def test_layer_combine_end_to_end():
     outs = layer.forward(hidden, ids)
     final = layer.combine(w)
     torch.cuda.synchronize()
+    assert torch.equal(layer(hidden, ids, w), final)              # the one-call form
+    outs = layer.state["out"]
     _, _, slot, recv = O.permute_by_expert(ids.numpy(), cfg.num_experts)
     rows = np.concatenate([o.cpu().numpy() for o in outs[:-1]])
     ref = O.unpermute_combine(rows, slot, w.numpy(), outs[-1].cpu().numpy())
