@@ -214,7 +214,7 @@ def main() -> int:
                     help="instead of the benchmark, run a plain device copy of BYTES bytes 5 times (reference point for the FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py measures one GPU: this build has no multi-GPU path (the layer would shard by expert; see DESIGN.md). Use --gpus 1.", file=sys.stderr)
+        print("bench.py measures one GPU: this build has no multi-GPU path (the layer would shard by expert, one all-to-all of rows either side of the launches). Use --gpus 1.", file=sys.stderr)
         return 2
 
     import torch

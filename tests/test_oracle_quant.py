@@ -97,7 +97,7 @@ def test_int_gemm_matches_python_int_bruteforce():
         for n in range(7):
             assert int(acc[m, n]) == sum(int(a[m, k]) * int(b[n, k]) for k in range(37))
     assert acc.dtype == np.int32 and acc.shape == (5, 7)                   # [M, N], not transposed
-    # worst-case magnitude at the largest BASELINE K stays inside int32
+    # worst-case magnitude at the largest K of the benchmark workloads (14336) stays inside int32
     k = 14336
     assert O.int_gemm(np.full((1, k), 127), np.full((1, k), -127))[0, 0] == -127 * 127 * k
 
