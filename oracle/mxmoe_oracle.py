@@ -22,6 +22,8 @@ fails a test in ``tests/test_oracle_*.py``):
 * ``permute_by_expert``   — brute force against a dict-of-lists.
 * ``tile_to_problem``     — every (problem, tile_m, tile_n) visited exactly once.
 * ``silu_mul``            — float64 ``x*sigmoid(x)*u`` within one fp16 ulp.
+* ``unpermute_combine``   — one-hot weights return the routed row bit for bit, dense float64 sum
+  within fp16 rounding (+ shared row), independence of the order of the sorted rows, dropped slots.
 
 Parity unpinned (see also the header of ``online_hadamard``): the reference's online rotation
 calls the third-party ``fast_hadamard_transform`` CUDA package (Dao-AILab, version unpinned,
