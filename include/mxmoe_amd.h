@@ -29,7 +29,7 @@ const char* mxmoe_kernel_name(int kernel_id);
 /* Index of the kernel whose name equals or ends with `name`, or -1. */
 int mxmoe_find_kernel(const char* name);
 /* Number of tile branches of a kernel, and the description of one:
- * out[0..7] = {format (0 fp16, 1 w8a8, 2 w4a4, 3 w4a16 g128, 4 w3a16 g128, 5 w2a16 g128), BM, BN, BK, WGM, WGN, lds_bytes, k_multiple}. */
+ * out[0..7] = {format (0 fp16, 1 w8a8, 2 w4a4, 3 w4a16 g128, 4 w3a16 g128, 5 w2a16 g128, 6 w4a4 g128), BM, BN, BK, WGM, WGN, lds_bytes, k_multiple}. */
 int mxmoe_kernel_num_branches(int kernel_id);
 int mxmoe_kernel_branch(int kernel_id, int branch, int32_t out[8]);
 
@@ -45,6 +45,7 @@ int mxmoe_kernel_branch(int kernel_id, int branch, int32_t out[8]);
  *   fp16              fp16 [M,K]                 fp16 [N,K]                          -               -
  *   w8a8_g-1_sym      int8 [M,K]                 fragment blocks of int8 [N,K]  (*)  fp16 [M]        fp16 [N]
  *   w4a4_g-1_sym      int4 [M,K/2] (even k low)  fragment blocks of int4 [N,K/2] (*) fp16 [M]        fp16 [N]
+ *   w4a4_g128_sym     int4 [M,K/2] (even k low)  fragment blocks of int4 [N,K/2] (*) fp16 [M,K/128]  fp16 [K/128,N] (group-major)
  *   w{4,3,2}a16_g128  fp16 [M,K]                 packed [N/16][K/128][64][w dwords]  -               fp16 [N/16][K/128][16][2]
  *
  * (*) weights of the integer formats are stored in MFMA fragment order: uint8 [ceil(N/32)][KB/64][2][64 lanes][16], KB = bytes per
@@ -53,7 +54,8 @@ int mxmoe_kernel_branch(int kernel_id, int branch, int32_t out[8]);
  *
  * kernel_id = -1 selects the first registered kernel that has a tile for every format in h_q.
  * acc_dump (optional, may be NULL) is a DEVICE array of per-problem int32 [M,N] buffers (entries may be NULL) that
- * receive the raw accumulators (int32 for w8a8 / w4a4, fp32 bit patterns otherwise); used by the parity tests.
+ * receive the raw accumulators (int32 for w8a8 / w4a4 per channel, fp32 bit patterns otherwise: for w4a4_g128 the fp32 sum over the
+ * groups of float(group's int32 sum) * (scale_a * scale_b), groups in ascending order); used by the parity tests.
  * Errors: 1 "quant type not supported" (same text as the reference launcher, compose_kernel.py:433), 2 bad kernel id,
  * 3 unsupported shape (K not a multiple of the tile's K step, N not a multiple of 8), 4 launch failure. */
 int mxmoe_group_gemm(int kernel_id, const void* const* As, const void* const* Bs, const void* const* scale_a, const void* const* scale_b,
@@ -83,8 +85,9 @@ int mxmoe_build_permutation(const int32_t* topk_ids, int num_tokens, int topk, i
  *
  * One workgroup per destination row; rows 0..R-1 are the routed rows in sorted order, rows R..R+T-1 (when has_shared) the
  * always-on shared expert, stored as expert index E.  exp_table is a DEVICE int64 [4][E(+1)] table: tag (0 fp16 copy,
- * 1 int8 per token, 2 int4 per token), first row, offset into inp_store and offset into scale_store, both offsets in fp16
- * elements exactly as ref_bind.cu:475-505 computes them (row strides K, K/2, K/4 halves; one scale per row).
+ * 1 int8 per token, 2 int4 per token, 3 int4 with one scale per 128 values), first row, offset into inp_store and offset into
+ * scale_store, both offsets in fp16 elements exactly as ref_bind.cu:475-505 computes them (row strides K, K/2, K/4, K/4 halves; one
+ * scale per row, K/128 scales per row for tag 3).
  * rotate: 0 no rotation, 1 rotate rows of quantised experts, 2 rotate every row, with y = (H_k kron H_{n/k}) x / sqrt(n)
  * (mxmoe/quant/hadamard_utils.py:96-106).  had_k = 1 for power-of-two rows; otherwise H_k = S_f kron B and had_signs is a
  * DEVICE float [(k/f)^2] array holding B as +-1.0 (mxmoe/quant/hadamard_utils.py:162-4379 tables).

@@ -6,7 +6,7 @@
 // The reference launches `quant_act_kernel` / `silu_mul_then_quant_kernel` (mxmoe/kernels/src/ref_bind.cu:531-544,
 // 701-716) whose source file (act_kernel.cuh) is absent from the reference; the contracts implemented here are the
 // launch arguments and the host offset builder of ref_bind.cu:461-505, 635-671: one workgroup per destination row,
-// rows grouped by expert, per-expert tag {0 fp16 copy, 1 int8, 2 int4}, row strides K, K/2, K/4 halves, one fp16
+// rows grouped by expert, per-expert tag {0 fp16 copy, 1 int8, 2 int4, 3 int4 with a scale per 128 values}, row strides K, K/2, K/4 halves, one fp16
 // scale per row.  The permutation replaces torch::sort + bincount of ref_bind.cu:47-64,449-453 with a STABLE order.
 //
 // Arithmetic is the exact operation sequence of the fp16 quantiser (mxmoe/quant/quant.py:68-84: absmax / upper,
@@ -399,6 +399,38 @@ __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
       }
       continue;
     }
+    if (tag == 3) {
+      // int4 with one scale per 128 values: a group is 16 consecutive chunks, i.e. the 16 lanes of an aligned lane group (the chunk
+      // index and the lane index agree modulo 16), so its absmax is a 4-step exchange inside those lanes.  Row: n / 2 bytes of codes,
+      // n / 128 scales.
+      uint8_t* out = a.inp_store + 2 * (inp_off + lrow * (n / 4));
+      _Float16* sout = a.scale_store + scale_off + lrow * (n >> 7);
+#pragma unroll
+      for (int i = 0; i < MAXC; ++i) {
+        const int c = tid + i * NT;
+        const bool live = c < nchunks;  // whole lane groups are live or not: n is a multiple of 128
+        float gmax = 0.0f;
+        if (live) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) gmax = fmaxf(gmax, fabsf(v[i][j]));
+        }
+#pragma unroll
+        for (int o = 8; o > 0; o >>= 1) gmax = fmaxf(gmax, __shfl_xor(gmax, o));
+        float scale = round_h(gmax / 7.0f);
+        if (scale == 0.0f) scale = 1.0f;
+        if (live) {
+          if ((c & 15) == 0) sout[c >> 4] = (_Float16)scale;
+          unsigned w = 0;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const float r = round_h(v[i][j] / scale);
+            w |= (unsigned)((int)rintf(fminf(fmaxf(r, -7.0f), 7.0f)) & 0xF) << (4 * j);
+          }
+          *reinterpret_cast<unsigned*>(out + c * 4) = w;
+        }
+      }
+      continue;
+    }
     float amax = 0.0f;
 #pragma unroll
     for (int i = 0; i < MAXC; ++i) {
@@ -537,6 +569,30 @@ __global__ void __launch_bounds__(256) row_quant_wave_kernel(const RowArgs a) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) o[j] = (_Float16)v[i][j];
         *reinterpret_cast<v8h*>(out + (lane + 64 * i) * 8) = o;
+      }
+      continue;
+    }
+    if (tag == 3) {  // int4, one scale per 128 values = the 16 chunks held by an aligned group of 16 lanes
+      uint8_t* out = a.inp_store + 2 * (inp_off + lrow * (n / 4));
+      _Float16* sout = a.scale_store + scale_off + lrow * (n >> 7);
+#pragma unroll
+      for (int i = 0; i < NI; ++i) {
+        const int c = lane + 64 * i;
+        float gmax = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) gmax = fmaxf(gmax, fabsf(v[i][j]));
+#pragma unroll
+        for (int o = 8; o > 0; o >>= 1) gmax = fmaxf(gmax, __shfl_xor(gmax, o));
+        float scale = round_h(gmax / 7.0f);
+        if (scale == 0.0f) scale = 1.0f;
+        if ((c & 15) == 0) sout[c >> 4] = (_Float16)scale;
+        unsigned w = 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float r = round_h(v[i][j] / scale);
+          w |= (unsigned)((int)rintf(fminf(fmaxf(r, -7.0f), 7.0f)) & 0xF) << (4 * j);
+        }
+        *reinterpret_cast<unsigned*>(out + c * 4) = w;
       }
       continue;
     }

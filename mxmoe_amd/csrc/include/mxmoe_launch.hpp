@@ -21,6 +21,7 @@
 #include <vector>
 
 #include "mxmoe_tiles.hpp"
+#include "mxmoe_grp_tiles.hpp"
 #include "mxmoe_wo_tiles.hpp"
 
 namespace mxmoe {
@@ -126,12 +127,13 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd<Tiles...>) fused_group
 
 // ------------------------------------------------------------------ host side ------------------------------------------------------------------
 
-enum class Fmt { FP16, W8A8, W4A4, W4A16, W3A16, W2A16, UNSUPPORTED };
+enum class Fmt { FP16, W8A8, W4A4, W4A16, W3A16, W2A16, W4A4G128, UNSUPPORTED };
 
 inline Fmt classify(const mxmoe_qparams& q) {
   if (q.a_bits >= 16 && q.w_bits >= 16) return Fmt::FP16;
   if (q.a_bits == 8 && q.w_bits == 8 && q.gsize == -1 && q.sym) return Fmt::W8A8;
   if (q.a_bits == 4 && q.w_bits == 4 && q.gsize == -1 && q.sym) return Fmt::W4A4;
+  if (q.a_bits == 4 && q.w_bits == 4 && q.gsize == 128 && q.sym) return Fmt::W4A4G128;
   if (q.a_bits >= 16 && q.w_bits == 4 && q.gsize == 128) return Fmt::W4A16;
   if (q.a_bits >= 16 && q.w_bits == 3 && q.gsize == 128) return Fmt::W3A16;
   if (q.a_bits >= 16 && q.w_bits == 2 && q.gsize == 128) return Fmt::W2A16;
@@ -146,6 +148,7 @@ inline const char* fmt_name(Fmt f, bool sym) {
     case Fmt::W4A16: return sym ? "w4a16_g128_sym" : "w4a16_g128_asym";
     case Fmt::W3A16: return sym ? "w3a16_g128_sym" : "w3a16_g128_asym";
     case Fmt::W2A16: return sym ? "w2a16_g128_sym" : "w2a16_g128_asym";
+    case Fmt::W4A4G128: return "w4a4_g128_sym";
     default: return "unsupported";
   }
 }
@@ -166,6 +169,13 @@ struct BranchOf<MfmaTile<OP, BM, BN, WGM, WGN>> {
     using T = MfmaTile<OP, BM, BN, WGM, WGN>;
     const Fmt f = OP == Op::I8 ? Fmt::W8A8 : (OP == Op::I4 ? Fmt::W4A4 : Fmt::FP16);
     return BranchInfo{f, BM, BN, T::BK, WGM, WGN, T::kLdsBytes, T::BK, 0};
+  }
+};
+template <int BM>
+struct BranchOf<WxAxGTile<BM>> {
+  static BranchInfo get() {
+    using T = WxAxGTile<BM>;
+    return BranchInfo{Fmt::W4A4G128, BM, T::BN, T::BK, 1, 4, T::kLdsBytes, T::BK, 0};
   }
 };
 template <Op OP, int BM, int BN>
@@ -259,6 +269,7 @@ inline double tile_cost(const BranchInfo& b) {
       {Fmt::W4A16, 16, 128, 0.37}, {Fmt::W4A16, 16, 64, 0.20}, {Fmt::W4A16, 128, 128, 1.00},
       {Fmt::W3A16, 16, 128, 0.31}, {Fmt::W3A16, 16, 64, 0.20}, {Fmt::W3A16, 128, 128, 1.00},
       {Fmt::W2A16, 16, 128, 0.25}, {Fmt::W2A16, 16, 64, 0.20}, {Fmt::W2A16, 128, 128, 1.00},
+      {Fmt::W4A4G128, 64, 256, 1.00}, {Fmt::W4A4G128, 32, 256, 0.60},
   };
   for (const Row& r : table)
     if (r.f == b.fmt && r.bm == b.BM && r.bn == b.BN) return r.c;
@@ -387,7 +398,7 @@ inline int group_gemm(int kernel_id, const void* const* As, const void* const* B
       }
       for (int j = 0; j < ns; ++j) {
         const BranchInfo& bi = k.branches[sg[j].branch];
-        if (sz.z == 0 || sz.z % bi.k_multiple != 0 || sz.y % 8 != 0 || (bi.fmt != Fmt::FP16 && bi.fmt != Fmt::W8A8 && bi.fmt != Fmt::W4A4 && sz.y % 16 != 0)) {
+        if (sz.z == 0 || sz.z % bi.k_multiple != 0 || sz.y % 8 != 0 || (bi.fmt != Fmt::FP16 && bi.fmt != Fmt::W8A8 && bi.fmt != Fmt::W4A4 && bi.fmt != Fmt::W4A4G128 && sz.y % 16 != 0)) {
           char buf[200];
           snprintf(buf, sizeof buf, "problem %d: shape [%u,%u,%u] not supported by tile %s (K %% %d, N %% 8)", base + i, sz.x, sz.y, sz.z, fmt_name(bi.fmt, true), bi.k_multiple);
           last_error() = buf;

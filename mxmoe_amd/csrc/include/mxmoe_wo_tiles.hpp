@@ -216,7 +216,10 @@ struct SkinnyWoTile {
         gstore<v4h>(t.C + (long)m * N + n, o);
         if (t.acc_dump) {
 #pragma unroll
-          for (int e = 0; e < 4; ++e) gstore<int>(t.acc_dump + (long)m * N + n + e, __builtin_bit_cast(int, sum[e]));
+          for (int e = 0; e < 4; ++e) {
+            const float f = sum[e];  // a copy: a bit cast applied to a vector element reads element 0
+            gstore<int>(t.acc_dump + (long)m * N + n + e, __float_as_int(f));
+          }
         }
       }
     }
@@ -367,7 +370,10 @@ struct WoMfmaTile {
           const int m = m0 + wm * 64 + mb * 16 + lm, n = n0 + wn * 64 + nb * 16 + lg * 4;
           if (m < M && n < N) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) gstore<int>(t.acc_dump + (long)m * N + n + e, __builtin_bit_cast(int, acc[nb][mb][e]));
+            for (int e = 0; e < 4; ++e) {
+              const float f = acc[nb][mb][e];
+              gstore<int>(t.acc_dump + (long)m * N + n + e, __float_as_int(f));
+            }
           }
         }
       }

@@ -62,8 +62,9 @@ def make_problem(entry: dict, gen: torch.Generator, device="cuda", keep_ref: boo
     pw = quantize_and_pack(b, qp)
     prob = {"size": (m, n, k), "q": qp, "B": pw.data, "sb": pw.scale, "C": torch.zeros(m, n, dtype=torch.float16, device=device)}
     if qp[0] < 16:
-        qa, sa, _ = quant_minmax(a, qp[0], -1, True) if m else (a, a[:, :1], None)
-        qi = qa.to(torch.int8)
+        ag = qp[2] if qp[2] > 0 else -1                      # group-quantised activations (w4a4_g128_sym): scales [M, K / 128]
+        qa, sa, _ = quant_minmax(a, qp[0], ag, True) if m else (a, a[:, :1], None)
+        qi = qa.reshape(m, k).to(torch.int8)
         prob["A"] = qi.contiguous() if qp[0] == 8 else pack.pack_int4_k(qi)
         prob["sa"] = sa.reshape(-1).contiguous()
     else:

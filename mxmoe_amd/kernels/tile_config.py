@@ -35,6 +35,7 @@ SUPPORTED_QCFG = [
     "fp16",
     "w8a8_g-1_sym",
     "w4a4_g-1_sym",
+    "w4a4_g128_sym",
     *[f"w{w}a16_g128_{s}" for w in (4, 3, 2) for s in ("sym", "asym")],
 ]
 
@@ -52,6 +53,7 @@ QCFG_TO_MMA = {
     "fp16": "MFMA_F32_32x32x16_F16",
     "w8a8_g-1_sym": "MFMA_I32_32x32x32_I8",
     "w4a4_g-1_sym": "MFMA_I32_32x32x32_I8_FROM_I4",
+    "w4a4_g128_sym": "MFMA_I32_32x32x32_I8_FROM_I4",
     **{f"w{w}a16_g128_{s}": "MFMA_F32_16x16x32_F16" for w in (4, 3, 2) for s in ("sym", "asym")},
 }
 
@@ -98,6 +100,7 @@ class QConfig(QConfigBase):
 
 QCFG_W8A8 = QConfig(QBITS=8, GSIZE=-1, SYM=True, PACK_DIM="PackDim::K")
 QCFG_W4A4 = QConfig(QBITS=4, GSIZE=-1, SYM=True, PACK_DIM="PackDim::K")
+QCFG_W4A4_G128 = QConfig(QBITS=4, GSIZE=128, SYM=True, PACK_DIM="PackDim::K")
 
 CFG_TEMPLATE = "TileConfig<{BM},{BN},{BK},{WM},{WN},{WK},{STAGE},{SPLITK},{MMA},{QCFGA},{QCFGB}>"
 
@@ -159,6 +162,10 @@ class TileConfig:
     def is_skinny(self) -> bool:
         return self.is_weight_only() and self.BM == 16
 
+    def is_group_wa(self) -> bool:
+        """Both operands int4 with a scale per 128-wide K group (w4a4_g128_sym)."""
+        return self.MMA == "MFMA_I32_32x32x32_I8_FROM_I4" and getattr(self.QCFGA, "GSIZE", -1) == 128
+
     def smem_bytes_scale(self):
         return 0  # scales are read straight from global memory in the epilogue / per group
 
@@ -168,6 +175,8 @@ class TileConfig:
             return 4 * (self.BN // 16) * (64 * 16 + 4 * 64)  # per-wave partial sums of the final reduction + (scale, zero) patches
         if self.is_weight_only():
             return 2 * self.BM * 256  # two stages of BM activation rows x one 128-wide k block
+        if self.is_group_wa():
+            return self.STAGE * self.BM * 64
         if self.MMA != "MFMA_F32_32x32x16_F16":  # activations only: 3 stages of BM x 64 B, or the epilogue patch if larger
             return max(self.STAGE * self.BM * 64, 4 * min(self.BM, 64) * (64 * 2 + 8))
         return self.STAGE * (self.BM + self.BN) * 64
@@ -179,6 +188,8 @@ class TileConfig:
         if self.is_weight_only():
             return f"WoMfmaTile<{self.QCFGB.QBITS}, {self.BM}, {self.BN}>"
         op = {"MFMA_F32_32x32x16_F16": "Op::F16", "MFMA_I32_32x32x32_I8": "Op::I8", "MFMA_I32_32x32x32_I8_FROM_I4": "Op::I4"}[self.MMA]
+        if self.is_group_wa():
+            return f"WxAxGTile<{self.BM}>"
         if op != "Op::F16":
             return f"WxAxTile<{op}, {self.BM}, {self.BN}>"
         return f"MfmaTile<{op}, {self.BM}, {self.BN}, {self.WM}, {self.WN}>"
@@ -193,6 +204,8 @@ class TileConfig:
         k_elems = {"MFMA_F32_32x32x16_F16": 32, "MFMA_I32_32x32x32_I8": 64, "MFMA_I32_32x32x32_I8_FROM_I4": 128}[self.MMA]
         if self.BK != k_elems or self.STAGE != 3 or self.WK != 1 or (self.BM // self.WM) % 32 or (self.BN // self.WN) % 32:
             raise ValueError(f"{self!r}: unsupported shape for {self.MMA} (BK must be {k_elems}, STAGE 3, wave tile a multiple of 32x32)")
+        if self.is_group_wa() and self.BM not in (32, 64):
+            raise ValueError(f"{self!r}: group-quantised int4 tiles are 32 x 256 or 64 x 256 (two sets of accumulators)")
         if self.MMA != "MFMA_F32_32x32x16_F16" and ((self.WM, self.WN) != (1, 4) or self.BN != 256 or self.BM not in (32, 64, 128)):
             raise ValueError(f"{self!r}: integer tiles are BM x 256 with 1 x 4 waves (each wave streams its own 64 weight channels), BM in 32 / 64 / 128")
 
@@ -216,6 +229,7 @@ QCFG_MAP = {
     "fp16": TileConfig(),
     "w8a8_g-1_sym": TileConfig(QCFGA=QCFG_W8A8, QCFGB=QCFG_W8A8),
     "w4a4_g-1_sym": TileConfig(QCFGA=QCFG_W4A4, QCFGB=QCFG_W4A4),
+    "w4a4_g128_sym": TileConfig(QCFGA=QCFG_W4A4_G128, QCFGB=QCFG_W4A4_G128),
     **{k: TileConfig(QCFGB=build_qcfgb_from_str(k)) for k in [f"w{w}a16_g128_{s}" for w in (4, 3, 2) for s in ("sym", "asym")]},
 }
 
@@ -235,6 +249,8 @@ def get_possible_tile_list(arch: str, qcfg: str) -> list:
     bk = {"MFMA_F32_32x32x16_F16": 32, "MFMA_I32_32x32x32_I8": 64, "MFMA_I32_32x32x32_I8_FROM_I4": 128}[mma]
     if mma == "MFMA_F32_32x32x16_F16":
         shapes = [(128, 256, 2, 2), (64, 256, 1, 4), (32, 256, 1, 4), (128, 128, 2, 2), (256, 128, 2, 2)]
+    elif qcfg == "w4a4_g128_sym":
+        shapes = [(64, 256, 1, 4), (32, 256, 1, 4)]
     else:
         shapes = [(128, 256, 1, 4), (64, 256, 1, 4), (32, 256, 1, 4)]
     return [_with_q(TileConfig(BM=bm, BN=bn, BK=bk, WM=wm, WN=wn, WK=1, STAGE=3, MMA=mma), qcfg) for bm, bn, wm, wn in shapes]

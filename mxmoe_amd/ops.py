@@ -70,11 +70,13 @@ def _offsets(recv_cpu, num_tokens: int, num_experts: int, has_shared: bool, qpar
     for e in range(et):
         a_bits, _w, g, _s = qparams_per_exp[e]
         tag = act_tag(int(a_bits), int(g))
-        if tag not in (0, 1, 2):
+        if tag not in (0, 1, 2, 3):
             raise RuntimeError("quant type not supported")
         width = ld_shared if e == num_experts else ld
+        if tag == 3 and width % 128:
+            raise RuntimeError(f"group-128 activations need a row length that is a multiple of 128, got {width}")
         qld = width if tag == 0 else (width // 2 if tag == 1 else width // 4)
-        sld = 0 if tag == 0 else 1
+        sld = 0 if tag == 0 else (width // 128 if tag == 3 else 1)    # scales per row (ref_bind.cu:492)
         n = num_tokens if e == num_experts else int(recv_list[e])
         for c, v in zip(cols, (tag, acc, io, so)):
             c.append(v)

@@ -136,7 +136,7 @@ def profile_qcfg(qcfg: str, arch: str = "gfx950", slots=SLOTS, waves=WAVES, rebu
 
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(description="Regenerate the kernel-profile table on this GPU")
-    ap.add_argument("--qcfgs", nargs="+", default=["w4a4_g-1_sym", "w8a8_g-1_sym", "w4a16_g128_asym", "w3a16_g128_asym", "w2a16_g128_asym", "fp16"])
+    ap.add_argument("--qcfgs", nargs="+", default=["w4a4_g-1_sym", "w8a8_g-1_sym", "w4a16_g128_asym", "w3a16_g128_asym", "w2a16_g128_asym", "w4a4_g128_sym", "fp16"])
     ap.add_argument("--slots", nargs="+", default=list(SLOTS))
     ap.add_argument("--out", default="perf/performance_table.json")
     ap.add_argument("--build-only", action="store_true", help="compile the single-tile kernel libraries and stop (needs no GPU)")

@@ -22,6 +22,8 @@ W8A8 = (8, 8, -1, True)
 FP16 = (16, 16, -1, True)
 W4A16 = (16, 4, 128, False)
 W3A16 = (16, 3, 128, False)
+W2A16 = (16, 2, 128, False)
+W4A4G128 = (4, 4, 128, True)
 
 
 def qcfg_str(qp) -> str:

@@ -36,6 +36,13 @@ def quantize_and_pack(w: torch.Tensor, qparams, keep_codes: bool = False) -> Pac
     if w_bits >= 16:
         return PackedWeight(w.contiguous(), None, tuple(qparams), n, k)
     q, scale, zp = quant_minmax(w, w_bits, gsize, sym)
+    if a_bits < 16 and gsize == 128:
+        # w4a4_g128_sym: codes as for w4a4, one scale per channel and 128-wide K group, stored group-major [K/128, N] so that a
+        # tile reads the scales of its channels for one group as one contiguous run
+        assert sym and w_bits == 4 and a_bits == 4 and k % 128 == 0, "group-quantised w-a format: w4a4_g128_sym"
+        qi = q.reshape(n, k).to(torch.int8)
+        data = pack.pack_wxax_fragments(pack.pack_int4_k(qi))
+        return PackedWeight(data, scale.reshape(n, k // 128).t().contiguous(), tuple(qparams), n, k, qi if keep_codes else None)
     if a_bits < 16:
         assert gsize == -1 and sym, "w-a formats are per-channel symmetric"
         qi = q.to(torch.int8)

@@ -14,6 +14,8 @@ fails a test in ``tests/test_oracle_*.py``):
   form, invariants (|q| <= upper, absmax -> +-upper, group min -> 0, max -> 2^b-1).
 * ``int_gemm``            — exact integer arithmetic vs a python-int brute force.
 * ``epilogue_wxax``       — closed form incl. the sa = sb = 1 special case (int -> fp16 convert).
+* ``int_gemm_grouped`` / ``epilogue_grouped`` — groups sum to ``int_gemm``; one group reduces to
+  ``epilogue_wxax``; unit scales give the exact integer product; float64 sum within fp32 rounding.
 * ``sylvester_fwht``      — scipy.linalg.hadamard dense product, involution, H e_0, Parseval.
 * ``had_table``           — H H^T = K I and all entries +-1.
 * ``online_hadamard``     — dense kron(H_K, H_{n/K}) / sqrt(n) in float64.
@@ -130,6 +132,29 @@ def epilogue_wxax(acc: np.ndarray, sa: np.ndarray, sb: np.ndarray, scale_product
     b = sb.astype(F16).reshape(1, -1)
     s = (a * b).astype(F16).astype(F32) if scale_product == "fp16" else (a.astype(F32) * b.astype(F32)).astype(F32)
     return (acc.astype(F32) * s).astype(F32).astype(F16)
+
+
+def int_gemm_grouped(qa: np.ndarray, qb: np.ndarray, gsize: int) -> np.ndarray:
+    """Integer accumulators of a group-quantised mainloop, one per K group: ``acc[g,m,n] = sum_{k in group g} qa[m,k] qb[n,k]``
+    (cta_gemm.cuh:613-772 keeps one integer fragment per group before rescaling it)."""
+    k = qa.shape[-1]
+    assert k % gsize == 0
+    return np.stack([int_gemm(qa[:, g * gsize:(g + 1) * gsize], qb[:, g * gsize:(g + 1) * gsize]) for g in range(k // gsize)])
+
+
+def epilogue_grouped(acc: np.ndarray, sa: np.ndarray, sb: np.ndarray) -> np.ndarray:
+    """Group-quantised w-a epilogue: ``half( sum_g float(acc[g]) * (sa[m,g] * sb[n,g]) )``.
+
+    acc [G,M,N] int32, sa [M,G], sb [N,G] fp16.  Per group the product of the two fp16 scales is exact in fp32, the converted
+    accumulator is multiplied by it (one fp32 rounding) and added to the running fp32 sum, groups in ascending order, starting from
+    0 (one rounding per addition); one final rounding to fp16.  The reference rescales each group's integer fragment into an fp32
+    fragment in the same ascending order (cta_gemm.cuh:613-772)."""
+    g, m, n = acc.shape
+    out = np.zeros((m, n), dtype=F32)
+    for i in range(g):
+        s = (sa[:, i].astype(F32).reshape(-1, 1) * sb[:, i].astype(F32).reshape(1, -1)).astype(F32)
+        out = (out + (acc[i].astype(F32) * s).astype(F32)).astype(F32)
+    return out.astype(F16), out
 
 
 def gemm_fakequant(xq: np.ndarray, wq: np.ndarray) -> np.ndarray:
@@ -419,6 +444,15 @@ def linear_block(x: np.ndarray, w: np.ndarray, qp, rotate: bool):
     * weight-only (a_bits == 16, w_bits < 16): ``out = x @ fake_quant(w).T``; fp16: plain GEMM.
     """
     a_bits, w_bits, g, sym = qp
+    if a_bits < 16 and g > 0:
+        # group-quantised on both sides (w4a4_g128_sym): acc is the [G, M, N] stack of per-group accumulators
+        xr = online_hadamard(x) if rotate else x
+        qa, sa, _ = quant_minmax(xr, a_bits, g, True)
+        qb, sb, _ = quant_minmax(w, w_bits, g, True)
+        acc = int_gemm_grouped(qa, qb, g)
+        out_k, _ = epilogue_grouped(acc, sa.reshape(x.shape[0], -1), sb.reshape(w.shape[0], -1))
+        out_f = gemm_fakequant(dequant(qa, sa, 0 * sa, g), dequant(qb, sb, 0 * sb, g))
+        return out_k, out_f, acc
     if a_bits < 16:
         xr = online_hadamard(x) if rotate else x
         qa, sa, _ = quant_minmax(xr, a_bits, -1, True)

@@ -87,7 +87,7 @@ def test_plan_bounds_on_random_problem_lists(lib):
 
     rnd = random.Random(7)
     fmts = [((4, 4, -1, True), 128), ((8, 8, -1, True), 64), ((16, 4, 128, False), 128), ((16, 3, 128, False), 128), ((16, 2, 128, True), 128),
-            ((16, 16, -1, True), 32)]
+            ((16, 16, -1, True), 32), ((4, 4, 128, True), 128)]
     out = (C.c_int32 * 8)()
     for trial in range(40):
         nprob = rnd.choice([1, 3, 17, 60, 121, 260])
@@ -107,9 +107,9 @@ def test_plan_bounds_on_random_problem_lists(lib):
             assert lib.mxmoe_kernel_branch(kid, b, out) == 0
             shapes.append((out[0], out[1], out[2]))
         lo = hi = 0
-        fmt_id = {(4, 4): 2, (8, 8): 1, (16, 4): 3, (16, 3): 4, (16, 2): 5, (16, 16): 0}
+        fmt_id = {(4, 4, -1): 2, (8, 8, -1): 1, (16, 4, 128): 3, (16, 3, 128): 4, (16, 2, 128): 5, (16, 16, -1): 0, (4, 4, 128): 6}
         for (m, n, k), q in probs:
-            mine = [(bm, bn) for f, bm, bn in shapes if f == fmt_id[(q[0], q[1])]]
+            mine = [(bm, bn) for f, bm, bn in shapes if f == fmt_id[(q[0], q[1], q[2])]]
             assert mine, "the chosen kernel has a tile for every format of the list"
             if m == 0:
                 continue

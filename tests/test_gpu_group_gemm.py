@@ -108,6 +108,42 @@ def test_more_problems_than_one_launch_holds():
         assert np.array_equal(out.view(np.uint16), p["out"].view(np.uint16)), f"problem {i} {p['size']}"
 
 
+def _grouped_problem(rng, m, n, k):
+    """w4a4_g128_sym: codes and group scales from the oracle quantiser, expected fp32 sums and fp16 outputs from its epilogue."""
+    from mxmoe_amd import pack
+
+    x = rng.standard_normal((m, k)).astype(F16)
+    w = (rng.standard_normal((n, k)) * 0.02).astype(F16)
+    qa, sa, _ = O.quant_minmax(x, 4, 128, True)
+    qb, sb, _ = O.quant_minmax(w, 4, 128, True)
+    sa, sb = sa.reshape(m, k // 128), sb.reshape(n, k // 128)
+    out, f32 = O.epilogue_grouped(O.int_gemm_grouped(qa, qb, 128), sa, sb)
+    ta, tb = pack.pack_int4_k(torch.from_numpy(qa.astype(np.int8))), pack.pack_wxax_fragments(pack.pack_int4_k(torch.from_numpy(qb.astype(np.int8))))
+    return dict(A=ta.to(DEV), B=tb.to(DEV), sa=torch.from_numpy(sa.copy()).to(DEV), sb=torch.from_numpy(np.ascontiguousarray(sb.T)).to(DEV),
+                acc=f32.view(np.int32), out=out, fq=O.gemm_fakequant(O.dequant(qa, sa.reshape(-1, 1), 0 * sa.reshape(-1, 1), 128), O.dequant(qb, sb.reshape(-1, 1), 0 * sb.reshape(-1, 1), 128)),
+                size=(m, n, k), q=(4, 4, 128, True))
+
+
+def test_group_quantised_w4a4_bit_exact():
+    """w4a4_g128_sym: the fp32 sums over the groups (dumped as bit patterns) and the fp16 outputs equal the oracle's bit for bit, alone
+    and mixed with the per-channel formats in one launch."""
+    rng = np.random.default_rng(13)
+    shapes = [(1, 256, 128), (33, 384, 1408), (64, 2816, 2048), (130, 256, 256), (17, 264, 128), (300, 768, 384), (5, 2048, 1408)]
+    probs = [_grouped_problem(rng, m, n, k) for (m, n, k) in shapes]
+    _, outs, accs = _launch(probs)
+    for p, out, acc in zip(probs, outs, accs):
+        assert np.array_equal(acc, p["acc"]), f"fp32 group sums differ for {p['size']}"
+        assert np.array_equal(out.view(np.uint16), p["out"].view(np.uint16)), f"fp16 outputs differ for {p['size']}"
+        assert _rel(out, p["fq"]) <= 1e-2
+    mixed = [probs[1], _wxax_problem(rng, 40, 512, 256, 4), probs[3], _wxax_problem(rng, 70, 256, 128, 8)]
+    g, outs, accs = _launch(mixed)
+    from mxmoe_amd import _lib
+
+    assert b"fused_all" in _lib.load().mxmoe_kernel_name(g.plan()[0])
+    for p, out, acc in zip(mixed, outs, accs):
+        assert np.array_equal(acc, p["acc"]) and np.array_equal(out.view(np.uint16), p["out"].view(np.uint16)), p["size"]
+
+
 def test_fp16_group_gemm():
     rng = np.random.default_rng(2)
     probs = []

@@ -69,6 +69,20 @@ def test_wxax_layer_is_bit_exact_end_to_end():
         assert _rel(r["g_out"], r["out_f"]) <= 1e-2                         # vs the fake-quant path
 
 
+def test_layer_with_group_quantised_experts_is_bit_exact():
+    """Experts in w4a4_g128_sym next to per-channel ones: quantiser (one scale per 128 values), both GroupGEMMs and the fp16 results
+    equal the oracle's bit for bit (the accumulators of the group format are fp32 sums and are compared in the GroupGEMM's own test)."""
+    from mxmoe_amd import synth
+
+    cfg = synth.MoEConfig("t", "test", 4, 2, 256, 1408, 40, num_shared=0, rotate=1)
+    g = synth.W4A4G128
+    fm = [(g, g), (synth.W8A8, g), (g, synth.W4A4), (synth.W4A4, synth.W8A8)]
+    for r in _run(cfg, fm):
+        assert np.array_equal(r["g_mid"].view(np.uint16), r["mid"].view(np.uint16)), f"gate_up fp16, expert {r['e']}"
+        assert np.array_equal(r["g_out"].view(np.uint16), r["out"].view(np.uint16)), f"down fp16, expert {r['e']}"
+        assert _rel(r["g_out"], r["out_f"]) <= 1e-2
+
+
 def test_mixed_layer_with_shared_expert_within_tolerance():
     from mxmoe_amd import synth
 

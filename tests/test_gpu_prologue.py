@@ -52,7 +52,7 @@ def test_quant_inp_act_bit_exact(k, rotate):
     x[3] = 0                                                               # all-zero token: scale guard
     ids = _ids(rng, t, e, topk)
     ids[ids == 4] = 5 if False else ids[ids == 4]
-    qp = [(4, 4, -1, True), (8, 8, -1, True), (16, 4, 128, False), (4, 4, -1, True), (8, 8, -1, True), (16, 16, -1, True), (8, 8, -1, True)]
+    qp = [(4, 4, -1, True), (8, 8, -1, True), (16, 4, 128, False), (4, 4, 128, True), (8, 8, -1, True), (16, 16, -1, True), (8, 8, -1, True)]
     res = ops.quant_inp_act(torch.from_numpy(x).to(DEV), torch.from_numpy(ids).to(DEV), e, 1408, n_sh, qp, rotate=rotate)
     inp_list, scale_list, out_list, inp_store, scale_store, out_store, recv, perm, dst = res
     torch.cuda.synchronize()
@@ -76,7 +76,7 @@ def test_quant_inp_act_bit_exact(k, rotate):
         if tag == 0:
             assert np.array_equal(got.cpu().numpy().view(np.uint16), xr.view(np.uint16)), f"expert {ex} fp16 rows"
         else:
-            q, s, _ = O.quant_minmax(xr, a_bits, -1, True)
+            q, s, _ = O.quant_minmax(xr, a_bits, 128 if tag == 3 else -1, True)   # tag 3: one scale per 128 values, [M, K / 128]
             assert np.array_equal(scale_list[p].cpu().numpy().view(np.uint16), s.reshape(-1).view(np.uint16)), f"expert {ex} scales"
             assert np.array_equal(_unpack(got, tag, k), q.astype(np.int8)), f"expert {ex} codes"
         p += 1
@@ -95,7 +95,7 @@ def test_silu_mul_then_quant_bit_exact(n, n_sh, rotate):
     gu = (rng.standard_normal((r, 2 * n)) * 2).astype(F16)
     gu_sh = (rng.standard_normal((t, 2 * n * max(n_sh, 1))) * 2).astype(F16)
     flat = np.concatenate([gu.reshape(-1), gu_sh.reshape(-1)]) if n_sh else gu.reshape(-1)
-    qp = [(4, 4, -1, True), (8, 8, -1, True), (16, 4, 128, False), (4, 4, -1, True), (8, 8, -1, True)]
+    qp = [(4, 4, -1, True), (8, 8, -1, True), (16, 4, 128, False), (4, 4, 128, True), (8, 8, -1, True)]
     res = ops.silu_mul_then_quant(torch.from_numpy(flat).to(DEV), int((o_recv != 0).sum()), e, 2048, n, n_sh, t, topk,
                                   torch.from_numpy(o_dst).to(DEV), torch.from_numpy(o_recv), qp, rotate=rotate)
     inp_list, scale_list, out_list = res[:3]
@@ -118,7 +118,7 @@ def test_silu_mul_then_quant_bit_exact(n, n_sh, rotate):
         if tag == 0:
             assert np.array_equal(got.cpu().numpy().view(np.uint16), y.view(np.uint16)), f"expert {ex} fp16 rows"
         else:
-            q, s, _ = O.quant_minmax(y, a_bits, -1, True)
+            q, s, _ = O.quant_minmax(y, a_bits, 128 if tag == 3 else -1, True)
             assert np.array_equal(scale_list[p].cpu().numpy().view(np.uint16), s.reshape(-1).view(np.uint16)), f"expert {ex} scales"
             assert np.array_equal(_unpack(got, tag, y.shape[1]), q.astype(np.int8)), f"expert {ex} codes"
         p += 1

@@ -157,3 +157,37 @@ def test_exp_fixed_and_silu_mul():
     assert np.all(np.isinf(y[~fin]))
     # first half is the gate: swapping halves changes the answer
     assert not np.array_equal(y, O.silu_mul(np.concatenate([gu[:, 32:], gu[:, :32]], axis=1)))
+
+
+def test_grouped_accumulators_and_epilogue():
+    rng = np.random.default_rng(21)
+    m, n, k, g = 5, 7, 384, 128
+    qa = rng.integers(-7, 8, (m, k)).astype(np.float16)
+    qb = rng.integers(-7, 8, (n, k)).astype(np.float16)
+    acc = O.int_gemm_grouped(qa, qb, g)
+    assert acc.shape == (3, m, n)
+    assert np.array_equal(acc.sum(axis=0), O.int_gemm(qa, qb))                       # the groups partition K
+    assert np.array_equal(acc[1], O.int_gemm(qa[:, 128:256], qb[:, 128:256]))
+    ones_a, ones_b = np.ones((m, 3), np.float16), np.ones((n, 3), np.float16)
+    h, f = O.epilogue_grouped(acc, ones_a, ones_b)
+    assert np.array_equal(f, O.int_gemm(qa, qb).astype(np.float32))                  # unit scales: the exact integer product
+    sa = rng.uniform(0.01, 0.2, (m, 3)).astype(np.float16)
+    sb = rng.uniform(0.001, 0.02, (n, 3)).astype(np.float16)
+    h1, _ = O.epilogue_grouped(acc[:1], sa[:, :1], sb[:, :1])                        # one group: the per-token / per-channel epilogue
+    assert np.array_equal(h1.view(np.uint16), O.epilogue_wxax(acc[0], sa[:, 0], sb[:, 0]).view(np.uint16))
+    h, f = O.epilogue_grouped(acc, sa, sb)
+    exact = sum(acc[i].astype(np.float64) * sa[:, i].astype(np.float64)[:, None] * sb[:, i].astype(np.float64)[None, :] for i in range(3))
+    assert np.abs(f - exact).max() <= 4 * 2.0 ** -24 * np.abs(exact).max() + 1e-12
+    # a sign error or a transposed scale fails: swap sa's groups
+    h_bad, _ = O.epilogue_grouped(acc, sa[:, ::-1].copy(), sb)
+    assert not np.array_equal(h_bad, h)
+
+
+def test_linear_block_group_format_agrees_with_fake_quant():
+    rng = np.random.default_rng(22)
+    x = rng.standard_normal((6, 256)).astype(np.float16)
+    w = (rng.standard_normal((16, 256)) * 0.02).astype(np.float16)
+    out_k, out_f, acc = O.linear_block(x, w, (4, 4, 128, True), rotate=True)
+    assert acc.shape == (2, 6, 16)
+    rel = np.abs(out_k.astype(np.float64) - out_f.astype(np.float64)).max() / np.abs(out_f.astype(np.float64)).max()
+    assert rel <= 1e-2
