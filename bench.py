@@ -153,6 +153,13 @@ def cpu_baseline(cfg, budget_s: float = 20.0):
         ops += 2 * m * (2 * cfg.inter * cfg.hidden + cfg.hidden * cfg.inter)
         used.append(int(e))
     cores = os.cpu_count() or 1
+    try:  # the threads the BLAS behind numpy actually runs (the box caps them below the core count)
+        from threadpoolctl import threadpool_info
+
+        blas = [int(p["num_threads"]) for p in threadpool_info() if p.get("user_api") == "blas"]
+        cores = max(blas) if blas else cores
+    except ImportError:
+        pass
     return {"value": round(ops / spent / 1e12, 5), "unit": "TOPS", "cores": cores, "kind": "port",
             "sample": f"{len(used)} busiest experts of {cfg.name} ({sum(int(recv[e]) for e in used)} of {cfg.rows} routed rows), "
                       f"activation fake-quant + fp32 matmuls + SiLU timed, {spent:.1f} s"}
@@ -161,7 +168,7 @@ def cpu_baseline(cfg, budget_s: float = 20.0):
 def time_whole_layer(cfg, layer, reps: int = 7) -> dict:
     """Wall time of the whole layer forward as a caller of the ops sees it (permute + rotate + quantise, gate_up launch, SiLU*up +
     rotate + quantise, down launch, un-permute + combine), including the host work of the ops (offset tables, allocations); median of
-    `reps` repetitions.
+    `reps` repetitions, step by step with a synchronisation after each (`*_ms`, `layer_ms`) and as the layer's one-call form (`one_call_ms`).
     Reported next to the GroupGEMM figure, never as `value`."""
     import torch
 
@@ -185,6 +192,15 @@ def time_whole_layer(cfg, layer, reps: int = 7) -> dict:
     parts = {k: sorted(v)[len(v) // 2] for k, v in samples.items()}
     out = {f"{k}_ms": round(v, 4) for k, v in parts.items()}
     out["layer_ms"] = round(sum(parts.values()), 4)
+    # the same forward as one call (all host tables in one pass, no synchronisation between the steps)
+    whole = []
+    for rep in range(reps + 2):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        layer(hidden, ids, w)
+        torch.cuda.synchronize()
+        whole.append((time.perf_counter() - t0) * 1e3)
+    out["one_call_ms"] = round(sorted(whole[2:])[len(whole[2:]) // 2], 4)
     return out
 
 

@@ -5,9 +5,14 @@ packaged so the pointer tables of both launches are built once and every later s
 """
 from __future__ import annotations
 
+import ctypes as C
+
+import numpy as np
 import torch
 
-from . import ops
+from . import _lib, ops
+from . import layer_tables as LT
+from .hadamard import device_signs
 from .synth import MoEConfig, draw_formats, expert_weights
 from .weights import quantize_and_pack
 
@@ -37,6 +42,7 @@ class MxMoELayer:
         self.qp_gate_up = [f[0] for f in self.formats]
         self.qp_down = [f[1] for f in self.formats]
         self.state = None
+        self._static = None
 
     @property
     def weight_bytes(self) -> int:
@@ -92,11 +98,89 @@ class MxMoELayer:
         self.down()
         return self.state["out"]
 
+    def _static_tables(self):
+        """Per-expert constants of both linear blocks (formats, row lengths, weight addresses), built once."""
+        if self._static is None:
+            cfg = self.cfg
+            sh = [cfg.num_shared] if cfg.num_shared else []
+            i_sh = cfg.inter * max(cfg.num_shared, 1)
+            gu_w = [cfg.hidden] * self.n_exp_total
+            gu_n = [2 * cfg.inter] * cfg.num_experts + [2 * i_sh for _ in sh]
+            dn_w = [cfg.inter] * cfg.num_experts + [i_sh for _ in sh]
+            dn_n = [cfg.hidden] * self.n_exp_total
+
+            def ptrs(ws):
+                return [w.data.data_ptr() for w in ws], [0 if w.scale is None else w.scale.data_ptr() for w in ws]
+
+            self._static = (LT.static_block(self.qp_gate_up, gu_w, gu_n, *ptrs(self.w13)), LT.static_block(self.qp_down, dn_w, dn_n, *ptrs(self.w2)))
+        return self._static
+
     def __call__(self, hidden: torch.Tensor, topk_ids: torch.Tensor, topk_weights: torch.Tensor) -> torch.Tensor:
         """The whole MoE MLP, `(hidden [T, K] fp16, topk_ids [T, k] int32, topk_weights [T, k] fp32) -> [T, K] fp16`: what a serving
-        framework's fused-MoE operator computes after routing (permute, quantise, gate_up, SiLU * up, down, un-permute + combine)."""
-        self.forward(hidden, topk_ids)
-        return self.combine(topk_weights)
+        framework's fused-MoE operator computes after routing (permute, quantise, gate_up, SiLU * up, down, un-permute + combine).
+
+        Same kernels and results as `forward` + `combine`, but the host side is one pass: after the single device-to-host copy of
+        the tokens-per-expert counts every table of both launches is computed with array arithmetic and sent in one copy."""
+        cfg, dev = self.cfg, self.device
+        lib = _lib.load()
+        hidden = hidden.to(dev).contiguous()
+        ids = topk_ids.to(dev).to(torch.int32).contiguous()
+        w = topk_weights.to(dev).to(torch.float32).contiguous()
+        t, k_hid = hidden.shape
+        topk = ids.shape[1]
+        assert hidden.dtype == torch.float16 and k_hid == cfg.hidden and w.shape == ids.shape
+        e_cnt, has_shared = cfg.num_experts, cfg.num_shared > 0
+        gu, dn = self._static_tables()
+        dst, perm, slot, recv = ops.build_permutation(ids, e_cnt)
+        rows = np.empty(self.n_exp_total, np.int64)
+        rows[:e_cnt] = recv.cpu().numpy()                     # the one synchronisation of the forward (as ref_bind.cu:451)
+        if has_shared:
+            rows[e_cnt] = t
+        routed = int(rows[:e_cnt].sum())
+        t1, t2 = LT.block_tables(gu, rows), LT.block_tables(dn, rows)
+
+        def f16(n):
+            return torch.empty(max(n, 1), dtype=torch.float16, device=dev)
+
+        inp1, sa1, mid = f16(t1.inp_total), f16(t1.scale_total), f16(t1.out_total)
+        inp2, sa2, out = f16(t2.inp_total), f16(t2.scale_total), f16(t2.out_total)
+        p1, s1, q1 = LT.launch_tables(gu, rows, t1, inp1.data_ptr(), sa1.data_ptr(), mid.data_ptr())
+        p2, s2, q2 = LT.launch_tables(dn, rows, t2, inp2.data_ptr(), sa2.data_ptr(), out.data_ptr())
+        staging, off = LT.pack_staging([t1.table, t2.table, p1, p2, s1, s2])
+        d_tab = torch.from_numpy(staging).to(dev)
+        base = d_tab.data_ptr()
+        count = p1.shape[1]
+        stream = torch.cuda.current_stream().cuda_stream
+        final = torch.empty((t, cfg.hidden), dtype=torch.float16, device=dev)
+        if count == 0:
+            return final.zero_()
+
+        def signs(n, n_shared):
+            if not cfg.rotate:
+                return 1, 1, None
+            hk, hf, sg = device_signs(n, dev)
+            if has_shared and device_signs(n_shared, dev)[0] != hk:
+                raise RuntimeError("routed and shared intermediate sizes need the same Hadamard order")
+            return hk, hf, None if sg is None else sg.data_ptr()
+
+        def launch(ptr_off, sizes_off, h_sizes, h_q):
+            row = lambda i: base + ptr_off + i * count * 8  # noqa: E731
+            _lib.check(lib, lib.mxmoe_group_gemm(-1, row(0), row(1), row(2), row(3), row(4), row(4), None, None, None, None, base + sizes_off,
+                                                 h_sizes.ctypes.data_as(C.POINTER(_lib.Dim3)), None, h_q.ctypes.data_as(C.POINTER(_lib.QParams)), count, None, stream))
+
+        hk, hf, sg = signs(cfg.hidden, cfg.hidden)
+        _lib.check(lib, lib.mxmoe_quant_act(hidden.data_ptr(), inp1.data_ptr(), sa1.data_ptr(), dst.data_ptr(), perm.data_ptr(), base + off[0],
+                                            cfg.hidden, routed, t, e_cnt, int(has_shared), cfg.rotate, hk, hf, sg, stream))
+        launch(off[2], off[4], s1, q1)
+        i_sh = cfg.inter * max(cfg.num_shared, 1)
+        hk, hf, sg = signs(cfg.inter, i_sh)
+        _lib.check(lib, lib.mxmoe_silu_mul_quant(mid.data_ptr(), mid.data_ptr() + routed * 2 * cfg.inter * 2, inp2.data_ptr(), sa2.data_ptr(), dst.data_ptr(), base + off[1],
+                                                 cfg.inter, i_sh, routed, t, e_cnt, int(has_shared), cfg.rotate, hk, hf, sg, stream))
+        launch(off[3], off[5], s2, q2)
+        ws = torch.empty(lib.mxmoe_combine_workspace_bytes(t, topk), dtype=torch.uint8, device=dev)
+        shared_ptr = out.data_ptr() + routed * cfg.hidden * 2 if has_shared else None
+        _lib.check(lib, lib.mxmoe_unpermute_combine(out.data_ptr(), shared_ptr, w.data_ptr(), slot.data_ptr(), routed, t, topk, cfg.hidden, final.data_ptr(), ws.data_ptr(), stream))
+        return final
 
     # ---- accounting -----------------------------------------------------------------------------------------
     def gemm_ops(self) -> int:

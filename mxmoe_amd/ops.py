@@ -38,7 +38,8 @@ def gg_permute_inp(hidden: torch.Tensor, topk_ids: torch.Tensor, E: int):
     """ref_bind.cu:47-64 -> (num_problems, inp_buffer [R, K], perm_indices [R], recv_tokens_per_exp [E] int64 CPU)."""
     dst, perm, _slot, recv = build_permutation(topk_ids, E)
     recv_cpu = recv.cpu()
-    return int((recv_cpu != 0).sum()), hidden.index_select(0, perm), perm, recv_cpu
+    routed = int(recv_cpu.sum())                            # entries past this were never written (ids out of range are dropped)
+    return int((recv_cpu != 0).sum()), hidden.index_select(0, perm[:routed]), perm, recv_cpu
 
 
 def build_permutation(topk_ids: torch.Tensor, num_experts: int):
@@ -122,8 +123,9 @@ def quant_inp_act(hidden, topk_ids, num_experts: int, N: int, num_shared_experts
     out_store = torch.empty((num_shared_experts + topk) * t * N * 2, dtype=torch.float16, device=dev)
     d_table = table.to(dev)
     hk, hf, signs = device_signs(k, dev) if rotate else (1, 1, None)
+    routed = int(recv_cpu.sum())                            # rows whose expert id was in range; the sorted arrays hold exactly these
     _lib.check(lib, lib.mxmoe_quant_act(hidden.data_ptr(), inp_store.data_ptr(), scale_store.data_ptr(), dst.data_ptr(), perm.data_ptr(), d_table.data_ptr(),
-                                        k, t * topk, t, num_experts, int(has_shared), rotate, hk, hf, None if signs is None else signs.data_ptr(), _stream()))
+                                        k, routed, t, num_experts, int(has_shared), rotate, hk, hf, None if signs is None else signs.data_ptr(), _stream()))
     inp_list, scale_list = _views(inp_store, scale_store, table, rows, inp_sizes, scale_sizes, lds)
     out_list, off = [], 0
     for e, n in enumerate(rows):
@@ -145,9 +147,9 @@ def silu_mul_then_quant(inp, num_problems: int, num_experts: int, K: int, N: int
     out_list[p] is the [M_p, K] buffer of the down projection."""
     lib = _lib.load()
     has_shared = num_shared_experts > 0
-    r = num_tokens * topk
     dev = inp.device
     recv_cpu = recv_tokens_per_exp.cpu()
+    r = int(recv_cpu.sum())                                 # routed rows in the store (ids out of range were dropped by the permutation)
     table, rows, inp_sizes, scale_sizes, lds, io, so = _offsets(recv_cpu, num_tokens, num_experts, has_shared, qparams_per_exp, N, N * max(num_shared_experts, 1))
     inp_store = torch.empty(io, dtype=torch.float16, device=dev)
     scale_store = torch.empty(so, dtype=torch.float16, device=dev)

@@ -135,6 +135,34 @@ def test_layer_combine_end_to_end():
     assert np.array_equal(final.cpu().numpy().view(np.uint16), ref.view(np.uint16))
 
 
+@pytest.mark.parametrize("num_shared,rotate,drop", [(0, 1, False), (2, 1, False), (1, 0, True), (0, 2, True)])
+def test_one_call_form_equals_the_stepwise_forward(num_shared, rotate, drop):
+    """`layer(hidden, ids, weights)` builds all host tables in one pass; it must give exactly the result of the operator-by-operator
+    path for every format family, with a shared expert, with experts that receive no row and with expert ids out of range (dropped)."""
+    from mxmoe_amd import synth
+    from mxmoe_amd.layer import MxMoELayer
+
+    cfg = synth.MoEConfig("t", "test", 8, 2, 256, 1408, 40, num_shared=num_shared, rotate=rotate)
+    g = synth.W4A4G128
+    fm = [(synth.W4A4, synth.W8A8), (synth.W8A8, synth.W4A4), (g, g), (synth.W4A16, synth.W3A16), (synth.FP16, synth.FP16), (synth.W4A4, synth.W4A4),
+          (synth.W8A8, g), (synth.W3A16, synth.W4A16)]
+    if num_shared:
+        fm.append((synth.W4A16, synth.W4A16) if rotate == 0 else (synth.W8A8, synth.W4A4))
+    hidden = synth.make_hidden(cfg)
+    ids, w = synth.make_routing(cfg)
+    ids = torch.where(ids == 5, torch.full_like(ids, 1), ids)      # expert 5 receives nothing
+    if drop:
+        ids = torch.where(ids == 3, torch.full_like(ids, cfg.num_experts), ids)   # as on a GPU that does not own expert 3
+    layer = MxMoELayer(cfg, formats=fm)
+    layer.forward(hidden, ids)
+    stepwise = layer.combine(w).clone()
+    one_call = layer(hidden, ids, w)
+    torch.cuda.synchronize()
+    assert int(layer.state["recv"][5]) == 0
+    assert torch.equal(one_call, stepwise)
+    assert torch.equal(layer(hidden, ids, w), stepwise)            # and again: nothing is left over from the previous call
+
+
 def test_layer_from_checkpoint_file_keeps_the_function(tmp_path):
     """fp16 weights -> rotate + quantise + pack -> file -> layer: identical to packing in place, and (the weight rotation cancelling
     the online rotation of the activations) still the function of the fp16 MLP up to w8a8 quantisation noise."""
