@@ -1,6 +1,7 @@
 /* C-ABI of the MI355X-native mixed-precision MoE GroupGEMM library (libmxmoe_amd.so).
  *
- * Plain pointers and sizes only.  Every function returns 0 on success and a non-zero code on failure;
+ * Plain pointers and sizes only.  Every function returns 0 on success and a non-zero code on failure
+ * (1 format not supported, 2 bad kernel or branch id, 3 bad size or shape, 4 the launch failed, 5 a required pointer is NULL);
  * mxmoe_last_error() then returns a message for the calling thread.  All device pointers must belong to the
  * current HIP device; `stream` is a hipStream_t passed as void* (NULL = the default stream).  Nothing here
  * allocates device memory or synchronises the stream.
@@ -57,7 +58,8 @@ int mxmoe_kernel_branch(int kernel_id, int branch, int32_t out[8]);
  * receive the raw accumulators (int32 for w8a8 / w4a4 per channel, fp32 bit patterns otherwise: for w4a4_g128 the fp32 sum over the
  * groups of float(group's int32 sum) * (scale_a * scale_b), groups in ascending order); used by the parity tests.
  * Errors: 1 "quant type not supported" (same text as the reference launcher, compose_kernel.py:433), 2 bad kernel id,
- * 3 unsupported shape (K not a multiple of the tile's K step, N not a multiple of 8), 4 launch failure. */
+ * 3 unsupported shape (K not a multiple of the tile's K step, N not a multiple of 8), 4 launch failure, 5 a required array is NULL
+ * (the scale arrays are required as soon as one non-empty problem is quantised). */
 int mxmoe_group_gemm(int kernel_id, const void* const* As, const void* const* Bs, const void* const* scale_a, const void* const* scale_b,
                      void* const* Cs, void* const* Ds, const int64_t* lda, const int64_t* ldb, const int64_t* ldc, const int64_t* ldd,
                      const mxmoe_dim3* d_sizes, const mxmoe_dim3* h_sizes, const mxmoe_qparams* d_q, const mxmoe_qparams* h_q, int problem_count,

@@ -764,6 +764,10 @@ int mxmoe_build_permutation(const int32_t* topk_ids, int num_tokens, int topk, i
     last_error() = "bad permutation size";
     return 3;
   }
+  if (!topk_ids || !dst_exp_sorted || !perm_indices || !src_slot || !recv_tokens_per_exp || !workspace) {
+    last_error() = "null pointer";
+    return 5;
+  }
   hipStream_t s = (hipStream_t)stream;
   const int blocks = (total + kPermChunk - 1) / kPermChunk;
   int32_t* hist = reinterpret_cast<int32_t*>(workspace);
@@ -802,6 +806,14 @@ static int fill_common(RowArgs& a, int n, int n_shared, int had_k, int had_f, co
 
 int mxmoe_quant_act(const void* hidden, void* inp_store, void* scale_store, const int32_t* dst_exp_sorted, const int64_t* perm_indices, const int64_t* exp_table,
                     int K, int rows_routed, int num_tokens, int num_experts, int has_shared, int rotate, int had_k, int had_f, const float* had_signs, void* stream) {
+  if (rows_routed < 0 || num_tokens < 0 || num_experts <= 0) {
+    last_error() = "bad row or expert count";
+    return 3;
+  }
+  if (!hidden || !inp_store || !scale_store || !exp_table || (rows_routed > 0 && (!dst_exp_sorted || !perm_indices))) {
+    last_error() = "null pointer";
+    return 5;
+  }
   RowArgs a{};
   a.src = a.src_shared = reinterpret_cast<const _Float16*>(hidden);
   a.inp_store = reinterpret_cast<uint8_t*>(inp_store);
@@ -824,6 +836,14 @@ int mxmoe_quant_act(const void* hidden, void* inp_store, void* scale_store, cons
 int mxmoe_silu_mul_quant(const void* gate_up, const void* gate_up_shared, void* inp_store, void* scale_store, const int32_t* dst_exp_sorted, const int64_t* exp_table,
                          int N, int N_shared, int rows_routed, int num_tokens, int num_experts, int has_shared, int rotate, int had_k, int had_f,
                          const float* had_signs, void* stream) {
+  if (rows_routed < 0 || num_tokens < 0 || num_experts <= 0) {
+    last_error() = "bad row or expert count";
+    return 3;
+  }
+  if (!gate_up || !inp_store || !scale_store || !exp_table || (rows_routed > 0 && !dst_exp_sorted) || (has_shared && !gate_up_shared)) {
+    last_error() = "null pointer";
+    return 5;
+  }
   RowArgs a{};
   a.src = reinterpret_cast<const _Float16*>(gate_up);
   a.src_shared = reinterpret_cast<const _Float16*>(gate_up_shared);

@@ -54,6 +54,10 @@ int mxmoe_group_gemm(int kernel_id, const void* const* As, const void* const* Bs
 
 int mxmoe_group_gemm_plan(int kernel_id, const mxmoe_dim3* h_sizes, const mxmoe_qparams* h_q, int problem_count, int32_t* branch_out, int32_t* tiles_out) {
   auto& reg = registry();
+  if (problem_count < 0 || (problem_count > 0 && (!h_sizes || !h_q))) {
+    last_error() = "null argument";
+    return 5;
+  }
   if (kernel_id < 0) {
     for (int i = 0; i < (int)reg.size() && kernel_id < 0; ++i)
       if (kernel_covers(reg[i], h_q, problem_count)) kernel_id = i;

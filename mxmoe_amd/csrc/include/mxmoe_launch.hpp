@@ -370,6 +370,15 @@ inline int group_gemm(int kernel_id, const void* const* As, const void* const* B
     return 2;
   }
   const FusedKernel& k = reg[kernel_id];
+  for (int i = 0; i < count; ++i) {  // the tiles read the scales unconditionally: refuse a launch whose scale arrays are missing
+    const Fmt f = classify(h_q[i]);
+    const bool wa = f == Fmt::W8A8 || f == Fmt::W4A4 || f == Fmt::W4A4G128;
+    const bool wo = f == Fmt::W4A16 || f == Fmt::W3A16 || f == Fmt::W2A16;
+    if (h_sizes[i].x != 0 && ((wa && (!sa || !sb)) || (wo && !sb))) {
+      last_error() = "scale arrays are required for quantised formats";
+      return 5;
+    }
+  }
   for (int base = 0; base < count; base += kMaxProblems) {
     const int n = std::min(kMaxProblems, count - base);
     FusedArgs a;

@@ -116,3 +116,31 @@ def test_plan_bounds_on_random_problem_lists(lib):
             lo += min(-(-m // bm) * -(-n // bn) for bm, bn in mine if bm == max(x for x, _ in mine))
             hi += max(-(-m // bm) * -(-n // bn) for bm, bn in mine)
         assert lo <= tiles <= hi, (trial, lo, tiles, hi)
+
+
+def test_missing_arrays_are_refused_before_any_launch(lib):
+    """A quantised problem without scale arrays, or a plan without its host arrays, fails on the host with code 5."""
+    from mxmoe_amd import _lib
+
+    sizes = (_lib.Dim3 * 1)(_lib.Dim3(8, 256, 128))
+    q = (_lib.QParams * 1)(_lib.QParams(4, 4, -1, 1))
+    one = (C.c_void_p * 1)(0)
+    addr = C.addressof(one)
+    rc = lib.mxmoe_group_gemm(0, addr, addr, None, None, addr, addr, None, None, None, None, addr, sizes, None, q, 1, None, None)
+    assert rc == 5 and b"scale arrays" in lib.mxmoe_last_error()
+    rc = lib.mxmoe_group_gemm(0, None, addr, addr, addr, addr, addr, None, None, None, None, addr, sizes, None, q, 1, None, None)
+    assert rc == 5 and b"null argument" in lib.mxmoe_last_error()
+    assert lib.mxmoe_group_gemm_plan(-1, None, None, 1, None, None) == 5
+
+
+def test_prologue_entry_points_validate_on_the_host(lib):
+    one = (C.c_int64 * 8)()
+    a = C.addressof(one)
+    assert lib.mxmoe_quant_act(None, a, a, a, a, a, 256, 4, 2, 2, 0, 0, 1, 1, None, None) == 5 and b"null" in lib.mxmoe_last_error()
+    assert lib.mxmoe_quant_act(a, a, a, None, a, a, 256, 4, 2, 2, 0, 0, 1, 1, None, None) == 5
+    assert lib.mxmoe_quant_act(a, a, a, a, a, a, 256, -1, 2, 2, 0, 0, 1, 1, None, None) == 3
+    assert lib.mxmoe_quant_act(a, a, a, a, a, a, 260, 4, 2, 2, 0, 0, 1, 1, None, None) == 3 and b"multiple of 8" in lib.mxmoe_last_error()
+    assert lib.mxmoe_silu_mul_quant(a, None, a, a, a, a, 256, 256, 4, 2, 2, 1, 0, 1, 1, None, None) == 5
+    assert lib.mxmoe_silu_mul_quant(a, a, a, a, a, a, 1408, 1408, 4, 2, 2, 0, 1, 176, 4, None, None) == 3 and b"sign table" in lib.mxmoe_last_error()
+    assert lib.mxmoe_build_permutation(None, 4, 2, 8, a, a, a, a, a, None) == 5
+    assert lib.mxmoe_build_permutation(a, 0, 2, 8, a, a, a, a, a, None) == 3
