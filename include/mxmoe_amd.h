@@ -96,7 +96,8 @@ int mxmoe_build_permutation(const int32_t* topk_ids, int num_tokens, int topk, i
  *
  * mxmoe_quant_act gathers row perm_indices[r] of hidden [T, K] (shared rows read token r - R).
  * mxmoe_silu_mul_quant reads gate_up [R, 2N] (first half gate, second half up; shared rows from gate_up_shared [T, 2*N_shared]),
- * computes silu(gate) * up in fp32 rounded once to fp16, then rotates / quantises / packs like mxmoe_quant_act. */
+ * computes silu(gate) * up in fp32 rounded once to fp16, then rotates / quantises / packs like mxmoe_quant_act.
+ * scale_store may be NULL when every tag is 0 (no expert quantises its activations). */
 int mxmoe_quant_act(const void* hidden, void* inp_store, void* scale_store, const int32_t* dst_exp_sorted, const int64_t* perm_indices, const int64_t* exp_table,
                     int K, int rows_routed, int num_tokens, int num_experts, int has_shared, int rotate, int had_k, int had_f, const float* had_signs, void* stream);
 int mxmoe_silu_mul_quant(const void* gate_up, const void* gate_up_shared, void* inp_store, void* scale_store, const int32_t* dst_exp_sorted, const int64_t* exp_table,

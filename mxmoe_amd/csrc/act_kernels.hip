@@ -810,7 +810,7 @@ int mxmoe_quant_act(const void* hidden, void* inp_store, void* scale_store, cons
     last_error() = "bad row or expert count";
     return 3;
   }
-  if (!hidden || !inp_store || !scale_store || !exp_table || (rows_routed > 0 && (!dst_exp_sorted || !perm_indices))) {
+  if (!hidden || !inp_store || !exp_table || (rows_routed > 0 && (!dst_exp_sorted || !perm_indices))) {
     last_error() = "null pointer";
     return 5;
   }
@@ -840,7 +840,7 @@ int mxmoe_silu_mul_quant(const void* gate_up, const void* gate_up_shared, void* 
     last_error() = "bad row or expert count";
     return 3;
   }
-  if (!gate_up || !inp_store || !scale_store || !exp_table || (rows_routed > 0 && !dst_exp_sorted) || (has_shared && !gate_up_shared)) {
+  if (!gate_up || !inp_store || !exp_table || (rows_routed > 0 && !dst_exp_sorted) || (has_shared && !gate_up_shared)) {
     last_error() = "null pointer";
     return 5;
   }

@@ -83,12 +83,23 @@ def layer_weights(cfg, e):
     return w13.numpy(), w2.numpy()
 
 
+def _one_call_equals_stepwise(cfg, hidden, ids, layer):
+    """Size-independent property: the whole forward as one call gives the bits of the operator-by-operator forward + combine."""
+    from mxmoe_amd import synth
+
+    _, w = synth.make_routing(cfg)
+    stepwise = layer.combine(w).clone()
+    assert torch.equal(layer(hidden, ids, w), stepwise)
+    assert stepwise.shape == (cfg.tokens, cfg.hidden) and bool(torch.isfinite(stepwise).all())
+
+
 def test_c2_uniform_w4a4_full_size():
     cfg, hidden, ids, layer, outs, recv, prob_of = _build("c2")
     assert int(recv.sum()) == cfg.tokens * cfg.topk == sum(o.shape[0] for o in outs)
     assert all(o.shape == (int(recv[e]), cfg.hidden) for e, o in zip(sorted(prob_of), outs))
     _check_wxax_experts(cfg, hidden, ids, layer, recv, prob_of, [0, 31, 59])
     assert all(bool(torch.isfinite(o).all()) for o in outs)
+    _one_call_equals_stepwise(cfg, hidden, ids, layer)
 
 
 def test_c3_mixed_zipf_full_size():
@@ -123,6 +134,7 @@ def test_c4_weight_only_decode_full_size():
         out = O.gemm_fakequant(y, O.fake_quant(w2, b2, g2, s2))
         assert _rel(outs[p].cpu().numpy(), out) <= 1e-2, f"down, expert {e}"
     assert {f[0][1] for f in layer.formats} == {3, 4}
+    _one_call_equals_stepwise(cfg, hidden, ids, layer)
 
 
 def test_c1_fp16_full_size():
