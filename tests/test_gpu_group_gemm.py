@@ -208,6 +208,54 @@ def test_weight_only_many_tokens():
         assert _rel(out, p["ref"]) <= 1e-2, (p["size"], p["q"], _rel(out, p["ref"]))
 
 
+def _any_problem(rng, fmt, m, n, k):
+    from mxmoe_amd.weights import quantize_and_pack
+
+    if fmt in ("w4a4", "w8a8"):
+        return _wxax_problem(rng, m, n, k, 4 if fmt == "w4a4" else 8)
+    if fmt == "w4a4g":
+        return _grouped_problem(rng, m, n, k)
+    x = rng.standard_normal((m, k)).astype(F16)
+    w = (rng.standard_normal((n, k)) * 0.02).astype(F16)
+    if fmt == "fp16":
+        return dict(A=torch.from_numpy(x).to(DEV), B=torch.from_numpy(w).to(DEV), ref=O.gemm_fp16(x, w), size=(m, n, k), q=(16, 16, -1, True))
+    bits, sym = int(fmt[1]), fmt.endswith("s")
+    pw = quantize_and_pack(torch.from_numpy(w), (16, bits, 128, sym))
+    q, sc, z = O.quant_minmax(w, bits, 128, sym)
+    return dict(A=torch.from_numpy(x).to(DEV), B=pw.data.to(DEV), sb=pw.scale.to(DEV), ref=O.gemm_fakequant(x, O.dequant(q, sc, z, 128)),
+                size=(m, n, k), q=(16, bits, 128, sym))
+
+
+@pytest.mark.parametrize("seed", [101, 102, 103])
+def test_random_shapes_every_format_in_mixed_launches(seed):
+    """Seeded sweep over ragged shapes: any M (empty problems, one row, tile sizes +- 1), N any multiple of the format's step (not of a
+    tile), K any multiple of the format's slice, formats mixed in one launch.  Integer formats bit-exact, the others within 1e-2."""
+    rng = np.random.default_rng(seed)
+    k_step = {"w4a4": 128, "w8a8": 64, "w4a4g": 128, "fp16": 32, "w4a": 128, "w3a": 128, "w2s": 128, "w4s": 128}
+    n_step = {"w4a4": 8, "w8a8": 8, "w4a4g": 8, "fp16": 8}
+    fmts = list(k_step)
+    probs = []
+    for _ in range(14):
+        fmt = fmts[int(rng.integers(len(fmts)))]
+        m = int(rng.choice([1, 2, 15, 16, 17, 31, 32, 33, 63, 64, 65, 127, 128, 129, 200, 257]))
+        n = n_step.get(fmt, 16) * int(rng.integers(1, 60))
+        k = k_step[fmt] * int(rng.integers(1, 1 + 1536 // k_step[fmt]))
+        probs.append(_any_problem(rng, fmt, m, n, k))
+    empty = dict(probs[0])
+    empty.update(A=torch.zeros((0, 8), dtype=torch.int8, device=DEV), sa=torch.zeros(0, dtype=torch.float16, device=DEV), size=(0,) + probs[0]["size"][1:])
+    probs.insert(3, empty)
+    g, outs, accs = _launch(probs)
+    print("seed", seed, "kernel", g.plan()[0], [(p["q"], p["size"]) for p in probs])
+    for i, (p, out, acc) in enumerate(zip(probs, outs, accs)):
+        if p["size"][0] == 0:
+            continue
+        if "acc" in p:
+            assert np.array_equal(acc, p["acc"]), (i, p["size"], p["q"])
+            assert np.array_equal(out.view(np.uint16), p["out"].view(np.uint16)), (i, p["size"], p["q"])
+        else:
+            assert np.isfinite(out).all() and _rel(out, p["ref"]) <= 1e-2, (i, p["size"], p["q"], _rel(out, p["ref"]))
+
+
 def test_unsupported_format_raises_reference_message():
     rng = np.random.default_rng(4)
     p = _wxax_problem(rng, 4, 256, 128, 8)
