@@ -21,7 +21,7 @@ PEAK = {"int8": 5000.0, "fp16": 2500.0, "hbm": 8000.0}  # MI355X: TOP/s dense in
 
 # HBM bytes per launch of the dominant (gate_up) kernel, from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE runs scaled by the
 # same counters on a plain 256 MiB copy (summaries: profiles/fused_group_gemm_<workload>.txt, profiles/counter_calibration_copy_256MiB.txt)
-TRAFFIC = {"c2": 571311932, "c3": 793819758, "c4": 190296938}
+TRAFFIC = {"c2": 572434874, "c3": 789254059, "c4": 190260813}
 
 
 def build_layer(name: str, tokens: int | None):
@@ -74,14 +74,14 @@ def time_layer(layer, steps: int, warmup: int):
     return wall / steps, up, dn
 
 
-def launch_duration(plan, n: int = 20) -> float:
+def launch_duration(plan, n: int = 20, warm: int = 100) -> float:
     """Average duration (ms) of one launch: n back-to-back launches between two HIP events on the launch stream (no event
     between launches, so dispatch gaps of a few microseconds do not count as kernel time)."""
     import torch
 
     a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    plan.run()
-    torch.cuda.synchronize()
+    for _ in range(warm):  # the GPU needs tens of milliseconds of continuous work to settle at its sustained clock
+        plan.run()
     a.record()
     for _ in range(n):
         plan.run()
@@ -204,7 +204,7 @@ def time_whole_layer(cfg, layer, reps: int = 7) -> dict:
     return out
 
 
-def run_workload(name: str, steps: int, warmup: int, tokens=None):
+def run_workload(name: str, steps: int, warmup: int, tokens=None, whole: bool = True):
     cfg, layer = build_layer(name, tokens)
     ms, up, dn = time_layer(layer, steps, warmup)
     ops = layer.gemm_ops()
@@ -213,19 +213,20 @@ def run_workload(name: str, steps: int, warmup: int, tokens=None):
         "workload": name, "tops": round(ops / (ms * 1e-3) / 1e12, 2), "ms_per_step": round(ms, 4),
         "gate_up_us": round(up * 1e3, 2), "down_us": round(dn * 1e3, 2),
         "gate_up_tops": round(st["gg1"].ops / (up * 1e-3) / 1e12, 2), "down_tops": round(st["gg2"].ops / (dn * 1e-3) / 1e12, 2),
-        "ops": ops, "roofline": roofline_of(cfg, layer, up, dn), "whole_layer": time_whole_layer(cfg, layer),
+        "ops": ops, "whole_layer": time_whole_layer(cfg, layer) if whole else None, "roofline": roofline_of(cfg, layer, up, dn),
     }
 
 
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=300, help="untimed steps first: the GPU takes tens of milliseconds of continuous work to reach its sustained clock")
     ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
     ap.add_argument("--also", default="c3,c4", help="comma-separated extra workloads reported under 'also' (empty to skip)")
     ap.add_argument("--tokens", type=int, default=None)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-whole-layer", action="store_true", help="skip the wall-clock timing of the whole forward (profiling runs: the trace then ends with the launches the roofline entry is measured on)")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="BYTES",
                     help="instead of the benchmark, run a plain device copy of BYTES bytes 5 times (reference point for the FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -249,12 +250,12 @@ def main() -> int:
         return 0
     from mxmoe_amd import synth
 
-    cfg, layer, main_res = run_workload(args.workload, args.steps, args.warmup, args.tokens)
+    cfg, layer, main_res = run_workload(args.workload, args.steps, args.warmup, args.tokens, not args.no_whole_layer)
     also = {}
     del layer
     torch.cuda.empty_cache()
     for extra in [w for w in args.also.split(",") if w and w != args.workload]:
-        _, lay, res = run_workload(extra, max(10, args.steps // 2), max(5, args.warmup // 2))
+        _, lay, res = run_workload(extra, max(10, args.steps // 2), max(5, args.warmup // 2), whole=not args.no_whole_layer)
         also[extra] = res
         del lay
         torch.cuda.empty_cache()
