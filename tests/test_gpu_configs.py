@@ -114,6 +114,7 @@ def test_c3_mixed_zipf_full_size():
     _check_wxax_experts(cfg, hidden, ids, layer, recv, prob_of, sorted(want))
     assert {f[0][1] for f in fm} == {4, 8} and {f[1][1] for f in fm} == {4, 8}
     assert all(bool(torch.isfinite(o).all()) for o in outs)
+    _one_call_equals_stepwise(cfg, hidden, ids, layer)
 
 
 def test_c4_weight_only_decode_full_size():
@@ -152,6 +153,7 @@ def test_c1_fp16_full_size():
         g, u = st["mid"][p].float()[:, :cfg.inter], st["mid"][p].float()[:, cfg.inter:]
         y = (g * torch.sigmoid(g) * u).half().float()
         assert _rel(outs[p].float().cpu().numpy(), (y @ w2.T).cpu().numpy()) <= 1e-2
+    _one_call_equals_stepwise(cfg, hidden, ids, layer)
 
 
 def layer_weights_t(cfg, e):
@@ -190,3 +192,16 @@ def test_c5_shaped_layer_reduced():
             assert np.array_equal(r["g_out"].view(np.uint16), out_k.view(np.uint16)), f"down fp16, expert {r['e']}"
         else:
             assert _rel(r["g_out"], r["out"]) <= 1e-2, f"down, expert {r['e']}"
+
+
+def test_c5_one_call_equals_stepwise_at_real_row_lengths():
+    """Mixtral row lengths (4096 and 14336 = 28 x 512) with a tenth of the tokens: the one-call forward against the stepwise one."""
+    from mxmoe_amd import synth
+    from mxmoe_amd.layer import MxMoELayer
+
+    cfg = synth.get_config("c5", 512)
+    hidden = synth.make_hidden(cfg)
+    ids, _ = synth.make_routing(cfg)
+    layer = MxMoELayer(cfg)
+    layer.forward(hidden, ids)
+    _one_call_equals_stepwise(cfg, hidden, ids, layer)
