@@ -76,7 +76,9 @@ def main(argv=None) -> int:
     exact = False
     if args.synthetic:
         cfg, trace, synthetic_qcfg = materialise_synthetic(args.synthetic, None if "--bs" not in (argv or sys.argv) else bs)
-        args.qconfig = args.qconfig or synthetic_qcfg  # e.g. a qconfig the allocator (mxmoe_amd.bits_solver) wrote for this workload
+        # an explicit --qconfig (e.g. one the allocator, mxmoe_amd.bits_solver, wrote for this workload) or --qstr (one format for every
+        # block) wins over the configuration's own seeded formats
+        args.qconfig = args.qconfig or (None if args.qstr is not None else synthetic_qcfg)
         model_id, dataset, bs, layer, exact = cfg.model, "synthetic", cfg.tokens, 0, True
 
     if args.qconfig is not None:
