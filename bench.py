@@ -42,7 +42,7 @@ def build_layer(name: str, tokens: int | None):
     return cfg, layer
 
 
-def time_layer(layer, steps: int, warmup: int):
+def time_layer(layer, steps: int, warmup: int, settle_s: float = 0.15):
     """K steps of (gate_up launch, down launch); returns (ms_per_step, avg gate_up ms, avg down ms).
 
     The timed region holds nothing but the 2K launches (events between launches open gaps of several microseconds, which are not
@@ -51,6 +51,14 @@ def time_layer(layer, steps: int, warmup: int):
 
     st = layer.state
     g1, g2 = st["gg1"], st["gg2"]
+    # After an idle period the GPU needs tens of milliseconds of continuous work to reach its sustained clock; bring it there
+    # before the warm-up steps, whatever their number, so that a short --warmup does not time the ramp.
+    t_settle = time.perf_counter()
+    while time.perf_counter() - t_settle < settle_s:
+        for _ in range(20):
+            g1.run()
+            g2.run()
+        torch.cuda.synchronize()
     for _ in range(warmup):
         g1.run()
         g2.run()
@@ -221,7 +229,7 @@ def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=300, help="untimed steps first: the GPU takes tens of milliseconds of continuous work to reach its sustained clock")
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
     ap.add_argument("--also", default="c3,c4", help="comma-separated extra workloads reported under 'also' (empty to skip)")
     ap.add_argument("--tokens", type=int, default=None)
