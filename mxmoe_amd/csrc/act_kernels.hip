@@ -161,6 +161,21 @@ __device__ __forceinline__ float exp_fixed(float t) {
 
 __device__ __forceinline__ float round_h(float v) { return (float)(_Float16)v; }
 
+// v / s in fp32 for fp16-valued v and s, given r = 1.0f / s: the rounded product v * r corrected once with its exact remainder.
+// With r the correctly rounded reciprocal this is the correctly rounded quotient, i.e. bit for bit what the division instruction
+// sequence returns, for every pair of fp16 values (checked with exact integer arithmetic over all 2^20 mantissa pairs in
+// tests/test_oracle_quant.py); a row's elements share one scale, so the division proper is done once per row.
+// An infinite scale (a row that already holds an infinity) keeps the plain result: finite / inf = 0.
+struct ScaleDiv {
+  float r, s;
+  __device__ __forceinline__ explicit ScaleDiv(float scale) : r(1.0f / scale), s(__builtin_isinf(scale) ? 0.0f : scale) {}
+  __device__ __forceinline__ float operator()(float v) const {
+    const float q0 = v * r;
+    const float e = __builtin_fmaf(-s, q0, v);
+    return __builtin_fmaf(e, r, q0);
+  }
+};
+
 // NT threads per workgroup (256, or 192 when that wastes fewer lanes: a 1408-element row is 176 chunks of 8).
 template <int MAXC, bool SILU, int NT>
 __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
@@ -299,9 +314,9 @@ __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
           if (c < nchunks) {
             float o[8];
             get(c ^ hc, o);
-            const bool upper = c & hc;
+            const float sgn = (c & hc) ? -1.0f : 1.0f;  // upper half of a pair: other - own, lower half: own + other
 #pragma unroll
-            for (int j = 0; j < 8; ++j) v[i][j] = upper ? o[j] - v[i][j] : v[i][j] + o[j];
+            for (int j = 0; j < 8; ++j) v[i][j] = __builtin_fmaf(sgn, v[i][j], o[j]);  // +-own is exact, so this is the plain sum / difference
           }
         }
         __syncthreads();
@@ -372,8 +387,9 @@ __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
               const bool upper = ((c / (pl.kb * mc)) & hh) != 0;
               float o[8];
               get(upper ? c - hc : c + hc, o);
+              const float sgn = upper ? -1.0f : 1.0f;
 #pragma unroll
-              for (int j = 0; j < 8; ++j) v[i][j] = upper ? o[j] - v[i][j] : v[i][j] + o[j];
+              for (int j = 0; j < 8; ++j) v[i][j] = __builtin_fmaf(sgn, v[i][j], o[j]);
             }
           }
         }
@@ -418,12 +434,13 @@ __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
         for (int o = 8; o > 0; o >>= 1) gmax = fmaxf(gmax, __shfl_xor(gmax, o));
         float scale = round_h(gmax / 7.0f);
         if (scale == 0.0f) scale = 1.0f;
+        const ScaleDiv div(scale);
         if (live) {
           if ((c & 15) == 0) sout[c >> 4] = (_Float16)scale;
           unsigned w = 0;
 #pragma unroll
           for (int j = 0; j < 8; ++j) {
-            const float r = round_h(v[i][j] / scale);
+            const float r = round_h(div(v[i][j]));
             w |= (unsigned)((int)rintf(fminf(fmaxf(r, -7.0f), 7.0f)) & 0xF) << (4 * j);
           }
           *reinterpret_cast<unsigned*>(out + c * 4) = w;
@@ -451,6 +468,7 @@ __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
     const float upper = tag == 1 ? 127.0f : 7.0f;
     float scale = round_h(amax / upper);   // fp16 division: fp32 quotient of two fp16 values, rounded to fp16
     if (scale == 0.0f) scale = 1.0f;       // quantize.cuh:258
+    const ScaleDiv div(scale);
     if (tid == 0) a.scale_store[scale_off + lrow] = (_Float16)scale;
     uint8_t* out = a.inp_store + 2 * (inp_off + lrow * (tag == 1 ? n / 2 : n / 4));
 #pragma unroll
@@ -460,7 +478,7 @@ __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
         int q[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-          const float r = round_h(v[i][j] / scale);
+          const float r = round_h(div(v[i][j]));
           q[j] = (int)rintf(fminf(fmaxf(r, -upper), upper));
         }
         if (tag == 1) {
@@ -535,13 +553,15 @@ __global__ void __launch_bounds__(256) row_quant_wave_kernel(const RowArgs a) {
             }
 #pragma unroll
       for (int m = 1; m < 64; m <<= 1) {
-        const bool upper = lane & m;
+        // upper half of a pair: other - own, lower half: own + other; one fused multiply-add with own's sign, which rounds once
+        // exactly like the sum / difference (the product with +-1 is exact)
+        const float sgn = (lane & m) ? -1.0f : 1.0f;
 #pragma unroll
         for (int i = 0; i < NI; ++i)
 #pragma unroll
           for (int j = 0; j < 8; ++j) {
             const float o = __shfl_xor(v[i][j], m);
-            v[i][j] = upper ? o - v[i][j] : v[i][j] + o;
+            v[i][j] = __builtin_fmaf(sgn, v[i][j], o);
           }
       }
 #pragma unroll
@@ -585,11 +605,12 @@ __global__ void __launch_bounds__(256) row_quant_wave_kernel(const RowArgs a) {
         for (int o = 8; o > 0; o >>= 1) gmax = fmaxf(gmax, __shfl_xor(gmax, o));
         float scale = round_h(gmax / 7.0f);
         if (scale == 0.0f) scale = 1.0f;
+        const ScaleDiv div(scale);
         if ((c & 15) == 0) sout[c >> 4] = (_Float16)scale;
         unsigned w = 0;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-          const float r = round_h(v[i][j] / scale);
+          const float r = round_h(div(v[i][j]));
           w |= (unsigned)((int)rintf(fminf(fmaxf(r, -7.0f), 7.0f)) & 0xF) << (4 * j);
         }
         *reinterpret_cast<unsigned*>(out + c * 4) = w;
@@ -606,6 +627,7 @@ __global__ void __launch_bounds__(256) row_quant_wave_kernel(const RowArgs a) {
     const float upper = tag == 1 ? 127.0f : 7.0f;
     float scale = round_h(amax / upper);   // fp16 division: fp32 quotient of two fp16 values, rounded to fp16
     if (scale == 0.0f) scale = 1.0f;       // quantize.cuh:258
+    const ScaleDiv div(scale);
     if (lane == 0) a.scale_store[scale_off + lrow] = (_Float16)scale;
     uint8_t* out = a.inp_store + 2 * (inp_off + lrow * (tag == 1 ? n / 2 : n / 4));
 #pragma unroll
@@ -614,7 +636,7 @@ __global__ void __launch_bounds__(256) row_quant_wave_kernel(const RowArgs a) {
       int q[8];
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        const float r = round_h(v[i][j] / scale);
+        const float r = round_h(div(v[i][j]));
         q[j] = (int)rintf(fminf(fmaxf(r, -upper), upper));
       }
       if (tag == 1) {

@@ -191,3 +191,69 @@ def test_linear_block_group_format_agrees_with_fake_quant():
     assert acc.shape == (2, 6, 16)
     rel = np.abs(out_k.astype(np.float64) - out_f.astype(np.float64)).max() / np.abs(out_f.astype(np.float64)).max()
     assert rel <= 1e-2
+
+
+# ---- the quantiser kernels divide a row by its scale with one shared reciprocal: exactness of that scheme ----
+def _rne_shift(x, sh):
+    """round-to-nearest-even of x / 2^sh for non-negative int64 arrays (sh array or scalar >= 1)"""
+    sh = np.asarray(sh, dtype=np.int64)
+    half = np.int64(1) << (sh - 1)
+    q = x >> sh
+    r = x & ((np.int64(1) << sh) - 1)
+    up = (r > half) | ((r == half) & ((q & 1) == 1))
+    return q + up.astype(np.int64)
+
+
+def _rn24(x):
+    """(mantissa in [2^23, 2^24), exponent e) with value ~= m * 2^e of the positive int64 array x rounded to 24 significant bits"""
+    nb = np.floor(np.log2(x.astype(np.float64))).astype(np.int64) + 1          # bit length (exact for < 2^53; values here are)
+    # fix possible off-by-one of the float log
+    nb = np.where((np.int64(1) << (nb - 1)) > x, nb - 1, nb)
+    nb = np.where((np.int64(1) << nb) <= x, nb + 1, nb)
+    sh = nb - 24
+    m = np.where(sh > 0, _rne_shift(x, np.maximum(sh, 1)), x << np.maximum(-sh, 0))
+    e = sh.copy()
+    over = m == (1 << 24)
+    m = np.where(over, m >> 1, m); e = np.where(over, e + 1, e)
+    return m, e
+
+
+def test_shared_reciprocal_division_is_exact_for_all_fp16_pairs():
+    """v / s as the kernels compute it (r = RN(1 / s) once per row; q0 = RN(v * r); e = v - s * q0 exactly, one fused operation;
+    q = RN(q0 + e * r), one fused operation) against the correctly rounded quotient, in exact integer arithmetic, for every pair of
+    11-bit mantissas: fp16 values are such mantissas times powers of two (subnormals have trailing zeros), signs are symmetric and
+    no intermediate leaves the normal fp32 range, so this covers every finite fp16 pair.  Without the correction step the rounded
+    product alone is wrong for a large share of the pairs, so the check can fail."""
+    a, b = np.meshgrid(np.arange(1024, 2048, dtype=np.int64), np.arange(1024, 2048, dtype=np.int64), indexing="ij")
+    a = a.ravel(); b = b.ravel()
+    # y = RN24(1/b): 2^34 / b lies in (2^23, 2^24]
+    num = np.int64(1) << 34
+    yq, yr = num // b, num % b
+    Y = yq + ((2 * yr > b) | ((2 * yr == b) & (yq & 1 == 1))).astype(np.int64)       # value y = Y * 2^-34 (Y = 2^24 only for b = 1024)
+    # q0 = RN24(a * y)
+    P = a * Y                                                                       # value a*y = P * 2^-34
+    m0, e0 = _rn24(P)                                                                # q0 = m0 * 2^(e0 - 34)
+    # e = a - b*q0 exactly, in units of 2^(e0-34)
+    E = (a << (34 - e0)) - b * m0
+    assert (np.abs(E) < (1 << 24)).all(), "remainder representable in fp32"
+    # q1 = RN24(q0 + e*y): units of 2^(e0-34-34)
+    S = (m0 << 34) + E * Y
+    m1, e1 = _rn24(S)                                                                # q1 = m1 * 2^(e1 + e0 - 68)
+    # true quotient RN24(a/b): a/b in (0.5, 2)
+    big = a << 40
+    tq, tr = big // b, big % b                                                      # a/b = (tq + tr/b) * 2^-40, tq < 2^41
+    nb = np.where(tq >= (np.int64(1) << 40), 41, 40)
+    sh = nb - 24
+    mt = tq >> sh
+    rem_hi = tq & ((np.int64(1) << sh) - 1)
+    half = np.int64(1) << (sh - 1)
+    gt = (rem_hi > half) | ((rem_hi == half) & (tr > 0))
+    tie = (rem_hi == half) & (tr == 0)
+    mt = mt + (gt | (tie & ((mt & 1) == 1))).astype(np.int64)
+    et = sh - 40
+    over = mt == (1 << 24); mt = np.where(over, mt >> 1, mt); et = np.where(over, et + 1, et)
+
+    same = (m1 == mt) & ((e1 + e0 - 68) == et)
+    assert same.all(), (a[~same][:5], b[~same][:5])
+    plain = (m0 == mt) & ((e0 - 34) == et)
+    assert 0.05 < (~plain).mean() < 0.6
