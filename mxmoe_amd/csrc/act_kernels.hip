@@ -13,6 +13,7 @@
 // x / scale, clamp, round-half-even, all rounded to fp16) and of a fixed-order fp32 Hadamard transform, so integer
 // codes are reproducible bit for bit on a CPU; this file must be compiled with FMA contraction off.
 #include <hip/hip_runtime.h>
+#include <type_traits>
 #include <stdint.h>
 
 #include <cmath>
@@ -497,6 +498,28 @@ __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
   }
 }
 
+// Value of lane (l ^ M).  Distances 1 .. 8 stay inside a row of 16 lanes and are data-parallel-primitive moves in the vector ALU
+// (quad permutations; l ^ 4 = mirror of 8 lanes, then of 4; l ^ 8 = mirror of 16 lanes, then of 8); 16 and 32 go through the LDS
+// crossbar, whose throughput is what bounds this kernel once the arithmetic is trimmed.
+template <int M>
+__device__ __forceinline__ float lane_xor(float v) {
+  int x = __float_as_int(v);
+  if constexpr (M == 1) {
+    x = __builtin_amdgcn_update_dpp(0, x, 0xB1, 0xF, 0xF, true);   // quad_perm [1,0,3,2]
+  } else if constexpr (M == 2) {
+    x = __builtin_amdgcn_update_dpp(0, x, 0x4E, 0xF, 0xF, true);   // quad_perm [2,3,0,1]
+  } else if constexpr (M == 4) {
+    x = __builtin_amdgcn_update_dpp(0, x, 0x141, 0xF, 0xF, true);  // row_half_mirror: l ^ 7
+    x = __builtin_amdgcn_update_dpp(0, x, 0x1B, 0xF, 0xF, true);   // quad_perm [3,2,1,0]: l ^ 3
+  } else if constexpr (M == 8) {
+    x = __builtin_amdgcn_update_dpp(0, x, 0x140, 0xF, 0xF, true);  // row_mirror: l ^ 15
+    x = __builtin_amdgcn_update_dpp(0, x, 0x141, 0xF, 0xF, true);  // row_half_mirror: l ^ 7
+  } else {
+    return __shfl_xor(v, M);
+  }
+  return __int_as_float(x);
+}
+
 // One row per WAVE, for rows whose rotation is a pure Sylvester transform (n = 512 * NI, NI a power of two): lane l holds the NI
 // 8-element chunks l + 64*i.  The butterfly strides map to three levels, taken in the same ascending order as everywhere else:
 // 1, 2, 4 inside a chunk (registers), 8 .. 256 across the lanes (cross-lane exchange, no LDS staging, no barrier),
@@ -551,19 +574,22 @@ __global__ void __launch_bounds__(256) row_quant_wave_kernel(const RowArgs a) {
               v[i][j] = p + q;
               v[i][j + h] = p - q;
             }
-#pragma unroll
-      for (int m = 1; m < 64; m <<= 1) {
+      auto lane_stage = [&](auto mc) {
+        constexpr int m = decltype(mc)::value;
         // upper half of a pair: other - own, lower half: own + other; one fused multiply-add with own's sign, which rounds once
         // exactly like the sum / difference (the product with +-1 is exact)
         const float sgn = (lane & m) ? -1.0f : 1.0f;
 #pragma unroll
         for (int i = 0; i < NI; ++i)
 #pragma unroll
-          for (int j = 0; j < 8; ++j) {
-            const float o = __shfl_xor(v[i][j], m);
-            v[i][j] = __builtin_fmaf(sgn, v[i][j], o);
-          }
-      }
+          for (int j = 0; j < 8; ++j) v[i][j] = __builtin_fmaf(sgn, v[i][j], lane_xor<m>(v[i][j]));
+      };
+      lane_stage(std::integral_constant<int, 1>{});
+      lane_stage(std::integral_constant<int, 2>{});
+      lane_stage(std::integral_constant<int, 4>{});
+      lane_stage(std::integral_constant<int, 8>{});
+      lane_stage(std::integral_constant<int, 16>{});
+      lane_stage(std::integral_constant<int, 32>{});
 #pragma unroll
       for (int hi = 1; hi < NI; hi <<= 1)
 #pragma unroll
