@@ -177,6 +177,28 @@ struct ScaleDiv {
   }
 };
 
+// Value of lane (l ^ M).  Distances 1 .. 8 stay inside a row of 16 lanes and are data-parallel-primitive moves in the vector ALU
+// (quad permutations; l ^ 4 = mirror of 8 lanes, then of 4; l ^ 8 = mirror of 16 lanes, then of 8); 16 and 32 go through the LDS
+// crossbar, whose throughput is what bounds this kernel once the arithmetic is trimmed.
+template <int M>
+__device__ __forceinline__ float lane_xor(float v) {
+  int x = __float_as_int(v);
+  if constexpr (M == 1) {
+    x = __builtin_amdgcn_update_dpp(0, x, 0xB1, 0xF, 0xF, true);   // quad_perm [1,0,3,2]
+  } else if constexpr (M == 2) {
+    x = __builtin_amdgcn_update_dpp(0, x, 0x4E, 0xF, 0xF, true);   // quad_perm [2,3,0,1]
+  } else if constexpr (M == 4) {
+    x = __builtin_amdgcn_update_dpp(0, x, 0x141, 0xF, 0xF, true);  // row_half_mirror: l ^ 7
+    x = __builtin_amdgcn_update_dpp(0, x, 0x1B, 0xF, 0xF, true);   // quad_perm [3,2,1,0]: l ^ 3
+  } else if constexpr (M == 8) {
+    x = __builtin_amdgcn_update_dpp(0, x, 0x140, 0xF, 0xF, true);  // row_mirror: l ^ 15
+    x = __builtin_amdgcn_update_dpp(0, x, 0x141, 0xF, 0xF, true);  // row_half_mirror: l ^ 7
+  } else {
+    return __shfl_xor(v, M);
+  }
+  return __int_as_float(x);
+}
+
 // NT threads per workgroup (256, or 192 when that wastes fewer lanes: a 1408-element row is 176 chunks of 8).
 template <int MAXC, bool SILU, int NT>
 __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
@@ -185,7 +207,7 @@ __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
   const int nmax = max(a.plan.n, a.plan_shared.n);
   float* x = lds;                  // [nmax]
   float* sg = lds + nmax;          // [kb*kb]
-  float* red = sg + a.plan.kb * a.plan.kb;  // [8]
+  float* red = sg + a.plan.kb * a.plan.kb;  // [16]: one slot per wave
   // A chunk of 8 values lives in two planes of 16 bytes (values 0-3, values 4-7): consecutive lanes then touch consecutive 16-byte
   // words and a wave's 128-bit accesses spread over all banks (32-byte lane strides would hit every bank twice).
   float4* xlo = reinterpret_cast<float4*>(x);
@@ -306,8 +328,37 @@ __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
 
     if (rot) {
       // Sylvester strides 8 .. m/2 through LDS (ascending)
+      bool lds_stale = false;  // registers ahead of the copy in LDS
       for (int h = 8; h < pl.m; h <<= 1) {
         const int hc = h >> 3;
+        if (hc < 64) {
+          // the partner chunk c ^ hc sits in the same wave, hc lanes away (NT is a multiple of 64): exchange in registers
+          const float sgn = (tid & hc) ? -1.0f : 1.0f;
+          auto stage = [&](auto mc) {
+#pragma unroll
+            for (int i = 0; i < MAXC; ++i)
+#pragma unroll
+              for (int j = 0; j < 8; ++j) v[i][j] = __builtin_fmaf(sgn, v[i][j], lane_xor<decltype(mc)::value>(v[i][j]));
+          };
+          switch (hc) {
+            case 1: stage(std::integral_constant<int, 1>{}); break;
+            case 2: stage(std::integral_constant<int, 2>{}); break;
+            case 4: stage(std::integral_constant<int, 4>{}); break;
+            case 8: stage(std::integral_constant<int, 8>{}); break;
+            case 16: stage(std::integral_constant<int, 16>{}); break;
+            default: stage(std::integral_constant<int, 32>{}); break;
+          }
+          lds_stale = true;
+          continue;
+        }
+        if (lds_stale) {  // every thread rewrites its own chunks only, which nobody reads before the barrier below
+#pragma unroll
+          for (int i = 0; i < MAXC; ++i) {
+            const int c = tid + i * NT;
+            if (c < nchunks) put(c, v[i]);
+          }
+          lds_stale = false;
+        }
         __syncthreads();
 #pragma unroll
         for (int i = 0; i < MAXC; ++i) {
@@ -496,28 +547,6 @@ __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
       }
     }
   }
-}
-
-// Value of lane (l ^ M).  Distances 1 .. 8 stay inside a row of 16 lanes and are data-parallel-primitive moves in the vector ALU
-// (quad permutations; l ^ 4 = mirror of 8 lanes, then of 4; l ^ 8 = mirror of 16 lanes, then of 8); 16 and 32 go through the LDS
-// crossbar, whose throughput is what bounds this kernel once the arithmetic is trimmed.
-template <int M>
-__device__ __forceinline__ float lane_xor(float v) {
-  int x = __float_as_int(v);
-  if constexpr (M == 1) {
-    x = __builtin_amdgcn_update_dpp(0, x, 0xB1, 0xF, 0xF, true);   // quad_perm [1,0,3,2]
-  } else if constexpr (M == 2) {
-    x = __builtin_amdgcn_update_dpp(0, x, 0x4E, 0xF, 0xF, true);   // quad_perm [2,3,0,1]
-  } else if constexpr (M == 4) {
-    x = __builtin_amdgcn_update_dpp(0, x, 0x141, 0xF, 0xF, true);  // row_half_mirror: l ^ 7
-    x = __builtin_amdgcn_update_dpp(0, x, 0x1B, 0xF, 0xF, true);   // quad_perm [3,2,1,0]: l ^ 3
-  } else if constexpr (M == 8) {
-    x = __builtin_amdgcn_update_dpp(0, x, 0x140, 0xF, 0xF, true);  // row_mirror: l ^ 15
-    x = __builtin_amdgcn_update_dpp(0, x, 0x141, 0xF, 0xF, true);  // row_half_mirror: l ^ 7
-  } else {
-    return __shfl_xor(v, M);
-  }
-  return __int_as_float(x);
 }
 
 // One row per WAVE, for rows whose rotation is a pure Sylvester transform (n = 512 * NI, NI a power of two): lane l holds the NI
@@ -726,9 +755,11 @@ static int launch_rows(const RowArgs& a, int lds_bytes, hipStream_t s) {
   }
   // workgroup size and chunks per thread with the fewest idle lanes
   const int nchunks = nmax / 8;
-  static const int kShapes[][2] = {{192, 1}, {256, 1}, {192, 2}, {256, 2}, {192, 3}, {256, 3}, {256, 7}};
+  // long rows take 512 threads rather than more chunks per thread: a thread's chunks live in registers (with the next row's
+  // already on their way), and seven of them leave room for one wave per SIMD only
+  static const int kShapes[][2] = {{192, 1}, {256, 1}, {192, 2}, {256, 2}, {192, 3}, {256, 3}, {512, 2}, {512, 3}, {512, 4}};
   int pick = -1;
-  for (int i = 0; i < 7 && pick < 0; ++i)
+  for (int i = 0; i < 9 && pick < 0; ++i)
     if (kShapes[i][0] * kShapes[i][1] >= nchunks) pick = i;
   switch (pick) {
     case 0: hipLaunchKernelGGL((row_quant_kernel<1, SILU, 192>), dim3(grid), dim3(192), lds_bytes, s, a); break;
@@ -737,7 +768,9 @@ static int launch_rows(const RowArgs& a, int lds_bytes, hipStream_t s) {
     case 3: hipLaunchKernelGGL((row_quant_kernel<2, SILU, 256>), dim3(grid), dim3(256), lds_bytes, s, a); break;
     case 4: hipLaunchKernelGGL((row_quant_kernel<3, SILU, 192>), dim3(grid), dim3(192), lds_bytes, s, a); break;
     case 5: hipLaunchKernelGGL((row_quant_kernel<3, SILU, 256>), dim3(grid), dim3(256), lds_bytes, s, a); break;
-    case 6: hipLaunchKernelGGL((row_quant_kernel<7, SILU, 256>), dim3(grid), dim3(256), lds_bytes, s, a); break;
+    case 6: hipLaunchKernelGGL((row_quant_kernel<2, SILU, 512>), dim3(grid), dim3(512), lds_bytes, s, a); break;
+    case 7: hipLaunchKernelGGL((row_quant_kernel<3, SILU, 512>), dim3(grid), dim3(512), lds_bytes, s, a); break;
+    case 8: hipLaunchKernelGGL((row_quant_kernel<4, SILU, 512>), dim3(grid), dim3(512), lds_bytes, s, a); break;
     default:
       last_error() = "row too long for the activation kernels";
       return 3;
@@ -877,7 +910,7 @@ int mxmoe_quant_act(const void* hidden, void* inp_store, void* scale_store, cons
   a.rotate = rotate;
   if (a.rows == 0) return 0;
   if (const int rc = fill_common(a, K, K, rotate ? had_k : 1, rotate ? had_f : 1, had_signs)) return rc;
-  const int lds = (K + a.plan.kb * a.plan.kb + 8) * (int)sizeof(float);
+  const int lds = (K + a.plan.kb * a.plan.kb + 16) * (int)sizeof(float);
   return launch_rows<false>(a, lds, (hipStream_t)stream);
 }
 
@@ -909,7 +942,7 @@ int mxmoe_silu_mul_quant(const void* gate_up, const void* gate_up_shared, void* 
   if (a.rows == 0) return 0;
   if (const int rc = fill_common(a, N, has_shared ? N_shared : N, rotate ? had_k : 1, rotate ? had_f : 1, had_signs)) return rc;
   const int nmax = N > a.plan_shared.n ? N : a.plan_shared.n;
-  const int lds = (nmax + a.plan.kb * a.plan.kb + 8) * (int)sizeof(float);
+  const int lds = (nmax + a.plan.kb * a.plan.kb + 16) * (int)sizeof(float);
   return launch_rows<true>(a, lds, (hipStream_t)stream);
 }
 

@@ -42,7 +42,7 @@ def _unpack(store_view, tag, n):
     return np.where(q >= 8, q - 16, q).astype(np.int8)
 
 
-@pytest.mark.parametrize("k,rotate", [(2048, 1), (4096, 1), (256, 0), (2048, 2), (512, 1), (1024, 2), (2048, 0)])
+@pytest.mark.parametrize("k,rotate", [(2048, 1), (4096, 1), (256, 0), (2048, 2), (512, 1), (1024, 2), (2048, 0), (256, 1), (8192, 1), (2816, 2), (14336, 1)])
 def test_quant_inp_act_bit_exact(k, rotate):
     from mxmoe_amd import ops
 
