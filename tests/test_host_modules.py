@@ -253,3 +253,14 @@ def test_build_refuses_compiler_memory_instructions_in_hand_counted_loops():
         chk(mk(wait + ["\tglobal_load_dword v40, v[2:3], off"] + load))
     # loops without hand-tracked loads may hold any memory instruction
     chk("_Z6kernelv:\n" + "\n".join(head + ["\tglobal_load_dword v40, v[2:3], off"] + tail) + "\n\ts_endpgm\n")
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU; asked for more it says so and exits non-zero without touching a device."""
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    root = Path(__file__).resolve().parent.parent
+    res = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert res.returncode == 2 and "one GPU" in res.stderr and res.stdout.strip() == ""
