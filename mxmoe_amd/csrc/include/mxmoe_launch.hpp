@@ -70,11 +70,29 @@ struct Dispatch<I, T, Rest...> {
   __device__ static __forceinline__ void go(int branch, TileArgs& t, int local, uint8_t* smem) {
     if (branch == I) {
       // local index -> (row tile, column tile) as tile_scheduler.cuh:40-49, but row tile fastest: neighbouring workgroups then share
-      // one block of weight rows (the large operand: it is fetched once per expert) and sweep the expert's activations, which
-      // are small enough to stay in L2
+      // one block of weight rows and sweep the problem's activations.  The 64 workgroups that an XCD runs at a time only share
+      // what its 4 MB L2 still holds, and they drift apart along K, so a problem whose activations exceed the L2 ends up
+      // streaming them once per column tile.  Such a problem is walked in groups of row tiles holding at most 2 MB of
+      // activations, each group against all column tiles: the group's activations stay resident whatever the drift, and a block
+      // of weights is fetched once per group by row tiles that start together.  The plain order is kept where the estimate of
+      // its traffic (activations once per 64 / grid_m column tiles, weights once) is below half of the grouped order's (weights
+      // once per group, activations once): very long rows, of which only one or two row tiles fit.
       const int grid_m = (t.M - t.row0 + T::BM - 1) / T::BM;
-      t.tile_n = local / grid_m;
-      t.tile_m = local - t.tile_n * grid_m;
+      const int grid_n = (t.N + T::BN - 1) / T::BN;
+      const int tile_bytes = max(T::BM * (t.K / 8) * T::kABits, 1);
+      int rg = min(max((2 << 20) / tile_bytes, 1), grid_m);  // row tiles per group
+      if (rg < grid_m) {
+        const float a_bytes = (float)grid_m * (float)tile_bytes;
+        const float b_bytes = (float)t.N * (float)(t.K / 8) * (float)T::kWBits;
+        const float grouped = (float)((grid_m + rg - 1) / rg) * b_bytes + a_bytes;
+        const float plain = fmaxf((float)grid_n * (float)grid_m * (1.0f / 64.0f), 1.0f) * a_bytes + b_bytes;
+        if (grouped >= 2.0f * plain || tile_bytes > (2 << 20)) rg = grid_m;  // (a single row tile beyond the budget cannot stay resident either)
+      }
+      const int per_group = rg * grid_n;
+      const int g = local / per_group, r = local - g * per_group;
+      const int rows_g = min(rg, grid_m - g * rg);
+      t.tile_n = r / rows_g;
+      t.tile_m = g * rg + (r - t.tile_n * rows_g);
       T::run(t, smem);
     } else {
       Dispatch<I + 1, Rest...>::go(branch, t, local, smem);

@@ -40,6 +40,7 @@ struct SkinnyWoTile {
   static constexpr int kScaleBytes = NB * KP * 64;         // per-wave patch of (scale, zero) pairs of one pass
   static constexpr int kLdsBytes = kRedBytes + kWaves * kScaleBytes;
   static constexpr int kAccRegs = NB * 4;
+  static constexpr int kABits = 16, kWBits = WBITS;  // fp16 activations, packed weights
   static constexpr int kLaneBytes = WBITS * 4;       // packed bytes per lane per (channel block, k block)
   static constexpr int kBlockBytes = 64 * kLaneBytes;
   static constexpr int kRing = 12;                   // packed blocks in flight per wave
@@ -243,6 +244,7 @@ struct WoMfmaTile {
   static constexpr int kStageBytes = BM * 256;
   static constexpr int kLdsBytes = 2 * kStageBytes;
   static constexpr int kAccRegs = 64;
+  static constexpr int kABits = 16, kWBits = WBITS;  // fp16 activations, packed weights
   static constexpr int kLaneBytes = Sk::kLaneBytes, kBlockBytes = Sk::kBlockBytes;
   static constexpr int kDma = kStageBytes / 1024 / kWaves;  // direct-to-LDS loads per wave per stage
 
