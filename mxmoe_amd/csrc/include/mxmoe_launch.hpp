@@ -59,6 +59,11 @@ struct FusedArgs {
 };
 static_assert(sizeof(FusedArgs) <= 4096, "kernel arguments are limited to 4 KB");
 
+// Activation bytes that a group of row tiles may hold (see Dispatch::go): half of an XCD's 4 MB L2.
+#ifndef MXMOE_GROUP_BYTES
+#define MXMOE_GROUP_BYTES (2 << 20)
+#endif
+
 template <int I, class... Tiles>
 struct Dispatch;
 template <int I>
@@ -80,13 +85,13 @@ struct Dispatch<I, T, Rest...> {
       const int grid_m = (t.M - t.row0 + T::BM - 1) / T::BM;
       const int grid_n = (t.N + T::BN - 1) / T::BN;
       const int tile_bytes = max(T::BM * (t.K / 8) * T::kABits, 1);
-      int rg = min(max((2 << 20) / tile_bytes, 1), grid_m);  // row tiles per group
+      int rg = min(max(MXMOE_GROUP_BYTES / tile_bytes, 1), grid_m);  // row tiles per group
       if (rg < grid_m) {
         const float a_bytes = (float)grid_m * (float)tile_bytes;
         const float b_bytes = (float)t.N * (float)(t.K / 8) * (float)T::kWBits;
         const float grouped = (float)((grid_m + rg - 1) / rg) * b_bytes + a_bytes;
         const float plain = fmaxf((float)grid_n * (float)grid_m * (1.0f / 64.0f), 1.0f) * a_bytes + b_bytes;
-        if (grouped >= 2.0f * plain || tile_bytes > (2 << 20)) rg = grid_m;  // (a single row tile beyond the budget cannot stay resident either)
+        if (grouped >= 2.0f * plain || tile_bytes > MXMOE_GROUP_BYTES) rg = grid_m;  // (a single row tile beyond the budget cannot stay resident either)
       }
       const int per_group = rg * grid_n;
       const int g = local / per_group, r = local - g * per_group;
