@@ -104,24 +104,32 @@ def _default_tokens(name: str) -> int:
     return synth.CONFIGS[name].tokens if name in synth.CONFIGS else -1
 
 
-def roofline_of(cfg, layer, up_ms: float, dn_ms: float):
-    """Roofline entry of the dominant launch.  Compute-bound layers (w-a formats at thousands of tokens): ops of the
-    gate_up launch against the int8 (or fp16) MFMA peak.  Skinny weight-only layers: algorithmic bytes against HBM."""
+def roofline_entry(cfg, layer, name: str) -> dict:
+    """Roofline entry of one launch ("gate_up" or "down").  Compute-bound layers (w-a formats at thousands of tokens): ops of the
+    launch against the int8 (or fp16) MFMA peak.  Skinny weight-only layers: algorithmic bytes against HBM."""
     st = layer.state
     by = layer.algorithmic_bytes()
-    name, plan = ("gate_up", st["gg1"]) if up_ms >= dn_ms else ("down", st["gg2"])
+    plan = st["gg1"] if name == "gate_up" else st["gg2"]
     ms = launch_duration(plan)
     traffic = TRAFFIC.get(cfg.name) if name == "gate_up" and cfg.tokens == _default_tokens(cfg.name) else None
+    # `traffic` is not measured by this run: it is the figure of the rocprofv3 --pmc summary named here (same command, same seeds)
+    src = {"traffic_source": f"profiles/fused_group_gemm_{cfg.name}.txt"} if traffic is not None else {}
     fmts = {q[:2] for q in plan.qparams}
     compute_bound = cfg.tokens * cfg.topk / cfg.num_experts >= 128
     if compute_bound:
         peak = PEAK["fp16"] if all(a >= 16 for a, _ in fmts) else PEAK["int8"]
         ach = plan.ops / (ms * 1e-3) / 1e12
         return {"kernel": f"fused_group_gemm[{name}]", "bound": "mfma", "achieved": round(ach, 2), "peak": peak, "unit": "TFLOP/s",
-                "frac": round(ach / peak, 4), "traffic": traffic, "launch_us": round(ms * 1e3, 2), "algorithmic_bytes": by[name]["total"]}
+                "frac": round(ach / peak, 4), "traffic": traffic, **src, "launch_us": round(ms * 1e3, 2), "algorithmic_bytes": by[name]["total"]}
     ach = by[name]["total"] / (ms * 1e-3) / 1e9
     return {"kernel": f"fused_group_gemm[{name}]", "bound": "hbm", "achieved": round(ach, 1), "peak": PEAK["hbm"], "unit": "GB/s",
-            "frac": round(ach / PEAK["hbm"], 4), "traffic": traffic, "launch_us": round(ms * 1e3, 2), "algorithmic_bytes": by[name]["total"]}
+            "frac": round(ach / PEAK["hbm"], 4), "traffic": traffic, **src, "launch_us": round(ms * 1e3, 2), "algorithmic_bytes": by[name]["total"]}
+
+
+def roofline_of(cfg, layer, up_ms: float, dn_ms: float):
+    """(entry of the dominant launch, entry of the other launch)."""
+    names = ("gate_up", "down") if up_ms >= dn_ms else ("down", "gate_up")
+    return tuple(roofline_entry(cfg, layer, n) for n in names)
 
 
 def cpu_baseline(cfg, budget_s: float = 20.0):
@@ -217,11 +225,12 @@ def run_workload(name: str, steps: int, warmup: int, tokens=None, whole: bool = 
     ms, up, dn = time_layer(layer, steps, warmup)
     ops = layer.gemm_ops()
     st = layer.state
+    roof = roofline_of(cfg, layer, up, dn)
     return cfg, layer, {
         "workload": name, "tops": round(ops / (ms * 1e-3) / 1e12, 2), "ms_per_step": round(ms, 4),
         "gate_up_us": round(up * 1e3, 2), "down_us": round(dn * 1e3, 2),
         "gate_up_tops": round(st["gg1"].ops / (up * 1e-3) / 1e12, 2), "down_tops": round(st["gg2"].ops / (dn * 1e-3) / 1e12, 2),
-        "ops": ops, "whole_layer": time_whole_layer(cfg, layer) if whole else None, "roofline": roofline_of(cfg, layer, up, dn),
+        "ops": ops, "whole_layer": time_whole_layer(cfg, layer) if whole else None, "roofline": roof[0], "roofline_other_launch": roof[1],
     }
 
 
@@ -230,8 +239,8 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
-    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
-    ap.add_argument("--also", default="c3,c4", help="comma-separated extra workloads reported under 'also' (empty to skip)")
+    ap.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--also", default="c2,c4", help="comma-separated extra workloads reported under 'also' (empty to skip)")
     ap.add_argument("--tokens", type=int, default=None)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-whole-layer", action="store_true", help="skip the wall-clock timing of the whole forward (profiling runs: the trace then ends with the launches the roofline entry is measured on)")
@@ -285,7 +294,7 @@ def main() -> int:
         "config": {"workload": f"{args.workload}: {cfg.description}", "experts": cfg.num_experts, "topk": cfg.topk, "hidden": cfg.hidden,
                    "intermediate": cfg.inter, "tokens": cfg.tokens, "formats": fm, "step": "gate_up GroupGEMM launch + down GroupGEMM launch"},
         "roofline": main_res["roofline"],
-        "detail": {k: main_res[k] for k in ("gate_up_us", "down_us", "gate_up_tops", "down_tops", "ops", "whole_layer")},
+        "detail": {k: main_res[k] for k in ("gate_up_us", "down_us", "gate_up_tops", "down_tops", "ops", "whole_layer", "roofline_other_launch")},
         "also": also,
     }
     if not args.no_cpu_baseline:

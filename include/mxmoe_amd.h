@@ -39,8 +39,12 @@ int mxmoe_kernel_branch(int kernel_id, int branch, int32_t out[8]);
  *
  * One launch computes Cs[p][M,N] = As[p][M,K] * Bs[p][N,K]^T for every problem p in its own format.
  * As, Bs, scale_a, scale_b, Cs, Ds, d_sizes and d_q are DEVICE arrays of `problem_count` entries; h_sizes and h_q are
- * their HOST mirrors (as in the reference).  Ds must alias Cs; lda/ldb/ldc/ldd and d_q are accepted for signature
- * compatibility and ignored (leading dimensions are K, K, N; the reference passes nullptr, ref_bind.cu:413).
+ * their HOST mirrors (as in the reference).  Ds must be the same array as Cs or NULL (anything else is error 3: results are written
+ * to Cs only); lda/ldb/ldc/ldd and d_q are DEVICE arrays accepted for signature compatibility and never read (leading dimensions are
+ * K, K, N; the reference's kernels ignore them as well and its caller passes nullptr, ref_bind.cu:413).
+ * A kernel registered with the sequential or the multi-stream policy (mxmoe_kernel_policy) runs the same problem list as one launch
+ * per run of consecutive problems of equal format, on `stream` or on up to 4 library-owned side streams that fork from and join
+ * `stream` (the reference's ablation launchers, kernel_sketch.py:148-274, 277-406); kernel_id = -1 only ever selects a fused kernel.
  *
  *   format            As[p]                      Bs[p]                               scale_a[p]      scale_b[p]
  *   fp16              fp16 [M,K]                 fp16 [N,K]                          -               -
@@ -58,12 +62,28 @@ int mxmoe_kernel_branch(int kernel_id, int branch, int32_t out[8]);
  * receive the raw accumulators (int32 for w8a8 / w4a4 per channel, fp32 bit patterns otherwise: for w4a4_g128 the fp32 sum over the
  * groups of float(group's int32 sum) * (scale_a * scale_b), groups in ascending order); used by the parity tests.
  * Errors: 1 "quant type not supported" (same text as the reference launcher, compose_kernel.py:433), 2 bad kernel id,
- * 3 unsupported shape (K not a multiple of the tile's K step, N not a multiple of 8), 4 launch failure, 5 a required array is NULL
+ * 3 unsupported shape (K not a multiple of the tile's K step, N not a multiple of 8) or Ds differs from Cs, 4 launch failure, 5 a required array is NULL
  * (the scale arrays are required as soon as one non-empty problem is quantised). */
 int mxmoe_group_gemm(int kernel_id, const void* const* As, const void* const* Bs, const void* const* scale_a, const void* const* scale_b,
                      void* const* Cs, void* const* Ds, const int64_t* lda, const int64_t* ldb, const int64_t* ldc, const int64_t* ldd,
                      const mxmoe_dim3* d_sizes, const mxmoe_dim3* h_sizes, const mxmoe_qparams* d_q, const mxmoe_qparams* h_q, int problem_count,
                      int32_t* const* acc_dump, void* stream);
+
+/* ---- the kernels as functions of the reference's own type: replaces KernelRegistry::Kernel::func and the registry loop of
+ *      mxmoe/kernels/src/test.cu:793-815 (FuncType, mxmoe/kernels/src/include/registry.cuh:28-39,72-107) ----
+ *
+ * mxmoe_kernel_func(i) / mxmoe_get_kernel(name) return kernel i (the kernel whose registry name equals or ends with `name`) as a
+ * function taking exactly FuncType's 15 arguments, or NULL.  Such a call launches on the stream last given to mxmoe_set_stream by
+ * the calling thread (initially the default stream, where the reference launches, kernel_sketch.py:123).  FuncType returns void:
+ * a failing call prints its message to stderr (the reference's launcher does the same and then exits, helper.h:186-193; here the
+ * process lives on) and mxmoe_last_status() returns the code of the calling thread's last FuncType call (0 = launched).
+ * mxmoe_kernel_policy: 0 fused, 1 sequential, 2 multi-stream (-1 bad id). */
+mxmoe_func_t mxmoe_kernel_func(int kernel_id);
+mxmoe_func_t mxmoe_get_kernel(const char* name);
+int mxmoe_kernel_policy(int kernel_id);
+void mxmoe_set_stream(void* stream);
+void* mxmoe_get_stream(void);
+int mxmoe_last_status(void);
 
 /* Tile count and branch choice the launcher would make, without launching.  The launcher runs the rows of a problem as at
  * most two segments (whole tiles of the largest shape, then the remainder with the cheapest shape that covers it):

@@ -32,6 +32,12 @@ SIGNATURES = {
     "mxmoe_quant_act": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P]),
     "mxmoe_silu_mul_quant": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P]),
     "mxmoe_group_gemm_plan": (_I, [_I, C.POINTER(Dim3), C.POINTER(QParams), _I, C.POINTER(C.c_int32), C.POINTER(C.c_int32)]),
+    "mxmoe_kernel_func": (_P, [_I]),
+    "mxmoe_get_kernel": (_P, [C.c_char_p]),
+    "mxmoe_kernel_policy": (_I, [_I]),
+    "mxmoe_set_stream": (None, [_P]),
+    "mxmoe_get_stream": (_P, []),
+    "mxmoe_last_status": (_I, []),
     "mxmoe_combine_workspace_bytes": (C.c_size_t, [_I, _I]),
     "mxmoe_unpermute_combine": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P]),
 }
@@ -40,16 +46,22 @@ _cached = {}
 
 
 GEMM_ONLY = ("mxmoe_last_error", "mxmoe_num_kernels", "mxmoe_kernel_name", "mxmoe_find_kernel", "mxmoe_kernel_num_branches", "mxmoe_kernel_branch",
-             "mxmoe_group_gemm", "mxmoe_group_gemm_plan")
+             "mxmoe_group_gemm", "mxmoe_group_gemm_plan", "mxmoe_kernel_func", "mxmoe_get_kernel", "mxmoe_kernel_policy", "mxmoe_set_stream", "mxmoe_get_stream",
+             "mxmoe_last_status")
+
+# the reference's FuncType (registry.cuh:28-39): 15 arguments, no return value
+FUNC_TYPE = C.CFUNCTYPE(None, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, C.POINTER(Dim3), _P, C.POINTER(QParams), _I)
 
 
 def load(path: str | Path | None = None) -> C.CDLL:
     """Load the library and attach the C-ABI signatures.  A generated library (`path` given) carries the GroupGEMM entry
     points only; the default library must export everything the header declares."""
     p = Path(path) if path is not None else LIB_PATH
-    key = str(p)
-    if key in _cached:
-        return _cached[key]
+    if p.exists():  # a library rebuilt under the same name (a generated one, per format set) is a different library
+        st = p.stat()
+        key = (str(p), st.st_mtime_ns, st.st_ino)
+        if key in _cached:
+            return _cached[key]
     if not p.exists():
         raise RuntimeError(
             f"{p} is missing: build it with `python -m mxmoe_amd.build` (hipcc, gfx950). "

@@ -159,10 +159,36 @@ def hipcc_build(sources, out: Path, extra=(), verbose: bool = False, jobs: int =
 
 
 def build_default(verbose: bool = False) -> Path:
-    """Compile every .hip translation unit of the package into libmxmoe_amd.so."""
-    sources = sorted(CSRC.glob("*.hip"))
+    """Compile every .hip translation unit of the package, and the generator's registration unit of the default kernels, into
+    libmxmoe_amd.so."""
+    from .kernels.compose_kernel import emit_default_library
+
+    sources = sorted(CSRC.glob("*.hip")) + [emit_default_library()]
     return hipcc_build(sources, LIB, verbose=verbose)
+
+
+def sample_generator():
+    """The generator run whose library ships prebuilt next to the default one: {w4a4, w8a8} with two shapes per format as
+    one-tile-per-format combinations (4 kernels) plus one kernel carrying both formats' shape sets.  The GPU tests load it, so
+    the flow generator -> hipcc -> registry -> launch is exercised without compiling on the GPU machine."""
+    from .kernels.compose_kernel import GEN_DIR, KernelType, TemplateGenerator
+    from .kernels.tile_config import get_possible_tile_list
+
+    tiles = {q: [t for t in get_possible_tile_list("gfx950", q) if t.BM in (128, 32)] for q in ("w4a4_g-1_sym", "w8a8_g-1_sym")}
+    for q in tiles:
+        tiles[q] = tiles[q] + [tuple(tiles[q])]
+    gen = TemplateGenerator("gfx950", list(tiles), KernelType.Fused, tiles, out_dir=GEN_DIR / "sample_w4a4_w8a8")
+    combos = [c for c in gen.get_tile_configs() if sum(isinstance(t, tuple) for t in c.values()) in (0, len(c))]
+    gen.get_tile_configs = lambda: combos
+    return gen
+
+
+def build_generated_sample(verbose: bool = False) -> Path:
+    gen = sample_generator()
+    gen.generate_source_code()
+    return gen.build()
 
 
 if __name__ == "__main__":
     print(build_default(verbose=True))
+    print(build_generated_sample(verbose=True))

@@ -44,13 +44,31 @@ int mxmoe_group_gemm(int kernel_id, const void* const* As, const void* const* Bs
                      void* const* Cs, void* const* Ds, const int64_t* lda, const int64_t* ldb, const int64_t* ldc, const int64_t* ldd,
                      const mxmoe_dim3* d_sizes, const mxmoe_dim3* h_sizes, const mxmoe_qparams* d_q, const mxmoe_qparams* h_q, int problem_count,
                      int32_t* const* acc_dump, void* stream) {
-  (void)Ds; (void)lda; (void)ldb; (void)ldc; (void)ldd; (void)d_q;
-  if (problem_count < 0 || (problem_count > 0 && (!As || !Bs || !Cs || !d_sizes || !h_sizes || !h_q))) {
-    last_error() = "null argument";
-    return 5;
-  }
-  return group_gemm(kernel_id, As, Bs, scale_a, scale_b, Cs, acc_dump, d_sizes, h_sizes, h_q, problem_count, (hipStream_t)stream);
+  // lda..ldd and d_q are device arrays the kernels never read (as in the reference, whose callers pass nullptr, ref_bind.cu:413):
+  // leading dimensions are K, K, N
+  (void)lda; (void)ldb; (void)ldc; (void)ldd; (void)d_q;
+  return checked_group_gemm(kernel_id, As, Bs, scale_a, scale_b, Cs, Ds, acc_dump, d_sizes, h_sizes, h_q, problem_count, (hipStream_t)stream);
 }
+
+mxmoe_func_t mxmoe_kernel_func(int kernel_id) {
+  if (kernel_id < 0 || kernel_id >= (int)registry().size()) { last_error() = "kernel id out of range"; return nullptr; }
+  return registry()[kernel_id].func;
+}
+
+mxmoe_func_t mxmoe_get_kernel(const char* name) {
+  const int id = mxmoe_find_kernel(name);
+  if (id < 0) { last_error() = std::string("no kernel named ") + (name ? name : "(null)"); return nullptr; }
+  return registry()[id].func;
+}
+
+int mxmoe_kernel_policy(int kernel_id) {
+  if (kernel_id < 0 || kernel_id >= (int)registry().size()) return -1;
+  return (int)registry()[kernel_id].policy;
+}
+
+void mxmoe_set_stream(void* stream) { func_stream() = (hipStream_t)stream; }
+void* mxmoe_get_stream(void) { return (void*)func_stream(); }
+int mxmoe_last_status(void) { return func_status(); }
 
 int mxmoe_group_gemm_plan(int kernel_id, const mxmoe_dim3* h_sizes, const mxmoe_qparams* h_q, int problem_count, int32_t* branch_out, int32_t* tiles_out) {
   auto& reg = registry();
@@ -60,7 +78,7 @@ int mxmoe_group_gemm_plan(int kernel_id, const mxmoe_dim3* h_sizes, const mxmoe_
   }
   if (kernel_id < 0) {
     for (int i = 0; i < (int)reg.size() && kernel_id < 0; ++i)
-      if (kernel_covers(reg[i], h_q, problem_count)) kernel_id = i;
+      if (reg[i].policy == Policy::Fused && kernel_covers(reg[i], h_q, problem_count)) kernel_id = i;
     if (kernel_id < 0) { last_error() = "quant type not supported"; return 1; }
   }
   if (kernel_id >= (int)reg.size()) { last_error() = "kernel id out of range"; return 2; }

@@ -218,11 +218,20 @@ struct BranchOf<SkinnyWoTile<WBITS, BN>> {
 
 using LaunchFn = hipError_t (*)(const FusedArgs&, int grid, int lds, hipStream_t);
 
+// How a registered kernel walks a problem list (the reference generates one host launcher per policy, kernel_sketch.py:82-145
+// fused, :148-274 sequential, :277-406 multi-stream):
+//   Fused       one launch over all problems;
+//   Sequential  one launch per run of consecutive problems of equal format, all on the caller's stream;
+//   MultiStream the same launches dealt round-robin to side streams that fork from and join the caller's stream.
+enum class Policy { Fused = 0, Sequential = 1, MultiStream = 2 };
+
 struct FusedKernel {
   std::string name;  // "[qcfg: (BM,BN,BK) (WGM,WGN,1) 2], ...<fn name>" — same shape as registry.cuh:42-70
   std::vector<BranchInfo> branches;
   int lds_bytes;
   LaunchFn launch;
+  Policy policy;
+  mxmoe_func_t func;  // the kernel as a function of the reference's FuncType (registry.cuh:28-39)
 };
 
 inline std::vector<FusedKernel>& registry() {
@@ -260,9 +269,53 @@ hipError_t launch_fused(const FusedArgs& a, int grid, int lds, hipStream_t s) {
   return hipGetLastError();
 }
 
+inline int group_gemm(int kernel_id, const void* const* As, const void* const* Bs, const void* const* sa, const void* const* sb, void* const* Cs,
+                      int32_t* const* acc, const mxmoe_dim3* d_sizes, const mxmoe_dim3* h_sizes, const mxmoe_qparams* h_q, int count, hipStream_t stream);
+
+// Stream the FuncType functions launch on (that type has no stream argument; the reference launches on stream 0,
+// kernel_sketch.py:123), and the status of the calling thread's last FuncType call (that type returns void).
+inline hipStream_t& func_stream() {
+  static thread_local hipStream_t s = nullptr;
+  return s;
+}
+inline int& func_status() {
+  static thread_local int rc = 0;
+  return rc;
+}
+
+inline int checked_group_gemm(int kernel_id, const void* const* As, const void* const* Bs, const void* const* sa, const void* const* sb, void* const* Cs,
+                              void* const* Ds, int32_t* const* acc, const mxmoe_dim3* d_sizes, const mxmoe_dim3* h_sizes, const mxmoe_qparams* h_q, int count,
+                              hipStream_t stream) {
+  if (count < 0 || (count > 0 && (!As || !Bs || !Cs || !d_sizes || !h_sizes || !h_q))) {
+    last_error() = "null argument";
+    return 5;
+  }
+  if (Ds && Ds != Cs) {  // the kernels write Cs only: a caller that expects its results in a different Ds would read stale memory
+    last_error() = "Ds must be the same array as Cs (or NULL)";
+    return 3;
+  }
+  return group_gemm(kernel_id, As, Bs, sa, sb, Cs, acc, d_sizes, h_sizes, h_q, count, stream);
+}
+
+// One C function of the reference's FuncType per registered kernel: the template instance is the function, its static member the
+// registry index it launches.  A failure is reported like the reference's launcher reports CUDA errors (message on stderr,
+// helper.h:186-193) but the process is left alive; mxmoe_last_status() returns the code.
+template <int POLICY, class... Tiles>
+struct FuncThunk {
+  static inline int kernel_id = -1;
+  static void call(mxmoe_half** As, mxmoe_half** Bs, mxmoe_half** sa, mxmoe_half** sb, mxmoe_half** Cs, mxmoe_half** Ds, int64_t*, int64_t*, int64_t*, int64_t*,
+                   mxmoe_dim3* d_sizes, mxmoe_dim3* h_sizes, mxmoe_qparams*, mxmoe_qparams* h_q, int problem_count) {
+    const int rc = checked_group_gemm(kernel_id, (const void* const*)As, (const void* const*)Bs, (const void* const*)sa, (const void* const*)sb, (void* const*)Cs,
+                                      (void* const*)Ds, nullptr, d_sizes, h_sizes, h_q, problem_count, func_stream());
+    func_status() = rc;
+    if (rc != 0) fprintf(stderr, "mxmoe: %s\n", last_error().c_str());
+  }
+};
+
 template <class... Tiles>
-int register_fused(const char* fn_name) {
+int register_fused(const char* fn_name, Policy policy = Policy::Fused) {
   FusedKernel k;
+  k.policy = policy;
   k.branches = {BranchOf<Tiles>::get()...};
   k.lds_bytes = 0;
   std::string n;
@@ -274,8 +327,14 @@ int register_fused(const char* fn_name) {
   }
   k.name = n + fn_name;
   k.launch = &launch_fused<Tiles...>;
+  const int id = (int)registry().size();
+  switch (policy) {
+    case Policy::Fused: FuncThunk<0, Tiles...>::kernel_id = id; k.func = &FuncThunk<0, Tiles...>::call; break;
+    case Policy::Sequential: FuncThunk<1, Tiles...>::kernel_id = id; k.func = &FuncThunk<1, Tiles...>::call; break;
+    default: FuncThunk<2, Tiles...>::kernel_id = id; k.func = &FuncThunk<2, Tiles...>::call; break;
+  }
   registry().push_back(k);
-  return (int)registry().size() - 1;
+  return id;
 }
 
 // Run time of one tile of a branch relative to the 128 x 256 tile of the same format (same K), from the kernel-profile table
@@ -374,6 +433,107 @@ inline bool kernel_covers(const FusedKernel& k, const mxmoe_qparams* q, int coun
   return true;
 }
 
+// One launch over problems [base, base + n) of the caller's arrays with kernel `k` (n <= kMaxProblems).
+inline int launch_range(const FusedKernel& k, const void* const* As, const void* const* Bs, const void* const* sa, const void* const* sb, void* const* Cs,
+                        int32_t* const* acc, const mxmoe_dim3* d_sizes, const mxmoe_dim3* h_sizes, const mxmoe_qparams* h_q, int base, int n, hipStream_t stream) {
+  FusedArgs a;
+  std::memset(&a, 0, sizeof a);
+  a.As = reinterpret_cast<const uint8_t* const*>(As);
+  a.Bs = reinterpret_cast<const uint8_t* const*>(Bs);
+  a.sa = reinterpret_cast<const _Float16* const*>(sa);
+  a.sb = reinterpret_cast<const _Float16* const*>(sb);
+  a.Cs = reinterpret_cast<_Float16* const*>(Cs);
+  a.acc = acc;
+  a.sizes = d_sizes;
+  a.problem_offset = base;
+  struct Entry {
+    int row0, rows, problem, branch, tiles;
+  };
+  Entry entries[kMaxEntries];
+  int nent = 0;
+  for (int i = 0; i < n; ++i) {
+    const mxmoe_dim3& sz = h_sizes[base + i];
+    const Fmt f = classify(h_q[base + i]);
+    Segment sg[2];
+    const int ns = f == Fmt::UNSUPPORTED ? -1 : plan_segments(k, f, (int)sz.x, (int)sz.y, sg);
+    if (ns < 0) {
+      last_error() = "quant type not supported";
+      return 1;
+    }
+    for (int j = 0; j < ns; ++j) {
+      const BranchInfo& bi = k.branches[sg[j].branch];
+      if (sz.z == 0 || sz.z % bi.k_multiple != 0 || sz.y % 8 != 0 || (bi.fmt != Fmt::FP16 && bi.fmt != Fmt::W8A8 && bi.fmt != Fmt::W4A4 && bi.fmt != Fmt::W4A4G128 && sz.y % 16 != 0)) {
+        char buf[200];
+        snprintf(buf, sizeof buf, "problem %d: shape [%u,%u,%u] not supported by tile %s (K %% %d, N %% 8)", base + i, sz.x, sz.y, sz.z, fmt_name(bi.fmt, true), bi.k_multiple);
+        last_error() = buf;
+        return 3;
+      }
+      entries[nent++] = Entry{sg[j].row0, sg[j].rows, i, sg[j].branch, ((sg[j].rows + bi.BM - 1) / bi.BM) * (int)((sz.y + bi.BN - 1) / bi.BN)};
+    }
+  }
+  // most expensive tile shape first; problems keep their order inside a shape (neighbouring tiles share operands)
+  constexpr int kMaxBranches = 32;
+  int order[kMaxBranches];
+  const int nb = std::min((int)k.branches.size(), kMaxBranches);
+  for (int b = 0; b < nb; ++b) order[b] = b;
+  std::stable_sort(order, order + nb, [&](int x, int y) { return branch_cost(k.branches[x]) > branch_cost(k.branches[y]); });
+  int total = 0, ne = 0, wg = 0, np = 0;
+  for (int oi = 0; oi < nb; ++oi) {
+    const int b = order[oi];
+    const int tile0 = total;
+    for (int ei = 0; ei < nent; ++ei) {
+      const Entry& en = entries[ei];
+      if (en.branch != b || en.tiles == 0) continue;
+      a.entry[ne] = FusedArgs::Entry{total, en.row0, en.rows, en.problem | (en.branch << 16)};
+      total += en.tiles;
+      ++ne;
+    }
+    if (total == tile0) continue;
+    // shapes beyond the phase table share the last phase (their relative order is kept)
+    if (np < kMaxPhases) {
+      a.phase_tile0[np] = tile0;
+      a.phase_wg0[np] = wg;
+      ++np;
+    }
+    const int p0 = a.phase_tile0[np - 1];
+    wg = a.phase_wg0[np - 1] + (total - p0 + kNumXcd - 1) / kNumXcd * kNumXcd;
+  }
+  a.num_entries = ne;
+  if (total == 0) return 0;
+  a.total_tiles = total;
+  a.num_phases = np;
+  a.phase_tile0[np] = total;
+  a.phase_wg0[np] = wg;
+  const hipError_t e = k.launch(a, wg, k.lds_bytes, stream);
+  if (e != hipSuccess) {
+    last_error() = std::string("kernel launch failed: ") + hipGetErrorString(e);
+    return 4;
+  }
+  return 0;
+}
+
+// Side streams of the multi-stream policy, created on first use per device (default priority, non-blocking) and kept for the
+// life of the process, with the events that fork them from and join them to the caller's stream.
+constexpr int kSideStreams = 4;
+struct SideStreams {
+  hipStream_t stream[kSideStreams];
+  hipEvent_t fork, join[kSideStreams];
+  bool ready;
+};
+inline SideStreams* side_streams() {
+  static SideStreams pool[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+  SideStreams& p = pool[dev];
+  if (!p.ready) {
+    if (hipEventCreateWithFlags(&p.fork, hipEventDisableTiming) != hipSuccess) return nullptr;
+    for (int i = 0; i < kSideStreams; ++i)
+      if (hipStreamCreateWithFlags(&p.stream[i], hipStreamNonBlocking) != hipSuccess || hipEventCreateWithFlags(&p.join[i], hipEventDisableTiming) != hipSuccess) return nullptr;
+    p.ready = true;
+  }
+  return &p;
+}
+
 // Host launcher.  Array arguments as in the reference FuncType (registry.cuh:28-39): every pointer array and
 // d_sizes / d_q live in device memory, h_sizes / h_q are their host mirrors.  ld* and d_q are accepted and unused.
 inline int group_gemm(int kernel_id, const void* const* As, const void* const* Bs, const void* const* sa, const void* const* sb, void* const* Cs,
@@ -382,7 +542,7 @@ inline int group_gemm(int kernel_id, const void* const* As, const void* const* B
   auto& reg = registry();
   if (kernel_id < 0) {
     for (int i = 0; i < (int)reg.size() && kernel_id < 0; ++i)
-      if (kernel_covers(reg[i], h_q, count)) kernel_id = i;
+      if (reg[i].policy == Policy::Fused && kernel_covers(reg[i], h_q, count)) kernel_id = i;
     if (kernel_id < 0) {
       last_error() = "quant type not supported";  // same message as the reference launcher (compose_kernel.py:433)
       return 1;
@@ -402,83 +562,45 @@ inline int group_gemm(int kernel_id, const void* const* As, const void* const* B
       return 5;
     }
   }
-  for (int base = 0; base < count; base += kMaxProblems) {
-    const int n = std::min(kMaxProblems, count - base);
-    FusedArgs a;
-    std::memset(&a, 0, sizeof a);
-    a.As = reinterpret_cast<const uint8_t* const*>(As);
-    a.Bs = reinterpret_cast<const uint8_t* const*>(Bs);
-    a.sa = reinterpret_cast<const _Float16* const*>(sa);
-    a.sb = reinterpret_cast<const _Float16* const*>(sb);
-    a.Cs = reinterpret_cast<_Float16* const*>(Cs);
-    a.acc = acc;
-    a.sizes = d_sizes;
-    a.problem_offset = base;
-    struct Entry {
-      int row0, rows, problem, branch, tiles;
-    };
-    Entry entries[kMaxEntries];
-    int nent = 0;
-    for (int i = 0; i < n; ++i) {
-      const mxmoe_dim3& sz = h_sizes[base + i];
-      const Fmt f = classify(h_q[base + i]);
-      Segment sg[2];
-      const int ns = f == Fmt::UNSUPPORTED ? -1 : plan_segments(k, f, (int)sz.x, (int)sz.y, sg);
-      if (ns < 0) {
-        last_error() = "quant type not supported";
-        return 1;
-      }
-      for (int j = 0; j < ns; ++j) {
-        const BranchInfo& bi = k.branches[sg[j].branch];
-        if (sz.z == 0 || sz.z % bi.k_multiple != 0 || sz.y % 8 != 0 || (bi.fmt != Fmt::FP16 && bi.fmt != Fmt::W8A8 && bi.fmt != Fmt::W4A4 && bi.fmt != Fmt::W4A4G128 && sz.y % 16 != 0)) {
-          char buf[200];
-          snprintf(buf, sizeof buf, "problem %d: shape [%u,%u,%u] not supported by tile %s (K %% %d, N %% 8)", base + i, sz.x, sz.y, sz.z, fmt_name(bi.fmt, true), bi.k_multiple);
-          last_error() = buf;
-          return 3;
-        }
-        entries[nent++] = Entry{sg[j].row0, sg[j].rows, i, sg[j].branch, ((sg[j].rows + bi.BM - 1) / bi.BM) * (int)((sz.y + bi.BN - 1) / bi.BN)};
-      }
-    }
-    // most expensive tile shape first; problems keep their order inside a shape (neighbouring tiles share operands)
-    constexpr int kMaxBranches = 32;
-    int order[kMaxBranches];
-    const int nb = std::min((int)k.branches.size(), kMaxBranches);
-    for (int b = 0; b < nb; ++b) order[b] = b;
-    std::stable_sort(order, order + nb, [&](int x, int y) { return branch_cost(k.branches[x]) > branch_cost(k.branches[y]); });
-    int total = 0, ne = 0, wg = 0, np = 0;
-    for (int oi = 0; oi < nb; ++oi) {
-      const int b = order[oi];
-      const int tile0 = total;
-      for (int ei = 0; ei < nent; ++ei) {
-        const Entry& en = entries[ei];
-        if (en.branch != b || en.tiles == 0) continue;
-        a.entry[ne] = FusedArgs::Entry{total, en.row0, en.rows, en.problem | (en.branch << 16)};
-        total += en.tiles;
-        ++ne;
-      }
-      if (total == tile0) continue;
-      // shapes beyond the phase table share the last phase (their relative order is kept)
-      if (np < kMaxPhases) {
-        a.phase_tile0[np] = tile0;
-        a.phase_wg0[np] = wg;
-        ++np;
-      }
-      const int p0 = a.phase_tile0[np - 1];
-      wg = a.phase_wg0[np - 1] + (total - p0 + kNumXcd - 1) / kNumXcd * kNumXcd;
-    }
-    a.num_entries = ne;
-    if (total == 0) continue;
-    a.total_tiles = total;
-    a.num_phases = np;
-    a.phase_tile0[np] = total;
-    a.phase_wg0[np] = wg;
-    const hipError_t e = k.launch(a, wg, k.lds_bytes, stream);
-    if (e != hipSuccess) {
-      last_error() = std::string("kernel launch failed: ") + hipGetErrorString(e);
+  auto run = [&](int base, int n, hipStream_t s) { return launch_range(k, As, Bs, sa, sb, Cs, acc, d_sizes, h_sizes, h_q, base, n, s); };
+  if (k.policy == Policy::Fused) {
+    for (int base = 0; base < count; base += kMaxProblems)
+      if (const int rc = run(base, std::min(kMaxProblems, count - base), stream)) return rc;
+    return 0;
+  }
+  // runs of consecutive problems of equal format (kernel_sketch.py:192-246 compares the QParams of neighbours the same way)
+  auto same = [&](int x, int y) { return h_q[x].a_bits == h_q[y].a_bits && h_q[x].w_bits == h_q[y].w_bits && h_q[x].gsize == h_q[y].gsize && h_q[x].sym == h_q[y].sym; };
+  SideStreams* side = nullptr;
+  if (k.policy == Policy::MultiStream) {
+    side = side_streams();
+    if (!side || hipEventRecord(side->fork, stream) != hipSuccess) {
+      last_error() = "could not set up the side streams of the multi-stream policy";
       return 4;
     }
   }
-  return 0;
+  int nrun = 0, rc = 0;
+  unsigned used = 0;
+  for (int base = 0; base < count && rc == 0;) {
+    int n = 1;
+    while (base + n < count && n < kMaxProblems && same(base, base + n)) ++n;
+    hipStream_t s = stream;
+    if (side) {
+      const int si = nrun % kSideStreams;
+      s = side->stream[si];
+      if (!(used >> si & 1) && hipStreamWaitEvent(s, side->fork, 0) != hipSuccess) rc = 4;
+      used |= 1u << si;
+    }
+    if (rc == 0) rc = run(base, n, s);
+    base += n;
+    ++nrun;
+  }
+  if (side) {  // join whatever was forked, also after a failure, so that the caller's stream stays ordered after the side work
+    for (int si = 0; si < kSideStreams; ++si)
+      if (used >> si & 1)
+        if (hipEventRecord(side->join[si], side->stream[si]) != hipSuccess || hipStreamWaitEvent(stream, side->join[si], 0) != hipSuccess) rc = rc ? rc : 4;
+    if (rc == 4 && last_error().empty()) last_error() = "stream fork / join failed";
+  }
+  return rc;
 }
 
 }  // namespace mxmoe

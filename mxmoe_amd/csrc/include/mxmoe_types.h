@@ -22,6 +22,15 @@ typedef struct mxmoe_qparams {
   uint8_t _pad[3];
 } mxmoe_qparams;
 
+// fp16 storage as the C-ABI names it (the reference's `half`); only ever used behind pointers.
+typedef uint16_t mxmoe_half;
+
+// The reference's kernel function type (`FuncType`, mxmoe/kernels/src/include/registry.cuh:28-39) with this library's plain-C
+// stand-ins for half, dim3 and QParams (same sizes and layouts, so a caller may cast between the two pointer types).
+typedef void (*mxmoe_func_t)(mxmoe_half** ptr_As, mxmoe_half** ptr_Bs, mxmoe_half** ptr_scale_a, mxmoe_half** ptr_scale_b, mxmoe_half** ptr_Cs, mxmoe_half** ptr_Ds,
+                             int64_t* ldas, int64_t* ldbs, int64_t* ldcs, int64_t* ldds, mxmoe_dim3* device_problem_sizes, mxmoe_dim3* host_problem_sizes,
+                             mxmoe_qparams* device_qbits_list, mxmoe_qparams* host_qbits_list, int problem_count);
+
 #ifdef __cplusplus
 }
 #endif

@@ -6,8 +6,9 @@ Per (layer, "gate_up" | "down") problem list: fp16 operands ~ U(-1, 1) (seed 42)
 every registered fused kernel that covers the formats is timed (<= 30 warm-up, <= 50 timed launches, HIP events, median)
 and reported as `kernel_name, avg_time (ms), TFLOPS, speedup` against the best fp16 grouped GEMM of the same shapes (the
 reference's CUTLASS baseline; here the fp16 MFMA kernel), written to `<output>-<layer>-<gate_up|down>.csv`.
-Sequential and multi-stream launches (one launch per contiguous run of equal-format problems, on one stream or one
-stream per run — the reference's ablation launchers, kernel_sketch.py:148-406) are timed next to the fused launch.
+Sequential and multi-stream launches (one launch per contiguous run of equal-format problems, on one stream or dealt to
+side streams — the reference's ablation launchers, kernel_sketch.py:148-406, here policies of the C++ host launcher) are
+timed next to the fused launch.
 """
 from __future__ import annotations
 
@@ -91,6 +92,26 @@ def _runs_of_equal_format(probs):
     return runs
 
 
+POLICY_KERNEL = {"seq": b"groupgemm_seq_launch_all", "ms": b"groupgemm_ms_launch_all"}
+
+
+def launch_policy(probs, policy: str, lib=None):
+    """A callable that runs the problem list once under `policy`: "fused" (one launch, the library's first kernel that covers the
+    formats), "seq" or "ms" (the default library's sequential / multi-stream launchers, the reference's ablation baselines
+    kernel_sketch.py:148-406: one launch per run of consecutive equal-format problems, on the current stream or on the
+    library's side streams)."""
+    if policy == "fused":
+        g = _launch_of(probs, lib or _lib.load())
+    else:
+        lib = _lib.load()
+        kid = lib.mxmoe_find_kernel(POLICY_KERNEL[policy])
+        if kid < 0 or lib.mxmoe_kernel_policy(kid) != {"seq": 1, "ms": 2}[policy]:
+            raise RuntimeError(f"the library has no {policy} launcher")
+        g = _launch_of(probs, lib, kid)
+    g.plan()
+    return g.run
+
+
 def tflops(probs, ms: float) -> float:
     return sum(2 * m * n * k for (m, n, k) in (p["size"] for p in probs)) / (ms * 1e-3) / 1e12
 
@@ -141,32 +162,14 @@ def bench_one_case(entries, lib=None, mode: str = "bench", filters=(), out_file:
 
     if rows:
         results["mxmoe-hz"] = min(rows)
-    # ablation launch policies with the best kernel library-wide: one launch per contiguous run of equal-format problems
-    runs = [_launch_of(r, lib) for r in _runs_of_equal_format(probs)]
-    try:
-        for r in runs:
-            r.plan()
-
-        def seq():
-            for r in runs:
-                r.run()
-
-        ms = bench_func(seq)["median"]
-        results["mxmoe-seq"] = (ms, tflops(probs, ms), f"seq_launch x{len(runs)}")
-        streams = [torch.cuda.Stream() for _ in runs]
-
-        def multi():
-            cur = torch.cuda.current_stream()
-            for s, r in zip(streams, runs):
-                s.wait_stream(cur)
-                r.run(stream=s.cuda_stream)
-            for s in streams:
-                cur.wait_stream(s)
-
-        ms = bench_func(multi)["median"]
-        results["mxmoe-ms"] = (ms, tflops(probs, ms), f"ms_launch x{len(runs)}")
-    except RuntimeError:
-        pass
+    # ablation launch policies (the library's sequential and multi-stream launchers over the same tiles)
+    for impl, policy in (("mxmoe-seq", "seq"), ("mxmoe-ms", "ms")):
+        try:
+            run = launch_policy(probs, policy)
+        except RuntimeError:
+            continue  # a format outside the every-format kernel
+        ms = bench_func(run)["median"]
+        results[impl] = (ms, tflops(probs, ms), f"{policy}_launch x{len(_runs_of_equal_format(probs))}")
 
     base_tf = results["fp16-baseline"][1]
     for impl, (ms, tf, name) in results.items():

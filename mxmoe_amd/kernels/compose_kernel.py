@@ -6,8 +6,14 @@ emits `generated/hz_fused_decl.hpp` + one `generated/hz_fused_<i>.hip` per fusio
 qcfg (cartesian product filtered by equal wavefront count, compose_kernel.py:87-108), each registering
 `groupgemm_hz_fused_<i>`.  `build()` then replaces the reference's cmake + ninja step (run_mxmoe_gg.py:109-111).
 
-`KernelType.Sequential` / `MultiStream` (the reference's ablation launchers, kernel_sketch.py:148-406) emit one
-single-format kernel per qcfg; the launch policy for them lives in mxmoe_amd.harness.
+A qcfg's entry in `tile_configs` may also be a tuple of TileConfig (a *shape set*): the kernel then carries every shape of
+the set as a branch of that format and its host launcher picks the shapes per problem from the row count (whole tiles of the
+cheapest shape per row, the remainder with the shape that covers it most cheaply).  The kernels of the default library
+(`default_kernel_specs`) are such sets; `emit_default_library` writes their translation unit, which the package build compiles.
+
+`KernelType.Sequential` / `MultiStream` (the reference's ablation launchers, kernel_sketch.py:148-406) emit the same
+combinations registered with the sequential / multi-stream launch policy of the C++ host launcher: one launch per run of
+consecutive problems of equal format, on the caller's stream or on side streams.
 """
 from __future__ import annotations
 
@@ -42,8 +48,20 @@ BRANCH_CONDITION_MAP = {"fp16": "(a_bits == 16 && w_bits == 16)", **{k: _gen_con
 GEN_DIR = Path(__file__).resolve().parent.parent / "csrc" / "generated"
 
 
+POLICY = {"hz_fused": "Policy::Fused", "seq_launch": "Policy::Sequential", "ms_launch": "Policy::MultiStream"}
+
+
+def _flat(items):
+    """Tiles of a combination, shape sets expanded."""
+    out = []
+    for it in items:
+        out += list(it) if isinstance(it, (tuple, list)) else [it]
+    return out
+
+
 def is_fusion_compatible(tile_cfgs) -> bool:
-    return all(tile_cfgs[0].num_warps == c.num_warps for c in tile_cfgs)
+    tiles = _flat(tile_cfgs)
+    return all(tiles[0].num_warps == c.num_warps for c in tiles)
 
 
 class TemplateGenerator:
@@ -64,27 +82,21 @@ class TemplateGenerator:
         else:
             per_q = OrderedDict((q, get_possible_tile_list(self.arch, q)) for q in self.qcfgs)
         for tiles in per_q.values():
-            for t in tiles:
+            for t in _flat(tiles):
                 t.validate()
-        if self.kernel_type == KernelType.Fused:
-            combos = [c for c in product(*per_q.values()) if is_fusion_compatible(c)]
-            return [OrderedDict(zip(per_q.keys(), c)) for c in combos]
-        # one single-format kernel per (qcfg, tile)
-        return [OrderedDict([(q, t)]) for q, tiles in per_q.items() for t in tiles]
+        combos = [c for c in product(*per_q.values()) if is_fusion_compatible(c)]
+        return [OrderedDict(zip(per_q.keys(), c)) for c in combos]
 
     def get_smem_size(self, tile_cfg_dict) -> tuple:
-        return max(t.smem_bytes_tile() for t in tile_cfg_dict.values()), max(t.smem_bytes_scale() for t in tile_cfg_dict.values())
+        tiles = _flat(tile_cfg_dict.values())
+        return max(t.smem_bytes_tile() for t in tiles), max(t.smem_bytes_scale() for t in tiles)
 
     def cvt_qcfg_str_to_condition(self, qcfg: str) -> str:
         assert qcfg in self.qcfgs, f"Invalid qcfg: {qcfg}"
         return BRANCH_CONDITION_MAP[qcfg]
 
     def build_single_kernel(self, tile_cfg: OrderedDict, kname: str):
-        tiles = ", ".join(t.cpp_type() for t in tile_cfg.values())
-        comment = "; ".join(f"{q} if {BRANCH_CONDITION_MAP[q]} -> {t.to_str()}" for q, t in tile_cfg.items())
-        defn = KERNEL_DEFINITION_TEMPLATE.substitute(KernelName=kname, Tiles=tiles, Comment=comment)
-        decl = f"//   {kname}: " + ", ".join(f"[{q}: ({t.BM},{t.BN},{t.BK}) ({t.WM},{t.WN},{t.WK}) {t.STAGE}]" for q, t in tile_cfg.items())
-        return decl, defn
+        return build_kernel_source(tile_cfg, kname, self.kernel_type)
 
     def generate_source_code(self) -> list:
         combos = self.get_tile_configs()
@@ -114,6 +126,62 @@ class TemplateGenerator:
         """hipcc the generated translation units into one shared library exporting the C-ABI."""
         out = Path(out) if out else self.out_dir / f"libmxmoe_{self.kernel_type}.so"
         return _build.hipcc_build(self.files, out)
+
+
+def build_kernel_source(tile_cfg, kname: str, kernel_type: KernelType = KernelType.Fused):
+    """(declaration comment, translation unit) of one kernel; `tile_cfg` maps qcfg -> TileConfig or tuple of TileConfig."""
+    pairs = [(q, t) for q, item in tile_cfg.items() for t in _flat([item])]
+    tiles = ", ".join(t.cpp_type() for _, t in pairs)
+    comment = "; ".join(f"{q} if {BRANCH_CONDITION_MAP[q]} -> {t.to_str()}" for q, t in pairs)
+    defn = KERNEL_DEFINITION_TEMPLATE.substitute(KernelName=kname, Tiles=tiles, Comment=comment, Policy=POLICY[str(kernel_type)])
+    decl = f"//   {kname}: " + ", ".join(f"[{q}: ({t.BM},{t.BN},{t.BK}) ({t.WM},{t.WN},{t.WK}) {t.STAGE}]" for q, t in pairs)
+    return decl, defn
+
+
+def _pick(arch: str, qcfg: str, *shapes):
+    """Candidate tiles of `qcfg` with the given (BM, BN) shapes, in that order."""
+    by_shape = {(t.BM, t.BN): t for t in get_possible_tile_list(arch, qcfg)}
+    return tuple(by_shape[s] for s in shapes)
+
+
+def default_kernel_specs(arch: str = "gfx950"):
+    """The kernels of libmxmoe_amd.so: (function name, kernel type, {qcfg: shape set}) in registry order."""
+    w4, w8 = "w4a4_g-1_sym", "w8a8_g-1_sym"
+    wo = OrderedDict((f"w{b}a16_g128_asym", _pick(arch, f"w{b}a16_g128_asym", (16, 128))) for b in (4, 3, 2))
+    wo_big = OrderedDict((f"w{b}a16_g128_asym", _pick(arch, f"w{b}a16_g128_asym", (128, 128))) for b in (4, 3, 2))
+    wo_all = OrderedDict((q, wo[q] + wo_big[q]) for q in wo)
+    everything = OrderedDict([(w4, _pick(arch, w4, (128, 256), (32, 256))), (w8, _pick(arch, w8, (128, 256), (32, 256))),
+                              ("fp16", _pick(arch, "fp16", (128, 256), (32, 256))), *wo_all.items(), ("w4a4_g128_sym", _pick(arch, "w4a4_g128_sym", (64, 256)))])
+    return [
+        ("groupgemm_hz_fused_wxax", KernelType.Fused, OrderedDict([(w4, _pick(arch, w4, (128, 256), (64, 256), (32, 256))), (w8, _pick(arch, w8, (128, 256), (64, 256), (32, 256)))])),
+        ("groupgemm_hz_fused_fp16", KernelType.Fused, OrderedDict([("fp16", _pick(arch, "fp16", (128, 256), (64, 256), (32, 256)))])),
+        ("groupgemm_hz_fused_wo", KernelType.Fused, wo_all),
+        ("groupgemm_hz_fused_wxax_g128", KernelType.Fused, OrderedDict([("w4a4_g128_sym", _pick(arch, "w4a4_g128_sym", (64, 256), (32, 256)))])),
+        # every format in one launch (layers that mix weight-only, w-a and fp16 blocks), and the same kernel behind the two ablation policies
+        ("groupgemm_hz_fused_all", KernelType.Fused, everything),
+        ("groupgemm_seq_launch_all", KernelType.Sequential, everything),
+        ("groupgemm_ms_launch_all", KernelType.MultiStream, everything),
+    ]
+
+
+def emit_default_library(out_dir: str | os.PathLike | None = None, arch: str = "gfx950") -> Path:
+    """Write the translation unit that registers the default kernels (one file: the seven registrations share their tile
+    instantiations) and return its path."""
+    out_dir = Path(out_dir) if out_dir else GEN_DIR
+    out_dir.mkdir(parents=True, exist_ok=True)
+    body = []
+    for kname, ktype, tile_cfg in default_kernel_specs(arch):
+        for t in _flat(tile_cfg.values()):
+            t.validate()
+        if not is_fusion_compatible(list(tile_cfg.values())):
+            raise ValueError(f"{kname}: branches disagree on the wavefront count")
+        _decl, defn = build_kernel_source(tile_cfg, kname, ktype)
+        body.append(defn.replace('#include "mxmoe_launch.hpp"\n', ""))
+    path = out_dir / "default_kernels.hip"
+    text = '#include "mxmoe_launch.hpp"\n' + "".join(body)
+    if not path.exists() or path.read_text() != text:
+        path.write_text(text)
+    return path
 
 
 def main(argv=None) -> int:

@@ -99,7 +99,7 @@ def build_qcfg_lib(qcfg: str, arch: str = "gfx950", rebuild: bool = False):
     An existing library is reused unless `rebuild`, so it can be compiled on a machine without a GPU beforehand."""
     from .kernels.compose_kernel import GEN_DIR
 
-    gen = TemplateGenerator(arch, [qcfg], KernelType.Sequential, out_dir=GEN_DIR / f"perf_{qcfg}")
+    gen = TemplateGenerator(arch, [qcfg], KernelType.Fused, out_dir=GEN_DIR / f"perf_{qcfg}")  # one qcfg: one single-tile kernel per candidate
     gen.generate_source_code()
     so = gen.out_dir / f"libmxmoe_{gen.kernel_type}.so"
     if rebuild or not so.exists():

@@ -100,26 +100,27 @@ def main(argv=None) -> int:
 
     from mxmoe_amd import harness
 
+    # the kernel library depends on the format set only: generate and build it once, not per layer
+    print(f"qcfg_list: {sorted(qcfg_list)}")
+    gpu_info = get_gpu_info()
+    tile_configs = None
+    if args.tile_config is not None:
+        with open(args.tile_config) as f:
+            tile_configs = load_tile_configs(json.load(f), qcfg_list)
+    generator = TemplateGenerator(gpu_info["cc"], qcfg_list, KernelType.Fused, tile_configs)
+    if args.max_kernels:
+        combos = generator.get_tile_configs()[: args.max_kernels]
+        generator.get_tile_configs = lambda: combos
+    generator.generate_source_code()
+    lib_path = generator.build()
+
+    from mxmoe_amd import _lib
+
+    lib = _lib.load(lib_path)
+    os.makedirs(f"{CUR_DIR}/out/bench", exist_ok=True)
+    bench_save = f"{CUR_DIR}/out/bench/{model_id}-{dataset}-{bs}{workload_suffix.replace('.json', '')}"
     for lyr in layers:
         generate_workload_from_gate_trace(trace, bs, lyr, workload_path, args.qconfig, args.qstr if args.qconfig is None else None, exact_counts=exact)
-        print(f"qcfg_list: {sorted(qcfg_list)}")
-        gpu_info = get_gpu_info()
-        tile_configs = None
-        if args.tile_config is not None:
-            with open(args.tile_config) as f:
-                tile_configs = load_tile_configs(json.load(f), qcfg_list)
-        generator = TemplateGenerator(gpu_info["cc"], qcfg_list, KernelType.Fused, tile_configs)
-        if args.max_kernels:
-            combos = generator.get_tile_configs()[: args.max_kernels]
-            generator.get_tile_configs = lambda: combos
-        generator.generate_source_code()
-        lib_path = generator.build()
-
-        from mxmoe_amd import _lib
-
-        lib = _lib.load(lib_path)
-        os.makedirs(f"{CUR_DIR}/out/bench", exist_ok=True)
-        bench_save = f"{CUR_DIR}/out/bench/{model_id}-{dataset}-{bs}{workload_suffix.replace('.json', '')}"
         harness.bench_input_file(workload_path, bench_save, lib=lib, mode=args.mode)
     return 0
 

@@ -133,6 +133,46 @@ def test_missing_arrays_are_refused_before_any_launch(lib):
     assert lib.mxmoe_group_gemm_plan(-1, None, None, 1, None, None) == 5
 
 
+def test_ds_must_alias_cs(lib):
+    """Results are written to Cs only, so a caller handing over a different Ds array is refused instead of being left with
+    stale memory (the reference passes the same array twice, ref_bind.cu:413)."""
+    from mxmoe_amd import _lib
+
+    sizes = (_lib.Dim3 * 1)(_lib.Dim3(8, 256, 128))
+    q = (_lib.QParams * 1)(_lib.QParams(4, 4, -1, 1))
+    one, other = (C.c_void_p * 1)(0), (C.c_void_p * 1)(0)
+    a, b = C.addressof(one), C.addressof(other)
+    rc = lib.mxmoe_group_gemm(0, a, a, a, a, a, b, None, None, None, None, a, sizes, None, q, 1, None, None)
+    assert rc == 3 and b"Ds" in lib.mxmoe_last_error()
+
+
+def test_kernels_are_exported_with_the_reference_function_type(lib):
+    """One function of the reference's FuncType per kernel, by index and by name; a failing call reports through
+    mxmoe_last_status (the type returns void).  Host-only: the call below fails validation before any launch."""
+    from mxmoe_amd import _lib
+
+    n = lib.mxmoe_num_kernels()
+    funcs = [lib.mxmoe_kernel_func(i) for i in range(n)]
+    assert all(funcs) and len(set(funcs)) == n                              # every kernel its own function
+    assert lib.mxmoe_kernel_func(n) is None and lib.mxmoe_get_kernel(b"nope") is None
+    assert lib.mxmoe_get_kernel(b"groupgemm_hz_fused_wxax") == funcs[0]
+    assert lib.mxmoe_get_kernel(lib.mxmoe_kernel_name(2)) == funcs[2]       # the full registry key works as well
+    assert {lib.mxmoe_kernel_policy(i) for i in range(n)} == {0, 1, 2} and lib.mxmoe_kernel_policy(-1) == -1
+    assert lib.mxmoe_get_stream() is None
+    lib.mxmoe_set_stream(0x10)
+    assert lib.mxmoe_get_stream() == 0x10
+    lib.mxmoe_set_stream(None)
+    fn = _lib.FUNC_TYPE(funcs[1])                                           # the fp16 kernel, asked to run a w4a4 problem
+    sizes = (_lib.Dim3 * 1)(_lib.Dim3(8, 256, 128))
+    q = (_lib.QParams * 1)(_lib.QParams(4, 4, -1, 1))
+    one = (C.c_void_p * 1)(0)
+    a = C.addressof(one)
+    fn(a, a, a, a, a, a, None, None, None, None, a, sizes, None, q, 1)
+    assert lib.mxmoe_last_status() == 1 and lib.mxmoe_last_error() == b"quant type not supported"
+    fn(a, a, a, a, a, a, None, None, None, None, a, sizes, None, q, 0)      # an empty problem list is a successful no-op
+    assert lib.mxmoe_last_status() == 0
+
+
 def test_prologue_entry_points_validate_on_the_host(lib):
     one = (C.c_int64 * 8)()
     a = C.addressof(one)

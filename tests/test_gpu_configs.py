@@ -139,6 +139,8 @@ def test_c4_weight_only_decode_full_size():
 
 
 def test_c1_fp16_full_size():
+    """fp16 GroupGEMM at full size against an fp32 matmul of the same fp16 operands computed by the GPU's BLAS library (the plain
+    fp32 reference of a floating-point kernel; the oracle's `gemm_fp16` covers the small fp16 cases of test_gpu_group_gemm.py)."""
     cfg, hidden, ids, layer, outs, recv, prob_of = _build("c1", dump=False)
     st = layer.state
     _, perm, _, _ = O.permute_by_expert(ids.numpy(), cfg.num_experts)
@@ -192,6 +194,52 @@ def test_c5_shaped_layer_reduced():
             assert np.array_equal(r["g_out"].view(np.uint16), out_k.view(np.uint16)), f"down fp16, expert {r['e']}"
         else:
             assert _rel(r["g_out"], r["out"]) <= 1e-2, f"down, expert {r['e']}"
+
+
+def test_c5_full_size():
+    """Mixtral at its own dimensions (K = 4096 / 14336, 8192 tokens): the largest accumulators of the five workloads and the grouped
+    tile order of long-row problems, against exact products.  Per launch of each sampled expert: integer formats compare every
+    int32 accumulator of the expert with the exact integer product of the codes the launch read, and the first rows with the
+    complete oracle chain from the fp16 inputs; the weight-only block compares its first rows with the oracle's fake-quant
+    product to max-abs-rel 1e-2."""
+    cfg, hidden, ids, layer, outs, recv, prob_of = _build("c5")
+    assert int(recv.sum()) == cfg.tokens * cfg.topk == sum(o.shape[0] for o in outs)
+    st, fm = layer.state, layer.formats
+    _, perm, _, _ = O.permute_by_expert(ids.numpy(), cfg.num_experts)
+    starts = np.concatenate([[0], np.cumsum(recv)])
+    h = hidden.numpy()
+    busiest = int(np.argmax(recv))
+    want = {busiest}
+    want.add(next(e for e in prob_of if fm[e][0][0] == 4))           # a w4a4 gate_up
+    want.add(next(e for e in prob_of if fm[e][0][0] == 8))           # a w8a8 gate_up
+    want.add(next(e for e in prob_of if fm[e][1][0] == 4))           # a w4a4 down
+    want.add(next(e for e in prob_of if fm[e][1][0] == 8))           # a w8a8 down
+    want.add(next(e for e in prob_of if fm[e][0][0] >= 16))          # the weight-only gate_up
+    rows_oracle = 16
+    for e in sorted(want):
+        p = prob_of[e]
+        gu, dn = fm[e]
+        m = min(int(recv[e]), rows_oracle)
+        x = h[perm[starts[e]:starts[e] + m]]
+        w13, w2 = layer_weights(cfg, e)
+        if gu[0] < 16:
+            assert torch.equal(_exact_acc(_codes(st["inp"][p], gu[0]), layer.w13[e].q), st["acc1"][p]), f"gate_up accumulators, expert {e}"
+            mid_k, mid_f, acc1 = O.linear_block(x, w13, gu, cfg.rotate >= 1)
+            assert np.array_equal(st["acc1"][p][:m].cpu().numpy(), acc1), f"oracle gate_up accumulators, expert {e}"
+            assert np.array_equal(st["mid"][p][:m].cpu().numpy().view(np.uint16), mid_k.view(np.uint16)), f"oracle gate_up fp16, expert {e}"
+            assert _rel(mid_k, mid_f) <= 1e-2
+        else:
+            mid = O.gemm_fakequant(x, O.fake_quant(w13, gu[1], gu[2], gu[3]))
+            assert _rel(st["mid"][p][:m].cpu().numpy(), mid) <= 1e-2, f"weight-only gate_up, expert {e}"
+        if dn[0] < 16:
+            assert torch.equal(_exact_acc(_codes(st["inp2"][p], dn[0]), layer.w2[e].q), st["acc2"][p]), f"down accumulators, expert {e}"
+            # the oracle's down block from the GPU's own intermediate rows (isolates the activation step and the down launch)
+            out_k, out_f, acc2 = O.linear_block(O.silu_mul(st["mid"][p][:m].cpu().numpy()), w2, dn, cfg.rotate >= 1)
+            assert np.array_equal(st["acc2"][p][:m].cpu().numpy(), acc2), f"oracle down accumulators, expert {e}"
+            assert np.array_equal(outs[p][:m].cpu().numpy().view(np.uint16), out_k.view(np.uint16)), f"oracle down fp16, expert {e}"
+            assert _rel(out_k, out_f) <= 1e-2
+    assert {f[0] for f in fm} | {f[1] for f in fm} == {(4, 4, -1, True), (8, 8, -1, True), (16, 4, 128, False)}
+    assert all(bool(torch.isfinite(o).all()) for o in outs)
 
 
 def test_c5_one_call_equals_stepwise_at_real_row_lengths():

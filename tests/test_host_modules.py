@@ -84,13 +84,43 @@ def test_template_generator_product_and_sources(tmp_path):
     files = g.generate_source_code()
     assert len(g.combos) == 6 and len(files) == 7                          # 3 x 2 combinations + the ABI unit
     src = (tmp_path / "hz_fused_4.hip").read_text()
-    assert 'register_fused<WxAxTile<Op::I4, 32, 256>, WxAxTile<Op::I8, 128, 256>>("groupgemm_hz_fused_4")' in src
+    assert 'register_fused<WxAxTile<Op::I4, 32, 256>, WxAxTile<Op::I8, 128, 256>>("groupgemm_hz_fused_4", Policy::Fused)' in src
     assert "(a_bits == 4 && w_bits == 4 && gsize == -1 && sym == true)" in src
     assert "groupgemm_hz_fused_5" in (tmp_path / "hz_fused_decl.hpp").read_text()
+    # the ablation launchers are the same combinations behind another launch policy (kernel_sketch.py:148-406)
     seq = TemplateGenerator("gfx950", ["w8a8_g-1_sym", "w4a4_g-1_sym"], KernelType.Sequential, tiles, out_dir=tmp_path / "seq")
-    assert len(seq.get_tile_configs()) == 5                                # one single-format kernel per (qcfg, tile)
+    assert len(seq.get_tile_configs()) == 6
+    seq.generate_source_code()
+    assert '("groupgemm_seq_launch_0", Policy::Sequential)' in (tmp_path / "seq" / "seq_launch_0.hip").read_text()
+    # a tuple of tiles is a shape set: one kernel carrying every shape of the set as a branch of that format
+    sets = {"w4a4_g-1_sym": [tuple(tiles["w4a4_g-1_sym"])], "w8a8_g-1_sym": [tuple(tiles["w8a8_g-1_sym"]), tiles["w8a8_g-1_sym"][0]]}
+    g2 = TemplateGenerator("gfx950", ["w8a8_g-1_sym", "w4a4_g-1_sym"], KernelType.MultiStream, sets, out_dir=tmp_path / "sets")
+    g2.generate_source_code()
+    assert len(g2.combos) == 2
+    assert ('register_fused<WxAxTile<Op::I4, 128, 256>, WxAxTile<Op::I4, 64, 256>, WxAxTile<Op::I4, 32, 256>, WxAxTile<Op::I8, 128, 256>, '
+            'WxAxTile<Op::I8, 64, 256>>("groupgemm_ms_launch_0", Policy::MultiStream)') in (tmp_path / "sets" / "ms_launch_0.hip").read_text()
     with pytest.raises(ValueError, match="Unsupported qcfg"):
         TemplateGenerator("gfx950", ["w2a16_g-1_sym"])
+
+
+def test_default_library_is_generator_output(tmp_path, lib):
+    """The kernels libmxmoe_amd.so registers are the generator's `default_kernel_specs`, name for name and branch for branch."""
+    from mxmoe_amd.kernels import compose_kernel as ck
+
+    specs = ck.default_kernel_specs()
+    src = ck.emit_default_library(tmp_path).read_text()
+    assert lib.mxmoe_num_kernels() == len(specs)
+    policy = {ck.KernelType.Fused: 0, ck.KernelType.Sequential: 1, ck.KernelType.MultiStream: 2}
+    import ctypes as C
+
+    out = (C.c_int32 * 8)()
+    for i, (name, ktype, tile_cfg) in enumerate(specs):
+        assert lib.mxmoe_kernel_name(i).decode().endswith(name) and f'"{name}", {ck.POLICY[str(ktype)]}' in src
+        assert lib.mxmoe_kernel_policy(i) == policy[ktype]
+        tiles = ck._flat(tile_cfg.values())
+        assert lib.mxmoe_kernel_num_branches(i) == len(tiles)
+        for b, t in enumerate(tiles):
+            assert lib.mxmoe_kernel_branch(i, b, out) == 0 and (out[1], out[2], out[3]) == (t.BM, t.BN, t.BK)
 
 
 def test_run_mxmoe_gg_helpers(tmp_path):
