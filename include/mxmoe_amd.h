@@ -102,6 +102,16 @@ size_t mxmoe_permute_workspace_bytes(int total_rows, int num_experts);
 int mxmoe_build_permutation(const int32_t* topk_ids, int num_tokens, int topk, int num_experts, int32_t* dst_exp_sorted, int64_t* perm_indices,
                             int64_t* src_slot, int64_t* recv_tokens_per_exp, void* workspace, void* stream);
 
+/* The same permutation for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  No counterpart in the reference.  The per-block histograms that the `workspace` argument
+ * above brings in live in a static device array of mxmoe_static_scratch_bytes() bytes (1 MiB per GPU, held until the process
+ * ends) instead; the call allocates and frees nothing.  Sizes whose mxmoe_permute_workspace_bytes() exceeds it (more than
+ * 262144 / num_experts - 1 blocks of 256 rows) are refused with error 3.  All calls on one GPU share that array: calls that overlap
+ * in time on one GPU (different streams or threads) race and must be serialised by the caller.  Same outputs as above. */
+size_t mxmoe_static_scratch_bytes(void);
+int mxmoe_build_permutation_static(const int32_t* topk_ids, int num_tokens, int topk, int num_experts, int32_t* dst_exp_sorted, int64_t* perm_indices,
+                                   int64_t* src_slot, int64_t* recv_tokens_per_exp, void* stream);
+
 /* ---- activation quantisers: replace the launches of quant_act_kernel and silu_mul_then_quant_kernel
  *      (mxmoe/kernels/src/ref_bind.cu:524-544 and 691-716; their source, act_kernel.cuh, is absent from the reference) ----
  *

@@ -838,20 +838,10 @@ size_t mxmoe_permute_workspace_bytes(int total, int num_experts) {
   return (blocks * num_experts + num_experts) * sizeof(int32_t);
 }
 
-int mxmoe_build_permutation(const int32_t* topk_ids, int num_tokens, int topk, int num_experts, int32_t* dst_exp_sorted, int64_t* perm_indices,
-                            int64_t* src_slot, int64_t* recv_tokens_per_exp, void* workspace, void* stream) {
+static int build_permutation_impl(const int32_t* topk_ids, int num_tokens, int topk, int num_experts, int32_t* dst_exp_sorted, int64_t* perm_indices,
+                                  int64_t* src_slot, int64_t* recv_tokens_per_exp, int32_t* hist, hipStream_t s) {
   const int total = num_tokens * topk;
-  if (total <= 0 || num_experts <= 0 || num_experts > 4096) {
-    last_error() = "bad permutation size";
-    return 3;
-  }
-  if (!topk_ids || !dst_exp_sorted || !perm_indices || !src_slot || !recv_tokens_per_exp || !workspace) {
-    last_error() = "null pointer";
-    return 5;
-  }
-  hipStream_t s = (hipStream_t)stream;
   const int blocks = (total + kPermChunk - 1) / kPermChunk;
-  int32_t* hist = reinterpret_cast<int32_t*>(workspace);
   int nbits = 1;
   while ((1 << nbits) <= num_experts) ++nbits;  // ids 0..E (E = parked lanes)
   const size_t lds = (size_t)num_experts * sizeof(int32_t);
@@ -865,6 +855,67 @@ int mxmoe_build_permutation(const int32_t* topk_ids, int num_tokens, int topk, i
     return 4;
   }
   return 0;
+}
+
+static int check_permutation_args(const int32_t* topk_ids, int num_tokens, int topk, int num_experts, const int32_t* dst_exp_sorted, const int64_t* perm_indices,
+                                  const int64_t* src_slot, const int64_t* recv_tokens_per_exp) {
+  if (num_tokens <= 0 || topk <= 0 || (long)num_tokens * topk > (1l << 30) || num_experts <= 0 || num_experts > 4096) {
+    last_error() = "bad permutation size";
+    return 3;
+  }
+  if (!topk_ids || !dst_exp_sorted || !perm_indices || !src_slot || !recv_tokens_per_exp) {
+    last_error() = "null pointer";
+    return 5;
+  }
+  return 0;
+}
+
+int mxmoe_build_permutation(const int32_t* topk_ids, int num_tokens, int topk, int num_experts, int32_t* dst_exp_sorted, int64_t* perm_indices,
+                            int64_t* src_slot, int64_t* recv_tokens_per_exp, void* workspace, void* stream) {
+  if (const int rc = check_permutation_args(topk_ids, num_tokens, topk, num_experts, dst_exp_sorted, perm_indices, src_slot, recv_tokens_per_exp)) return rc;
+  if (!workspace) {
+    last_error() = "null pointer";
+    return 5;
+  }
+  return build_permutation_impl(topk_ids, num_tokens, topk, num_experts, dst_exp_sorted, perm_indices, src_slot, recv_tokens_per_exp,
+                                reinterpret_cast<int32_t*>(workspace), (hipStream_t)stream);
+}
+
+// ---- the permutation for callers that may not allocate: the per-block histograms live in a static device array ----
+constexpr size_t kStaticScratchInts = 256 * 1024;  // 1 MiB per device, held until the process ends
+static __device__ __align__(256) int32_t scratch[kStaticScratchInts];
+
+size_t mxmoe_static_scratch_bytes(void) { return kStaticScratchInts * sizeof(int32_t); }
+
+int mxmoe_build_permutation_static(const int32_t* topk_ids, int num_tokens, int topk, int num_experts, int32_t* dst_exp_sorted, int64_t* perm_indices,
+                                   int64_t* src_slot, int64_t* recv_tokens_per_exp, void* stream) {
+  if (const int rc = check_permutation_args(topk_ids, num_tokens, topk, num_experts, dst_exp_sorted, perm_indices, src_slot, recv_tokens_per_exp)) return rc;
+  const size_t need = mxmoe_permute_workspace_bytes(num_tokens * topk, num_experts);
+  if (need > mxmoe_static_scratch_bytes()) {
+    char buf[200];
+    snprintf(buf, sizeof buf, "permutation of %d rows over %d experts needs %zu bytes of scratch, the static buffer holds %zu: use mxmoe_build_permutation with a workspace",
+             num_tokens * topk, num_experts, need, mxmoe_static_scratch_bytes());
+    last_error() = buf;
+    return 3;
+  }
+  // every device has its own copy of the array at its own address; `scratch` itself is only a host-side handle for the lookup
+  static int32_t* device_ptr[64] = {};
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+    last_error() = "no current HIP device";
+    return 4;
+  }
+  if (!device_ptr[dev]) {
+    void* p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) {
+      last_error() = std::string("hipGetSymbolAddress(scratch) failed: ") + hipGetErrorString(e);
+      return 4;
+    }
+    device_ptr[dev] = reinterpret_cast<int32_t*>(p);
+  }
+  // nothing needs clearing: perm_hist_kernel writes every counter the later kernels read
+  return build_permutation_impl(topk_ids, num_tokens, topk, num_experts, dst_exp_sorted, perm_indices, src_slot, recv_tokens_per_exp, device_ptr[dev], (hipStream_t)stream);
 }
 
 static int fill_common(RowArgs& a, int n, int n_shared, int had_k, int had_f, const float* signs) {
