@@ -45,15 +45,31 @@ def check_no_spills(remarks: str) -> None:
                                f"register ring or lower its waves per SIMD")
 
 
+_VMEM = re.compile(r"(global_|buffer_|flat_|scratch_)(load|store|atomic)")
+
+
 def check_untracked_load_copies(asm: str) -> None:
-    """Refuse device code in which a register is moved by the compiler while a hand-tracked load into it is in flight.
+    """Refuse device code in which the compiler touches a register while a hand-tracked load into it is in flight, or adds a
+    vector-memory instruction of its own where vector-memory instructions are counted by hand.
 
     The weight fragments of the WxAxTile kernels are loaded by inline-assembly `global_load_dwordx4` whose completion only the
-    hand-placed `s_waitcnt vmcnt(N) ; landed v[a:b]` knows about.  A register-to-register copy (or a spill) of such a register,
-    which the register allocator is free to insert wherever the value is live across a branch or a loop edge, copies whatever the
-    register holds at that moment.  `asm` is hipcc's -S output for the device.  Every kernel is walked in layout order with the set
-    of registers in flight (added by an inline-assembly load, removed by the wait that names them); loop bodies are walked twice,
-    so that loads issued at the bottom of an iteration are in flight at its top."""
+    hand-placed `s_waitcnt vmcnt(N) ; landed v[a:b]` knows about, and N is the exact number of younger vector-memory instructions
+    (fragment loads and direct-to-LDS loads, all inline assembly).  `asm` is hipcc's -S output for the device.  Every kernel is
+    cut into basic blocks and the set of registers possibly in flight (added by an inline-assembly load, removed by the wait that
+    names them) is propagated along its branches to a fixed point, so loads issued at the bottom of a loop iteration are in flight
+    at its top and code the compiler lays out elsewhere is judged by how control reaches it.  Refused:
+
+    * ANY compiler-generated instruction (whatever its mnemonic: a move, a spill, a permute, an ordinary ALU operation reading or
+      overwriting it) that names a register in flight: it would read stale data, or its result would be overwritten when the load
+      lands;
+    * any compiler-generated vector-memory instruction, inside a loop or not, while a hand-tracked load is in flight: it would be
+      one more instruction in the queue than the hand-computed N assumes;
+    * a compiler-generated store, atomic or scratch access while direct-to-LDS loads (inline assembly too, awaited by hand-placed
+      counts) may be outstanding, i.e. since the last hand-placed wait for vmcnt(0): writes retire out of order with the loads, so
+      a count that includes one says nothing about the loads.  Compiler-generated LOADS are allowed there: loads retire in
+      order, so one more younger load makes a hand-placed wait last longer, never shorter (the weight-only MFMA tile counts on
+      exactly that: its weight loads are the compiler's, its activation loads go straight to LDS);
+    * a load that is never waited for."""
     lines = asm.splitlines()
     starts = [i for i, l in enumerate(lines) if re.match(r"^_Z\w+:", l)]
 
@@ -66,52 +82,88 @@ def check_untracked_load_copies(asm: str) -> None:
 
     for si, start in enumerate(starts):
         end = starts[si + 1] if si + 1 < len(starts) else len(lines)
+        end = next((i for i in range(start, end) if lines[i].startswith(".Lfunc_end")), end)
         kernel = lines[start].split(":")[0]
-        # loop regions: header line .. end of the last block that names the header
-        label_lines = [i for i in range(start, end) if re.match(r"^\.LBB\d+_\d+:", lines[i])]
-        regions = []
-        for h in (i for i in range(start, end) if "Loop Header" in lines[i]):
-            name = lines[h].split(":")[0].strip().lstrip(".L")
-            members = [i for i in range(start, end) if re.search(rf"Header={name}\b", lines[i])]
-            last = max([h] + members)
-            nxt = next((i for i in label_lines if i > last), end)
-            regions.append((min([h] + members), nxt))
-        order, pos = [], start
-        for lo, hi in sorted(regions):
-            if lo < pos:
+        # basic blocks: (instructions as (line number, text, inside inline assembly), successor labels, falls through)
+        blocks, label_of, cur, inside = [], {}, None, False
+
+        def new_block():
+            blocks.append({"ins": [], "succ": [], "fall": True})
+            return blocks[-1]
+
+        cur = new_block()
+        for i in range(start + 1, end):
+            raw = lines[i]
+            t = raw.strip()
+            m = re.match(r"^(\.LBB\d+_\d+):", raw)
+            if m:
+                if cur["ins"] or cur["succ"] or len(blocks) == 1:
+                    cur = new_block()
+                label_of[m.group(1)] = len(blocks) - 1
                 continue
-            order += list(range(pos, lo)) + list(range(lo, hi)) * 2
-            pos = hi
-        order += list(range(pos, end))
-        # a loop that issues hand-tracked loads counts every vector-memory instruction: the compiler must not add its own there
-        for lo, hi in regions:
-            body = [lines[i].strip() for i in range(lo, hi)]
-            tracked, inside = False, False
-            for t in body:
-                inside = True if t.startswith(";;#ASMSTART") else False if t.startswith(";;#ASMEND") else inside
-                tracked |= inside and t.startswith("global_load")
-            inside = False
-            for k, t in enumerate(body):
-                inside = True if t.startswith(";;#ASMSTART") else False if t.startswith(";;#ASMEND") else inside
-                if tracked and not inside and re.match(r"(global_|buffer_|flat_|scratch_)(load|store|atomic)", t):
-                    raise RuntimeError(f"{kernel}: line {lo + k + 1} `{t}`: compiler-generated vector-memory instruction inside a loop whose "
-                                       f"loads are counted by hand")
-        inflight, in_asm = set(), False
-        for i in order:
-            t = lines[i].strip()
             if t.startswith(";;#ASMSTART"):
-                in_asm = True
-            elif t.startswith(";;#ASMEND"):
-                in_asm = False
-            elif in_asm and t.startswith("global_load"):
-                inflight |= regs_of(t.split(",")[0])
-            elif in_asm and t.startswith("s_waitcnt") and "; landed" in t:
-                inflight -= regs_of(t.split("; landed")[1])
-            elif not in_asm and inflight and re.match(r"(v_mov_b|v_accvgpr_|scratch_|v_swap_)", t) and regs_of(t) & inflight:
-                raise RuntimeError(f"{kernel}: line {i + 1} `{t}` moves a register while a hand-tracked load into it is in flight; "
-                                   f"restructure the tile so that no fragment register is live across a branch")
-        if inflight:
-            raise RuntimeError(f"{kernel}: hand-tracked loads into v{sorted(inflight)} are never waited for")
+                inside = True
+                continue
+            if t.startswith(";;#ASMEND"):
+                inside = False
+                continue
+            if not t or t.startswith(";") or t.startswith("."):
+                continue
+            cur["ins"].append((i, t, inside))
+            if inside:
+                continue
+            m = re.match(r"s_(c?branch)\w*\s+(\.LBB\d+_\d+)", t)
+            if m:
+                cur["succ"].append(m.group(2))
+                cur["fall"] = m.group(1) == "cbranch"
+                cur = new_block()
+            elif re.match(r"s_(endpgm|setpc_b64|trap)", t):
+                cur["fall"] = False
+                cur = new_block()
+
+        def successors(b):
+            out = [label_of[l] for l in blocks[b]["succ"] if l in label_of]
+            if blocks[b]["fall"] and b + 1 < len(blocks):
+                out.append(b + 1)
+            return out
+
+        # Forward may-analysis over the control-flow graph to a fixed point.  State at a block's entry: registers with a hand-tracked
+        # load possibly in flight, and `lds_pending` (direct-to-LDS loads, counted by hand as well but landing in no register, may
+        # be outstanding: only a hand-placed wait for vmcnt(0) is known to have drained them).
+        state_in = {0: (frozenset(), False)}
+        work = [0]
+        while work:
+            b = work.pop()
+            inflight, lds_pending = set(state_in[b][0]), state_in[b][1]
+            for i, t, in_asm in blocks[b]["ins"]:
+                if in_asm:
+                    if t.startswith("global_load"):
+                        inflight |= regs_of(t.split(",")[0])
+                    elif _VMEM.match(t):
+                        lds_pending = True
+                    elif t.startswith("s_waitcnt"):
+                        if "; landed" in t:
+                            inflight -= regs_of(t.split("; landed")[1])
+                        if re.search(r"vmcnt\(0\)", t):  # every vector-memory instruction issued so far has completed
+                            inflight.clear()
+                            lds_pending = False
+                elif _VMEM.match(t) and (inflight or (lds_pending and not re.match(r"(global|buffer|flat)_load", t))):
+                    raise RuntimeError(f"{kernel}: line {i + 1} `{t}`: compiler-generated vector-memory instruction while vector-memory "
+                                       f"instructions are counted by hand (loads in flight: v{sorted(inflight)}, direct-to-LDS loads pending: {lds_pending})")
+                elif inflight and regs_of(t.split(";")[0]) & inflight:
+                    raise RuntimeError(f"{kernel}: line {i + 1} `{t}` touches a register while a hand-tracked load into it is in flight; "
+                                       f"restructure the tile so that no fragment register is live across a branch")
+                elif inflight and t.startswith("s_endpgm"):
+                    raise RuntimeError(f"{kernel}: hand-tracked loads into v{sorted(inflight)} are never waited for")
+            succ = successors(b)
+            if inflight and not succ and not any(t.startswith("s_endpgm") for _, t, _ in blocks[b]["ins"]):
+                raise RuntimeError(f"{kernel}: hand-tracked loads into v{sorted(inflight)} are never waited for")
+            for n in succ:
+                old = state_in.get(n)
+                new = (frozenset(inflight) | (old[0] if old else frozenset()), lds_pending or (old[1] if old else False))
+                if new != old:
+                    state_in[n] = new
+                    work.append(n)
 
 
 def hipcc_build(sources, out: Path, extra=(), verbose: bool = False, jobs: int = 8) -> Path:

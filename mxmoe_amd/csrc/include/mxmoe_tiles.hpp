@@ -624,10 +624,14 @@ struct WxAxTile {
     }
     if constexpr (OP == Op::I4) widen(pbq[0][0][0], bop[0]);
 
-    // ---- one K slice; P = kt % kDepth (compile-time, so the ring slots are fixed registers)
+    // ---- one K slice; P = kt % kDepth (compile-time, so the ring slots are fixed registers).  The loop below always runs whole
+    // groups of kDepth slices.  A slice past the end of K (`live` false) issues the same loads and passes the same waits and
+    // barriers as any other (its activation loads have zero length, its weight loads re-read the last slice), so the hand-computed
+    // counts hold on every path through the loop; it only skips the LDS reads, the widening and the matrix instructions.
     auto slice = [&](auto parc, int kt, const uint8_t* sc, const uint8_t* sn, int nstage) {
       constexpr int P = decltype(parc)::value;
       constexpr int Pprev = (P + kDepth - 1) % kDepth, Pnext = (P + 1) % kDepth;
+      const bool live = kt < KT;
       static_for<U>([&](auto uc) {
         constexpr int u = decltype(uc)::value;
         constexpr int step = u / FN, j = u % FN;
@@ -643,35 +647,36 @@ struct WxAxTile {
         if constexpr (u == 0) pbq[Pprev][1][1] = load_b(1, 1, kt - 1 + kDepth);
         else pbq[P][(u - 1) % FN][(u - 1) / FN] = load_b((u - 1) % FN, (u - 1) / FN, kt + kDepth);
         asm volatile("" ::: "memory");
-        // activation fragments of the next k-step
-        if (j == 0) {
-#pragma unroll
-          for (int i = 0; i < FM; ++i) {
-            const v4i p = step == 0 ? lds_a(sc, 1, i) : lds_a(sn, 0, i);
-            if constexpr (OP == Op::I4) pa[i] = p; else aop[step ^ 1][i][0] = p;
-          }
-        }
         if constexpr (OP == Op::I4) {
           // weight operands of unit u+1
-          if constexpr (u + 1 < U) {
-            ready(std::integral_constant<int, u + 1>{}, pbq[P][(u + 1) % FN][(u + 1) / FN]);
-            widen(pbq[P][(u + 1) % FN][(u + 1) / FN], bop[(u + 1) & 1]);
-          } else {
-            ready(std::integral_constant<int, 0>{}, pbq[Pnext][0][0]);
-            widen(pbq[Pnext][0][0], bop[0]);
-          }
-#pragma unroll
-          for (int i = 0; i < FM; ++i) {
-            mma(acc[i][j], aop[0][i], bop[u & 1]);
-            if (j == FN - 1) widen(pa[i], aop[0][i]);  // next k-step's operand, right after the last use of this one
-          }
-          __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
-          __builtin_amdgcn_sched_group_barrier(0x100, FM, 0);
-          sched_mfma_valu<12 + (j == FN - 1 ? 12 * FM : 0), 2 * FM, 0>();
+          if constexpr (u + 1 < U) ready(std::integral_constant<int, u + 1>{}, pbq[P][(u + 1) % FN][(u + 1) / FN]);
+          else ready(std::integral_constant<int, 0>{}, pbq[Pnext][0][0]);
         } else {
           ready(uc, pbq[P][j][step]);
+        }
+        if (live) {
+          // activation fragments of the next k-step
+          if (j == 0) {
 #pragma unroll
-          for (int i = 0; i < FM; ++i) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(pbq[P][j][step], aop[step][i][0], acc[i][j], 0, 0, 0);
+            for (int i = 0; i < FM; ++i) {
+              const v4i p = step == 0 ? lds_a(sc, 1, i) : lds_a(sn, 0, i);
+              if constexpr (OP == Op::I4) pa[i] = p; else aop[step ^ 1][i][0] = p;
+            }
+          }
+          if constexpr (OP == Op::I4) {
+            if constexpr (u + 1 < U) widen(pbq[P][(u + 1) % FN][(u + 1) / FN], bop[(u + 1) & 1]);
+            else widen(pbq[Pnext][0][0], bop[0]);
+#pragma unroll
+            for (int i = 0; i < FM; ++i) {
+              mma(acc[i][j], aop[0][i], bop[u & 1]);
+              if (j == FN - 1) widen(pa[i], aop[0][i]);  // next k-step's operand, right after the last use of this one
+            }
+            __builtin_amdgcn_sched_group_barrier(0x100, FM, 0);
+            sched_mfma_valu<12 + (j == FN - 1 ? 12 * FM : 0), 2 * FM, 0>();
+          } else {
+#pragma unroll
+            for (int i = 0; i < FM; ++i) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(pbq[P][j][step], aop[step][i][0], acc[i][j], 0, 0, 0);
+          }
         }
         __builtin_amdgcn_sched_barrier(0);
       });
@@ -682,12 +687,10 @@ struct WxAxTile {
     for (int kt0 = 0; kt0 < KT; kt0 += kDepth) {
       static_for<kDepth>([&](auto dc) {
         constexpr int d = decltype(dc)::value;
-        if (kt0 + d < KT) {
-          const int nidx = sidx == 2 ? 0 : sidx + 1;
-          const int nn = nidx == 2 ? 0 : nidx + 1;
-          slice(dc, kt0 + d, smem + sidx * kStageBytes, smem + nidx * kStageBytes, nn);
-          sidx = nidx;
-        }
+        const int nidx = sidx == 2 ? 0 : sidx + 1;
+        const int nn = nidx == 2 ? 0 : nidx + 1;
+        slice(dc, kt0 + d, smem + sidx * kStageBytes, smem + nidx * kStageBytes, nn);
+        sidx = nidx;
       });
     }
     // Nothing may still land in LDS once the epilogue reuses it, and nothing in registers either: the fragments fetched past the

@@ -261,6 +261,13 @@ def test_build_refuses_moves_of_registers_with_loads_in_flight():
         chk(kernel(load + move + wait))
     with pytest.raises(RuntimeError, match="never waited"):
         chk(kernel(load))
+    # whatever the mnemonic: a permute or an ordinary ALU operation reading the register, or anything overwriting it
+    for bad in ("\tv_perm_b32 v40, v11, v41, v42", "\tv_and_b32_e32 v5, v10, v4", "\tv_pk_mov_b32 v[40:41], v[12:13], v[12:13]",
+                "\tv_readlane_b32 s4, v13, 3", "\tv_add_u32_e32 v12, v40, v41", "\tds_write_b128 v50, v[10:13]"):
+        with pytest.raises(RuntimeError, match="in flight"):
+            chk(kernel(load + [bad] + wait))
+        chk(kernel(load + wait + [bad]))
+    chk(kernel(load + ["\tv_and_b32_e32 v5, v110, v4 ; v10 in a comment"] + wait))
     # loop: the load at the bottom of an iteration is in flight at the top of the next one
     loop = [".LBB0_1:                                ; =>This Inner Loop Header: Depth=1"] + move + wait + ["\tv_and_b32_e32 v5, v10, v4"] + load + \
            ["\ts_cbranch_scc1 .LBB0_1", ".LBB0_2:"] + wait
@@ -280,9 +287,38 @@ def test_build_refuses_compiler_memory_instructions_in_hand_counted_loops():
     mk = lambda body: "_Z6kernelv:\n" + "\n".join(load + head + body + tail + wait) + "\n\ts_endpgm\n"
     chk(mk(wait + load))
     with pytest.raises(RuntimeError, match="counted by hand"):
-        chk(mk(wait + ["\tglobal_load_dword v40, v[2:3], off"] + load))
-    # loops without hand-tracked loads may hold any memory instruction
+        chk(mk(wait + load + ["\tglobal_load_dword v40, v[2:3], off"]))     # in flight around the back edge
+    chk(mk(wait + ["\tglobal_load_dword v40, v[2:3], off"] + load))         # between the wait and the next load nothing is in flight
+    # kernels without hand-tracked loads may hold any memory instruction
     chk("_Z6kernelv:\n" + "\n".join(head + ["\tglobal_load_dword v40, v[2:3], off"] + tail) + "\n\ts_endpgm\n")
+    # outside loops as well: between the first hand-counted load and the last hand-placed wait nothing may be added ...
+    dma = ["\t;;#ASMSTART", "\ts_mov_b32 m0, s4", "\tbuffer_load_dwordx4 v1, s[8:11], s5 offen lds", "\t;;#ASMEND"]
+    plain_wait = ["\t;;#ASMSTART", "\ts_waitcnt vmcnt(0)", "\t;;#ASMEND"]
+    straight = lambda body: "_Z6kernelv:\n" + "\n".join(body) + "\n\ts_endpgm\n"
+    for extra in ("\tglobal_load_dword v40, v[2:3], off", "\tglobal_store_dword v[2:3], v40, off", "\tbuffer_load_dword v40, v41, s[8:11], 0 offen",
+                  "\tscratch_store_dword off, v40, s32"):
+        with pytest.raises(RuntimeError, match="counted by hand"):
+            chk(straight(load + [extra] + wait))
+        # direct-to-LDS loads land in no register: compiler loads behind them only lengthen the hand-placed wait (loads retire in
+        # order), but writes retire out of order with loads and would make the count meaningless
+        if "_load" in extra and not extra.strip().startswith("scratch"):
+            chk(straight(dma + [extra] + plain_wait))
+        else:
+            with pytest.raises(RuntimeError, match="counted by hand"):
+                chk(straight(dma + [extra] + plain_wait))
+        # before the first and after the last of them the compiler is free
+        chk(straight([extra] + load + wait + [extra]))
+        chk(straight([extra] + dma + plain_wait + [extra]))
+    # the state follows the branches, not the layout: a block laid out after the wait but entered from before it is judged in flight
+    cold = "_Z6kernelv:\n" + "\n".join(load + ["\ts_cbranch_scc1 .LBB0_9", ".LBB0_1:"] + wait + ["\ts_endpgm", ".LBB0_9:",
+                                                "\tv_mov_b32_e32 v40, v11", "\ts_branch .LBB0_1"]) + "\n"
+    with pytest.raises(RuntimeError, match="in flight"):
+        chk(cold)
+    # ... and a block laid out in the middle of the loads but only reached after the wait is not
+    chk("_Z6kernelv:\n" + "\n".join(["\ts_branch .LBB0_2", ".LBB0_1:", "\tv_mov_b32_e32 v40, v11", "\ts_endpgm", ".LBB0_2:"] + load + wait +
+                                    ["\ts_branch .LBB0_1"]) + "\n")
+    # a hand-placed wait for vmcnt(0) lands everything
+    chk(straight(load + plain_wait + ["\tv_mov_b32_e32 v40, v11"]))
 
 
 def test_bench_refuses_more_than_one_gpu():
