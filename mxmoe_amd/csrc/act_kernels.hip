@@ -143,20 +143,21 @@ struct RowArgs {
   RotPlan plan, plan_shared;
 };
 
-// fixed fp32 op sequence for exp(t), identical to the CPU restatement
+// fixed fp32 op sequence for exp(t), identical to the CPU restatement: every step is one correctly rounded operation (the
+// multiply-adds are fused: one rounding each)
 __device__ __forceinline__ float exp_fixed(float t) {
   t = fminf(fmaxf(t, -87.0f), 87.0f);
   const float k = rintf(t * 1.4426950408889634f);
-  float r = t - k * 0.693145751953125f;
-  r = r - k * 1.428606765330187e-06f;
+  float r = __builtin_fmaf(-k, 0.693145751953125f, t);
+  r = __builtin_fmaf(-k, 1.428606765330187e-06f, r);
   float p = 0.0001984127f;
-  p = p * r + 0.0013888889f;
-  p = p * r + 0.008333334f;
-  p = p * r + 0.041666668f;
-  p = p * r + 0.16666667f;
-  p = p * r + 0.5f;
-  p = p * r + 1.0f;
-  p = p * r + 1.0f;
+  p = __builtin_fmaf(p, r, 0.0013888889f);
+  p = __builtin_fmaf(p, r, 0.008333334f);
+  p = __builtin_fmaf(p, r, 0.041666668f);
+  p = __builtin_fmaf(p, r, 0.16666667f);
+  p = __builtin_fmaf(p, r, 0.5f);
+  p = __builtin_fmaf(p, r, 1.0f);
+  p = __builtin_fmaf(p, r, 1.0f);
   return ldexpf(p, (int)k);
 }
 
@@ -174,6 +175,18 @@ struct ScaleDiv {
     const float q0 = v * r;
     const float e = __builtin_fmaf(-s, q0, v);
     return __builtin_fmaf(e, r, q0);
+  }
+};
+
+// Power-of-two factors of the dense stage of the non-power-of-two rotations for a row whose largest magnitude is mx (an fp16
+// value held in fp32): with mx < 2^E, to_grid = 2^(17-E) turns the row into integers of magnitude <= 2^17 and from_grid = 2^(E-17)
+// turns sums of them back.  Taken from the exponent field of mx; an all-zero row gets 1 and 1.
+struct DenseGrid {
+  float to_grid, from_grid;
+  __device__ __forceinline__ explicit DenseGrid(float mx) {
+    const int e_field = __float_as_int(mx) >> 23;  // mx >= 0
+    to_grid = e_field == 0 ? 1.0f : __int_as_float((270 - e_field) << 23);
+    from_grid = e_field == 0 ? 1.0f : __int_as_float(max(e_field - 16, 1) << 23);
   }
 };
 
@@ -388,11 +401,30 @@ __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
 
       if (pl.kb > 1) {
         const int mc = pl.m >> 3;  // chunks per k row
+        // snap the row to the grid of step 2^(E-17), max|v| < 2^E: the sums of the dense stage are then sums of integers below
+        // 2^17, exact in fp32 in any order
+        float mx = 0.0f;
+#pragma unroll
+        for (int i = 0; i < MAXC; ++i) {
+          if (tid + i * NT < nchunks) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) mx = fmaxf(mx, fabsf(v[i][j]));
+          }
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+        if ((tid & 63) == 0) red[tid >> 6] = mx;
         __syncthreads();
+        mx = red[0];
+#pragma unroll
+        for (int w = 1; w < NT / 64; ++w) mx = fmaxf(mx, red[w]);
+        const DenseGrid grid(mx);
 #pragma unroll
         for (int i = 0; i < MAXC; ++i) {
           const int c = tid + i * NT;
           if (c < nchunks) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[i][j] = rintf(v[i][j] * grid.to_grid);
             put(c, v[i]);
           }
         }
@@ -417,7 +449,7 @@ __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
               for (int j = 0; j < 8; ++j) acc[j] = __builtin_fmaf(s, vv[j], acc[j]);  // s = +-1: the product is exact, so this is acc + s*v
             }
 #pragma unroll
-            for (int j = 0; j < 8; ++j) v[i][j] = acc[j];
+            for (int j = 0; j < 8; ++j) v[i][j] = acc[j] * grid.from_grid;  // exact: an integer below 2^24 times a power of two
           }
         }
         // S_f butterflies across blocks of kb rows (ascending)
@@ -709,6 +741,307 @@ __global__ void __launch_bounds__(256) row_quant_wave_kernel(const RowArgs a) {
   }
 }
 
+// One row per WAVE for rotations H_K kron H_8 with a table-driven factor (K = f * kb, H_K = S_f kron B, f <= 4, kb <= 64; a 1408-value
+// row is 176 x 8 with f = 4, kb = 44): lane l holds the chunks l + 64 i, a chunk being the 8 values of one k.  The Sylvester part
+// (H_8) stays inside a chunk.  The dense stage t[b][col] = sum_b' B[b][b'] q[b'][col] over the 8 f columns col = blk * 8 + j runs on the
+// matrix cores: the row, snapped to integers of at most 18 bits (DenseGrid) and divided by 16 so that every value is an fp16 number,
+// is written to LDS transposed ([col][b'], b' contiguous), B (+-1, zero padded) is the first operand held in registers for the
+// whole kernel, and the fp32 results are exact whatever order the hardware adds in.  Results return through LDS in row order, so
+// the quantise / pack / store code sees the same chunk-per-lane layout as in the other kernels and writes 16 bytes per lane.
+// Four independent rows per workgroup; no barrier (each wave owns its piece of LDS).
+constexpr int kDensePitch = 144;             // bytes per column of the transposed row: 64 fp16 + 16 (16 lanes read 16 distinct bank groups)
+constexpr int kDenseWaveLds = 32 * kDensePitch + (2048 + 8) * 2;  // transposed row + the rotated row in row order (+ a slot for discarded values)
+template <int MAXC, bool SILU>
+__global__ void __launch_bounds__(256) row_quant_dense_kernel(const RowArgs a) {
+  extern __shared__ __align__(16) uint8_t dlds[];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int lm = lane & 15, lg = lane >> 4;
+  uint8_t* xt = dlds + wave * kDenseWaveLds;           // [32 columns][kDensePitch]
+  uint8_t* yrow = xt + 32 * kDensePitch;               // [n] fp16, then the discard slot
+  const RotPlan pl = a.plan;
+  const int n = pl.n, nchunks = n >> 3, kb = pl.kb;
+  const int ksteps = (kb + 31) >> 5, mblocks = (kb + 15) >> 4;
+  // B as the first operand of v_mfma_f32_16x16x32_f16: lane holds row 16 mb + (lane & 15), k = 32 ks + 8 (lane >> 4) + 0..7
+  v8h bsign[4][2];
+#pragma unroll
+  for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      const int b = 16 * mb + lm;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        // unconditional loads (index clamped into the table, the value dropped afterwards): all of them are in flight together
+        const int bp = 32 * ks + 8 * lg + i;
+        const float sv = a.signs[min(b, kb - 1) * kb + min(bp, kb - 1)];
+        bsign[mb][ks][i] = (b < kb && bp < kb) ? (_Float16)sv : (_Float16)0.0f;
+      }
+    }
+  // columns and k positions that no row ever writes must read as zero
+  for (int i = lane; i < 32 * kDensePitch / 16; i += 64) reinterpret_cast<v4i*>(xt)[i] = v4i{0, 0, 0, 0};
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_wave_barrier();
+
+  struct RowMeta {
+    int tag;
+    long lrow, inp_off, scale_off;
+    const _Float16* srow;
+  };
+  auto load_meta = [&](int row) {
+    RowMeta m;
+    const bool shared_row = row >= a.R;
+    const int e = shared_row ? a.E : a.dst_exp[row];
+    m.tag = (int)a.table[e];
+    m.lrow = row - a.table[a.Et + e];
+    m.inp_off = a.table[2 * a.Et + e];
+    m.scale_off = a.table[3 * a.Et + e];
+    if (SILU) {
+      m.srow = shared_row ? a.src_shared + (long)(row - a.R) * 2 * n : a.src + (long)row * 2 * n;
+    } else {
+      m.srow = a.src + (shared_row ? (long)(row - a.R) : (long)a.perm[row]) * n;
+    }
+    return m;
+  };
+  auto load_data = [&](const RowMeta& m, v8h (&g)[MAXC], v8h (&u)[MAXC]) {
+#pragma unroll
+    for (int i = 0; i < MAXC; ++i) {
+      const int c = min(lane + 64 * i, nchunks - 1);  // lanes past the row re-read its last chunk (never used)
+      g[i] = *reinterpret_cast<const v8h*>(m.srow + c * 8);
+      if (SILU) u[i] = *reinterpret_cast<const v8h*>(m.srow + n + c * 8);
+    }
+  };
+  const int stride_rows = gridDim.x * 4;
+  RowMeta next_meta;
+  v8h next_g[MAXC], next_u[MAXC];
+  const int row0 = blockIdx.x * 4 + wave;
+  if (row0 < a.rows) {
+    next_meta = load_meta(row0);
+    load_data(next_meta, next_g, next_u);
+  }
+  for (int row = row0; row < a.rows; row += stride_rows) {
+    const RowMeta cur = next_meta;
+    v8h cur_g[MAXC], cur_u[MAXC];
+#pragma unroll
+    for (int i = 0; i < MAXC; ++i) {
+      cur_g[i] = next_g[i];
+      if (SILU) cur_u[i] = next_u[i];
+    }
+    if (row + stride_rows < a.rows) {  // the next row's bookkeeping and data are fetched under this row's arithmetic
+      next_meta = load_meta(row + stride_rows);
+      load_data(next_meta, next_g, next_u);
+    }
+    const int tag = cur.tag;
+    const bool rot = a.rotate == 2 || (a.rotate == 1 && tag != 0);
+    float v[MAXC][8];
+#pragma unroll
+    for (int i = 0; i < MAXC; ++i) {
+      const bool live = lane + 64 * i < nchunks;
+      const v8h g = cur_g[i];
+      if (SILU) {
+        const v8h u = cur_u[i];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float gf = (float)g[j];
+          const float sl = gf / (1.0f + exp_fixed(-gf));
+          v[i][j] = round_h(keep_f32(sl * (float)u[j]));
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[i][j] = (float)g[j];
+      }
+      if (!live) {  // chunks past the row count as zeros (in the row's maxima) and are never stored
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[i][j] = 0.0f;
+      }
+    }
+    if (rot) {
+      // H_8 inside the chunk (strides 1, 2, 4), scale, round to fp16
+      float mx = 0.0f;
+#pragma unroll
+      for (int i = 0; i < MAXC; ++i) {
+#pragma unroll
+        for (int h = 1; h < 8; h <<= 1)
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            if (!(j & h)) {
+              const float p = v[i][j], q = v[i][j + h];
+              v[i][j] = p + q;
+              v[i][j + h] = p - q;
+            }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          v[i][j] = round_h(keep_f32(v[i][j] * pl.scale));
+          mx = fmaxf(mx, fabsf(v[i][j]));
+        }
+      }
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+      const DenseGrid grid(mx);
+      const float to16 = grid.to_grid * 0.0625f;  // exact (a power of two well inside the range); rint(v * to_grid) / 16 below
+      // transposed write: chunk c = blk * kb + b' -> columns blk * 8 + j, position b'
+#pragma unroll
+      for (int i = 0; i < MAXC; ++i) {
+        const int c = lane + 64 * i;
+        if (c < nchunks) {
+          const int blk = c / kb, bp = c - blk * kb;
+          uint8_t* dst = xt + (blk * 8) * kDensePitch + bp * 2;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) *reinterpret_cast<_Float16*>(dst + j * kDensePitch) = (_Float16)(rintf(v[i][j] * grid.to_grid) * 0.0625f);
+        }
+      }
+      (void)to16;
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_wave_barrier();
+      // lane holds column col = 16 nb + (lane & 15), i.e. blk = 2 nb + ((lane >> 3) & 1), j = lane & 7, and rows
+      // b = 16 mb + 4 (lane >> 4) + r of every 16 x 16 block
+      v4f acc[4][2];
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) acc[mb][nb] = v4f{0.f, 0.f, 0.f, 0.f};
+      const int ncols = pl.f > 2 ? 2 : 1;
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) {
+        if (ks < ksteps) {
+#pragma unroll
+          for (int nb = 0; nb < 2; ++nb) {
+            if (nb < ncols) {
+              const v8h xf = *reinterpret_cast<const v8h*>(xt + (nb * 16 + lm) * kDensePitch + ks * 64 + lg * 16);
+#pragma unroll
+              for (int mb = 0; mb < 4; ++mb)
+                if (mb < mblocks) acc[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(bsign[mb][ks], xf, acc[mb][nb], 0, 0, 0);
+            }
+          }
+        }
+      }
+      // back to the row's scale, S_f butterflies across blk (bit 0 = lane bit 3, bit 1 = the column block; ascending), one rounding to
+      // fp16, and the value goes to its place in the row (values of rows or blocks that do not exist go to the discard slot)
+      const float back = grid.from_grid * 16.0f;
+      const float sgn8 = (lane & 8) ? -1.0f : 1.0f;
+      const int blk0 = (lane >> 3) & 1, jj = lane & 7;
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb) {
+        if (mb < mblocks) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            float t0 = acc[mb][0][r] * back, t1 = acc[mb][1][r] * back;
+            if (pl.f > 1) {
+              t0 = __builtin_fmaf(sgn8, t0, lane_xor<8>(t0));
+              if (pl.f > 2) {
+                t1 = __builtin_fmaf(sgn8, t1, lane_xor<8>(t1));
+                const float p = t0, q = t1;
+                t0 = p + q;
+                t1 = p - q;
+              }
+            }
+            const int b = 16 * mb + 4 * lg + r;
+            const bool ok0 = b < kb && blk0 < pl.f;
+            const int i0 = ok0 ? (((blk0 * kb + b) << 3) + jj) : 2048;
+            *reinterpret_cast<_Float16*>(yrow + i0 * 2) = (_Float16)t0;
+            if (pl.f > 2) {
+              const int i1 = b < kb ? ((((blk0 + 2) * kb + b) << 3) + jj) : 2048;
+              *reinterpret_cast<_Float16*>(yrow + i1 * 2) = (_Float16)t1;
+            }
+          }
+        }
+      }
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int i = 0; i < MAXC; ++i) {
+        const int c = min(lane + 64 * i, nchunks - 1);
+        const bool live = lane + 64 * i < nchunks;
+        const v8h y = *reinterpret_cast<const v8h*>(yrow + c * 16);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[i][j] = live ? (float)y[j] : 0.0f;
+      }
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_wave_barrier();  // the next row's writes come after these reads
+    }
+
+    // ---- store: fp16 copy or symmetric quantisation (as in the other row kernels) ----
+    const long lrow = cur.lrow, inp_off = cur.inp_off, scale_off = cur.scale_off;
+    if (tag == 0) {
+      _Float16* out = reinterpret_cast<_Float16*>(a.inp_store) + inp_off + lrow * n;
+#pragma unroll
+      for (int i = 0; i < MAXC; ++i) {
+        const int c = lane + 64 * i;
+        if (c < nchunks) {
+          v8h o;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) o[j] = (_Float16)v[i][j];
+          *reinterpret_cast<v8h*>(out + c * 8) = o;
+        }
+      }
+      continue;
+    }
+    if (tag == 3) {  // int4, one scale per 128 values = the 16 chunks held by an aligned group of 16 lanes
+      uint8_t* out = a.inp_store + 2 * (inp_off + lrow * (n / 4));
+      _Float16* sout = a.scale_store + scale_off + lrow * (n >> 7);
+#pragma unroll
+      for (int i = 0; i < MAXC; ++i) {
+        const int c = lane + 64 * i;
+        const bool live = c < nchunks;  // whole lane groups are live or not: n is a multiple of 128
+        float gmax = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) gmax = fmaxf(gmax, fabsf(v[i][j]));
+#pragma unroll
+        for (int o = 8; o > 0; o >>= 1) gmax = fmaxf(gmax, __shfl_xor(gmax, o));
+        float scale = round_h(gmax / 7.0f);
+        if (scale == 0.0f) scale = 1.0f;
+        const ScaleDiv div(scale);
+        if (live) {
+          if ((c & 15) == 0) sout[c >> 4] = (_Float16)scale;
+          unsigned w = 0;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const float r = round_h(div(v[i][j]));
+            w |= (unsigned)((int)rintf(fminf(fmaxf(r, -7.0f), 7.0f)) & 0xF) << (4 * j);
+          }
+          *reinterpret_cast<unsigned*>(out + c * 4) = w;
+        }
+      }
+      continue;
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < MAXC; ++i)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[i][j]));  // chunks past the row hold zeros
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
+    const float upper = tag == 1 ? 127.0f : 7.0f;
+    float scale = round_h(amax / upper);   // fp16 division: fp32 quotient of two fp16 values, rounded to fp16
+    if (scale == 0.0f) scale = 1.0f;       // quantize.cuh:258
+    const ScaleDiv div(scale);
+    if (lane == 0) a.scale_store[scale_off + lrow] = (_Float16)scale;
+    uint8_t* out = a.inp_store + 2 * (inp_off + lrow * (tag == 1 ? n / 2 : n / 4));
+#pragma unroll
+    for (int i = 0; i < MAXC; ++i) {
+      const int c = lane + 64 * i;
+      if (c < nchunks) {
+        int q[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float r = round_h(div(v[i][j]));
+          q[j] = (int)rintf(fminf(fmaxf(r, -upper), upper));
+        }
+        if (tag == 1) {
+          uint2 w;
+          w.x = (q[0] & 0xFF) | ((q[1] & 0xFF) << 8) | ((q[2] & 0xFF) << 16) | ((unsigned)(q[3] & 0xFF) << 24);
+          w.y = (q[4] & 0xFF) | ((q[5] & 0xFF) << 8) | ((q[6] & 0xFF) << 16) | ((unsigned)(q[7] & 0xFF) << 24);
+          *reinterpret_cast<uint2*>(out + c * 8) = w;
+        } else {
+          unsigned w = 0;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) w |= (unsigned)(q[j] & 0xF) << (4 * j);
+          *reinterpret_cast<unsigned*>(out + c * 4) = w;
+        }
+      }
+    }
+  }
+}
+
 static int make_plan(int n, int had_k, int had_f, bool rotate, RotPlan* p) {
   p->n = n;
   p->scale = 1.0f / sqrtf((float)n);
@@ -745,6 +1078,23 @@ static int launch_rows(const RowArgs& a, int lds_bytes, hipStream_t s) {
       case 2: hipLaunchKernelGGL((row_quant_wave_kernel<2, SILU>), dim3(wgrid), dim3(256), 0, s, a); break;
       case 4: hipLaunchKernelGGL((row_quant_wave_kernel<4, SILU>), dim3(wgrid), dim3(256), 0, s, a); break;
       default: hipLaunchKernelGGL((row_quant_wave_kernel<8, SILU>), dim3(wgrid), dim3(256), 0, s, a); break;
+    }
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+      last_error() = std::string("kernel launch failed: ") + hipGetErrorString(e);
+      return 4;
+    }
+    return 0;
+  }
+  // table-driven factor times H_8, one size of row: one row per wave, dense stage on the matrix cores
+  if (a.plan.kb > 1 && a.plan.m == 8 && a.plan.f <= 4 && a.plan.kb <= 64 && n <= 2048 && a.plan_shared.n == n && a.plan_shared.kb == a.plan.kb && a.rotate != 0) {
+    const int wgrid = (a.rows + 3) / 4 < cus * 4 ? (a.rows + 3) / 4 : cus * 4;
+    const int dlds = 4 * kDenseWaveLds;
+    switch ((n / 8 + 63) / 64) {
+      case 1: hipLaunchKernelGGL((row_quant_dense_kernel<1, SILU>), dim3(wgrid), dim3(256), dlds, s, a); break;
+      case 2: hipLaunchKernelGGL((row_quant_dense_kernel<2, SILU>), dim3(wgrid), dim3(256), dlds, s, a); break;
+      case 3: hipLaunchKernelGGL((row_quant_dense_kernel<3, SILU>), dim3(wgrid), dim3(256), dlds, s, a); break;
+      default: hipLaunchKernelGGL((row_quant_dense_kernel<4, SILU>), dim3(wgrid), dim3(256), dlds, s, a); break;
     }
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) {

@@ -180,20 +180,41 @@ _LN2_LO = F32(1.428606765330187e-06)      # ln2 - LN2_HI
 _EXP_C = [F32(c) for c in (1.0, 1.0, 0.5, 0.16666667, 0.041666668, 0.008333334, 0.0013888889, 0.0001984127)]
 
 
-def exp_f32_fixed(t: np.ndarray) -> np.ndarray:
-    """exp(t) in fp32 as a FIXED sequence of individually rounded fp32 mul/add ops (no FMA).
+def fma_f32(a, b, c) -> np.ndarray:
+    """Fused multiply-add on float32 values: ``a * b + c`` rounded ONCE to float32 (what the GPU's v_fma_f32 computes).
 
-    ``k = rint(t*log2e)``, ``r = (t - k*LN2_HI) - k*LN2_LO``, degree-7 Horner polynomial, exact
-    scaling by 2^k.  The HIP kernels run the identical op sequence (contraction off), which is
-    what makes ``silu_mul`` bit-reproducible between CPU and GPU.  Relative error < 2e-7.
+    The product of two float32 values is exact in float64; the sum is taken in float64 with its exact rounding error (TwoSum),
+    and an inexact sum gets its last bit set (round to odd), after which the rounding to float32 cannot go wrong (53 >= 2*24 + 2).
+    """
+    a = np.asarray(a, F32).astype(np.float64)
+    b = np.asarray(b, F32).astype(np.float64)
+    c = np.asarray(c, F32).astype(np.float64)
+    with np.errstate(invalid="ignore", over="ignore"):
+        p = a * b
+        s = p + c
+        bb = s - p
+        err = (p - (s - bb)) + (c - bb)
+        bits = s.view(np.int64)
+        fix = (err != 0) & ((bits & 1) == 0) & np.isfinite(s)
+        up = (err > 0) == (s > 0)
+        bits = np.where(fix, np.where(up, bits + 1, bits - 1), bits)
+        return bits.view(np.float64).astype(F32)
+
+
+def exp_f32_fixed(t: np.ndarray) -> np.ndarray:
+    """exp(t) in fp32 as a FIXED sequence of correctly rounded fp32 operations.
+
+    ``k = rint(t*log2e)``, ``r = fma(-k, LN2_LO, fma(-k, LN2_HI, t))``, degree-7 Horner polynomial of fused multiply-adds,
+    exact scaling by 2^k.  The HIP kernels run the identical op sequence, which is what makes ``silu_mul`` bit-reproducible
+    between CPU and GPU.  Relative error < 2e-7.
     """
     t = np.clip(t.astype(F32), F32(-87.0), F32(87.0))
     k = np.rint((t * _LOG2E).astype(F32)).astype(F32)
-    r = (t - (k * _LN2_HI).astype(F32)).astype(F32)
-    r = (r - (k * _LN2_LO).astype(F32)).astype(F32)
+    r = fma_f32(-k, _LN2_HI, t)
+    r = fma_f32(-k, _LN2_LO, r)
     p = np.full_like(r, _EXP_C[7])
     for c in _EXP_C[6::-1]:
-        p = ((p * r).astype(F32) + c).astype(F32)
+        p = fma_f32(p, r, c)
     return np.ldexp(p, k.astype(np.int32)).astype(F32)
 
 
@@ -286,6 +307,21 @@ def had_factor(k: int):
     return f, kb, h[:kb, :kb].copy()
 
 
+def dense_grid(v: np.ndarray):
+    """Per-row power-of-two factors of the dense ``B`` stage of ``online_hadamard``: ``(to_grid, from_grid)`` float32 ``[rows, 1]``.
+
+    With ``max|v| < 2^E`` over the row (E from the exponent field of the fp32 maximum; NaNs are ignored), ``to_grid = 2^(17-E)``
+    maps the row onto integers of magnitude <= 2^17 and ``from_grid = 2^(E-13)`` maps sums of those integers divided by 16 (the
+    form the HIP kernel feeds to the fp16 matrix instruction: at most 11 significant bits, 2^-4 <= |.| <= 2^13) back.  An
+    all-zero row gets (1, 1).
+    """
+    mx = np.fmax.reduce(np.abs(v.astype(F32)), axis=1, keepdims=True).astype(F32)
+    e_field = (mx.view(np.uint32) >> 23).astype(np.int64)
+    to_grid = np.where(e_field == 0, 127 << 23, (270 - e_field) << 23).astype(np.uint32).view(F32)
+    from_grid = np.where(e_field == 0, 127 << 23, np.maximum(e_field - 12, 1) << 23).astype(np.uint32).view(F32)
+    return to_grid, from_grid
+
+
 def online_hadamard(x: np.ndarray) -> np.ndarray:
     """Online rotation of fp16 rows: ``y = (H_K kron H_{n/K}) x / sqrt(n)``, index ``p = k*(n/K) + j``.
 
@@ -294,9 +330,13 @@ def online_hadamard(x: np.ndarray) -> np.ndarray:
     PARITY UNPINNED at the last fp16 bit (third-party kernel + backend matmul order, see module
     header).  This build's definition, which the HIP kernels reproduce bit for bit:
       1. fp32 ``sylvester_fwht`` along ``n/K`` (ascending strides), one fp32 multiply by ``had_scale(n)``, round to fp16;
-      2. K > 1, with ``H_K = S_f kron B`` (``had_factor``): inside each of the f blocks of Kb rows,
-         ``t[b] = sum_{b'} B[b,b'] v[b']`` accumulated in fp32 from 0 over ``b' = 0..Kb-1`` in order; then the
-         ``S_f`` butterflies across blocks in fp32 (ascending strides); one rounding to fp16.
+      2. K > 1, with ``H_K = S_f kron B`` (``had_factor``): the row's fp16 values are snapped (round to nearest even) to the
+         grid of step ``2^(E-17)``, ``max|v| < 2^E`` over the row (``dense_grid``); inside each of the f blocks of Kb rows
+         ``t[b] = sum_{b'} B[b,b'] v[b']`` is then an EXACT sum (integers below 2^17 times Kb <= 64 < 2^7 terms stay below
+         2^24), so its value does not depend on the order or the width of the accumulation and the kernel may leave it to
+         the matrix cores; then the ``S_f`` butterflies across blocks in fp32 (ascending strides); one rounding to fp16.
+         Snapping moves a value by at most 2^-18 of the row's largest one, far below the fp16 rounding of step 1 and the
+         int4 / int8 quantisation step that follows.  Rows that hold an infinity or a NaN give unspecified values.
     """
     assert x.dtype == F16
     n = x.shape[-1]
@@ -307,11 +347,13 @@ def online_hadamard(x: np.ndarray) -> np.ndarray:
     if k == 1:
         return v.reshape(x.shape)
     f, kb, b = had_factor(k)
-    vf = v.astype(F32).reshape(-1, f, kb, m)
-    acc = np.zeros_like(vf)
-    for bp in range(kb):  # fixed sequential order
-        sgn = b[:, bp].astype(F32).reshape(1, 1, kb, 1)
-        acc = (acc + sgn * vf[:, :, bp:bp + 1, :]).astype(F32)
+    assert kb <= 64
+    rows = v.shape[0]
+    to_grid, from_grid = dense_grid(v.reshape(rows, n))
+    q = np.rint((v.astype(F32).reshape(rows, n) * to_grid).astype(F32)).reshape(rows, f, kb, m)  # integers, |q| <= 2^17
+    with np.errstate(invalid="ignore", over="ignore"):
+        t = np.einsum("cb,rfbm->rfcm", b.astype(np.float64), q.astype(np.float64) / 16.0)        # exact in float64
+        acc = (t.astype(F32) * from_grid.reshape(rows, 1, 1, 1)).astype(F32)                     # exact: |16 t| < 2^24, power-of-two factor
     # S_f butterflies across the block index (axis 1): move it last, transform, move back
     acc = np.moveaxis(sylvester_fwht(np.ascontiguousarray(np.moveaxis(acc, 1, -1))), -1, 1)
     return acc.astype(F16).reshape(x.shape)

@@ -42,7 +42,8 @@ def _unpack(store_view, tag, n):
     return np.where(q >= 8, q - 16, q).astype(np.int8)
 
 
-@pytest.mark.parametrize("k,rotate", [(2048, 1), (4096, 1), (256, 0), (2048, 2), (512, 1), (1024, 2), (2048, 0), (256, 1), (8192, 1), (2816, 2), (14336, 1)])
+@pytest.mark.parametrize("k,rotate", [(2048, 1), (4096, 1), (256, 0), (2048, 2), (512, 1), (1024, 2), (2048, 0), (256, 1), (8192, 1), (2816, 2), (14336, 1),
+                                      (1408, 1), (1408, 2), (224, 2), (96, 1)])
 def test_quant_inp_act_bit_exact(k, rotate):
     from mxmoe_amd import ops
 
@@ -53,6 +54,8 @@ def test_quant_inp_act_bit_exact(k, rotate):
     ids = _ids(rng, t, e, topk)
     ids[ids == 4] = 5 if False else ids[ids == 4]
     qp = [(4, 4, -1, True), (8, 8, -1, True), (16, 4, 128, False), (4, 4, 128, True), (8, 8, -1, True), (16, 16, -1, True), (8, 8, -1, True)]
+    if k % 128:                                                            # group-128 activations need rows that are multiples of 128
+        qp[3] = (4, 4, -1, True)
     res = ops.quant_inp_act(torch.from_numpy(x).to(DEV), torch.from_numpy(ids).to(DEV), e, 1408, n_sh, qp, rotate=rotate)
     inp_list, scale_list, out_list, inp_store, scale_store, out_store, recv, perm, dst = res
     torch.cuda.synchronize()
@@ -83,7 +86,7 @@ def test_quant_inp_act_bit_exact(k, rotate):
     assert p == len(inp_list)
 
 
-@pytest.mark.parametrize("n,n_sh,rotate", [(1408, 2, 2), (2048, 0, 1), (14336, 0, 1), (512, 1, 0)])
+@pytest.mark.parametrize("n,n_sh,rotate", [(1408, 2, 2), (2048, 0, 1), (14336, 0, 1), (512, 1, 0), (1408, 0, 1), (1408, 1, 2), (224, 0, 2), (96, 1, 1)])
 def test_silu_mul_then_quant_bit_exact(n, n_sh, rotate):
     from mxmoe_amd import ops
 
@@ -96,6 +99,8 @@ def test_silu_mul_then_quant_bit_exact(n, n_sh, rotate):
     gu_sh = (rng.standard_normal((t, 2 * n * max(n_sh, 1))) * 2).astype(F16)
     flat = np.concatenate([gu.reshape(-1), gu_sh.reshape(-1)]) if n_sh else gu.reshape(-1)
     qp = [(4, 4, -1, True), (8, 8, -1, True), (16, 4, 128, False), (4, 4, 128, True), (8, 8, -1, True)]
+    if n % 128:
+        qp[3] = (8, 8, -1, True)
     res = ops.silu_mul_then_quant(torch.from_numpy(flat).to(DEV), int((o_recv != 0).sum()), e, 2048, n, n_sh, t, topk,
                                   torch.from_numpy(o_dst).to(DEV), torch.from_numpy(o_recv), qp, rotate=rotate)
     inp_list, scale_list, out_list = res[:3]

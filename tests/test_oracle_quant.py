@@ -138,6 +138,38 @@ def test_fakequant_path_agrees_with_integer_path_within_tolerance():
         assert rel < 1e-2 and acc.dtype == np.int32
 
 
+def test_fma_f32_is_one_correct_rounding():
+    """The oracle's fused multiply-add against exact rational arithmetic, including products that cancel against the addend and
+    results that sit next to a float32 rounding boundary (where rounding the float64 sum a second time would go wrong)."""
+    from fractions import Fraction
+
+    rng = np.random.default_rng(8)
+    n = 3000
+    a = (rng.standard_normal(n) * 10.0 ** rng.integers(-6, 6, n)).astype(np.float32)
+    b = (rng.standard_normal(n) * 10.0 ** rng.integers(-6, 6, n)).astype(np.float32)
+    c = (rng.standard_normal(n) * 10.0 ** rng.integers(-8, 8, n)).astype(np.float32)
+    c[:1000] = (-(a[:1000].astype(np.float64) * b[:1000].astype(np.float64))).astype(np.float32)          # near-total cancellation
+    # a * b = (1 + 2^-12)^2 = 1 + 2^-11 + 2^-24; with c = 2^-24 + tiny the exact sum lies just above a float32 tie
+    a[1000:1010] = np.float32(1 + 2.0**-12)
+    b[1000:1010] = np.float32(1 + 2.0**-12)
+    c[1000:1010] = np.float32(2.0**-24) * np.float32(1 + 2.0**-20) * np.arange(1, 11, dtype=np.float32)
+    got = O.fma_f32(a, b, c)
+
+    def exact(x, y, z):
+        v = Fraction(float(x)) * Fraction(float(y)) + Fraction(float(z))
+        near = np.float32(float(v))
+        best = None
+        for cand in (near, np.nextafter(near, np.float32(np.inf)), np.nextafter(near, np.float32(-np.inf))):
+            key = (abs(Fraction(float(cand)) - v), int(np.asarray(cand).view(np.uint32)) & 1)   # nearest, ties to even
+            if best is None or key < best[0]:
+                best = (key, cand)
+        return best[1]
+
+    for i in range(n):
+        assert got[i] == exact(a[i], b[i], c[i]), i
+    assert O.fma_f32(np.float32(3), np.float32(4), np.float32(5)) == 17
+
+
 def test_exp_fixed_and_silu_mul():
     t = np.linspace(-87, 87, 20001).astype(np.float32)
     rel = np.abs(O.exp_f32_fixed(t).astype(np.float64) / np.exp(t.astype(np.float64)) - 1)
