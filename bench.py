@@ -208,15 +208,32 @@ def time_whole_layer(cfg, layer, reps: int = 7) -> dict:
     parts = {k: sorted(v)[len(v) // 2] for k, v in samples.items()}
     out = {f"{k}_ms": round(v, 4) for k, v in parts.items()}
     out["layer_ms"] = round(sum(parts.values()), 4)
-    # the same forward as one call (all host tables in one pass, no synchronisation between the steps)
-    whole = []
-    for rep in range(reps + 2):
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        layer(hidden, ids, w)
-        torch.cuda.synchronize()
-        whole.append((time.perf_counter() - t0) * 1e3)
-    out["one_call_ms"] = round(sorted(whole[2:])[len(whole[2:]) // 2], 4)
+    # the same forward as one call: tables planned on the device, no synchronisation, persistent buffers
+    out_buf = torch.empty((cfg.tokens, cfg.hidden), dtype=torch.float16, device="cuda")
+
+    def wall(fn):
+        ts = []
+        for rep in range(reps + 2):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            fn()
+            torch.cuda.synchronize()
+            ts.append((time.perf_counter() - t0) * 1e3)
+        ts = sorted(ts[2:])
+        return round(ts[len(ts) // 2], 4)
+
+    out["one_call_ms"] = wall(lambda: layer(hidden, ids, w, out=out_buf))
+    out["one_call_host_tables_ms"] = wall(lambda: layer.call_with_host_tables(hidden, ids, w))   # tables built on the host after reading the counts back
+    # ... and replayed from a HIP graph
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        layer(hidden, ids, w, out=out_buf)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        layer(hidden, ids, w, out=out_buf)
+    out["graph_replay_ms"] = wall(graph.replay)
     return out
 
 

@@ -146,6 +146,52 @@ size_t mxmoe_combine_workspace_bytes(int num_tokens, int topk);
 int mxmoe_unpermute_combine(const void* down_out, const void* shared_out, const float* topk_weights, const int64_t* src_slot, int rows, int num_tokens, int topk,
                             int K, void* out, void* workspace, void* stream);
 
+/* ---- a layer forward that never waits for its routing (no counterpart in the reference, whose operators copy the tokens-per-expert
+ *      counts to the host and build every table there: mxmoe/kernels/src/ref_bind.cu:451, 475-505, 362-404, kernel_sketch.py:89-104) ----
+ *
+ * For callers that cannot synchronise or must not let launch arguments depend on the data (HIP graph capture, serving loops): one
+ * small kernel per linear block derives, from recv_tokens_per_exp in DEVICE memory, everything the host launcher computes from its
+ * host copy (per-expert {tag, first row, offsets} table of the quantisers, the five pointer arrays, the sizes, the tile tables of the
+ * fused launch) into a plan buffer; the *_planned entry points read their tables from it.  Same kernels, same results.
+ *
+ * A block is described per expert by mxmoe_block_desc {QParams, N, K, packed weights, weight scales} (d_desc in device memory, h_desc
+ * its host mirror; the shared expert, when shared_rows > 0, is entry num_experts and has shared_rows rows).  At most 120 problems.
+ * Stores are laid out as the host path lays them out (experts in order, rows packed), so they must be sized for the worst case:
+ * capacity rows x the widest row of any expert.
+ *
+ *   mxmoe_plan_bytes(P)            size of a plan buffer for P problems (device memory, owned by the caller, reusable);
+ *   mxmoe_plan_offset(which, P)    byte offset inside it of: 1 the quantisers' int64 [4][P] table, 2 the pointer arrays void* [5][P]
+ *                                  (A, B, scale_a, scale_b, C), 3 two int64 {rows routed, address of the shared expert's output rows},
+ *                                  4 the sizes mxmoe_dim3 [P];
+ *   mxmoe_plan_select_kernel       the kernel (>= 0) that mxmoe_plan_block / mxmoe_plan_grid_bound use for these formats when given -1, after
+ *                                  checking formats and shapes; negative on error;
+ *   mxmoe_plan_grid_bound          workgroups that cover the launch whatever the routing, for at most routed_rows_max routed rows
+ *                                  (tokens x top-k): per expert tiles(M) <= tiles(1) + slope * (M - 1), summed over the non-empty experts
+ *                                  (workgroups past the planned tiles cost about 10 - 20 ns each, so the bound is kept tight);
+ *   mxmoe_plan_block               enqueue the planning kernel for one block (inp_store / scale_store: the packed activations and
+ *                                  their scales that the block reads, out_store: where its output rows go);
+ *   mxmoe_group_gemm_planned       the fused launch, grid from mxmoe_plan_grid_bound (workgroups past the planned tiles exit at once);
+ *   mxmoe_quant_act_planned, mxmoe_silu_mul_quant_planned, mxmoe_unpermute_combine_planned
+ *                                  as their namesakes, with d_plan in place of exp_table / row counts / shared-expert pointers;
+ *                                  rows_capacity = tokens x top-k (rows that were not routed because their expert id was out of
+ *                                  range are skipped on the device); d_plan_gate_up is the first launch's plan, whose output the
+ *                                  SiLU step reads. */
+size_t mxmoe_plan_bytes(int num_problems);
+size_t mxmoe_plan_offset(int which, int num_problems);
+int mxmoe_plan_select_kernel(int kernel_id, const mxmoe_block_desc* h_desc, int num_problems);
+int mxmoe_plan_grid_bound(int kernel_id, const mxmoe_block_desc* h_desc, int num_experts, int routed_rows_max, int shared_rows);
+int mxmoe_plan_block(int kernel_id, const int64_t* d_recv_tokens_per_exp, int num_experts, int shared_rows, const mxmoe_block_desc* d_desc,
+                     const mxmoe_block_desc* h_desc, const void* inp_store, const void* scale_store, void* out_store, void* d_plan, void* stream);
+int mxmoe_group_gemm_planned(int kernel_id, const void* d_plan, int grid, void* stream);
+int mxmoe_quant_act_planned(const void* hidden, void* inp_store, void* scale_store, const int32_t* dst_exp_sorted, const int64_t* perm_indices, const void* d_plan,
+                            int K, int rows_capacity, int num_tokens, int num_experts, int has_shared, int rotate, int had_k, int had_f, const float* had_signs,
+                            void* stream);
+int mxmoe_silu_mul_quant_planned(const void* gate_up, const void* d_plan_gate_up, void* inp_store, void* scale_store, const int32_t* dst_exp_sorted, const void* d_plan,
+                                 int N, int N_shared, int rows_capacity, int num_tokens, int num_experts, int has_shared, int rotate, int had_k, int had_f,
+                                 const float* had_signs, void* stream);
+int mxmoe_unpermute_combine_planned(const void* down_out, const void* d_plan_down, int num_problems, const float* topk_weights, const int64_t* src_slot, int num_tokens,
+                                    int topk, int K, void* out, void* workspace, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -11,6 +11,12 @@ class Dim3(C.Structure):
     _fields_ = [("x", C.c_uint32), ("y", C.c_uint32), ("z", C.c_uint32)]
 
 
+class BlockDesc(C.Structure):
+    """mxmoe_block_desc: one linear block of one expert for the device-side planner (40 bytes)."""
+    _fields_ = [("a_bits", C.c_int32), ("w_bits", C.c_int32), ("gsize", C.c_int32), ("sym", C.c_uint8), ("_pad", C.c_uint8 * 3),
+                ("N", C.c_uint32), ("K", C.c_uint32), ("B", C.c_void_p), ("scale_b", C.c_void_p)]
+
+
 class QParams(C.Structure):
     _fields_ = [("a_bits", C.c_int32), ("w_bits", C.c_int32), ("gsize", C.c_int32), ("sym", C.c_uint8), ("_pad", C.c_uint8 * 3)]
 
@@ -40,6 +46,15 @@ SIGNATURES = {
     "mxmoe_set_stream": (None, [_P]),
     "mxmoe_get_stream": (_P, []),
     "mxmoe_last_status": (_I, []),
+    "mxmoe_plan_bytes": (C.c_size_t, [_I]),
+    "mxmoe_plan_offset": (C.c_size_t, [_I, _I]),
+    "mxmoe_plan_select_kernel": (_I, [_I, _P, _I]),
+    "mxmoe_plan_grid_bound": (_I, [_I, _P, _I, _I, _I]),
+    "mxmoe_plan_block": (_I, [_I, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P]),
+    "mxmoe_group_gemm_planned": (_I, [_I, _P, _I, _P]),
+    "mxmoe_quant_act_planned": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P]),
+    "mxmoe_silu_mul_quant_planned": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P]),
+    "mxmoe_unpermute_combine_planned": (_I, [_P, _P, _I, _P, _P, _I, _I, _I, _P, _P, _P]),
     "mxmoe_combine_workspace_bytes": (C.c_size_t, [_I, _I]),
     "mxmoe_unpermute_combine": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P]),
 }

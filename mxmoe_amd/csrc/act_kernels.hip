@@ -21,6 +21,7 @@
 
 #include "../../include/mxmoe_amd.h"
 #include "include/mxmoe_launch.hpp"
+#include "include/mxmoe_plan.hpp"
 
 namespace mxmoe {
 
@@ -141,7 +142,18 @@ struct RowArgs {
   int rows;
   int rotate;  // 0 never, 1 rows of quantised experts, 2 every row
   RotPlan plan, plan_shared;
+  // Planned mode (the tables were written by the device-side planner, the host never saw the counts): R is then the CAPACITY of the
+  // routed part (tokens x top-k), rows routed .. R-1 do not exist when expert ids were dropped, and the shared expert's source rows
+  // are wherever the planner put them.  Both null otherwise.
+  const int64_t* routed_ptr;       // rows that were routed
+  const int64_t* shared_src_addr;  // address of the shared expert's source rows
 };
+
+// rows [routed, R) of a planned launch do not exist
+__device__ __forceinline__ bool row_exists(const RowArgs& a, int row) { return !a.routed_ptr || row >= a.R || row < (int)*a.routed_ptr; }
+__device__ __forceinline__ const _Float16* shared_src(const RowArgs& a) {
+  return a.shared_src_addr ? reinterpret_cast<const _Float16*>(*a.shared_src_addr) : a.src_shared;
+}
 
 // fixed fp32 op sequence for exp(t), identical to the CPU restatement: every step is one correctly rounded operation (the
 // multiply-adds are fused: one rounding each)
@@ -244,21 +256,23 @@ __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
     int e, tag;
     long start_row, inp_off, scale_off;
     const _Float16* srow;
-    bool shared_row;
+    bool shared_row, exists;
   };
+  const _Float16* const src_shared = shared_src(a);
   auto load_meta = [&](int row) {
     RowMeta m;
     m.shared_row = row >= a.R;
-    m.e = m.shared_row ? a.E : a.dst_exp[row];
+    m.exists = row_exists(a, row);
+    m.e = m.shared_row ? a.E : (m.exists ? a.dst_exp[row] : 0);
     m.tag = (int)a.table[m.e];
     m.start_row = a.table[a.Et + m.e];
     m.inp_off = a.table[2 * a.Et + m.e];
     m.scale_off = a.table[3 * a.Et + m.e];
     const int n = (m.shared_row ? a.plan_shared : a.plan).n;
     if (SILU) {
-      m.srow = m.shared_row ? a.src_shared + (long)(row - a.R) * 2 * n : a.src + (long)row * 2 * n;
+      m.srow = m.shared_row ? src_shared + (long)(row - a.R) * 2 * n : a.src + (long)row * 2 * n;
     } else {
-      m.srow = a.src + (m.shared_row ? (long)(row - a.R) : (long)a.perm[row]) * n;
+      m.srow = (m.shared_row ? src_shared : a.src) + (m.shared_row ? (long)(row - a.R) : (m.exists ? (long)a.perm[row] : 0l)) * n;
     }
     return m;
   };
@@ -292,6 +306,7 @@ __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
       next_meta = load_meta(row + gridDim.x);
       load_data(next_meta, next_g, next_u);
     }
+    if (!cur.exists) continue;  // (the whole workgroup: a row belongs to one workgroup)
     const bool shared_row = cur.shared_row;
     const RotPlan pl = shared_row ? a.plan_shared : a.plan;
     const int n = pl.n;
@@ -299,7 +314,7 @@ __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
     const int tag = cur.tag;
     const long inp_off = cur.inp_off;
     const long scale_off = cur.scale_off;
-    const long lrow = row - cur.start_row;
+    const long lrow = shared_row ? row - a.R : row - cur.start_row;  // (the shared expert's first row is R only when every row was routed)
     const bool rot = a.rotate == 2 || (a.rotate == 1 && tag != 0);
 
     float v[MAXC][8];
@@ -591,19 +606,21 @@ __global__ void __launch_bounds__(256) row_quant_wave_kernel(const RowArgs a) {
   const int wave = threadIdx.x >> 6;
   const int n = a.plan.n;  // == a.plan_shared.n == 512 * NI
   const int stride_rows = gridDim.x * 4;
+  const _Float16* const src_shared = shared_src(a);
   for (int row = blockIdx.x * 4 + wave; row < a.rows; row += stride_rows) {
+    if (!row_exists(a, row)) continue;
     const bool shared_row = row >= a.R;
     const int e = shared_row ? a.E : a.dst_exp[row];
     const int tag = (int)a.table[e];
-    const long lrow = row - a.table[a.Et + e];
+    const long lrow = shared_row ? row - a.R : row - a.table[a.Et + e];
     const long inp_off = a.table[2 * a.Et + e];
     const long scale_off = a.table[3 * a.Et + e];
     const bool rot = a.rotate == 2 || (a.rotate == 1 && tag != 0);
     const _Float16* srow;
     if (SILU) {
-      srow = shared_row ? a.src_shared + (long)(row - a.R) * 2 * n : a.src + (long)row * 2 * n;
+      srow = shared_row ? src_shared + (long)(row - a.R) * 2 * n : a.src + (long)row * 2 * n;
     } else {
-      srow = a.src + (shared_row ? (long)(row - a.R) : (long)a.perm[row]) * n;
+      srow = (shared_row ? src_shared : a.src) + (shared_row ? (long)(row - a.R) : (long)a.perm[row]) * n;
     }
     float v[NI][8];
 #pragma unroll
@@ -786,19 +803,22 @@ __global__ void __launch_bounds__(256) row_quant_dense_kernel(const RowArgs a) {
     int tag;
     long lrow, inp_off, scale_off;
     const _Float16* srow;
+    bool exists;
   };
+  const _Float16* const src_shared = shared_src(a);
   auto load_meta = [&](int row) {
     RowMeta m;
     const bool shared_row = row >= a.R;
-    const int e = shared_row ? a.E : a.dst_exp[row];
+    m.exists = row_exists(a, row);
+    const int e = shared_row ? a.E : (m.exists ? a.dst_exp[row] : 0);
     m.tag = (int)a.table[e];
-    m.lrow = row - a.table[a.Et + e];
+    m.lrow = shared_row ? row - a.R : row - a.table[a.Et + e];
     m.inp_off = a.table[2 * a.Et + e];
     m.scale_off = a.table[3 * a.Et + e];
     if (SILU) {
-      m.srow = shared_row ? a.src_shared + (long)(row - a.R) * 2 * n : a.src + (long)row * 2 * n;
+      m.srow = shared_row ? src_shared + (long)(row - a.R) * 2 * n : a.src + (long)row * 2 * n;
     } else {
-      m.srow = a.src + (shared_row ? (long)(row - a.R) : (long)a.perm[row]) * n;
+      m.srow = (shared_row ? src_shared : a.src) + (shared_row ? (long)(row - a.R) : (m.exists ? (long)a.perm[row] : 0l)) * n;
     }
     return m;
   };
@@ -830,6 +850,7 @@ __global__ void __launch_bounds__(256) row_quant_dense_kernel(const RowArgs a) {
       next_meta = load_meta(row + stride_rows);
       load_data(next_meta, next_g, next_u);
     }
+    if (!cur.exists) continue;
     const int tag = cur.tag;
     const bool rot = a.rotate == 2 || (a.rotate == 1 && tag != 0);
     float v[MAXC][8];
@@ -1145,8 +1166,10 @@ __global__ void combine_fill_kernel(int32_t* __restrict__ row_of_slot, int slots
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < slots) row_of_slot[i] = -1;
 }
-__global__ void combine_invert_kernel(const int64_t* __restrict__ src_slot, int rows, int slots, int32_t* __restrict__ row_of_slot) {
+__global__ void combine_invert_kernel(const int64_t* __restrict__ src_slot, int rows, int slots, int32_t* __restrict__ row_of_slot,
+                                      const int64_t* __restrict__ rows_ptr) {
   const int r = blockIdx.x * blockDim.x + threadIdx.x;
+  if (rows_ptr) rows = min(rows, (int)*rows_ptr);  // planned mode: `rows` is the capacity, the routed rows are counted on the device
   if (r < rows) {
     const int64_t sl = src_slot[r];
     if (sl >= 0 && sl < slots) row_of_slot[sl] = r;
@@ -1155,8 +1178,10 @@ __global__ void combine_invert_kernel(const int64_t* __restrict__ src_slot, int 
 // One workgroup per token: out[t] = half( sum_k w[t,k] * float(down[row(t,k)])  (k ascending, fp32: product rounded, then the
 // sum rounded)  + float(shared[t]) ).  Pure streaming: every down row is read once, 16 bytes per lane.
 __global__ void __launch_bounds__(256) combine_kernel(const _Float16* __restrict__ down, const _Float16* __restrict__ shared, const float* __restrict__ weights,
-                                                      const int32_t* __restrict__ row_of_slot, int topk, int K, _Float16* __restrict__ out) {
+                                                      const int32_t* __restrict__ row_of_slot, int topk, int K, _Float16* __restrict__ out,
+                                                      const int64_t* __restrict__ shared_addr) {
   const int t = blockIdx.x;
+  if (shared_addr) shared = reinterpret_cast<const _Float16*>(*shared_addr);  // planned mode: where the planner put the shared expert's rows (0: none)
   for (int c = threadIdx.x * 8; c < K; c += 256 * 8) {
     float acc[8];
 #pragma unroll
@@ -1347,6 +1372,77 @@ int mxmoe_silu_mul_quant(const void* gate_up, const void* gate_up_shared, void* 
   return launch_rows<true>(a, lds, (hipStream_t)stream);
 }
 
+// ---- the same three steps behind a device-side plan (mxmoe_plan_block): nothing here depends on the routing ----
+int mxmoe_quant_act_planned(const void* hidden, void* inp_store, void* scale_store, const int32_t* dst_exp_sorted, const int64_t* perm_indices, const void* d_plan,
+                            int K, int rows_capacity, int num_tokens, int num_experts, int has_shared, int rotate, int had_k, int had_f, const float* had_signs,
+                            void* stream) {
+  if (rows_capacity <= 0 || num_tokens < 0 || num_experts <= 0) {
+    last_error() = "bad row or expert count";
+    return 3;
+  }
+  if (!hidden || !inp_store || !d_plan || !dst_exp_sorted || !perm_indices) {
+    last_error() = "null pointer";
+    return 5;
+  }
+  const int et = num_experts + (has_shared ? 1 : 0);
+  const PlanLayout lay(et);
+  const uint8_t* plan = reinterpret_cast<const uint8_t*>(d_plan);
+  RowArgs a{};
+  a.src = a.src_shared = reinterpret_cast<const _Float16*>(hidden);
+  a.inp_store = reinterpret_cast<uint8_t*>(inp_store);
+  a.scale_store = reinterpret_cast<_Float16*>(scale_store);
+  a.dst_exp = dst_exp_sorted;
+  a.perm = perm_indices;
+  a.table = reinterpret_cast<const int64_t*>(plan + lay.table);
+  a.routed_ptr = reinterpret_cast<const int64_t*>(plan + lay.misc);
+  a.R = rows_capacity;
+  a.T = num_tokens;
+  a.E = num_experts;
+  a.Et = et;
+  a.rows = rows_capacity + (has_shared ? num_tokens : 0);
+  a.rotate = rotate;
+  if (const int rc = fill_common(a, K, K, rotate ? had_k : 1, rotate ? had_f : 1, had_signs)) return rc;
+  const int lds = (K + a.plan.kb * a.plan.kb + 16) * (int)sizeof(float);
+  return launch_rows<false>(a, lds, (hipStream_t)stream);
+}
+
+int mxmoe_silu_mul_quant_planned(const void* gate_up, const void* d_plan_gate_up, void* inp_store, void* scale_store, const int32_t* dst_exp_sorted, const void* d_plan,
+                                 int N, int N_shared, int rows_capacity, int num_tokens, int num_experts, int has_shared, int rotate, int had_k, int had_f,
+                                 const float* had_signs, void* stream) {
+  if (rows_capacity <= 0 || num_tokens < 0 || num_experts <= 0) {
+    last_error() = "bad row or expert count";
+    return 3;
+  }
+  if (!gate_up || !inp_store || !d_plan || !dst_exp_sorted || !d_plan_gate_up) {
+    last_error() = "null pointer";
+    return 5;
+  }
+  const int et = num_experts + (has_shared ? 1 : 0);
+  const PlanLayout lay(et);
+  const uint8_t* plan = reinterpret_cast<const uint8_t*>(d_plan);
+  RowArgs a{};
+  a.src = reinterpret_cast<const _Float16*>(gate_up);
+  a.src_shared = nullptr;
+  // the shared expert's gate_up rows are the output of problem E of the first launch: the planner of that launch left their address
+  a.shared_src_addr = has_shared ? reinterpret_cast<const int64_t*>(reinterpret_cast<const uint8_t*>(d_plan_gate_up) + lay.misc) + 1 : nullptr;
+  a.inp_store = reinterpret_cast<uint8_t*>(inp_store);
+  a.scale_store = reinterpret_cast<_Float16*>(scale_store);
+  a.dst_exp = dst_exp_sorted;
+  a.perm = nullptr;
+  a.table = reinterpret_cast<const int64_t*>(plan + lay.table);
+  a.routed_ptr = reinterpret_cast<const int64_t*>(plan + lay.misc);
+  a.R = rows_capacity;
+  a.T = num_tokens;
+  a.E = num_experts;
+  a.Et = et;
+  a.rows = rows_capacity + (has_shared ? num_tokens : 0);
+  a.rotate = rotate;
+  if (const int rc = fill_common(a, N, has_shared ? N_shared : N, rotate ? had_k : 1, rotate ? had_f : 1, had_signs)) return rc;
+  const int nmax = N > a.plan_shared.n ? N : a.plan_shared.n;
+  const int lds = (nmax + a.plan.kb * a.plan.kb + 16) * (int)sizeof(float);
+  return launch_rows<true>(a, lds, (hipStream_t)stream);
+}
+
 size_t mxmoe_combine_workspace_bytes(int num_tokens, int topk) { return (size_t)num_tokens * topk * sizeof(int32_t); }
 
 int mxmoe_unpermute_combine(const void* down_out, const void* shared_out, const float* topk_weights, const int64_t* src_slot, int rows, int num_tokens, int topk,
@@ -1363,9 +1459,35 @@ int mxmoe_unpermute_combine(const void* down_out, const void* shared_out, const 
   const int slots = num_tokens * topk;
   int32_t* row_of_slot = reinterpret_cast<int32_t*>(workspace);
   hipLaunchKernelGGL(combine_fill_kernel, dim3((slots + 255) / 256), dim3(256), 0, s, row_of_slot, slots);
-  if (rows > 0) hipLaunchKernelGGL(combine_invert_kernel, dim3((rows + 255) / 256), dim3(256), 0, s, src_slot, rows, slots, row_of_slot);
+  if (rows > 0) hipLaunchKernelGGL(combine_invert_kernel, dim3((rows + 255) / 256), dim3(256), 0, s, src_slot, rows, slots, row_of_slot, (const int64_t*)nullptr);
   hipLaunchKernelGGL(combine_kernel, dim3(num_tokens), dim3(256), 0, s, reinterpret_cast<const _Float16*>(down_out), reinterpret_cast<const _Float16*>(shared_out),
-                     topk_weights, row_of_slot, topk, K, reinterpret_cast<_Float16*>(out));
+                     topk_weights, row_of_slot, topk, K, reinterpret_cast<_Float16*>(out), (const int64_t*)nullptr);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    last_error() = std::string("kernel launch failed: ") + hipGetErrorString(e);
+    return 4;
+  }
+  return 0;
+}
+
+int mxmoe_unpermute_combine_planned(const void* down_out, const void* d_plan_down, int num_problems, const float* topk_weights, const int64_t* src_slot, int num_tokens,
+                                    int topk, int K, void* out, void* workspace, void* stream) {
+  if (num_tokens <= 0 || topk <= 0 || K <= 0 || K % 8 || num_problems <= 0) {
+    last_error() = "bad combine size (K must be a multiple of 8)";
+    return 3;
+  }
+  if (!down_out || !d_plan_down || !topk_weights || !src_slot || !out || !workspace) {
+    last_error() = "null pointer";
+    return 5;
+  }
+  hipStream_t s = (hipStream_t)stream;
+  const int slots = num_tokens * topk;
+  const int64_t* misc = reinterpret_cast<const int64_t*>(reinterpret_cast<const uint8_t*>(d_plan_down) + PlanLayout(num_problems).misc);
+  int32_t* row_of_slot = reinterpret_cast<int32_t*>(workspace);
+  hipLaunchKernelGGL(combine_fill_kernel, dim3((slots + 255) / 256), dim3(256), 0, s, row_of_slot, slots);
+  hipLaunchKernelGGL(combine_invert_kernel, dim3((slots + 255) / 256), dim3(256), 0, s, src_slot, slots, slots, row_of_slot, misc);
+  hipLaunchKernelGGL(combine_kernel, dim3(num_tokens), dim3(256), 0, s, reinterpret_cast<const _Float16*>(down_out), (const _Float16*)nullptr, topk_weights, row_of_slot,
+                     topk, K, reinterpret_cast<_Float16*>(out), misc + 1);
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     last_error() = std::string("kernel launch failed: ") + hipGetErrorString(e);

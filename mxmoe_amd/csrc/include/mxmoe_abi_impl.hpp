@@ -87,9 +87,9 @@ int mxmoe_group_gemm_plan(int kernel_id, const mxmoe_dim3* h_sizes, const mxmoe_
   for (int i = 0; i < problem_count; ++i) {
     const Fmt f = classify(h_q[i]);
     Segment sg[2];
-    const int ns = f == Fmt::UNSUPPORTED ? -1 : plan_segments(k, f, (int)h_sizes[i].x, (int)h_sizes[i].y, sg);
+    const int ns = f == Fmt::UNSUPPORTED ? -1 : plan_segments(plan_of(k), (int)f, (int)h_sizes[i].x, (int)h_sizes[i].y, sg);
     if (ns < 0) { last_error() = "quant type not supported"; return 1; }
-    if (branch_out) branch_out[i] = ns ? sg[0].branch : pick_branch(k, f, 1, (int)h_sizes[i].y);
+    if (branch_out) branch_out[i] = ns ? sg[0].branch : pick_branch(plan_of(k), (int)f, 1, (int)h_sizes[i].y);
     for (int j = 0; j < ns; ++j) {
       const BranchInfo& bi = k.branches[sg[j].branch];
       total += ((sg[j].rows + bi.BM - 1) / bi.BM) * (int)((h_sizes[i].y + bi.BN - 1) / bi.BN);

@@ -110,42 +110,74 @@ struct Dispatch<I, T, Rest...> {
 template <class... Tiles>
 constexpr int kWavesPerSimd = ((Tiles::kAccRegs > 128) || ...) ? 1 : 2;
 
-template <class... Tiles>
-__global__ void __launch_bounds__(kThreads, kWavesPerSimd<Tiles...>) fused_group_gemm_kernel(const FusedArgs args) {
-  extern __shared__ __align__(16) uint8_t smem[];
+// Tables are read through the constant address space: what a workgroup reads from them is the same for all lanes and is not
+// written while the kernel runs (a planned launch's tables were written by the planning kernel before it), so every read is a
+// scalar load, whether the table came in the kernel arguments or lies in device memory.
+#define MXMOE_CONST __attribute__((address_space(4)))
+template <class T>
+__device__ __forceinline__ T cload(const T* p) {
+  return *(const MXMOE_CONST T*)(p);
+}
+__device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
+
+template <class ArgsPtr, class... Tiles>
+__device__ __forceinline__ void fused_body(ArgsPtr args, uint8_t* smem) {
   const int wg = blockIdx.x;
+  const int num_phases = uni(args->num_phases);
   int ph = 0;
-  while (ph + 1 < args.num_phases && wg >= args.phase_wg0[ph + 1]) ++ph;
-  const int v = wg - args.phase_wg0[ph];
-  const int ntiles = args.phase_tile0[ph + 1] - args.phase_tile0[ph];
+  while (ph + 1 < num_phases && wg >= uni(args->phase_wg0[ph + 1])) ++ph;
+  const int v = wg - uni(args->phase_wg0[ph]);
+  const int tile0 = uni(args->phase_tile0[ph]);
+  const int ntiles = uni(args->phase_tile0[ph + 1]) - tile0;
   const int chunk = (ntiles + kNumXcd - 1) / kNumXcd;
   const int pt = (v % kNumXcd) * chunk + v / kNumXcd;
   if (pt >= ntiles) return;
-  const int tile = args.phase_tile0[ph] + pt;
+  const int tile = tile0 + pt;
   // tile_scheduler.cuh:25-37 — the entry that holds the tile: last entry whose first tile is <= tile (binary search here; all
-  // indices are wave-uniform, so these are scalar loads from the argument block)
-  int lo = 0, hi = args.num_entries - 1;
+  // indices are wave-uniform, so these are scalar loads)
+  int lo = 0, hi = uni(args->num_entries) - 1;
   while (lo < hi) {
     const int mid = (lo + hi + 1) >> 1;
-    if (args.entry[mid].first <= tile) lo = mid; else hi = mid - 1;
+    if (uni(args->entry[mid].first) <= tile) lo = mid; else hi = mid - 1;
   }
-  const FusedArgs::Entry en = args.entry[lo];
-  const int local = tile - en.first;
-  const int gp = args.problem_offset + (en.problem_branch & 0xFFFF);
-  const mxmoe_dim3 sz = args.sizes[gp];
+  const int en_first = uni(args->entry[lo].first), en_row0 = uni(args->entry[lo].row0), en_rows = uni(args->entry[lo].rows), en_pb = uni(args->entry[lo].problem_branch);
+  const int local = tile - en_first;
+  const int gp = uni(args->problem_offset) + (en_pb & 0xFFFF);
+  const mxmoe_dim3* sizes = args->sizes;
+  const uint8_t* const* As = args->As;
+  const uint8_t* const* Bs = args->Bs;
+  const _Float16* const* sa = args->sa;
+  const _Float16* const* sb = args->sb;
+  _Float16* const* Cs = args->Cs;
+  int32_t* const* acc = args->acc;
   TileArgs t;
-  t.A = args.As[gp];
-  t.B = args.Bs[gp];
-  t.sa = args.sa ? args.sa[gp] : nullptr;
-  t.sb = args.sb ? args.sb[gp] : nullptr;
-  t.C = args.Cs[gp];
-  t.acc_dump = args.acc ? args.acc[gp] : nullptr;
-  t.row0 = en.row0;
-  t.M = t.row0 + en.rows;  // rows past the segment are treated like rows past the problem
-  t.N = (int)sz.y;
-  t.K = (int)sz.z;
+  t.A = cload(As + gp);
+  t.B = cload(Bs + gp);
+  t.sa = sa ? cload(sa + gp) : nullptr;
+  t.sb = sb ? cload(sb + gp) : nullptr;
+  t.C = cload(Cs + gp);
+  t.acc_dump = acc ? cload(acc + gp) : nullptr;
+  t.row0 = en_row0;
+  t.M = t.row0 + en_rows;  // rows past the segment are treated like rows past the problem
+  t.N = uni((int)cload(&sizes[gp].y));
+  t.K = uni((int)cload(&sizes[gp].z));
   t.tile_m = t.tile_n = 0;
-  Dispatch<0, Tiles...>::go(en.problem_branch >> 16, t, local, smem);
+  Dispatch<0, Tiles...>::go(en_pb >> 16, t, local, smem);
+}
+
+template <class... Tiles>
+__global__ void __launch_bounds__(kThreads, kWavesPerSimd<Tiles...>) fused_group_gemm_kernel(const FusedArgs args) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  fused_body<const FusedArgs*, Tiles...>(&args, smem);
+}
+
+// The same kernel with its tables in device memory, where a planning kernel wrote them from the tokens-per-expert counts: the
+// host then needs no copy of the counts, so a layer forward neither synchronises nor depends on its routing when it is enqueued
+// (or captured into a graph).  The grid is sized for the worst case; workgroups past the planned tiles leave at once.
+template <class... Tiles>
+__global__ void __launch_bounds__(kThreads, kWavesPerSimd<Tiles...>) fused_group_gemm_planned_kernel(const FusedArgs* __restrict__ args) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  fused_body<const MXMOE_CONST FusedArgs*, Tiles...>((const MXMOE_CONST FusedArgs*)args, smem);
 }
 
 // ------------------------------------------------------------------ host side ------------------------------------------------------------------
@@ -217,6 +249,7 @@ struct BranchOf<SkinnyWoTile<WBITS, BN>> {
 };
 
 using LaunchFn = hipError_t (*)(const FusedArgs&, int grid, int lds, hipStream_t);
+using LaunchPlannedFn = hipError_t (*)(const FusedArgs* d_args, int grid, int lds, hipStream_t);
 
 // How a registered kernel walks a problem list (the reference generates one host launcher per policy, kernel_sketch.py:82-145
 // fused, :148-274 sequential, :277-406 multi-stream):
@@ -232,6 +265,8 @@ struct FusedKernel {
   LaunchFn launch;
   Policy policy;
   mxmoe_func_t func;  // the kernel as a function of the reference's FuncType (registry.cuh:28-39)
+  LaunchPlannedFn launch_planned;  // the same kernel reading its tables from device memory (device-side planning)
+  int plan_index;                  // index into plan_infos()
 };
 
 inline std::vector<FusedKernel>& registry() {
@@ -252,6 +287,127 @@ struct BranchOf<WoMfmaTile<WBITS, BM, BN>> {
   }
 };
 
+// Run time of one tile of a branch relative to the 128 x 256 tile of the same format (same K), from the kernel-profile table
+// measured on MI355X (ms per 256 tiles at K = 2048).  Small tiles pay a fixed prologue / epilogue and use the matrix pipe less
+// well; the weight-only entries compare the skinny streaming tile with the 128 x 128 dequantise-to-fp16 tile.
+inline double tile_cost(const BranchInfo& b) {
+  struct Row { Fmt f; int bm, bn; double c; };
+  static const Row table[] = {
+      // (inside a fused kernel the small integer tiles run at the occupancy of the largest one, which costs them part of the
+      // advantage they show as single-tile kernels in the profile table)
+      {Fmt::W4A4, 128, 256, 1.00}, {Fmt::W4A4, 64, 256, 0.58}, {Fmt::W4A4, 32, 256, 0.48},
+      {Fmt::W8A8, 128, 256, 1.00}, {Fmt::W8A8, 64, 256, 0.74}, {Fmt::W8A8, 32, 256, 0.56},
+      {Fmt::FP16, 128, 256, 1.00}, {Fmt::FP16, 64, 256, 0.69}, {Fmt::FP16, 32, 256, 0.53}, {Fmt::FP16, 128, 128, 0.57}, {Fmt::FP16, 256, 128, 1.09},
+      {Fmt::W4A16, 16, 128, 0.37}, {Fmt::W4A16, 16, 64, 0.20}, {Fmt::W4A16, 128, 128, 1.00},
+      {Fmt::W3A16, 16, 128, 0.31}, {Fmt::W3A16, 16, 64, 0.20}, {Fmt::W3A16, 128, 128, 1.00},
+      {Fmt::W2A16, 16, 128, 0.25}, {Fmt::W2A16, 16, 64, 0.20}, {Fmt::W2A16, 128, 128, 1.00},
+      {Fmt::W4A4G128, 64, 256, 1.00}, {Fmt::W4A4G128, 32, 256, 0.60},
+  };
+  for (const Row& r : table)
+    if (r.f == b.fmt && r.bm == b.BM && r.bn == b.BN) return r.c;
+  return (0.22 + 0.78 * b.BM / 128.0) * b.BN / 256.0;  // shapes without a measurement
+}
+
+// Rough run time of one tile across formats, used only to order the tile list (expensive shapes first): the matrix pipe runs
+// fp16 at half the int8 rate, and int4 operands are widened to int8.
+inline double branch_cost(const BranchInfo& b) {
+  const double per_k = b.fmt == Fmt::FP16 ? 2.0 : (b.fmt == Fmt::W4A16 || b.fmt == Fmt::W3A16 || b.fmt == Fmt::W2A16) ? 1.2 : (b.fmt == Fmt::W8A8 ? 1.25 : 1.0);
+  return tile_cost(b) * per_k;
+}
+
+// What the planners (the host launcher and the device-side planning kernel) need to know of a kernel's branches, as plain data.
+constexpr int kMaxBranches = 32;
+struct PlanBranch {
+  int fmt, BM, BN, k_multiple;
+  double cost;  // tile_cost
+};
+struct PlanInfo {
+  int nb;                    // branches
+  int order[kMaxBranches];   // branch indices, most expensive tile first (branch_cost); ties keep the registration order
+  PlanBranch b[kMaxBranches];
+};
+
+// Cheapest branch of format `f` for a block of `rows` x `N` run with one tile shape: cost = row tiles * column tiles * tile_cost.
+__host__ __device__ inline int pick_branch(const PlanInfo& k, int f, int rows, int N) {
+  int best = -1;
+  double best_cost = 0;
+  for (int i = 0; i < k.nb; ++i) {
+    const PlanBranch& b = k.b[i];
+    if (b.fmt != f) continue;
+    const double c = (double)((rows + b.BM - 1) / b.BM) * ((N + b.BN - 1) / b.BN) * b.cost;
+    if (best < 0 || c < best_cost - 1e-9 || (c < best_cost + 1e-9 && b.BM > k.b[best].BM)) {
+      best = i;
+      best_cost = c;
+    }
+  }
+  return best;
+}
+
+struct Segment {
+  int row0, rows, branch;
+};
+
+// Split the M rows of an M x N problem into at most two segments: whole tiles of the shape that is cheapest per output element,
+// then the remainder with the shape that covers it most cheaply.  Returns the number of segments (0 for M == 0), or -1 when
+// the kernel has no tile for `f`.
+__host__ __device__ inline int plan_segments(const PlanInfo& k, int f, int M, int N, Segment out[2]) {
+  int big = -1;
+  double big_unit = 0;
+  for (int i = 0; i < k.nb; ++i) {
+    const PlanBranch& b = k.b[i];
+    if (b.fmt != f) continue;
+    const double unit = b.cost * ((N + b.BN - 1) / b.BN) / b.BM;  // cost per row of the problem
+    if (big < 0 || unit < big_unit - 1e-12 || (unit < big_unit + 1e-12 && b.BM > k.b[big].BM)) {
+      big = i;
+      big_unit = unit;
+    }
+  }
+  if (big < 0) return -1;
+  if (M <= 0) return 0;
+  auto cost_of = [&](int branch, int rows) {
+    const PlanBranch& b = k.b[branch];
+    return (double)((rows + b.BM - 1) / b.BM) * ((N + b.BN - 1) / b.BN) * b.cost;
+  };
+  const int bm = k.b[big].BM;
+  const int full = (M / bm) * bm, rem = M - full;
+  const int whole = pick_branch(k, f, M, N);
+  if (rem == 0 || full == 0) {
+    out[0] = Segment{0, M, whole};
+    return 1;
+  }
+  const int rb = pick_branch(k, f, rem, N);
+  if (cost_of(whole, M) <= cost_of(big, full) + cost_of(rb, rem) + 1e-9 || rb == big) {
+    out[0] = Segment{0, M, rb == big ? big : whole};
+    return 1;
+  }
+  out[0] = Segment{0, full, big};
+  out[1] = Segment{full, rem, rb};
+  return 2;
+}
+
+__host__ __device__ inline int segment_tiles(const PlanInfo& k, const Segment& sg, int N) {
+  const PlanBranch& b = k.b[sg.branch];
+  return ((sg.rows + b.BM - 1) / b.BM) * ((N + b.BN - 1) / b.BN);
+}
+
+inline PlanInfo make_plan_info(const std::vector<BranchInfo>& branches) {
+  PlanInfo k;
+  std::memset(&k, 0, sizeof k);
+  k.nb = std::min((int)branches.size(), kMaxBranches);
+  for (int i = 0; i < k.nb; ++i) {
+    k.b[i] = PlanBranch{(int)branches[i].fmt, branches[i].BM, branches[i].BN, branches[i].k_multiple, tile_cost(branches[i])};
+    k.order[i] = i;
+  }
+  std::stable_sort(k.order, k.order + k.nb, [&](int x, int y) { return branch_cost(branches[x]) > branch_cost(branches[y]); });
+  return k;
+}
+
+inline std::vector<PlanInfo>& plan_infos() {
+  static std::vector<PlanInfo> v;
+  return v;
+}
+inline const PlanInfo& plan_of(const FusedKernel& k) { return plan_infos()[k.plan_index]; }
+
 template <class... Tiles>
 hipError_t launch_fused(const FusedArgs& a, int grid, int lds, hipStream_t s) {
   // more than 64 KB of dynamic LDS must be opted into, once per device (kept out of library load time: no HIP call before first use)
@@ -266,6 +422,22 @@ hipError_t launch_fused(const FusedArgs& a, int grid, int lds, hipStream_t s) {
     }
   }
   hipLaunchKernelGGL((fused_group_gemm_kernel<Tiles...>), dim3(grid), dim3(kThreads), lds, s, a);
+  return hipGetLastError();
+}
+
+template <class... Tiles>
+hipError_t launch_fused_planned(const FusedArgs* d_args, int grid, int lds, hipStream_t s) {
+  static bool lds_opted_in[64] = {};
+  if (lds > 64 * 1024) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return hipGetLastError();
+    if (dev >= 0 && dev < 64 && !lds_opted_in[dev]) {
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&fused_group_gemm_planned_kernel<Tiles...>), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+      if (e != hipSuccess) return e;
+      lds_opted_in[dev] = true;
+    }
+  }
+  hipLaunchKernelGGL((fused_group_gemm_planned_kernel<Tiles...>), dim3(grid), dim3(kThreads), lds, s, d_args);
   return hipGetLastError();
 }
 
@@ -327,6 +499,9 @@ int register_fused(const char* fn_name, Policy policy = Policy::Fused) {
   }
   k.name = n + fn_name;
   k.launch = &launch_fused<Tiles...>;
+  k.launch_planned = &launch_fused_planned<Tiles...>;
+  k.plan_index = (int)plan_infos().size();
+  plan_infos().push_back(make_plan_info(k.branches));
   const int id = (int)registry().size();
   switch (policy) {
     case Policy::Fused: FuncThunk<0, Tiles...>::kernel_id = id; k.func = &FuncThunk<0, Tiles...>::call; break;
@@ -337,100 +512,20 @@ int register_fused(const char* fn_name, Policy policy = Policy::Fused) {
   return id;
 }
 
-// Run time of one tile of a branch relative to the 128 x 256 tile of the same format (same K), from the kernel-profile table
-// measured on MI355X (ms per 256 tiles at K = 2048).  Small tiles pay a fixed prologue / epilogue and use the matrix pipe less
-// well; the weight-only entries compare the skinny streaming tile with the 128 x 128 dequantise-to-fp16 tile.
-inline double tile_cost(const BranchInfo& b) {
-  struct Row { Fmt f; int bm, bn; double c; };
-  static const Row table[] = {
-      // (inside a fused kernel the small integer tiles run at the occupancy of the largest one, which costs them part of the
-      // advantage they show as single-tile kernels in the profile table)
-      {Fmt::W4A4, 128, 256, 1.00}, {Fmt::W4A4, 64, 256, 0.58}, {Fmt::W4A4, 32, 256, 0.48},
-      {Fmt::W8A8, 128, 256, 1.00}, {Fmt::W8A8, 64, 256, 0.74}, {Fmt::W8A8, 32, 256, 0.56},
-      {Fmt::FP16, 128, 256, 1.00}, {Fmt::FP16, 64, 256, 0.69}, {Fmt::FP16, 32, 256, 0.53}, {Fmt::FP16, 128, 128, 0.57}, {Fmt::FP16, 256, 128, 1.09},
-      {Fmt::W4A16, 16, 128, 0.37}, {Fmt::W4A16, 16, 64, 0.20}, {Fmt::W4A16, 128, 128, 1.00},
-      {Fmt::W3A16, 16, 128, 0.31}, {Fmt::W3A16, 16, 64, 0.20}, {Fmt::W3A16, 128, 128, 1.00},
-      {Fmt::W2A16, 16, 128, 0.25}, {Fmt::W2A16, 16, 64, 0.20}, {Fmt::W2A16, 128, 128, 1.00},
-      {Fmt::W4A4G128, 64, 256, 1.00}, {Fmt::W4A4G128, 32, 256, 0.60},
-  };
-  for (const Row& r : table)
-    if (r.f == b.fmt && r.bm == b.BM && r.bn == b.BN) return r.c;
-  return (0.22 + 0.78 * b.BM / 128.0) * b.BN / 256.0;  // shapes without a measurement
-}
-
-// Rough run time of one tile across formats, used only to order the tile list (expensive shapes first): the matrix pipe runs
-// fp16 at half the int8 rate, and int4 operands are widened to int8.
-inline double branch_cost(const BranchInfo& b) {
-  const double per_k = b.fmt == Fmt::FP16 ? 2.0 : (b.fmt == Fmt::W4A16 || b.fmt == Fmt::W3A16 || b.fmt == Fmt::W2A16) ? 1.2 : (b.fmt == Fmt::W8A8 ? 1.25 : 1.0);
-  return tile_cost(b) * per_k;
-}
-
-// Cheapest branch of format `f` for a block of `rows` x `N` run with one tile shape: cost = row tiles * column tiles * tile_cost.
-inline int pick_branch(const FusedKernel& k, Fmt f, int rows, int N) {
-  int best = -1;
-  double best_cost = 0;
-  for (int i = 0; i < (int)k.branches.size(); ++i) {
-    const auto& b = k.branches[i];
-    if (b.fmt != f) continue;
-    const double c = (double)((rows + b.BM - 1) / b.BM) * ((N + b.BN - 1) / b.BN) * tile_cost(b);
-    if (best < 0 || c < best_cost - 1e-9 || (c < best_cost + 1e-9 && b.BM > k.branches[best].BM)) {
-      best = i;
-      best_cost = c;
-    }
-  }
-  return best;
-}
-
-struct Segment {
-  int row0, rows, branch;
-};
-
-// Split the M rows of an M x N problem into at most two segments: whole tiles of the shape that is cheapest per output element,
-// then the remainder with the shape that covers it most cheaply.  Returns the number of segments (0 for M == 0), or -1 when
-// the kernel has no tile for `f`.
-inline int plan_segments(const FusedKernel& k, Fmt f, int M, int N, Segment out[2]) {
-  int big = -1;
-  double big_unit = 0;
-  for (int i = 0; i < (int)k.branches.size(); ++i) {
-    const auto& b = k.branches[i];
-    if (b.fmt != f) continue;
-    const double unit = tile_cost(b) * ((N + b.BN - 1) / b.BN) / b.BM;  // cost per row of the problem
-    if (big < 0 || unit < big_unit - 1e-12 || (unit < big_unit + 1e-12 && b.BM > k.branches[big].BM)) {
-      big = i;
-      big_unit = unit;
-    }
-  }
-  if (big < 0) return -1;
-  if (M <= 0) return 0;
-  auto cost_of = [&](int branch, int rows) {
-    const auto& b = k.branches[branch];
-    return (double)((rows + b.BM - 1) / b.BM) * ((N + b.BN - 1) / b.BN) * tile_cost(b);
-  };
-  const int bm = k.branches[big].BM;
-  const int full = (M / bm) * bm, rem = M - full;
-  const int whole = pick_branch(k, f, M, N);
-  if (rem == 0 || full == 0) {
-    out[0] = Segment{0, M, whole};
-    return 1;
-  }
-  const int rb = pick_branch(k, f, rem, N);
-  if (cost_of(whole, M) <= cost_of(big, full) + cost_of(rb, rem) + 1e-9 || rb == big) {
-    out[0] = Segment{0, M, rb == big ? big : whole};
-    return 1;
-  }
-  out[0] = Segment{0, full, big};
-  out[1] = Segment{full, rem, rb};
-  return 2;
-}
-
 // A kernel can run a problem list when it has a branch for every format in it.
 inline bool kernel_covers(const FusedKernel& k, const mxmoe_qparams* q, int count) {
   for (int i = 0; i < count; ++i) {
     const Fmt f = classify(q[i]);
     Segment sg[2];
-    if (f == Fmt::UNSUPPORTED || plan_segments(k, f, 1, 256, sg) < 0) return false;
+    if (f == Fmt::UNSUPPORTED || plan_segments(plan_of(k), (int)f, 1, 256, sg) < 0) return false;
   }
   return true;
+}
+
+// K a multiple of the tile's K step, N a multiple of 8 (16 for the weight-only layouts)
+inline bool shape_ok(const BranchInfo& bi, const mxmoe_dim3& sz) {
+  const bool wo = bi.fmt == Fmt::W4A16 || bi.fmt == Fmt::W3A16 || bi.fmt == Fmt::W2A16;
+  return sz.z != 0 && sz.z % bi.k_multiple == 0 && sz.y % 8 == 0 && !(wo && sz.y % 16 != 0);
 }
 
 // One launch over problems [base, base + n) of the caller's arrays with kernel `k` (n <= kMaxProblems).
@@ -446,6 +541,7 @@ inline int launch_range(const FusedKernel& k, const void* const* As, const void*
   a.acc = acc;
   a.sizes = d_sizes;
   a.problem_offset = base;
+  const PlanInfo& pi = plan_of(k);
   struct Entry {
     int row0, rows, problem, branch, tiles;
   };
@@ -455,31 +551,26 @@ inline int launch_range(const FusedKernel& k, const void* const* As, const void*
     const mxmoe_dim3& sz = h_sizes[base + i];
     const Fmt f = classify(h_q[base + i]);
     Segment sg[2];
-    const int ns = f == Fmt::UNSUPPORTED ? -1 : plan_segments(k, f, (int)sz.x, (int)sz.y, sg);
+    const int ns = f == Fmt::UNSUPPORTED ? -1 : plan_segments(pi, (int)f, (int)sz.x, (int)sz.y, sg);
     if (ns < 0) {
       last_error() = "quant type not supported";
       return 1;
     }
     for (int j = 0; j < ns; ++j) {
       const BranchInfo& bi = k.branches[sg[j].branch];
-      if (sz.z == 0 || sz.z % bi.k_multiple != 0 || sz.y % 8 != 0 || (bi.fmt != Fmt::FP16 && bi.fmt != Fmt::W8A8 && bi.fmt != Fmt::W4A4 && bi.fmt != Fmt::W4A4G128 && sz.y % 16 != 0)) {
+      if (!shape_ok(bi, sz)) {
         char buf[200];
         snprintf(buf, sizeof buf, "problem %d: shape [%u,%u,%u] not supported by tile %s (K %% %d, N %% 8)", base + i, sz.x, sz.y, sz.z, fmt_name(bi.fmt, true), bi.k_multiple);
         last_error() = buf;
         return 3;
       }
-      entries[nent++] = Entry{sg[j].row0, sg[j].rows, i, sg[j].branch, ((sg[j].rows + bi.BM - 1) / bi.BM) * (int)((sz.y + bi.BN - 1) / bi.BN)};
+      entries[nent++] = Entry{sg[j].row0, sg[j].rows, i, sg[j].branch, segment_tiles(pi, sg[j], (int)sz.y)};
     }
   }
   // most expensive tile shape first; problems keep their order inside a shape (neighbouring tiles share operands)
-  constexpr int kMaxBranches = 32;
-  int order[kMaxBranches];
-  const int nb = std::min((int)k.branches.size(), kMaxBranches);
-  for (int b = 0; b < nb; ++b) order[b] = b;
-  std::stable_sort(order, order + nb, [&](int x, int y) { return branch_cost(k.branches[x]) > branch_cost(k.branches[y]); });
   int total = 0, ne = 0, wg = 0, np = 0;
-  for (int oi = 0; oi < nb; ++oi) {
-    const int b = order[oi];
+  for (int oi = 0; oi < pi.nb; ++oi) {
+    const int b = pi.order[oi];
     const int tile0 = total;
     for (int ei = 0; ei < nent; ++ei) {
       const Entry& en = entries[ei];

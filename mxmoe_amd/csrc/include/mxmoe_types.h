@@ -22,6 +22,15 @@ typedef struct mxmoe_qparams {
   uint8_t _pad[3];
 } mxmoe_qparams;
 
+// One linear block (gate_up or down) of one expert as the device-side planner sees it: format, output channels N, reduction
+// length K, packed weights and weight scales.  40 bytes.
+typedef struct mxmoe_block_desc {
+  mxmoe_qparams q;
+  uint32_t N, K;
+  const void* B;
+  const void* scale_b;
+} mxmoe_block_desc;
+
 // fp16 storage as the C-ABI names it (the reference's `half`); only ever used behind pointers.
 typedef uint16_t mxmoe_half;
 

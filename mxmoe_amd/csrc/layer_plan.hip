@@ -1,0 +1,402 @@
+// Device-side planning of the two fused launches of a layer forward.
+//
+// The reference's operators read the tokens-per-expert counts back to the host (`.cpu()`, mxmoe/kernels/src/ref_bind.cu:451) and
+// build every table there: the per-expert {tag, first row, offsets} table of the quantisers (ref_bind.cu:475-505), the five pointer
+// arrays and sizes of the launch (ref_bind.cu:362-404) and, in the generated launcher, the tile prefix sums
+// (mxmoe/kernels/kernel_sketch.py:89-104).  Here one small kernel derives all of them from the counts where they are, in device
+// memory, so that the host enqueues the whole forward without waiting for the routing: no synchronisation, nothing that depends
+// on the counts in any launch argument, and therefore a sequence that a HIP graph can hold.
+#include <hip/hip_runtime.h>
+
+#include "../../include/mxmoe_amd.h"
+#include "include/mxmoe_launch.hpp"
+#include "include/mxmoe_plan.hpp"
+
+namespace mxmoe {
+
+__host__ __device__ inline int act_tag_of(const mxmoe_qparams& q) {  // ref_bind.cu:461-473
+  if (q.a_bits >= 16) return 0;
+  if (q.a_bits == 8 && q.gsize == -1) return 1;
+  if (q.a_bits == 4 && q.gsize == -1) return 2;
+  if (q.a_bits == 4 && q.gsize == 128) return 3;
+  return -1;
+}
+
+__host__ __device__ inline int fmt_of(const mxmoe_qparams& q) {  // Fmt as an int (classify)
+  if (q.a_bits >= 16 && q.w_bits >= 16) return (int)Fmt::FP16;
+  if (q.a_bits == 8 && q.w_bits == 8 && q.gsize == -1 && q.sym) return (int)Fmt::W8A8;
+  if (q.a_bits == 4 && q.w_bits == 4 && q.gsize == -1 && q.sym) return (int)Fmt::W4A4;
+  if (q.a_bits == 4 && q.w_bits == 4 && q.gsize == 128 && q.sym) return (int)Fmt::W4A4G128;
+  if (q.a_bits >= 16 && q.w_bits == 4 && q.gsize == 128) return (int)Fmt::W4A16;
+  if (q.a_bits >= 16 && q.w_bits == 3 && q.gsize == 128) return (int)Fmt::W3A16;
+  if (q.a_bits >= 16 && q.w_bits == 2 && q.gsize == 128) return (int)Fmt::W2A16;
+  return (int)Fmt::UNSUPPORTED;
+}
+
+struct PlanParams {
+  const int64_t* recv;
+  const mxmoe_block_desc* desc;
+  const uint8_t* inp;
+  const uint8_t* scale;
+  uint8_t* out;
+  uint8_t* plan;
+  int E, Et, shared_rows;
+  PlanInfo info;
+};
+
+constexpr int kPlanThreads = 128;
+static_assert(kMaxProblems <= kPlanThreads, "one thread per problem");
+
+__device__ __forceinline__ long wave_excl_scan(long v, int lane, long* total) {
+  long inc = v;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const long t = __shfl_up(inc, o);
+    if (lane >= o) inc += t;
+  }
+  *total = __shfl(inc, 63);
+  return inc - v;
+}
+
+// One workgroup of two waves, thread e = expert e (the shared expert, if any, is expert E with `shared_rows` rows).  Everything the
+// host launcher computes (launch_range), with the same functions and in the same order, so the two produce identical tables;
+// prefix sums over experts are wave scans, and an entry finds its place from per-branch counts instead of a sequential walk.
+__global__ void __launch_bounds__(kPlanThreads) plan_block_kernel(const PlanParams p) {
+  __shared__ long s_tot[4][2];                       // per wave: rows, packed input, scales, output elements
+  __shared__ int s_cnt[kMaxBranches][2], s_til[kMaxBranches][2];  // per run-order rank and wave: entries, tiles
+  const int e = threadIdx.x, lane = e & 63, wave = e >> 6;
+  const PlanLayout lay(p.Et);
+  FusedArgs* fa = reinterpret_cast<FusedArgs*>(p.plan);
+  int64_t* table = reinterpret_cast<int64_t*>(p.plan + lay.table);
+  const void** ptrs = reinterpret_cast<const void**>(p.plan + lay.ptrs);
+  int64_t* misc = reinterpret_cast<int64_t*>(p.plan + lay.misc);
+  mxmoe_dim3* sizes = reinterpret_cast<mxmoe_dim3*>(p.plan + lay.sizes);
+
+  long rows = 0, qld = 0, sld = 0, out_ld = 0;
+  int tag = 0, fmt = 0, N = 0, K = 0;
+  mxmoe_block_desc d{};
+  if (e < p.Et) {
+    d = p.desc[e];
+    rows = e < p.E ? (long)p.recv[e] : (long)p.shared_rows;
+    tag = act_tag_of(d.q);
+    fmt = fmt_of(d.q);
+    N = (int)d.N;
+    K = (int)d.K;
+    qld = tag == 0 ? K : (tag == 1 ? K / 2 : K / 4);  // fp16 elements per packed activation row (ref_bind.cu:491)
+    sld = tag == 0 ? 0 : (tag == 3 ? K / 128 : 1);   // scales per row (ref_bind.cu:492)
+    out_ld = N;
+  }
+  // exclusive sums over the experts before this one
+  long tot[4], routed_tot;
+  long first_row = wave_excl_scan(rows, lane, &tot[0]);
+  long inp_off = wave_excl_scan(qld * rows, lane, &tot[1]);
+  long sc_off = wave_excl_scan(sld * rows, lane, &tot[2]);
+  long out_off = wave_excl_scan(out_ld * rows, lane, &tot[3]);
+  wave_excl_scan(e < p.E ? rows : 0, lane, &routed_tot);
+  if (lane == 0) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) s_tot[i][wave] = tot[i];
+  }
+  // segments of this problem and, per branch in run order, this wave's entries and tiles
+  Segment sg[2];
+  const int ns = e < p.Et ? plan_segments(p.info, fmt, (int)rows, N, sg) : 0;
+  int seg_tiles[2], seg_rank[2], seg_pos[2], seg_first[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    seg_tiles[j] = j < ns ? segment_tiles(p.info, sg[j], N) : 0;
+    seg_rank[j] = -1;
+    seg_pos[j] = seg_first[j] = 0;
+  }
+  for (int r = 0; r < p.info.nb; ++r) {
+    const int b = p.info.order[r];
+    int mine = 0, which = -1;
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+      if (j < ns && sg[j].branch == b && seg_tiles[j] > 0) {
+        mine = seg_tiles[j];
+        which = j;
+      }
+    // entries of this branch in this wave: position = matching lanes before this one, first tile = their tiles
+    const uint64_t has = __ballot(which >= 0);
+    int tc = 0, tt = 0;
+    if (has != 0) {  // (wave-uniform: most branches of a kernel are not used by a given launch)
+      tc = __popcll(has);
+      int inc = mine;
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        const int t = __shfl_up(inc, o);
+        if (lane >= o) inc += t;
+      }
+      tt = __shfl(inc, 63);
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        if (which == j) {
+          seg_rank[j] = r;
+          seg_pos[j] = __popcll(has & ((1ull << lane) - 1));
+          seg_first[j] = inc - mine;
+        }
+    }
+    if (lane == 0) {
+      s_cnt[r][wave] = tc;
+      s_til[r][wave] = tt;
+    }
+  }
+  __syncthreads();
+  if (wave == 1) {
+    first_row += s_tot[0][0];
+    inp_off += s_tot[1][0];
+    sc_off += s_tot[2][0];
+    out_off += s_tot[3][0];
+  }
+  if (e < p.Et) {
+    table[e] = tag;
+    table[p.Et + e] = first_row;
+    table[2 * p.Et + e] = inp_off;
+    table[3 * p.Et + e] = sc_off;
+    ptrs[e] = p.inp + 2 * inp_off;
+    ptrs[p.Et + e] = d.B;
+    ptrs[2 * p.Et + e] = sld > 0 ? p.scale + 2 * sc_off : nullptr;
+    ptrs[3 * p.Et + e] = d.scale_b;
+    ptrs[4 * p.Et + e] = p.out + 2 * out_off;
+    sizes[e] = mxmoe_dim3{(uint32_t)rows, (uint32_t)N, (uint32_t)K};
+    if (e == p.E) misc[1] = (int64_t)(p.out + 2 * out_off);
+  }
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    if (seg_rank[j] >= 0) {
+      int pos = seg_pos[j], first = seg_first[j];
+      for (int r = 0; r < seg_rank[j]; ++r) {
+        pos += s_cnt[r][0] + s_cnt[r][1];
+        first += s_til[r][0] + s_til[r][1];
+      }
+      if (wave == 1) {
+        pos += s_cnt[seg_rank[j]][0];
+        first += s_til[seg_rank[j]][0];
+      }
+      fa->entry[pos] = FusedArgs::Entry{first, sg[j].row0, sg[j].rows, e | (sg[j].branch << 16)};
+    }
+  }
+  if (e == 0) {
+    // rows routed = sum over the routed experts: wave 0's part is in routed_tot, wave 1 holds experts 64.. (all routed or shared)
+    misc[0] = s_tot[0][0] + s_tot[0][1] - (p.Et > p.E ? (long)p.shared_rows : 0);
+    if (p.Et == p.E) misc[1] = 0;
+    int total = 0, wg = 0, np = 0, ne = 0;
+    for (int r = 0; r < p.info.nb; ++r) {
+      const int tile0 = total;
+      total += s_til[r][0] + s_til[r][1];
+      ne += s_cnt[r][0] + s_cnt[r][1];
+      if (total == tile0) continue;
+      if (np < kMaxPhases) {  // shapes beyond the phase table share the last phase
+        fa->phase_tile0[np] = tile0;
+        fa->phase_wg0[np] = wg;
+        ++np;
+      }
+      const int p0 = fa->phase_tile0[np - 1];
+      wg = fa->phase_wg0[np - 1] + (total - p0 + kNumXcd - 1) / kNumXcd * kNumXcd;
+    }
+    fa->phase_tile0[np] = total;
+    fa->phase_wg0[np] = wg;
+    fa->num_phases = np;
+    fa->num_entries = ne;
+    fa->total_tiles = total;
+    fa->problem_offset = 0;
+    fa->As = reinterpret_cast<const uint8_t* const*>(ptrs);
+    fa->Bs = reinterpret_cast<const uint8_t* const*>(ptrs + p.Et);
+    fa->sa = reinterpret_cast<const _Float16* const*>(ptrs + 2 * p.Et);
+    fa->sb = reinterpret_cast<const _Float16* const*>(ptrs + 3 * p.Et);
+    fa->Cs = reinterpret_cast<_Float16* const*>(const_cast<void**>(ptrs + 4 * p.Et));
+    fa->acc = nullptr;
+    fa->sizes = sizes;
+  }
+  (void)routed_tot;
+}
+
+// Kernel for the formats of `h_desc`, checked once on the host: every problem's format has a branch and its shape fits it.
+static int resolve_kernel(int kernel_id, const mxmoe_block_desc* h_desc, int et) {
+  auto& reg = registry();
+  auto covers = [&](const FusedKernel& k) {
+    for (int i = 0; i < et; ++i) {
+      Segment sg[2];
+      const int f = fmt_of(h_desc[i].q);
+      if (f == (int)Fmt::UNSUPPORTED || plan_segments(plan_of(k), f, 1, 256, sg) < 0) return false;
+    }
+    return true;
+  };
+  if (kernel_id < 0) {
+    for (int i = 0; i < (int)reg.size() && kernel_id < 0; ++i)
+      if (reg[i].policy == Policy::Fused && covers(reg[i])) kernel_id = i;
+    if (kernel_id < 0) {
+      last_error() = "quant type not supported";
+      return -1;
+    }
+  }
+  if (kernel_id >= (int)reg.size()) {
+    last_error() = "kernel id out of range";
+    return -2;
+  }
+  const FusedKernel& k = reg[kernel_id];
+  if (!covers(k)) {
+    last_error() = "quant type not supported";
+    return -1;
+  }
+  for (int i = 0; i < et; ++i) {
+    const mxmoe_dim3 sz{1, h_desc[i].N, h_desc[i].K};
+    for (const BranchInfo& bi : k.branches)
+      if ((int)bi.fmt == fmt_of(h_desc[i].q) && !shape_ok(bi, sz)) {
+        char buf[200];
+        snprintf(buf, sizeof buf, "problem %d: shape [N %u, K %u] not supported by tile %s (K %% %d, N %% 8)", i, sz.y, sz.z, fmt_name(bi.fmt, true), bi.k_multiple);
+        last_error() = buf;
+        return -3;
+      }
+    const int tag = act_tag_of(h_desc[i].q);
+    if (tag < 0 || (tag == 3 && h_desc[i].K % 128)) {
+      last_error() = tag < 0 ? "quant type not supported" : "group-128 activations need a row length that is a multiple of 128";
+      return tag < 0 ? -1 : -3;
+    }
+  }
+  return kernel_id;
+}
+
+}  // namespace mxmoe
+
+using namespace mxmoe;
+
+extern "C" {
+
+size_t mxmoe_plan_bytes(int num_problems) { return PlanLayout(num_problems).total; }
+
+size_t mxmoe_plan_offset(int which, int num_problems) {
+  const PlanLayout lay(num_problems);
+  switch (which) {
+    case 0: return 0;
+    case 1: return lay.table;
+    case 2: return lay.ptrs;
+    case 3: return lay.misc;
+    case 4: return lay.sizes;
+    default: return lay.total;
+  }
+}
+
+int mxmoe_plan_select_kernel(int kernel_id, const mxmoe_block_desc* h_desc, int num_problems) {
+  if (!h_desc || num_problems <= 0 || num_problems > kMaxProblems) {
+    last_error() = "a planned launch holds 1 to 120 problems";
+    return -3;
+  }
+  return resolve_kernel(kernel_id, h_desc, num_problems);
+}
+
+int mxmoe_plan_grid_bound(int kernel_id, const mxmoe_block_desc* h_desc, int num_experts, int routed_rows_max, int shared_rows) {
+  const int et = num_experts + (shared_rows > 0 ? 1 : 0);
+  const int kid = mxmoe_plan_select_kernel(kernel_id, h_desc, et);
+  if (kid < 0) return kid;
+  const PlanInfo& pi = plan_of(registry()[kid]);
+  // For every routed expert tiles(M) <= first + slope * (M - 1) for all M >= 1, with first = tiles(1) and slope the steepest rise
+  // found by walking M over 64 rows of the format's largest tile (the planner's decisions repeat with that tile's period).  With at
+  // most n = min(experts, rows) experts non-empty, the launch has at most (sum of the n largest `first`) + max slope * (rows - n) tiles.
+  auto tiles_of = [&](int f, int m, int n) {
+    Segment sg[2];
+    const int ns = plan_segments(pi, f, m, n, sg);
+    int t = 0;
+    for (int j = 0; j < ns; ++j) t += segment_tiles(pi, sg[j], n);
+    return t;
+  };
+  // And tiles(M) <= extra + per_row * M, with per_row the columns per row of the shape that very long problems run on and extra the
+  // largest excess over it: the smaller of the two sums holds.
+  long shared_tiles = 0;
+  double slope = 0, per_row = 0;
+  long extras = 0;
+  std::vector<int> firsts;
+  struct Seen { int f, n, first, extra; double slope, per_row; };
+  std::vector<Seen> seen;
+  for (int e = 0; e < et; ++e) {
+    const int f = fmt_of(h_desc[e].q), n = (int)h_desc[e].N;
+    if (e >= num_experts) {  // the shared expert's row count is known
+      shared_tiles += tiles_of(f, shared_rows, n);
+      continue;
+    }
+    const Seen* hit = nullptr;
+    for (const Seen& sn : seen)
+      if (sn.f == f && sn.n == n) hit = &sn;
+    if (!hit) {
+      Segment sg[2];
+      plan_segments(pi, f, 1 << 20, n, sg);
+      const int bm = pi.b[sg[0].branch].BM, cols = (n + pi.b[sg[0].branch].BN - 1) / pi.b[sg[0].branch].BN;
+      Seen sn{f, n, tiles_of(f, 1, n), 0, 0.0, (double)cols / bm};
+      const int limit = std::min(std::max(routed_rows_max, 2), 64 * bm);
+      for (int m = 1; m <= limit; ++m) {
+        const int t = tiles_of(f, m, n);
+        if (m > 1) sn.slope = std::max(sn.slope, (double)(t - sn.first) / (m - 1));
+        sn.extra = std::max(sn.extra, t - (m / bm) * cols);
+      }
+      seen.push_back(sn);
+      hit = &seen.back();
+    }
+    firsts.push_back(hit->first);
+    slope = std::max(slope, hit->slope);
+    per_row = std::max(per_row, hit->per_row);
+    extras += hit->extra;
+  }
+  std::sort(firsts.begin(), firsts.end(), [](int x, int y) { return x > y; });
+  const int nonempty = std::min((int)firsts.size(), routed_rows_max);
+  long by_first = (long)(slope * (routed_rows_max - nonempty)) + 1;
+  for (int i = 0; i < nonempty; ++i) by_first += firsts[i];
+  const long by_rows = extras + (long)(per_row * routed_rows_max) + 1;
+  long bound = shared_tiles + std::min(by_first, by_rows);
+  bound += (long)kNumXcd * (kMaxPhases + 1);  // every phase is padded to a multiple of the XCD count
+  bound = (bound + kNumXcd - 1) / kNumXcd * kNumXcd;
+  if (bound > (1l << 30)) {
+    last_error() = "planned grid too large";
+    return -3;
+  }
+  return (int)bound;
+}
+
+int mxmoe_plan_block(int kernel_id, const int64_t* d_recv, int num_experts, int shared_rows, const mxmoe_block_desc* d_desc, const mxmoe_block_desc* h_desc,
+                     const void* inp_store, const void* scale_store, void* out_store, void* d_plan, void* stream) {
+  const int et = num_experts + (shared_rows > 0 ? 1 : 0);
+  if (!d_recv || !d_desc || !h_desc || !inp_store || !out_store || !d_plan) {
+    last_error() = "null pointer";
+    return 5;
+  }
+  const int kid = mxmoe_plan_select_kernel(kernel_id, h_desc, et);
+  if (kid < 0) return kid == -1 ? 1 : (kid == -2 ? 2 : 3);
+  PlanParams p;
+  p.recv = d_recv;
+  p.desc = d_desc;
+  p.inp = reinterpret_cast<const uint8_t*>(inp_store);
+  p.scale = reinterpret_cast<const uint8_t*>(scale_store);
+  p.out = reinterpret_cast<uint8_t*>(out_store);
+  p.plan = reinterpret_cast<uint8_t*>(d_plan);
+  p.E = num_experts;
+  p.Et = et;
+  p.shared_rows = shared_rows;
+  p.info = plan_of(registry()[kid]);
+  hipLaunchKernelGGL(plan_block_kernel, dim3(1), dim3(kPlanThreads), 0, (hipStream_t)stream, p);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    last_error() = std::string("kernel launch failed: ") + hipGetErrorString(e);
+    return 4;
+  }
+  return 0;
+}
+
+int mxmoe_group_gemm_planned(int kernel_id, const void* d_plan, int grid, void* stream) {
+  auto& reg = registry();
+  if (kernel_id < 0 || kernel_id >= (int)reg.size()) {
+    last_error() = "kernel id out of range";
+    return 2;
+  }
+  if (!d_plan || grid <= 0) {
+    last_error() = "null plan or empty grid";
+    return 5;
+  }
+  const FusedKernel& k = reg[kernel_id];
+  const hipError_t e = k.launch_planned(reinterpret_cast<const FusedArgs*>(d_plan), grid, k.lds_bytes, (hipStream_t)stream);
+  if (e != hipSuccess) {
+    last_error() = std::string("kernel launch failed: ") + hipGetErrorString(e);
+    return 4;
+  }
+  return 0;
+}
+
+}  // extern "C"

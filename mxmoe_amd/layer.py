@@ -115,8 +115,117 @@ class MxMoELayer:
             self._static = (LT.static_block(self.qp_gate_up, gu_w, gu_n, *ptrs(self.w13)), LT.static_block(self.qp_down, dn_w, dn_n, *ptrs(self.w2)))
         return self._static
 
-    def __call__(self, hidden: torch.Tensor, topk_ids: torch.Tensor, topk_weights: torch.Tensor) -> torch.Tensor:
+    # ---- the forward that never waits for its routing ---------------------------------------------------------
+    def _planned_setup(self, t: int, topk: int):
+        """Everything of the planned forward that depends only on the layer and on (tokens, top-k): block descriptors on both sides,
+        kernels, worst-case grids, plan buffers, and the stores sized for the worst case.  Built once and reused."""
+        key = (t, topk)
+        cache = self.__dict__.setdefault("_planned", {})
+        if key in cache:
+            return cache[key]
+        cfg, dev, lib = self.cfg, self.device, _lib.load()
+        e_cnt, has_shared = cfg.num_experts, cfg.num_shared > 0
+        et = self.n_exp_total
+        r_cap = t * topk
+        shared_rows = t if has_shared else 0
+        i_sh = cfg.inter * max(cfg.num_shared, 1)
+        ps = {"r_cap": r_cap, "shared_rows": shared_rows, "et": et}
+
+        def u8(n):
+            return torch.empty(max(int(n), 16), dtype=torch.uint8, device=dev)
+
+        def block(qps, ns, ks, ws):
+            h = (_lib.BlockDesc * et)()
+            for e in range(et):
+                a, w, g, sym = qps[e]
+                h[e] = _lib.BlockDesc(int(a), int(w), int(g), 1 if sym else 0, (C.c_uint8 * 3)(), int(ns[e]), int(ks[e]), ws[e].data.data_ptr(),
+                                      0 if ws[e].scale is None else ws[e].scale.data_ptr())
+            d = torch.frombuffer(bytearray(bytes(h)), dtype=torch.uint8).to(dev)
+            kid = lib.mxmoe_plan_select_kernel(-1, h, et)
+            if kid < 0:
+                raise RuntimeError(lib.mxmoe_last_error().decode())
+            grid = lib.mxmoe_plan_grid_bound(kid, h, e_cnt, r_cap, shared_rows)
+            if grid < 0:
+                raise RuntimeError(lib.mxmoe_last_error().decode())
+            # worst-case stores: every routed row as wide as the widest routed expert's packed row
+            tags = [ops.act_tag(int(q[0]), int(q[2])) for q in qps]
+            qld = [k if tg == 0 else (k // 2 if tg == 1 else k // 4) for tg, k in zip(tags, ks)]
+            sld = [0 if tg == 0 else (k // 128 if tg == 3 else 1) for tg, k in zip(tags, ks)]
+            sh = [e_cnt] if has_shared else []
+            inp = 2 * (max(qld[:e_cnt]) * r_cap + sum(qld[e] * shared_rows for e in sh))
+            sc = 2 * (max(sld[:e_cnt]) * r_cap + sum(sld[e] * shared_rows for e in sh))
+            out = 2 * (max(ns[:e_cnt]) * r_cap + sum(ns[e] * shared_rows for e in sh))
+            return {"h": h, "d": d, "kid": kid, "grid": grid, "plan": u8(lib.mxmoe_plan_bytes(et)), "inp": u8(inp), "scale": u8(sc), "out_bytes": out}
+
+        sh = [1] if has_shared else []
+        b1 = block(self.qp_gate_up, [2 * cfg.inter] * e_cnt + [2 * i_sh for _ in sh], [cfg.hidden] * et, self.w13)
+        b2 = block(self.qp_down, [cfg.hidden] * et, [cfg.inter] * e_cnt + [i_sh for _ in sh], self.w2)
+        ps["b1"], ps["b2"] = b1, b2
+        ps["mid"], ps["out"] = u8(b1["out_bytes"]), u8(b2["out_bytes"])
+        ps["dst"] = torch.empty(r_cap, dtype=torch.int32, device=dev)
+        ps["perm"] = torch.empty(r_cap, dtype=torch.int64, device=dev)
+        ps["slot"] = torch.empty(r_cap, dtype=torch.int64, device=dev)
+        ps["recv"] = torch.empty(e_cnt, dtype=torch.int64, device=dev)
+        ps["perm_ws"] = u8(lib.mxmoe_permute_workspace_bytes(r_cap, e_cnt))
+        ps["comb_ws"] = u8(lib.mxmoe_combine_workspace_bytes(t, topk))
+
+        def signs(n, n_shared):
+            if not cfg.rotate:
+                return 1, 1, None, None
+            hk, hf, sg = device_signs(n, dev)
+            if has_shared and device_signs(n_shared, dev)[0] != hk:
+                raise RuntimeError("routed and shared intermediate sizes need the same Hadamard order")
+            return hk, hf, sg, None if sg is None else sg.data_ptr()
+
+        ps["had1"], ps["had2"] = signs(cfg.hidden, cfg.hidden), signs(cfg.inter, i_sh)
+        cache[key] = ps
+        return ps
+
+    def __call__(self, hidden: torch.Tensor, topk_ids: torch.Tensor, topk_weights: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
         """The whole MoE MLP, `(hidden [T, K] fp16, topk_ids [T, k] int32, topk_weights [T, k] fp32) -> [T, K] fp16`: what a serving
+        framework's fused-MoE operator computes after routing (permute, quantise, gate_up, SiLU * up, down, un-permute + combine).
+
+        Same kernels and results as `forward` + `combine`, but nothing here waits for the routing: the tables of both launches are
+        derived from the tokens-per-expert counts by a planning kernel on the device (`mxmoe_plan_block`), the stores and plan
+        buffers are allocated once per (tokens, top-k) for the worst case, and every launch argument is independent of the data.
+        The call only enqueues nine kernels (no synchronisation, no allocation after the first call when `out` is given), so it can
+        be captured into a HIP graph.  Intermediate buffers belong to the layer and are reused by the next call of the same shape."""
+        cfg, dev = self.cfg, self.device
+        lib = _lib.load()
+        hidden = hidden.to(dev).contiguous()
+        ids = topk_ids.to(dev).to(torch.int32).contiguous()
+        w = topk_weights.to(dev).to(torch.float32).contiguous()
+        t, k_hid = hidden.shape
+        topk = ids.shape[1]
+        assert hidden.dtype == torch.float16 and k_hid == cfg.hidden and w.shape == ids.shape
+        e_cnt, has_shared = cfg.num_experts, int(cfg.num_shared > 0)
+        ps = self._planned_setup(t, topk)
+        b1, b2 = ps["b1"], ps["b2"]
+        stream = torch.cuda.current_stream().cuda_stream
+        final = out if out is not None else torch.empty((t, cfg.hidden), dtype=torch.float16, device=dev)
+        assert final.shape == (t, cfg.hidden) and final.dtype == torch.float16 and final.is_contiguous()
+        ck = lambda rc: _lib.check(lib, rc)  # noqa: E731
+        ck(lib.mxmoe_build_permutation(ids.data_ptr(), t, topk, e_cnt, ps["dst"].data_ptr(), ps["perm"].data_ptr(), ps["slot"].data_ptr(), ps["recv"].data_ptr(),
+                                       ps["perm_ws"].data_ptr(), stream))
+        ck(lib.mxmoe_plan_block(b1["kid"], ps["recv"].data_ptr(), e_cnt, ps["shared_rows"], b1["d"].data_ptr(), b1["h"], b1["inp"].data_ptr(), b1["scale"].data_ptr(),
+                                ps["mid"].data_ptr(), b1["plan"].data_ptr(), stream))
+        ck(lib.mxmoe_plan_block(b2["kid"], ps["recv"].data_ptr(), e_cnt, ps["shared_rows"], b2["d"].data_ptr(), b2["h"], b2["inp"].data_ptr(), b2["scale"].data_ptr(),
+                                ps["out"].data_ptr(), b2["plan"].data_ptr(), stream))
+        hk, hf, _sg, sgp = ps["had1"]
+        ck(lib.mxmoe_quant_act_planned(hidden.data_ptr(), b1["inp"].data_ptr(), b1["scale"].data_ptr(), ps["dst"].data_ptr(), ps["perm"].data_ptr(), b1["plan"].data_ptr(),
+                                       cfg.hidden, ps["r_cap"], t, e_cnt, has_shared, cfg.rotate, hk, hf, sgp, stream))
+        ck(lib.mxmoe_group_gemm_planned(b1["kid"], b1["plan"].data_ptr(), b1["grid"], stream))
+        i_sh = cfg.inter * max(cfg.num_shared, 1)
+        hk, hf, _sg, sgp = ps["had2"]
+        ck(lib.mxmoe_silu_mul_quant_planned(ps["mid"].data_ptr(), b1["plan"].data_ptr(), b2["inp"].data_ptr(), b2["scale"].data_ptr(), ps["dst"].data_ptr(), b2["plan"].data_ptr(),
+                                            cfg.inter, i_sh, ps["r_cap"], t, e_cnt, has_shared, cfg.rotate, hk, hf, sgp, stream))
+        ck(lib.mxmoe_group_gemm_planned(b2["kid"], b2["plan"].data_ptr(), b2["grid"], stream))
+        ck(lib.mxmoe_unpermute_combine_planned(ps["out"].data_ptr(), b2["plan"].data_ptr(), ps["et"], w.data_ptr(), ps["slot"].data_ptr(), t, topk, cfg.hidden,
+                                               final.data_ptr(), ps["comb_ws"].data_ptr(), stream))
+        return final
+
+    def call_with_host_tables(self, hidden: torch.Tensor, topk_ids: torch.Tensor, topk_weights: torch.Tensor) -> torch.Tensor:
+        """The whole MoE MLP with the tables of both launches built on the HOST (what the reference's operators do), `(hidden [T, K] fp16, topk_ids [T, k] int32, topk_weights [T, k] fp32) -> [T, K] fp16`: what a serving
         framework's fused-MoE operator computes after routing (permute, quantise, gate_up, SiLU * up, down, un-permute + combine).
 
         Same kernels and results as `forward` + `combine`, but the host side is one pass: after the single device-to-host copy of

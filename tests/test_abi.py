@@ -184,3 +184,55 @@ def test_prologue_entry_points_validate_on_the_host(lib):
     assert lib.mxmoe_silu_mul_quant(a, a, a, a, a, a, 1408, 1408, 4, 2, 2, 0, 1, 176, 4, None, None) == 3 and b"sign table" in lib.mxmoe_last_error()
     assert lib.mxmoe_build_permutation(None, 4, 2, 8, a, a, a, a, a, None) == 5
     assert lib.mxmoe_build_permutation(a, 0, 2, 8, a, a, a, a, a, None) == 3
+
+
+def test_planned_grid_bound_covers_every_routing(lib):
+    """The worst-case grid of a planned launch against the tile count the host launcher plans for random routings of the same
+    total: the bound must never be smaller (a smaller grid would silently drop tiles), and stays within a small factor."""
+    import random
+
+    from mxmoe_amd import _lib
+
+    rnd = random.Random(11)
+    cases = [([(4, 4, -1, True), (8, 8, -1, True)], 2816, 2048, 60, 32768, 0), ([(16, 4, 128, False), (16, 3, 128, False)], 2816, 2048, 64, 192, 32),
+             ([(4, 4, -1, True), (8, 8, -1, True), (16, 4, 128, False)], 28672, 4096, 8, 16384, 0), ([(16, 16, -1, True)], 2816, 2048, 60, 2048, 0),
+             ([(4, 4, 128, True), (4, 4, -1, True)], 2048, 1408, 17, 999, 7)]
+    for fmts, n, k, e_cnt, routed, shared_rows in cases:
+        et = e_cnt + (1 if shared_rows else 0)
+        qs = [rnd.choice(fmts) for _ in range(et)]
+        desc = (_lib.BlockDesc * et)(*[_lib.BlockDesc(q[0], q[1], q[2], int(q[3]), (C.c_uint8 * 3)(), n, k, 0, 0) for q in qs])
+        kid = lib.mxmoe_plan_select_kernel(-1, desc, et)
+        assert kid >= 0, lib.mxmoe_last_error()
+        bound = lib.mxmoe_plan_grid_bound(kid, desc, e_cnt, routed, shared_rows)
+        assert bound > 0, lib.mxmoe_last_error()
+        worst = 0
+        for trial in range(60):
+            style = trial % 4
+            if style == 0:                                          # everything on one expert
+                counts = [0] * e_cnt
+                counts[rnd.randrange(e_cnt)] = routed
+            elif style == 1:                                        # as even as possible
+                counts = [routed // e_cnt + (1 if i < routed % e_cnt else 0) for i in range(e_cnt)]
+            elif style == 2:                                        # many experts just past a tile boundary
+                unit = rnd.choice([1, 17, 33, 65, 129])
+                counts = [0] * e_cnt
+                left = routed
+                for i in range(e_cnt):
+                    take = min(left, unit)
+                    counts[i] = take
+                    left -= take
+                counts[0] += left
+            else:
+                cuts = sorted(rnd.randint(0, routed) for _ in range(e_cnt - 1))
+                counts = [b - a for a, b in zip([0] + cuts, cuts + [routed])]
+            assert sum(counts) == routed
+            rows = counts + ([shared_rows] if shared_rows else [])
+            rc, _, tiles = _plan(lib, kid, [((m, n, k), q) for m, q in zip(rows, qs)])
+            assert rc == 1000 + kid
+            worst = max(worst, tiles)
+            assert tiles + 8 * 9 <= bound, (fmts, counts[:6], tiles, bound)   # + the padding of every phase to the XCD count
+        assert bound <= 2.5 * worst + 600, (fmts, worst, bound)
+    bad = (_lib.BlockDesc * 1)(_lib.BlockDesc(8, 4, -1, 1, (C.c_uint8 * 3)(), 256, 128, 0, 0))
+    assert lib.mxmoe_plan_select_kernel(-1, bad, 1) < 0 and lib.mxmoe_last_error() == b"quant type not supported"
+    assert lib.mxmoe_plan_select_kernel(-1, desc, 121) < 0
+    assert lib.mxmoe_plan_bytes(60) >= 4096 + 60 * (32 + 40 + 12)

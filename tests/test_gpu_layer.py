@@ -198,3 +198,108 @@ def test_layer_from_checkpoint_file_keeps_the_function(tmp_path):
             g, u = h[:cfg.inter], h[cfg.inter:]
             ref[t] += float(w[t, j]) * (w2_.float() @ (g * torch.sigmoid(g) * u))
     assert _rel(a.float().numpy(), ref.numpy()) <= 5e-2
+
+
+def _small_layer(num_shared=1, rotate=1):
+    from mxmoe_amd import synth
+    from mxmoe_amd.layer import MxMoELayer
+
+    cfg = synth.MoEConfig("t", "test", 6, 2, 256, 1408, 96, num_shared=num_shared, rotate=rotate)
+    g = synth.W4A4G128
+    fm = [(synth.W4A4, synth.W8A8), (synth.W8A8, synth.W4A4), (g, g), (synth.W4A16, synth.W3A16), (synth.FP16, synth.FP16), (synth.W4A4, synth.W4A4),
+          (synth.W8A8, synth.W8A8)][: 6 + (1 if num_shared else 0)]
+    return cfg, MxMoELayer(cfg, formats=fm)
+
+
+@pytest.mark.parametrize("num_shared", [0, 1])
+def test_planned_forward_equals_the_host_planned_one(num_shared):
+    """The forward whose tables a device kernel derives from the counts (no synchronisation) against the forward whose tables the
+    host builds after reading the counts back, and against the stepwise operators: identical bits, every format in one layer; the
+    device-built tables themselves equal the host's."""
+    from mxmoe_amd import _lib, synth
+    from mxmoe_amd import layer_tables as LT
+
+    cfg, layer = _small_layer(num_shared)
+    hidden = synth.make_hidden(cfg)
+    ids, w = synth.make_routing(cfg)
+    ids[5:9, 0] = 2                                                     # one expert much busier than the others
+    layer.forward(hidden, ids)
+    want = layer.combine(w).clone()
+    got = layer(hidden, ids, w)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+    assert torch.equal(layer.call_with_host_tables(hidden, ids, w), want)
+    # the planner's tables: quantiser table, pointers and sizes of the first launch against the array-arithmetic version
+    lib = _lib.load()
+    ps = layer._planned_setup(cfg.tokens, cfg.topk)
+    et = layer.n_exp_total
+    raw = ps["b1"]["plan"].cpu().numpy()
+    off = [lib.mxmoe_plan_offset(i, et) for i in range(6)]
+    table = raw[off[1]:off[1] + 32 * et].view(np.int64).reshape(4, et)
+    ptrs = raw[off[2]:off[2] + 40 * et].view(np.int64).reshape(5, et)
+    misc = raw[off[3]:off[3] + 16].view(np.int64)
+    sizes = raw[off[4]:off[4] + 12 * et].view(np.uint32).reshape(et, 3)
+    gu, _dn = layer._static_tables()
+    rows = np.concatenate([np.bincount(ids.numpy().reshape(-1), minlength=cfg.num_experts), [cfg.tokens] * (1 if num_shared else 0)]).astype(np.int64)
+    bt = LT.block_tables(gu, rows)
+    assert np.array_equal(table, bt.table)
+    assert misc[0] == rows[: cfg.num_experts].sum()
+    assert np.array_equal(sizes, np.stack([rows, gu.n, gu.k], axis=1).astype(np.uint32))
+    b1 = ps["b1"]
+    assert np.array_equal(ptrs[0], b1["inp"].data_ptr() + 2 * bt.table[2]) and np.array_equal(ptrs[4], ps["mid"].data_ptr() + 2 * bt.out_off)
+    assert np.array_equal(ptrs[1], gu.b_ptr) and np.array_equal(ptrs[3], gu.sb_ptr)
+    assert np.array_equal(ptrs[2], np.where(gu.sld > 0, b1["scale"].data_ptr() + 2 * bt.table[3], 0))
+    assert misc[1] == (ptrs[4][-1] if num_shared else 0)
+
+
+def test_planned_forward_drops_out_of_range_experts_like_the_operators():
+    from mxmoe_amd import synth
+
+    cfg, layer = _small_layer(1)
+    hidden = synth.make_hidden(cfg)
+    ids, w = synth.make_routing(cfg)
+    ids[::7, 1] = cfg.num_experts + 2                                   # these slots belong to experts this GPU does not hold
+    layer.forward(hidden, ids)
+    want = layer.combine(w).clone()
+    got = layer(hidden, ids, w)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want) and bool(torch.isfinite(got).all())
+
+
+def test_planned_forward_replays_from_a_graph():
+    """The whole forward inside a HIP graph (nothing in it synchronises, allocates or depends on the routing): each replay, with new
+    routing and new hidden states written into the captured input buffers and eager work in between, equals the eager forward."""
+    from mxmoe_amd import synth
+
+    cfg, layer = _small_layer(1)
+    hidden = synth.make_hidden(cfg).cuda()
+    ids, w = synth.make_routing(cfg)
+    ids, w = ids.cuda(), w.cuda()
+    out = torch.empty((cfg.tokens, cfg.hidden), dtype=torch.float16, device="cuda")
+    layer(hidden, ids, w, out=out)                                      # first call: allocates the layer's buffers
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        layer(hidden, ids, w, out=out)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        layer(hidden, ids, w, out=out)
+    gen = torch.Generator(device="cpu")
+    for replay in range(4):
+        gen.manual_seed(100 + replay)
+        new_ids = torch.stack([torch.randperm(cfg.num_experts, generator=gen)[: cfg.topk] for _ in range(cfg.tokens)]).to(torch.int32)
+        if replay == 2:
+            new_ids[:, :] = torch.tensor([1, 3], dtype=torch.int32)     # all tokens on two experts: other experts empty
+        new_w = torch.rand(cfg.tokens, cfg.topk, generator=gen)
+        new_h = torch.randn(cfg.tokens, cfg.hidden, generator=gen).half()
+        layer.forward(new_h, new_ids)                                   # eager reference (and eager work between the replays)
+        want = layer.combine(new_w).clone()
+        hidden.copy_(new_h.cuda())
+        ids.copy_(new_ids.cuda())
+        w.copy_(new_w.cuda())
+        out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), f"replay {replay}"
