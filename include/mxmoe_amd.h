@@ -91,6 +91,11 @@ int mxmoe_last_status(void);
  * Host-only; used by the scheduler tests and the kernel-profile table.  Returns 1000 + kernel id on success. */
 int mxmoe_group_gemm_plan(int kernel_id, const mxmoe_dim3* h_sizes, const mxmoe_qparams* h_q, int problem_count, int32_t* branch_out, int32_t* tiles_out);
 
+/* The tile tables themselves (host-only; what the generated launcher keeps in its prefix-sum array, kernel_sketch.py:89-104): out receives
+ * {entries, tiles, phases, workgroups}, phase_tile0[9], phase_wg0[9], then per entry {first tile, first row, rows, problem | branch << 16}.
+ * At most 120 problems; used by the tests that compare the device-side planner with the host launcher. */
+int mxmoe_group_gemm_plan_tables(int kernel_id, const mxmoe_dim3* h_sizes, const mxmoe_qparams* h_q, int problem_count, int32_t* out, int out_ints);
+
 /* ---- token permutation: replaces gg_permute_inp and the sort / bincount prologue of quant_inp_act
  *      (mxmoe/kernels/src/ref_bind.cu:47-64, 449-453) ----
  *

@@ -1063,6 +1063,253 @@ __global__ void __launch_bounds__(256) row_quant_dense_kernel(const RowArgs a) {
   }
 }
 
+// One row per WORKGROUP of 8 waves for rotations B_kb kron H_512 (kb <= 32, no Sylvester factor in the table: a 14336-value row is
+// 28 x 512).  Wave w holds the k rows w, w + 8, w + 16, w + 24 of the [kb][512] view, lane l the chunk l of each, so the whole
+// Sylvester part runs inside a wave: strides 1, 2, 4 in a chunk, 8 .. 256 across lanes, no LDS and no barrier.  The dense stage is the
+// same exact integer sum as in row_quant_dense_kernel, on the matrix cores: the snapped row goes to LDS as it is ([k][column], one
+// 16-byte write per chunk), every wave gathers the second operand of its 64 columns from there (two bytes per read, each landing in
+// its half of the operand register) and multiplies B (first operand, in registers) into them, and the results return through LDS in
+// row order for the quantise / pack / store code.  Four barriers per row; two workgroups share a CU.
+constexpr int kWidePitch = 1024 + 8;                                 // bytes per k row of 512 fp16 in LDS: the 4 k groups (or row groups) that the
+                                                                     // lanes of a wave touch together land 8 or 16 banks apart
+constexpr int kWideLds = 2 * 32 * kWidePitch + 64;                   // snapped row, rotated row, reduction slots
+template <bool SILU>
+__global__ void __launch_bounds__(512) row_quant_wide_kernel(const RowArgs a) {
+  extern __shared__ __align__(16) uint8_t wlds[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int lm = lane & 15, lg = lane >> 4;
+  uint8_t* xt = wlds;                                   // [32 k rows][kWidePitch]: the snapped row
+  uint8_t* yrow = xt + 32 * kWidePitch;                 // [32 rows][kWidePitch]: the rotated row
+  float* red = reinterpret_cast<float*>(yrow + 32 * kWidePitch);  // [8] + [8]
+  const RotPlan pl = a.plan;
+  const int n = pl.n, kb = pl.kb;
+  constexpr int MAXC = 4;
+  // B as the first operand of v_mfma_f32_16x16x32_f16: lane holds row 16 mb + (lane & 15), k = 8 (lane >> 4) + 0..7
+  v8h bsign[2];
+#pragma unroll
+  for (int mb = 0; mb < 2; ++mb) {
+    const int b = 16 * mb + lm;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int bp = 8 * lg + i;
+      const float sv = a.signs[min(b, kb - 1) * kb + min(bp, kb - 1)];
+      bsign[mb][i] = (b < kb && bp < kb) ? (_Float16)sv : (_Float16)0.0f;
+    }
+  }
+  // k rows kb .. 31 are never written and must read as zero
+  for (int i = tid; i < 32 * kWidePitch / 8; i += 512) reinterpret_cast<uint2*>(xt)[i] = make_uint2(0, 0);
+  const _Float16* const src_shared = shared_src(a);
+  for (int row = blockIdx.x; row < a.rows; row += gridDim.x) {
+    if (!row_exists(a, row)) continue;
+    const bool shared_row = row >= a.R;
+    const int e = shared_row ? a.E : a.dst_exp[row];
+    const int tag = (int)a.table[e];
+    const long lrow = shared_row ? row - a.R : row - a.table[a.Et + e];
+    const long inp_off = a.table[2 * a.Et + e];
+    const long scale_off = a.table[3 * a.Et + e];
+    const bool rot = a.rotate == 2 || (a.rotate == 1 && tag != 0);
+    const _Float16* srow;
+    if (SILU) {
+      srow = shared_row ? src_shared + (long)(row - a.R) * 2 * n : a.src + (long)row * 2 * n;
+    } else {
+      srow = (shared_row ? src_shared : a.src) + (shared_row ? (long)(row - a.R) : (long)a.perm[row]) * n;
+    }
+    float v[MAXC][8];
+#pragma unroll
+    for (int i = 0; i < MAXC; ++i) {
+      const int kr = wave + 8 * i;
+      const bool live = kr < kb;
+      const int c = min(kr, kb - 1) * 64 + lane;  // chunk index in the row
+      const v8h g = *reinterpret_cast<const v8h*>(srow + c * 8);
+      if (SILU) {
+        const v8h u = *reinterpret_cast<const v8h*>(srow + n + c * 8);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float gf = (float)g[j];
+          const float sl = gf / (1.0f + exp_fixed(-gf));
+          v[i][j] = round_h(keep_f32(sl * (float)u[j]));
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[i][j] = (float)g[j];
+      }
+      if (!live) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[i][j] = 0.0f;
+      }
+    }
+    if (rot) {
+      // H_512 along each k row: strides 1, 2, 4 inside the chunk, 8 .. 256 across the lanes (ascending)
+#pragma unroll
+      for (int i = 0; i < MAXC; ++i)
+#pragma unroll
+        for (int h = 1; h < 8; h <<= 1)
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            if (!(j & h)) {
+              const float p = v[i][j], q = v[i][j + h];
+              v[i][j] = p + q;
+              v[i][j + h] = p - q;
+            }
+      auto lane_stage = [&](auto mc) {
+        constexpr int m = decltype(mc)::value;
+        const float sgn = (lane & m) ? -1.0f : 1.0f;
+#pragma unroll
+        for (int i = 0; i < MAXC; ++i)
+#pragma unroll
+          for (int j = 0; j < 8; ++j) v[i][j] = __builtin_fmaf(sgn, v[i][j], lane_xor<m>(v[i][j]));
+      };
+      lane_stage(std::integral_constant<int, 1>{});
+      lane_stage(std::integral_constant<int, 2>{});
+      lane_stage(std::integral_constant<int, 4>{});
+      lane_stage(std::integral_constant<int, 8>{});
+      lane_stage(std::integral_constant<int, 16>{});
+      lane_stage(std::integral_constant<int, 32>{});
+      float mx = 0.0f;
+#pragma unroll
+      for (int i = 0; i < MAXC; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          v[i][j] = round_h(keep_f32(v[i][j] * pl.scale));
+          mx = fmaxf(mx, fabsf(v[i][j]));
+        }
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+      if (lane == 0) red[wave] = mx;
+      __syncthreads();  // (also: the previous row's readers of xt / yrow are done)
+      mx = red[0];
+#pragma unroll
+      for (int w = 1; w < 8; ++w) mx = fmaxf(mx, red[w]);
+      const DenseGrid grid(mx);
+      // the snapped row, k row kr / chunk lane at its place
+#pragma unroll
+      for (int i = 0; i < MAXC; ++i) {
+        const int kr = wave + 8 * i;
+        if (kr < kb) {
+          v8h q;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) q[j] = (_Float16)(rintf(v[i][j] * grid.to_grid) * 0.0625f);
+          *reinterpret_cast<v8h*>(xt + kr * kWidePitch + lane * 16) = q;
+        }
+      }
+      __syncthreads();
+      // this wave's 64 columns: 4 column blocks x 2 row blocks; the second operand of a lane is column col, k = 8 (lane >> 4) + 0..7
+      const float back = grid.from_grid * 16.0f;
+#pragma unroll
+      for (int nb = 0; nb < 4; ++nb) {
+        const int col = wave * 64 + nb * 16 + lm;
+        v8h xf;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) xf[i] = *reinterpret_cast<const _Float16*>(xt + (8 * lg + i) * kWidePitch + col * 2);
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb) {
+          v4f acc = {0.f, 0.f, 0.f, 0.f};
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(bsign[mb], xf, acc, 0, 0, 0);
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int b = 16 * mb + 4 * lg + r;  // lane holds column col and rows b of the block (rows kb .. 31 are never read back)
+            *reinterpret_cast<_Float16*>(yrow + b * kWidePitch + col * 2) = (_Float16)(acc[r] * back);
+          }
+        }
+      }
+      __syncthreads();
+#pragma unroll
+      for (int i = 0; i < MAXC; ++i) {
+        const int kr = wave + 8 * i;
+        const v8h y = *reinterpret_cast<const v8h*>(yrow + min(kr, kb - 1) * kWidePitch + lane * 16);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[i][j] = kr < kb ? (float)y[j] : 0.0f;
+      }
+    }
+
+    // ---- store: fp16 copy or symmetric quantisation (as in the other row kernels); chunk c = kr * 64 + lane ----
+    if (tag == 0) {
+      _Float16* out = reinterpret_cast<_Float16*>(a.inp_store) + inp_off + lrow * n;
+#pragma unroll
+      for (int i = 0; i < MAXC; ++i) {
+        const int kr = wave + 8 * i;
+        if (kr < kb) {
+          v8h o;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) o[j] = (_Float16)v[i][j];
+          *reinterpret_cast<v8h*>(out + (kr * 64 + lane) * 8) = o;
+        }
+      }
+      continue;
+    }
+    if (tag == 3) {  // int4, one scale per 128 values = the 16 chunks held by an aligned group of 16 lanes
+      uint8_t* out = a.inp_store + 2 * (inp_off + lrow * (n / 4));
+      _Float16* sout = a.scale_store + scale_off + lrow * (n >> 7);
+#pragma unroll
+      for (int i = 0; i < MAXC; ++i) {
+        const int kr = wave + 8 * i;
+        const int c = kr * 64 + lane;
+        float gmax = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) gmax = fmaxf(gmax, fabsf(v[i][j]));
+#pragma unroll
+        for (int o = 8; o > 0; o >>= 1) gmax = fmaxf(gmax, __shfl_xor(gmax, o));
+        float scale = round_h(gmax / 7.0f);
+        if (scale == 0.0f) scale = 1.0f;
+        const ScaleDiv div(scale);
+        if (kr < kb) {
+          if ((c & 15) == 0) sout[c >> 4] = (_Float16)scale;
+          unsigned w = 0;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const float r = round_h(div(v[i][j]));
+            w |= (unsigned)((int)rintf(fminf(fmaxf(r, -7.0f), 7.0f)) & 0xF) << (4 * j);
+          }
+          *reinterpret_cast<unsigned*>(out + c * 4) = w;
+        }
+      }
+      continue;
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < MAXC; ++i)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[i][j]));
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
+    if (lane == 0) red[8 + wave] = amax;
+    __syncthreads();
+    amax = red[8];
+#pragma unroll
+    for (int w = 1; w < 8; ++w) amax = fmaxf(amax, red[8 + w]);
+    const float upper = tag == 1 ? 127.0f : 7.0f;
+    float scale = round_h(amax / upper);   // fp16 division: fp32 quotient of two fp16 values, rounded to fp16
+    if (scale == 0.0f) scale = 1.0f;       // quantize.cuh:258
+    const ScaleDiv div(scale);
+    if (tid == 0) a.scale_store[scale_off + lrow] = (_Float16)scale;
+    uint8_t* out = a.inp_store + 2 * (inp_off + lrow * (tag == 1 ? n / 2 : n / 4));
+#pragma unroll
+    for (int i = 0; i < MAXC; ++i) {
+      const int kr = wave + 8 * i;
+      if (kr < kb) {
+        const int c = kr * 64 + lane;
+        int q[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float r = round_h(div(v[i][j]));
+          q[j] = (int)rintf(fminf(fmaxf(r, -upper), upper));
+        }
+        if (tag == 1) {
+          uint2 w;
+          w.x = (q[0] & 0xFF) | ((q[1] & 0xFF) << 8) | ((q[2] & 0xFF) << 16) | ((unsigned)(q[3] & 0xFF) << 24);
+          w.y = (q[4] & 0xFF) | ((q[5] & 0xFF) << 8) | ((q[6] & 0xFF) << 16) | ((unsigned)(q[7] & 0xFF) << 24);
+          *reinterpret_cast<uint2*>(out + c * 8) = w;
+        } else {
+          unsigned w = 0;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) w |= (unsigned)(q[j] & 0xF) << (4 * j);
+          *reinterpret_cast<unsigned*>(out + c * 4) = w;
+        }
+      }
+    }
+  }
+}
+
 static int make_plan(int n, int had_k, int had_f, bool rotate, RotPlan* p) {
   p->n = n;
   p->scale = 1.0f / sqrtf((float)n);
@@ -1117,6 +1364,26 @@ static int launch_rows(const RowArgs& a, int lds_bytes, hipStream_t s) {
       case 3: hipLaunchKernelGGL((row_quant_dense_kernel<3, SILU>), dim3(wgrid), dim3(256), dlds, s, a); break;
       default: hipLaunchKernelGGL((row_quant_dense_kernel<4, SILU>), dim3(wgrid), dim3(256), dlds, s, a); break;
     }
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+      last_error() = std::string("kernel launch failed: ") + hipGetErrorString(e);
+      return 4;
+    }
+    return 0;
+  }
+  // table-driven order times H_512, one size of row: one row per 512-thread workgroup, Sylvester part inside the waves, dense stage on
+  // the matrix cores
+  if (a.plan.kb > 1 && a.plan.kb <= 32 && a.plan.m == 512 && a.plan.f == 1 && a.plan_shared.n == n && a.plan_shared.kb == a.plan.kb && a.rotate != 0) {
+    static bool opted_in[64] = {};
+    if (dev >= 0 && dev < 64 && !opted_in[dev]) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&row_quant_wide_kernel<SILU>), hipFuncAttributeMaxDynamicSharedMemorySize, kWideLds) != hipSuccess) {
+        last_error() = "could not reserve LDS for the wide-row quantiser";
+        return 4;
+      }
+      opted_in[dev] = true;
+    }
+    const int wgrid = a.rows < cus * 8 ? a.rows : cus * 8;
+    hipLaunchKernelGGL((row_quant_wide_kernel<SILU>), dim3(wgrid), dim3(512), kWideLds, s, a);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
       last_error() = std::string("kernel launch failed: ") + hipGetErrorString(e);

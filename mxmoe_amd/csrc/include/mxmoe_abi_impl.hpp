@@ -99,4 +99,29 @@ int mxmoe_group_gemm_plan(int kernel_id, const mxmoe_dim3* h_sizes, const mxmoe_
   return kernel_id + 1000;  // plan succeeded: 1000 + the kernel that would run
 }
 
+int mxmoe_group_gemm_plan_tables(int kernel_id, const mxmoe_dim3* h_sizes, const mxmoe_qparams* h_q, int problem_count, int32_t* out, int out_ints) {
+  auto& reg = registry();
+  if (problem_count <= 0 || problem_count > kMaxProblems || !h_sizes || !h_q || !out || kernel_id < 0 || kernel_id >= (int)reg.size()) {
+    last_error() = "bad argument";
+    return 5;
+  }
+  FusedArgs a;
+  std::memset(&a, 0, sizeof a);
+  int grid = 0;
+  if (const int rc = build_fused_tables(reg[kernel_id], h_sizes, h_q, 0, problem_count, a, &grid)) return rc;
+  const int need = 4 + 2 * (kMaxPhases + 1) + 4 * a.num_entries;
+  if (out_ints < need) {
+    last_error() = "output too small";
+    return 3;
+  }
+  int o = 0;
+  out[o++] = a.num_entries; out[o++] = a.total_tiles; out[o++] = a.num_phases; out[o++] = grid;
+  for (int i = 0; i <= kMaxPhases; ++i) out[o++] = a.phase_tile0[i];
+  for (int i = 0; i <= kMaxPhases; ++i) out[o++] = a.phase_wg0[i];
+  for (int i = 0; i < a.num_entries; ++i) {
+    out[o++] = a.entry[i].first; out[o++] = a.entry[i].row0; out[o++] = a.entry[i].rows; out[o++] = a.entry[i].problem_branch;
+  }
+  return 0;
+}
+
 }  // extern "C"

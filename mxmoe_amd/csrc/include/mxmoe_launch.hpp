@@ -49,6 +49,10 @@ struct FusedArgs {
   int num_phases;
   int phase_tile0[kMaxPhases + 1];
   int phase_wg0[kMaxPhases + 1];
+  // Bit p set: phase p maps workgroup v to tile v.  For the skinny weight-only tiles, which share no operand with their neighbours
+  // (every tile streams its own weights once): dealing them round-robin to the XCDs balances the memory traffic tile by tile,
+  // where contiguous runs would leave the XCD that holds a few long problems behind.
+  int phase_flat;
   // One entry per row segment of a problem, 16 bytes so that a workgroup fetches its entry with one scalar load: first tile of the
   // entry (exclusive prefix sum of tiles), first row of the segment inside its problem, rows of the segment, and
   // problem (relative to problem_offset) | tile type << 16.
@@ -130,7 +134,7 @@ __device__ __forceinline__ void fused_body(ArgsPtr args, uint8_t* smem) {
   const int tile0 = uni(args->phase_tile0[ph]);
   const int ntiles = uni(args->phase_tile0[ph + 1]) - tile0;
   const int chunk = (ntiles + kNumXcd - 1) / kNumXcd;
-  const int pt = (v % kNumXcd) * chunk + v / kNumXcd;
+  const int pt = (uni(args->phase_flat) >> ph & 1) ? v : (v % kNumXcd) * chunk + v / kNumXcd;
   if (pt >= ntiles) return;
   const int tile = tile0 + pt;
   // tile_scheduler.cuh:25-37 — the entry that holds the tile: last entry whose first tile is <= tile (binary search here; all
@@ -528,19 +532,11 @@ inline bool shape_ok(const BranchInfo& bi, const mxmoe_dim3& sz) {
   return sz.z != 0 && sz.z % bi.k_multiple == 0 && sz.y % 8 == 0 && !(wo && sz.y % 16 != 0);
 }
 
-// One launch over problems [base, base + n) of the caller's arrays with kernel `k` (n <= kMaxProblems).
-inline int launch_range(const FusedKernel& k, const void* const* As, const void* const* Bs, const void* const* sa, const void* const* sb, void* const* Cs,
-                        int32_t* const* acc, const mxmoe_dim3* d_sizes, const mxmoe_dim3* h_sizes, const mxmoe_qparams* h_q, int base, int n, hipStream_t stream) {
-  FusedArgs a;
-  std::memset(&a, 0, sizeof a);
-  a.As = reinterpret_cast<const uint8_t* const*>(As);
-  a.Bs = reinterpret_cast<const uint8_t* const*>(Bs);
-  a.sa = reinterpret_cast<const _Float16* const*>(sa);
-  a.sb = reinterpret_cast<const _Float16* const*>(sb);
-  a.Cs = reinterpret_cast<_Float16* const*>(Cs);
-  a.acc = acc;
-  a.sizes = d_sizes;
+// Tile tables of one launch over problems [base, base + n) (n <= kMaxProblems): entries, phases, totals of `a`; *grid receives the
+// workgroups to launch.  Host-only arithmetic.
+inline int build_fused_tables(const FusedKernel& k, const mxmoe_dim3* h_sizes, const mxmoe_qparams* h_q, int base, int n, FusedArgs& a, int* grid) {
   a.problem_offset = base;
+  a.phase_flat = 0;
   const PlanInfo& pi = plan_of(k);
   struct Entry {
     int row0, rows, problem, branch, tiles;
@@ -567,35 +563,60 @@ inline int launch_range(const FusedKernel& k, const void* const* As, const void*
       entries[nent++] = Entry{sg[j].row0, sg[j].rows, i, sg[j].branch, segment_tiles(pi, sg[j], (int)sz.y)};
     }
   }
-  // most expensive tile shape first; problems keep their order inside a shape (neighbouring tiles share operands)
+  // Most expensive tile shape first.  Inside a shape, the problems whose K is above the launch's smallest K go first (their tiles
+  // run longest: a shared expert with a wider intermediate, say; workgroups are dispatched in index order, and the longest
+  // jobs first is what keeps the tail of the launch short), then the others; problems keep their order otherwise (neighbouring tiles
+  // share operands).
+  uint32_t kmin = ~0u;
+  for (int i = 0; i < n; ++i) kmin = std::min(kmin, h_sizes[base + i].z);
   int total = 0, ne = 0, wg = 0, np = 0;
   for (int oi = 0; oi < pi.nb; ++oi) {
     const int b = pi.order[oi];
     const int tile0 = total;
-    for (int ei = 0; ei < nent; ++ei) {
-      const Entry& en = entries[ei];
-      if (en.branch != b || en.tiles == 0) continue;
-      a.entry[ne] = FusedArgs::Entry{total, en.row0, en.rows, en.problem | (en.branch << 16)};
-      total += en.tiles;
-      ++ne;
-    }
+    for (int pass = 0; pass < 2; ++pass)
+      for (int ei = 0; ei < nent; ++ei) {
+        const Entry& en = entries[ei];
+        if (en.branch != b || en.tiles == 0 || (h_sizes[base + en.problem].z > kmin) != (pass == 0)) continue;
+        a.entry[ne] = FusedArgs::Entry{total, en.row0, en.rows, en.problem | (en.branch << 16)};
+        total += en.tiles;
+        ++ne;
+      }
     if (total == tile0) continue;
     // shapes beyond the phase table share the last phase (their relative order is kept)
     if (np < kMaxPhases) {
       a.phase_tile0[np] = tile0;
       a.phase_wg0[np] = wg;
+      if (pi.b[b].BM <= 16) a.phase_flat |= 1 << np;
       ++np;
     }
     const int p0 = a.phase_tile0[np - 1];
     wg = a.phase_wg0[np - 1] + (total - p0 + kNumXcd - 1) / kNumXcd * kNumXcd;
   }
   a.num_entries = ne;
-  if (total == 0) return 0;
   a.total_tiles = total;
   a.num_phases = np;
   a.phase_tile0[np] = total;
   a.phase_wg0[np] = wg;
-  const hipError_t e = k.launch(a, wg, k.lds_bytes, stream);
+  *grid = wg;
+  return 0;
+}
+
+// One launch over problems [base, base + n) of the caller's arrays with kernel `k` (n <= kMaxProblems).
+inline int launch_range(const FusedKernel& k, const void* const* As, const void* const* Bs, const void* const* sa, const void* const* sb, void* const* Cs,
+                        int32_t* const* acc, const mxmoe_dim3* d_sizes, const mxmoe_dim3* h_sizes, const mxmoe_qparams* h_q, int base, int n, hipStream_t stream) {
+  FusedArgs a;
+  std::memset(&a, 0, sizeof a);
+  a.As = reinterpret_cast<const uint8_t* const*>(As);
+  a.Bs = reinterpret_cast<const uint8_t* const*>(Bs);
+  a.sa = reinterpret_cast<const _Float16* const*>(sa);
+  a.sb = reinterpret_cast<const _Float16* const*>(sb);
+  a.Cs = reinterpret_cast<_Float16* const*>(Cs);
+  a.acc = acc;
+  a.sizes = d_sizes;
+  int grid = 0;
+  if (const int rc = build_fused_tables(k, h_sizes, h_q, base, n, a, &grid)) return rc;
+  if (a.total_tiles == 0) return 0;
+  const hipError_t e = k.launch(a, grid, k.lds_bytes, stream);
   if (e != hipSuccess) {
     last_error() = std::string("kernel launch failed: ") + hipGetErrorString(e);
     return 4;

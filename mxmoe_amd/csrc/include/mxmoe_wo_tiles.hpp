@@ -113,14 +113,15 @@ struct SkinnyWoTile {
     const v8h bias = {(_Float16)1024.0f, (_Float16)1024.0f, (_Float16)64.0f, (_Float16)64.0f, (_Float16)1024.0f, (_Float16)1024.0f, (_Float16)64.0f, (_Float16)64.0f};
     constexpr int Q = NB * NKB;  // blocks of this pass, channel block major
 
-    // (scale, zero) pairs of the pass: 64 bytes per block, NKB consecutive blocks per channel block -> LDS [nb][s][64 B]
-    const uint8_t* sb = reinterpret_cast<const uint8_t*>(t.sb) + ((long)(n0 / 16) * KB + kb0) * 64;
+    // Everything the pass needs from memory is requested before anything is waited for, the weight ring first: the first blocks of
+    // the stream, the activations and the (scale, zero) pairs then arrive together, one memory latency after the pass began
+    // (waiting for the scales before requesting the weights costs a second one, which is a third of a short tile's life).
+    const uint8_t* wb = t.B + ((long)(n0 / 16) * KB + kb0) * kBlockBytes + lane * kLaneBytes;
+    auto w_of = [&](int q) { const int nb = q / NKB < nbv ? q / NKB : 0; return load_w(wb + ((long)nb * KB + q % NKB) * kBlockBytes); };
+    WReg wr[kRing];
 #pragma unroll
-    for (int c = lane; c < Q * 4; c += 64) {  // 16-byte pieces
-      const int nb = c / (NKB * 4), rest = c % (NKB * 4);
-      const v4i v = gload<v4i>(sb + ((long)(nb < nbv ? nb : 0) * KB) * 64 + rest * 16);
-      *reinterpret_cast<v4i*>(spatch + c * 16) = v;
-    }
+    for (int q = 0; q < kRing && q < Q; ++q) wr[q] = w_of(q);
+    __builtin_amdgcn_sched_barrier(0);
     // activations: lane holds row lm, k = 128*(kb0 + s) + 32*lg + 8*j + 0..7
     v8h xf[NKB][4];
     {
@@ -134,12 +135,22 @@ struct SkinnyWoTile {
           xf[s][j] = m < t.M ? __builtin_bit_cast(v8h, v) : v8h{};
         }
     }
-    const uint8_t* wb = t.B + ((long)(n0 / 16) * KB + kb0) * kBlockBytes + lane * kLaneBytes;
-    auto w_of = [&](int q) { const int nb = q / NKB < nbv ? q / NKB : 0; return load_w(wb + ((long)nb * KB + q % NKB) * kBlockBytes); };
-    WReg wr[kRing];
+    // (scale, zero) pairs of the pass: 64 bytes per block, NKB consecutive blocks per channel block -> LDS [nb][s][64 B]
+    const uint8_t* sb = reinterpret_cast<const uint8_t*>(t.sb) + ((long)(n0 / 16) * KB + kb0) * 64;
+    constexpr int kPieces = (Q * 4 + 63) / 64;  // 16-byte pieces per lane
+    v4i sv[kPieces];
 #pragma unroll
-    for (int q = 0; q < kRing && q < Q; ++q) wr[q] = w_of(q);
+    for (int i = 0; i < kPieces; ++i) {
+      const int c = min(lane + 64 * i, Q * 4 - 1);
+      const int nb = c / (NKB * 4), rest = c % (NKB * 4);
+      sv[i] = gload<v4i>(sb + ((long)(nb < nbv ? nb : 0) * KB) * 64 + rest * 16);
+    }
     __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < kPieces; ++i) {
+      const int c = lane + 64 * i;
+      if (c < Q * 4) *reinterpret_cast<v4i*>(spatch + c * 16) = sv[i];
+    }
 
     v4f sx[NKB], sxb[NKB];  // per k block: sum of x, sum of x * bias  (row = any channel, column = token)
 #pragma unroll

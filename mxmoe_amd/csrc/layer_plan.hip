@@ -64,6 +64,7 @@ __device__ __forceinline__ long wave_excl_scan(long v, int lane, long* total) {
 __global__ void __launch_bounds__(kPlanThreads) plan_block_kernel(const PlanParams p) {
   __shared__ long s_tot[4][2];                       // per wave: rows, packed input, scales, output elements
   __shared__ int s_cnt[kMaxBranches][2], s_til[kMaxBranches][2];  // per run-order rank and wave: entries, tiles
+  __shared__ int s_cnt_long[kMaxBranches][2], s_til_long[kMaxBranches][2];  // ... of which belong to long-K problems
   const int e = threadIdx.x, lane = e & 63, wave = e >> 6;
   const PlanLayout lay(p.Et);
   FusedArgs* fa = reinterpret_cast<FusedArgs*>(p.plan);
@@ -97,6 +98,16 @@ __global__ void __launch_bounds__(kPlanThreads) plan_block_kernel(const PlanPara
 #pragma unroll
     for (int i = 0; i < 4; ++i) s_tot[i][wave] = tot[i];
   }
+  // smallest K of the launch: problems above it run first inside their branch (see launch_range)
+  __shared__ int s_kmin[2];
+  {
+    int km = e < p.Et ? K : 0x7fffffff;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) km = min(km, __shfl_xor(km, o));
+    if (lane == 0) s_kmin[wave] = km;
+  }
+  __syncthreads();
+  const bool long_k = e < p.Et && K > min(s_kmin[0], s_kmin[1]);
   // segments of this problem and, per branch in run order, this wave's entries and tiles
   Segment sg[2];
   const int ns = e < p.Et ? plan_segments(p.info, fmt, (int)rows, N, sg) : 0;
@@ -116,29 +127,39 @@ __global__ void __launch_bounds__(kPlanThreads) plan_block_kernel(const PlanPara
         mine = seg_tiles[j];
         which = j;
       }
-    // entries of this branch in this wave: position = matching lanes before this one, first tile = their tiles
+    // entries of this branch in this wave, long-K problems first: position = matching lanes that run earlier, first tile = their tiles
     const uint64_t has = __ballot(which >= 0);
-    int tc = 0, tt = 0;
+    int tc = 0, tt = 0, tc_long = 0, tt_long = 0;
     if (has != 0) {  // (wave-uniform: most branches of a kernel are not used by a given launch)
+      const uint64_t has_long = __ballot(which >= 0 && long_k);
       tc = __popcll(has);
-      int inc = mine;
+      tc_long = __popcll(has_long);
+      int inc_long = long_k ? mine : 0, inc_rest = long_k ? 0 : mine;
 #pragma unroll
       for (int o = 1; o < 64; o <<= 1) {
-        const int t = __shfl_up(inc, o);
-        if (lane >= o) inc += t;
+        const int t0 = __shfl_up(inc_long, o), t1 = __shfl_up(inc_rest, o);
+        if (lane >= o) {
+          inc_long += t0;
+          inc_rest += t1;
+        }
       }
-      tt = __shfl(inc, 63);
+      tt_long = __shfl(inc_long, 63);
+      tt = tt_long + __shfl(inc_rest, 63);
+      const uint64_t before = (1ull << lane) - 1;
 #pragma unroll
       for (int j = 0; j < 2; ++j)
         if (which == j) {
           seg_rank[j] = r;
-          seg_pos[j] = __popcll(has & ((1ull << lane) - 1));
-          seg_first[j] = inc - mine;
+          // position / first tile inside this wave's entries of its own class; the other wave's and the other class's are added below
+          seg_pos[j] = long_k ? __popcll(has_long & before) : __popcll(has & ~has_long & before);
+          seg_first[j] = long_k ? inc_long - mine : inc_rest - mine;
         }
     }
     if (lane == 0) {
       s_cnt[r][wave] = tc;
       s_til[r][wave] = tt;
+      s_cnt_long[r][wave] = tc_long;
+      s_til_long[r][wave] = tt_long;
     }
   }
   __syncthreads();
@@ -169,9 +190,20 @@ __global__ void __launch_bounds__(kPlanThreads) plan_block_kernel(const PlanPara
         pos += s_cnt[r][0] + s_cnt[r][1];
         first += s_til[r][0] + s_til[r][1];
       }
-      if (wave == 1) {
-        pos += s_cnt[seg_rank[j]][0];
-        first += s_til[seg_rank[j]][0];
+      // inside the branch: [long-K entries of wave 0][of wave 1][other entries of wave 0][of wave 1]
+      const int r = seg_rank[j];
+      if (long_k) {
+        if (wave == 1) {
+          pos += s_cnt_long[r][0];
+          first += s_til_long[r][0];
+        }
+      } else {
+        pos += s_cnt_long[r][0] + s_cnt_long[r][1];
+        first += s_til_long[r][0] + s_til_long[r][1];
+        if (wave == 1) {
+          pos += s_cnt[r][0] - s_cnt_long[r][0];
+          first += s_til[r][0] - s_til_long[r][0];
+        }
       }
       fa->entry[pos] = FusedArgs::Entry{first, sg[j].row0, sg[j].rows, e | (sg[j].branch << 16)};
     }
@@ -180,7 +212,7 @@ __global__ void __launch_bounds__(kPlanThreads) plan_block_kernel(const PlanPara
     // rows routed = sum over the routed experts: wave 0's part is in routed_tot, wave 1 holds experts 64.. (all routed or shared)
     misc[0] = s_tot[0][0] + s_tot[0][1] - (p.Et > p.E ? (long)p.shared_rows : 0);
     if (p.Et == p.E) misc[1] = 0;
-    int total = 0, wg = 0, np = 0, ne = 0;
+    int total = 0, wg = 0, np = 0, ne = 0, flat = 0;
     for (int r = 0; r < p.info.nb; ++r) {
       const int tile0 = total;
       total += s_til[r][0] + s_til[r][1];
@@ -189,6 +221,7 @@ __global__ void __launch_bounds__(kPlanThreads) plan_block_kernel(const PlanPara
       if (np < kMaxPhases) {  // shapes beyond the phase table share the last phase
         fa->phase_tile0[np] = tile0;
         fa->phase_wg0[np] = wg;
+        if (p.info.b[p.info.order[r]].BM <= 16) flat |= 1 << np;
         ++np;
       }
       const int p0 = fa->phase_tile0[np - 1];
@@ -197,6 +230,7 @@ __global__ void __launch_bounds__(kPlanThreads) plan_block_kernel(const PlanPara
     fa->phase_tile0[np] = total;
     fa->phase_wg0[np] = wg;
     fa->num_phases = np;
+    fa->phase_flat = flat;
     fa->num_entries = ne;
     fa->total_tiles = total;
     fa->problem_offset = 0;

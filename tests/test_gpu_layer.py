@@ -252,6 +252,48 @@ def test_planned_forward_equals_the_host_planned_one(num_shared):
     assert misc[1] == (ptrs[4][-1] if num_shared else 0)
 
 
+def test_device_planner_writes_the_host_launchers_tile_tables():
+    """Entries, phases and totals that the planning kernel writes against the host launcher's for the same counts, on a layer whose
+    shared expert is twice as wide as the routed ones (its tiles run first inside their branch) and with experts left empty."""
+    import ctypes as C
+
+    from mxmoe_amd import _lib, synth
+    from mxmoe_amd.layer import MxMoELayer
+
+    cfg = synth.MoEConfig("t", "test", 9, 2, 256, 1408, 70, num_shared=2, formats=(synth.W4A16, synth.W3A16, synth.W4A4, synth.W8A8), format_probs=(0.3, 0.2, 0.3, 0.2))
+    layer = MxMoELayer(cfg)
+    hidden = synth.make_hidden(cfg)
+    ids, w = synth.make_routing(cfg)
+    ids = torch.where(ids == 4, torch.full_like(ids, 6), ids)            # expert 4 receives nothing
+    layer.forward(hidden, ids)
+    want = layer.combine(w).clone()
+    assert torch.equal(layer(hidden, ids, w), want)
+    lib = _lib.load()
+    ps = layer._planned_setup(cfg.tokens, cfg.topk)
+    et = layer.n_exp_total
+    rows = np.concatenate([np.bincount(ids.numpy().reshape(-1), minlength=cfg.num_experts), [cfg.tokens]])
+    for blk, qps in (("b1", layer.qp_gate_up), ("b2", layer.qp_down)):
+        b = ps[blk]
+        h_sizes = (_lib.Dim3 * et)(*[_lib.Dim3(int(rows[e]), b["h"][e].N, b["h"][e].K) for e in range(et)])
+        h_q = (_lib.QParams * et)(*[_lib.QParams(int(q[0]), int(q[1]), int(q[2]), 1 if q[3] else 0) for q in qps])
+        out = (C.c_int32 * 1200)()
+        assert lib.mxmoe_group_gemm_plan_tables(b["kid"], h_sizes, h_q, et, out, 1200) == 0, lib.mxmoe_last_error()
+        host = np.array(out[:], dtype=np.int32)
+        ne, tiles, nph, grid = host[:4]
+        hdr = b["plan"].cpu().numpy()[:4096].view(np.int32)
+        base = 56 // 4                                                  # seven pointers, then the integers of the table
+        assert (hdr[base], hdr[base + 1], hdr[base + 2], hdr[base + 3]) == (0, ne, tiles, nph)
+        assert np.array_equal(hdr[base + 4: base + 4 + nph + 1], host[4: 4 + nph + 1])                  # phase_tile0
+        assert np.array_equal(hdr[base + 13: base + 13 + nph + 1], host[13: 13 + nph + 1])              # phase_wg0
+        assert np.array_equal(hdr[base + 23: base + 23 + 4 * ne], host[22: 22 + 4 * ne])                # entries, in launch order (after phase_flat)
+        assert grid <= b["grid"]
+        if blk == "b2":                                                 # the shared expert's down block is the long one: first of its branch
+            first_problems = [int(host[22 + 4 * i + 3]) & 0xFFFF for i in range(ne)]
+            br = [int(host[22 + 4 * i + 3]) >> 16 for i in range(ne)]
+            sh_at = first_problems.index(cfg.num_experts)
+            assert sh_at == br.index(br[sh_at])
+
+
 def test_planned_forward_drops_out_of_range_experts_like_the_operators():
     from mxmoe_amd import synth
 
