@@ -237,6 +237,35 @@ def time_whole_layer(cfg, layer, reps: int = 7) -> dict:
     return out
 
 
+def mfma_probe(iters: int = 20000, workgroups: int = 512, repeats: int = 3):
+    """Rate and shader clock of a bare v_mfma_i32_32x32x32_i8 loop (512 workgroups = two per CU, 8 independent accumulators per wave) for
+    four operand patterns.  Each pattern runs `repeats` times back to back after a short warm-up launch; the last run is reported."""
+    import torch
+
+    from mxmoe_amd import _lib
+
+    lib = _lib.load()
+    src = torch.randint(0, 256, (65536,), dtype=torch.uint8, device="cuda", generator=torch.Generator("cuda").manual_seed(0))
+    out = torch.zeros(workgroups * 256 + 4, dtype=torch.int32, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    ops = 2 * 32 * 32 * 32 * 8 * iters * 4 * workgroups
+    res = {"probe": "bare v_mfma_i32_32x32x32_i8 loop", "workgroups": workgroups, "iters": iters, "ops_per_launch": ops, "peak_tops": PEAK["int8"], "modes": {}}
+    for mode, name in enumerate(["zero operands", "constant operands", "random 16*int4 operands", "random int8 operands", "random offset-binary int4 operands (0..15)", "random sign-extended int4 operands"]):
+        _lib.check(lib, lib.mxmoe_mfma_probe(mode, 100, workgroups, src.data_ptr(), out.data_ptr(), stream))
+        torch.cuda.synchronize()
+        for _ in range(repeats):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            _lib.check(lib, lib.mxmoe_mfma_probe(mode, iters, workgroups, src.data_ptr(), out.data_ptr(), stream))
+            e1.record()
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1)
+        rec = out[-4:].cpu().numpy().view("uint64")
+        res["modes"][name] = {"ms": round(ms, 3), "tops": round(ops / (ms * 1e-3) / 1e12, 1), "of_peak": round(ops / (ms * 1e-3) / 1e12 / PEAK["int8"], 3),
+                              "shader_clock_ghz": round(float(rec[0]) / (float(rec[1]) * 10.0), 3)}
+    return res
+
+
 def run_workload(name: str, steps: int, warmup: int, tokens=None, whole: bool = True):
     cfg, layer = build_layer(name, tokens)
     ms, up, dn = time_layer(layer, steps, warmup)
@@ -263,6 +292,8 @@ def main() -> int:
     ap.add_argument("--no-whole-layer", action="store_true", help="skip the wall-clock timing of the whole forward (profiling runs: the trace then ends with the launches the roofline entry is measured on)")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="BYTES",
                     help="instead of the benchmark, run a plain device copy of BYTES bytes 5 times (reference point for the FETCH_SIZE / WRITE_SIZE counters)")
+    ap.add_argument("--mfma-probe", action="store_true",
+                    help="instead of the benchmark, time a bare loop of int8 matrix instructions per operand pattern (the ceiling of the matrix pipes on this GPU)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (the layer would shard by expert, one all-to-all of rows either side of the launches). Use --gpus 1.", file=sys.stderr)
@@ -281,6 +312,9 @@ def main() -> int:
             dst.copy_(src)
         torch.cuda.synchronize()
         print(json.dumps({"copy_bytes": args.copy_calibration, "copies": 5}))
+        return 0
+    if args.mfma_probe:
+        print(json.dumps(mfma_probe()))
         return 0
     from mxmoe_amd import synth
 

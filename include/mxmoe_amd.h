@@ -197,6 +197,15 @@ int mxmoe_silu_mul_quant_planned(const void* gate_up, const void* d_plan_gate_up
 int mxmoe_unpermute_combine_planned(const void* down_out, const void* d_plan_down, int num_problems, const float* topk_weights, const int64_t* src_slot, int num_tokens,
                                     int topk, int K, void* out, void* workspace, void* stream);
 
+/* ---- diagnostic (no counterpart in the reference): the rate the int8 matrix pipes sustain on their own ----
+ * One launch of a bare loop of v_mfma_i32_32x32x32_i8 (8 independent accumulators per wave, two waves per SIMD, no memory traffic in
+ * the loop): `workgroups` x 256 threads, `iters` x 8 instructions per wave = 2*32*32*32 * 8 * iters * 4 * workgroups operations.
+ * mode: 0 all-zero operands, 1 a constant byte pattern, 2 random bytes 16*v (widened int4 codes),  3 random int8 bytes,
+ * 4 random bytes 0..15 (offset-binary int4), 5 random sign-extended int4 bytes.
+ * d_src: 65536 bytes of random data; d_out: (workgroups * 256 + 4) * 4 bytes; its last 16 bytes receive the shader-clock cycles and
+ * the 100 MHz real-time ticks of workgroup 0's loop (two uint64), which give the clock the chip ran at.  bench.py --mfma-probe. */
+int mxmoe_mfma_probe(int mode, int iters, int workgroups, const void* d_src, void* d_out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

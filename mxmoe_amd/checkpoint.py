@@ -18,7 +18,7 @@ import numpy as np
 import torch
 
 from .hadamard import get_hadK
-from .weights import PackedWeight, quantize_and_pack
+from .weights import PackedWeight, pack_codes, quantize_and_pack
 
 FORMAT_VERSION = 1
 MOE_MLP_NAME_MAP = {"ds2": "mlp", "qwen2_moe": "mlp", "qwen2_moe_57b": "mlp", "mixtral": "block_sparse_moe"}
@@ -66,18 +66,94 @@ def rotate_input_weights(w: torch.Tensor) -> torch.Tensor:
     return (w.to(torch.float64) @ q.T).to(w.dtype)
 
 
-def pack_layer(experts, formats, rotate: int = 0, model: str = "", layer: int = 0, num_shared: int = 0, device="cpu"):
+def recover_grid(w: torch.Tensor, bits: int, gsize: int, sym: bool):
+    """Codes, scale and zero point of a weight matrix that is ALREADY on a quantisation grid: every group of `w` [N, K] holds values
+    `scale * (q - zero)` with integer q in 0 .. 2^bits - 1 and an integer zero, stored in fp16 or bf16 (what a GPTQ run saves:
+    mxmoe/quant/gptq.py:21-25 is the grid, :539-546 the `state_dict` of fake-quantised weights).  Re-quantising such a matrix by
+    min / max would move it (its extreme codes need not be in use); this finds the grid itself.
+    -> (q [N, K] int, scale, zp) with value = q * scale + zp as `weights.pack_codes` takes them: signed codes and zp = 0 for symmetric
+    grids, codes from 0 and zp = (lowest value in use) otherwise.  Raises ValueError for a group that lies on no such grid.
+
+    Per group: the smallest non-zero magnitude is j * scale for a small j (weights cluster around zero, so j = 1 nearly always); for
+    j = 1, 2, ... the candidate is refined by least squares, first over the values within 8 steps of zero, then over the whole group
+    (a GPTQ scale is an fp32 number, and the stored values carry their type's rounding: an 8-bit code of 127 steps kept in bf16 is off
+    by up to half a step, so such a file does not determine its codes and the nearest ones are taken); the first candidate under which
+    every value is within 0.3 (plus the type's rounding) of an integer multiple and the integers span at most 2^bits - 1 is taken and
+    rounded to fp16, the type the kernels read scales in."""
+    n, k = w.shape
+    g = k if gsize == -1 else gsize
+    v = w.to(torch.float64).reshape(-1, g)
+    maxq = (1 << bits) - 1
+    # distance from an integer multiple that storage rounding alone explains: half the type's spacing at the largest multiple
+    eps = {torch.bfloat16: 2.0**-8, torch.float16: 2.0**-11}.get(w.dtype, 0.0)
+    tol = min(0.49, 0.3 + eps * maxq)
+    mag = v.abs()
+    vmin_nz = torch.where(mag > 0, mag, torch.full_like(mag, float("inf"))).amin(dim=1, keepdim=True)
+    flat = ~torch.isfinite(vmin_nz)                                       # all-zero groups: any scale does
+    vmin_nz = torch.where(flat, torch.ones_like(vmin_nz), vmin_nz)
+    scale = torch.zeros_like(vmin_nz)
+    done = torch.zeros_like(flat)
+    for j in range(1, 9):
+        cand = vmin_nz / j
+        t0 = v / cand
+        near = t0.abs() <= 8.5                                              # multiples small enough for the first guess to place
+        ok = (((t0 - t0.round()).abs() * near).amax(dim=1, keepdim=True) < 0.3)
+        ls = lambda t, m: ((v * t * m).sum(dim=1, keepdim=True) / (t * t * m).sum(dim=1, keepdim=True).clamp_min(1e-300))
+        s1 = torch.where(flat, torch.ones_like(cand), ls(t0.round(), near))
+        s2 = torch.where(flat, torch.ones_like(cand), ls((v / s1).round(), torch.ones_like(near)))
+        t2 = v / s2
+        ti = t2.round()
+        ok &= ((t2 - ti).abs().amax(dim=1, keepdim=True) < tol) & ((ti.amax(dim=1, keepdim=True) - ti.amin(dim=1, keepdim=True)) <= maxq)
+        take = ok & ~done
+        scale = torch.where(take, s2.to(torch.float16).to(torch.float64), scale)
+        done |= ok
+    if not bool(done.all()):
+        bad = int((~done).nonzero()[0, 0])
+        raise ValueError(f"group {bad} (channel {bad // (k // g)}) is not on a {bits}-bit grid")
+    t = (v / scale).round()
+    if bool(((t * scale - v).abs() > 0.5 * scale).any()):
+        raise ValueError("refined scale does not reproduce the stored values")
+    if sym:
+        lo, hi = -(1 << (bits - 1)), (1 << (bits - 1)) - 1
+        if bool((t.amin() < lo) | (t.amax() > hi)):
+            raise ValueError(f"symmetric {bits}-bit codes outside {lo} .. {hi}")
+        q, zp = t, torch.zeros_like(scale)
+    else:
+        tmin = t.amin(dim=1, keepdim=True)
+        q, zp = t - tmin, tmin * scale
+    return q.reshape(n, k), scale.to(torch.float16), zp.to(torch.float16)
+
+
+def ingest_fake_quant(w: torch.Tensor, qparams, keep_codes: bool = False) -> PackedWeight:
+    """Pack a fake-quantised weight matrix (GPTQ output) without quantising it again.  Symmetric weight-only formats are stored
+    offset-binary like their RTN counterparts."""
+    a_bits, w_bits, gsize, sym = qparams
+    n, k = w.shape
+    if w_bits >= 16:
+        return PackedWeight(w.to(torch.float16).contiguous(), None, tuple(qparams), n, k)
+    q, scale, zp = recover_grid(w, w_bits, gsize, sym)
+    return pack_codes(q, scale, zp, tuple(qparams), n, k, keep_codes)
+
+
+def load_fake_quant_state_dict(path: str) -> dict:
+    """The `.pt` file a GPTQ run writes (gptq.py:546: `torch.save(model.state_dict(), ...)`), read as tensors only."""
+    return torch.load(path, map_location="cpu", weights_only=True)
+
+
+def pack_layer(experts, formats, rotate: int = 0, model: str = "", layer: int = 0, num_shared: int = 0, device="cpu", fake_quant: bool = False):
     """experts: [(W13, W2)] fp16 (shared expert last when num_shared > 0); formats: [(gate_up qparams, down qparams)].
     rotate as in the operators: 0 never, 1 blocks with quantised activations, 2 every block.
+    fake_quant: the weights are a GPTQ run's fake-quantised output (rotated there already, if at all: gptq.py:525-528), so they are
+    neither rotated nor re-quantised here; their grid is recovered (`recover_grid`) and packed; `rotate` is only recorded.
     Returns ({tensor name: tensor}, metadata dict)."""
     tensors, meta_e = {}, []
     for e, ((w13, w2), (gu, dn)) in enumerate(zip(experts, formats)):
-        if rotate == 2 or (rotate == 1 and gu[0] < 16):
+        if not fake_quant and (rotate == 2 or (rotate == 1 and gu[0] < 16)):
             w13 = rotate_input_weights(w13)
-        if rotate == 2 or (rotate == 1 and dn[0] < 16):
+        if not fake_quant and (rotate == 2 or (rotate == 1 and dn[0] < 16)):
             w2 = rotate_input_weights(w2)
         for name, w, qp in (("w13", w13, gu), ("w2", w2, dn)):
-            p = quantize_and_pack(w.to(device), tuple(qp))
+            p = ingest_fake_quant(w.to(device), tuple(qp)) if fake_quant else quantize_and_pack(w.to(device), tuple(qp))
             tensors[f"e{e}.{name}.data"] = p.data.cpu().contiguous()
             if p.scale is not None:
                 tensors[f"e{e}.{name}.scale"] = p.scale.cpu().contiguous()

@@ -6,7 +6,9 @@ the reference keeps them as literal ``+1, -1`` tables in ``mxmoe/quant/hadamard_
 tables, checks ``H @ H.T == K * I`` for each, and stores them bit-packed (1 bit per entry, bit set
 means -1) so the product and the CPU oracle can load them without the reference being present.
 
-Run once, in the development container:  python mxmoe_amd/data/make_had_tables.py
+Run once, where a checkout of the reference exists; the table file is the argument:
+    python mxmoe_amd/data/make_had_tables.py <reference>/mxmoe/quant/hadamard_utils.py
+Nothing in the package imports this script or knows where a reference checkout lives.
 """
 import re
 import sys
@@ -14,12 +16,14 @@ from pathlib import Path
 
 import numpy as np
 
-SRC = Path("/root/reference/mxmoe/quant/hadamard_utils.py")
 OUT = Path(__file__).with_name("had_tables.npz")
 
 
 def main() -> int:
-    text = SRC.read_text()
+    if len(sys.argv) != 2:
+        print(__doc__)
+        return 2
+    text = Path(sys.argv[1]).read_text()
     blocks = re.split(r"^def get_had(\d+)\(\):", text, flags=re.M)
     tables = {}
     for name, body in zip(blocks[1::2], blocks[2::2]):

@@ -36,6 +36,13 @@ def quantize_and_pack(w: torch.Tensor, qparams, keep_codes: bool = False) -> Pac
     if w_bits >= 16:
         return PackedWeight(w.contiguous(), None, tuple(qparams), n, k)
     q, scale, zp = quant_minmax(w, w_bits, gsize, sym)
+    return pack_codes(q, scale, zp, qparams, n, k, keep_codes)
+
+
+def pack_codes(q: torch.Tensor, scale: torch.Tensor, zp: torch.Tensor, qparams, n: int, k: int, keep_codes: bool = False) -> PackedWeight:
+    """Pack integer codes `q` [N, K] with their fp16 `scale` / `zp` (one per channel, or per channel and group; value = q * scale + zp)
+    into the kernels' layouts.  Symmetric codes are signed, asymmetric ones 0 .. 2^bits - 1."""
+    a_bits, w_bits, gsize, sym = qparams
     if a_bits < 16 and gsize == 128:
         # w4a4_g128_sym: codes as for w4a4, one scale per channel and 128-wide K group, stored group-major [K/128, N] so that a
         # tile reads the scales of its channels for one group as one contiguous run

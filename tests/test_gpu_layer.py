@@ -200,6 +200,53 @@ def test_layer_from_checkpoint_file_keeps_the_function(tmp_path):
     assert _rel(a.float().numpy(), ref.numpy()) <= 5e-2
 
 
+def test_layer_from_fake_quantised_weights_is_their_function(tmp_path):
+    """Weights already on a quantisation grid (what a GPTQ run saves) are packed with their own codes: with fp16 activations
+    (w4a16 / w3a16 blocks) the layer is the MLP of exactly those weights, to fp16 rounding; re-quantising them by min / max would
+    add a second quantisation error."""
+    import sys, os
+    sys.path.insert(0, os.path.dirname(__file__))
+    from test_checkpoint import _gptq_like
+    from mxmoe_amd import checkpoint as C
+    from mxmoe_amd import synth
+    from mxmoe_amd.layer import MxMoELayer
+
+    cfg = synth.MoEConfig("t", "qwen2_moe", 4, 2, 256, 384, 48, rotate=0, formats=(synth.W4A16,), format_probs=(1.0,))
+    formats = [(synth.W4A16, synth.W3A16)] * cfg.num_experts
+    experts = []
+    for e in range(cfg.num_experts):
+        w13, _, _ = _gptq_like(2 * cfg.inter, cfg.hidden, 4, 128, False, torch.bfloat16, 100 + e)
+        w2, _, _ = _gptq_like(cfg.hidden, cfg.inter, 3, 128, False, torch.bfloat16, 200 + e)
+        experts.append((w13, w2))
+    tensors, meta = C.pack_layer(experts, formats, rotate=0, model="qwen2_moe", fake_quant=True)
+    path = str(tmp_path / "gptq_layer.safetensors")
+    C.save_layer(path, tensors, meta)
+    w13p, w2p, _ = C.load_layer(path, device="cuda")
+    hidden = synth.make_hidden(cfg)
+    ids, w = synth.make_routing(cfg)
+    layer = MxMoELayer(cfg, packed=(w13p, w2p))
+    out = layer(hidden, ids, w).float().cpu()
+
+    def mlp(ws):
+        x = hidden.float().cpu()
+        ref = torch.zeros(cfg.tokens, cfg.hidden)
+        for t in range(cfg.tokens):
+            for j in range(cfg.topk):
+                w13_, w2_ = ws[int(ids[t, j])]
+                h = (w13_.float() @ x[t]).half().float()
+                g, u = h[:cfg.inter], h[cfg.inter:]
+                ref[t] += float(w[t, j]) * (w2_.float() @ (g * torch.sigmoid(g) * u).half().float())
+        return ref
+
+    ref = mlp(experts)
+    err = _rel(out.numpy(), ref.numpy())
+    assert err <= 4e-3, err
+    # the same weights quantised a second time by min / max are measurably further from their own function
+    requant = MxMoELayer(cfg, formats=formats, weights=[(a.half(), b.half()) for a, b in experts])
+    err2 = _rel(requant(hidden, ids, w).float().cpu().numpy(), ref.numpy())
+    assert err2 > 3 * err, (err, err2)
+
+
 def _small_layer(num_shared=1, rotate=1):
     from mxmoe_amd import synth
     from mxmoe_amd.layer import MxMoELayer
