@@ -32,7 +32,13 @@ calls the third-party ``fast_hadamard_transform`` CUDA package (Dao-AILab, versi
 empty submodule in the reference) and an fp16 ``hadK @ x`` matmul whose accumulation order is
 backend dependent.  None of the reference's files pins their last fp16 bit.  The order used here
 is this build's own deterministic definition; agreement with the reference at that boundary is
-"equal up to fp16 rounding of the rotated activation".
+"equal up to fp16 rounding of the rotated activation".  Also unpinned: the rounding inside
+``silu_mul`` (the reference's kernel source for it, act_kernel.cuh, is absent; torch's fp16
+``act_fn(g) * u`` rounds the activation to fp16 before the multiply, here silu(g) stays in fp32
+and the product is rounded once), at most one fp16 ulp of the product apart.
+* ``dense_grid`` / the exact dense stage of ``online_hadamard`` — python-int sums in shuffled
+  orders give the same bits; grid edges (zero rows, subnormal and largest fp16 values).
+* ``fma_f32`` / ``exp_f32_fixed`` — one correct rounding against exact rational arithmetic.
 """
 from __future__ import annotations
 
