@@ -73,6 +73,12 @@ template <class T>
 __device__ __forceinline__ void gstore(void* p, const T& v) {
   *(MXMOE_GLOBAL T*)(p) = v;
 }
+// Output rows are written once and read by a later kernel: a streaming store keeps them from displacing the operands that the
+// workgroups of the launch still share in L2.
+template <class T>
+__device__ __forceinline__ void gstore_stream(void* p, const T& v) {
+  __builtin_nontemporal_store(v, (MXMOE_GLOBAL T*)(p));
+}
 
 // Raw buffer resource over `bytes` bytes at `p` (stride 0: offsets are plain byte offsets, loads past the end return zero).
 __device__ __forceinline__ v4i make_rsrc(const void* p, unsigned bytes) {
@@ -442,7 +448,7 @@ struct MfmaTile {
         const int m = m0 + wm * TM + i0 * 32 + ml;
         const int n = n0 + wn * TN + pc * 8;
         const v4i v = *reinterpret_cast<const v4i*>(patch + ml * kPitch + pc * 16);
-        if (m < M && n < N) gstore<v4i>(t.C + (long)m * N + n, v);
+        if (m < M && n < N) gstore_stream<v4i>(t.C + (long)m * N + n, v);
       }
     }
   }
@@ -763,7 +769,7 @@ struct WxAxTile {
         const int m = m0 + i0 * 32 + ml;
         const int n = n0 + wave * TN + pc * 8;
         const v4i v = *reinterpret_cast<const v4i*>(patch + ml * kPitch + pc * 16);
-        if (m < M && n < N) gstore<v4i>(t.C + (long)m * N + n, v);
+        if (m < M && n < N) gstore_stream<v4i>(t.C + (long)m * N + n, v);
       }
     }
   }

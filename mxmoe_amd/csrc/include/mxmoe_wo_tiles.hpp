@@ -396,7 +396,7 @@ struct WoMfmaTile {
       const int ml = r0 + pr;
       const int m = m0 + wm * 64 + ml, n = n0 + wn * 64 + pc * 8;
       const v4i v = *reinterpret_cast<const v4i*>(patch + ml * kPitch + pc * 16);
-      if (m < M && n < N) gstore<v4i>(t.C + (long)m * N + n, v);
+      if (m < M && n < N) gstore_stream<v4i>(t.C + (long)m * N + n, v);
     }
   }
 };
