@@ -266,6 +266,33 @@ def mfma_probe(iters: int = 20000, workgroups: int = 512, repeats: int = 3):
     return res
 
 
+def one_problem(spec: str):
+    """One problem of one format through the default integer kernel, timed with its quantised random operands, then with every code
+    byte set to one constant, then with all codes zero.  The launches are identical instruction for instruction; what differs is how
+    many operand bits toggle in the matrix pipes, and with it the clock the GPU sustains."""
+    import torch
+
+    from mxmoe_amd import _lib, harness
+
+    fmt, dims = spec.split(":")
+    m, n, k = (int(x) for x in dims.lower().split("x"))
+    bits = {"w4a4": 4, "w8a8": 8}[fmt]
+    lib = _lib.load()
+    prob = harness.make_problem({"shape": [m, n, k], "w_bits": bits, "a_bits": bits, "gsize": -1, "sym": True}, None)
+    launch = harness._launch_of([prob], lib, lib.mxmoe_find_kernel(b"groupgemm_hz_fused_wxax"))
+    res = {"problem": spec, "kernel": "groupgemm_hz_fused_wxax", "ops": 2 * m * n * k, "peak_tops": PEAK["int8"], "operands": {}}
+    for name in ("random codes", "constant codes", "zero codes"):
+        if name == "constant codes":
+            prob["A"].fill_(0x37)
+            prob["B"].fill_(0x5A)
+        elif name == "zero codes":
+            prob["A"].zero_()
+            prob["B"].zero_()
+        ms = harness.bench_func(launch.run, warmup=20, iters=30)["median"]
+        res["operands"][name] = {"us": round(ms * 1e3, 1), "tops": round(2 * m * n * k / ms / 1e9, 1), "of_peak": round(2 * m * n * k / ms / 1e9 / PEAK["int8"], 3)}
+    return res
+
+
 def run_workload(name: str, steps: int, warmup: int, tokens=None, whole: bool = True):
     cfg, layer = build_layer(name, tokens)
     ms, up, dn = time_layer(layer, steps, warmup)
@@ -292,6 +319,9 @@ def main() -> int:
     ap.add_argument("--no-whole-layer", action="store_true", help="skip the wall-clock timing of the whole forward (profiling runs: the trace then ends with the launches the roofline entry is measured on)")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="BYTES",
                     help="instead of the benchmark, run a plain device copy of BYTES bytes 5 times (reference point for the FETCH_SIZE / WRITE_SIZE counters)")
+    ap.add_argument("--one-problem", default="", metavar="FMT:MxNxK",
+                    help="instead of the benchmark, time one GroupGEMM problem (FMT w4a4 or w8a8, e.g. w4a4:32768x2048x4096) through the default "
+                         "kernel with random, constant and all-zero operand codes: the same instruction stream at three levels of operand toggling")
     ap.add_argument("--mfma-probe", action="store_true",
                     help="instead of the benchmark, time a bare loop of int8 matrix instructions per operand pattern (the ceiling of the matrix pipes on this GPU)")
     args = ap.parse_args()
@@ -315,6 +345,9 @@ def main() -> int:
         return 0
     if args.mfma_probe:
         print(json.dumps(mfma_probe()))
+        return 0
+    if args.one_problem:
+        print(json.dumps(one_problem(args.one_problem)))
         return 0
     from mxmoe_amd import synth
 
