@@ -175,6 +175,8 @@ int mxmoe_unpermute_combine(const void* down_out, const void* shared_out, const 
  *                                  (workgroups past the planned tiles cost about 10 - 20 ns each, so the bound is kept tight);
  *   mxmoe_plan_block               enqueue the planning kernel for one block (inp_store / scale_store: the packed activations and
  *                                  their scales that the block reads, out_store: where its output rows go);
+ *   mxmoe_plan_layer               the same for the two blocks of a layer (gate_up, down) in one launch: both plans depend on nothing
+ *                                  but the tokens-per-expert counts, and a forward of a few dozen microseconds feels every launch;
  *   mxmoe_group_gemm_planned       the fused launch, grid from mxmoe_plan_grid_bound (workgroups past the planned tiles exit at once);
  *   mxmoe_quant_act_planned, mxmoe_silu_mul_quant_planned, mxmoe_unpermute_combine_planned
  *                                  as their namesakes, with d_plan in place of exp_table / row counts / shared-expert pointers;
@@ -187,6 +189,7 @@ int mxmoe_plan_select_kernel(int kernel_id, const mxmoe_block_desc* h_desc, int 
 int mxmoe_plan_grid_bound(int kernel_id, const mxmoe_block_desc* h_desc, int num_experts, int routed_rows_max, int shared_rows);
 int mxmoe_plan_block(int kernel_id, const int64_t* d_recv_tokens_per_exp, int num_experts, int shared_rows, const mxmoe_block_desc* d_desc,
                      const mxmoe_block_desc* h_desc, const void* inp_store, const void* scale_store, void* out_store, void* d_plan, void* stream);
+int mxmoe_plan_layer(const mxmoe_plan_call* gate_up, const mxmoe_plan_call* down, const int64_t* d_recv_tokens_per_exp, int num_experts, int shared_rows, void* stream);
 int mxmoe_group_gemm_planned(int kernel_id, const void* d_plan, int grid, void* stream);
 int mxmoe_quant_act_planned(const void* hidden, void* inp_store, void* scale_store, const int32_t* dst_exp_sorted, const int64_t* perm_indices, const void* d_plan,
                             int K, int rows_capacity, int num_tokens, int num_experts, int has_shared, int rotate, int had_k, int had_f, const float* had_signs,

@@ -11,6 +11,12 @@ class Dim3(C.Structure):
     _fields_ = [("x", C.c_uint32), ("y", C.c_uint32), ("z", C.c_uint32)]
 
 
+class PlanCall(C.Structure):
+    """mxmoe_plan_call."""
+    _fields_ = [("kernel_id", C.c_int), ("d_desc", C.c_void_p), ("h_desc", C.c_void_p), ("inp_store", C.c_void_p), ("scale_store", C.c_void_p),
+                ("out_store", C.c_void_p), ("d_plan", C.c_void_p)]
+
+
 class BlockDesc(C.Structure):
     """mxmoe_block_desc: one linear block of one expert for the device-side planner (40 bytes)."""
     _fields_ = [("a_bits", C.c_int32), ("w_bits", C.c_int32), ("gsize", C.c_int32), ("sym", C.c_uint8), ("_pad", C.c_uint8 * 3),
@@ -52,6 +58,7 @@ SIGNATURES = {
     "mxmoe_plan_select_kernel": (_I, [_I, _P, _I]),
     "mxmoe_plan_grid_bound": (_I, [_I, _P, _I, _I, _I]),
     "mxmoe_plan_block": (_I, [_I, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P]),
+    "mxmoe_plan_layer": (_I, [_P, _P, _P, _I, _I, _P]),
     "mxmoe_group_gemm_planned": (_I, [_I, _P, _I, _P]),
     "mxmoe_quant_act_planned": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P]),
     "mxmoe_silu_mul_quant_planned": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P]),

@@ -40,6 +40,17 @@ typedef void (*mxmoe_func_t)(mxmoe_half** ptr_As, mxmoe_half** ptr_Bs, mxmoe_hal
                              int64_t* ldas, int64_t* ldbs, int64_t* ldcs, int64_t* ldds, mxmoe_dim3* device_problem_sizes, mxmoe_dim3* host_problem_sizes,
                              mxmoe_qparams* device_qbits_list, mxmoe_qparams* host_qbits_list, int problem_count);
 
+// One block (gate_up or down) of a layer for mxmoe_plan_layer: the arguments mxmoe_plan_block takes per block.
+typedef struct {
+  int kernel_id;                    // -1: chosen from the formats, as mxmoe_plan_select_kernel does
+  const mxmoe_block_desc* d_desc;   // device copy of the block descriptors [experts (+ 1 shared)]
+  const mxmoe_block_desc* h_desc;   // host copy of the same
+  const void* inp_store;            // packed activations the block reads
+  const void* scale_store;          // their scales (may be NULL for fp16 activations)
+  void* out_store;                  // where the block's output rows go
+  void* d_plan;                     // plan buffer of mxmoe_plan_bytes() bytes
+} mxmoe_plan_call;
+
 #ifdef __cplusplus
 }
 #endif

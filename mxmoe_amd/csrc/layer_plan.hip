@@ -61,7 +61,12 @@ __device__ __forceinline__ long wave_excl_scan(long v, int lane, long* total) {
 // One workgroup of two waves, thread e = expert e (the shared expert, if any, is expert E with `shared_rows` rows).  Everything the
 // host launcher computes (launch_range), with the same functions and in the same order, so the two produce identical tables;
 // prefix sums over experts are wave scans, and an entry finds its place from per-branch counts instead of a sequential walk.
-__global__ void __launch_bounds__(kPlanThreads) plan_block_kernel(const PlanParams p) {
+struct PlanPair {
+  PlanParams p[2];
+};
+
+__global__ void __launch_bounds__(kPlanThreads) plan_block_kernel(const PlanPair pair) {
+  const PlanParams& p = pair.p[blockIdx.x];  // one workgroup per block of the layer (gate_up, down): both only read the counts
   __shared__ long s_tot[4][2];                       // per wave: rows, packed input, scales, output elements
   __shared__ int s_cnt[kMaxBranches][2], s_til[kMaxBranches][2];  // per run-order rank and wave: entries, tiles
   __shared__ int s_cnt_long[kMaxBranches][2], s_til_long[kMaxBranches][2];  // ... of which belong to long-K problems
@@ -385,8 +390,8 @@ int mxmoe_plan_grid_bound(int kernel_id, const mxmoe_block_desc* h_desc, int num
   return (int)bound;
 }
 
-int mxmoe_plan_block(int kernel_id, const int64_t* d_recv, int num_experts, int shared_rows, const mxmoe_block_desc* d_desc, const mxmoe_block_desc* h_desc,
-                     const void* inp_store, const void* scale_store, void* out_store, void* d_plan, void* stream) {
+static int fill_plan_params(PlanParams& p, int kernel_id, const int64_t* d_recv, int num_experts, int shared_rows, const mxmoe_block_desc* d_desc,
+                            const mxmoe_block_desc* h_desc, const void* inp_store, const void* scale_store, void* out_store, void* d_plan) {
   const int et = num_experts + (shared_rows > 0 ? 1 : 0);
   if (!d_recv || !d_desc || !h_desc || !inp_store || !out_store || !d_plan) {
     last_error() = "null pointer";
@@ -394,7 +399,6 @@ int mxmoe_plan_block(int kernel_id, const int64_t* d_recv, int num_experts, int 
   }
   const int kid = mxmoe_plan_select_kernel(kernel_id, h_desc, et);
   if (kid < 0) return kid == -1 ? 1 : (kid == -2 ? 2 : 3);
-  PlanParams p;
   p.recv = d_recv;
   p.desc = d_desc;
   p.inp = reinterpret_cast<const uint8_t*>(inp_store);
@@ -405,13 +409,41 @@ int mxmoe_plan_block(int kernel_id, const int64_t* d_recv, int num_experts, int 
   p.Et = et;
   p.shared_rows = shared_rows;
   p.info = plan_of(registry()[kid]);
-  hipLaunchKernelGGL(plan_block_kernel, dim3(1), dim3(kPlanThreads), 0, (hipStream_t)stream, p);
+  return 0;
+}
+
+static int launch_plan(const PlanPair& pair, int blocks, void* stream) {
+  hipLaunchKernelGGL(plan_block_kernel, dim3(blocks), dim3(kPlanThreads), 0, (hipStream_t)stream, pair);
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     last_error() = std::string("kernel launch failed: ") + hipGetErrorString(e);
     return 4;
   }
   return 0;
+}
+
+int mxmoe_plan_block(int kernel_id, const int64_t* d_recv, int num_experts, int shared_rows, const mxmoe_block_desc* d_desc, const mxmoe_block_desc* h_desc,
+                     const void* inp_store, const void* scale_store, void* out_store, void* d_plan, void* stream) {
+  PlanPair pair;
+  const int rc = fill_plan_params(pair.p[0], kernel_id, d_recv, num_experts, shared_rows, d_desc, h_desc, inp_store, scale_store, out_store, d_plan);
+  if (rc) return rc;
+  pair.p[1] = pair.p[0];
+  return launch_plan(pair, 1, stream);
+}
+
+int mxmoe_plan_layer(const mxmoe_plan_call* gate_up, const mxmoe_plan_call* down, const int64_t* d_recv, int num_experts, int shared_rows, void* stream) {
+  if (!gate_up || !down) {
+    last_error() = "null pointer";
+    return 5;
+  }
+  PlanPair pair;
+  const mxmoe_plan_call* c[2] = {gate_up, down};
+  for (int i = 0; i < 2; ++i) {
+    const int rc = fill_plan_params(pair.p[i], c[i]->kernel_id, d_recv, num_experts, shared_rows, c[i]->d_desc, c[i]->h_desc, c[i]->inp_store, c[i]->scale_store,
+                                    c[i]->out_store, c[i]->d_plan);
+    if (rc) return rc;
+  }
+  return launch_plan(pair, 2, stream);
 }
 
 int mxmoe_group_gemm_planned(int kernel_id, const void* d_plan, int grid, void* stream) {

@@ -162,6 +162,9 @@ class MxMoELayer:
         b2 = block(self.qp_down, [cfg.hidden] * et, [cfg.inter] * e_cnt + [i_sh for _ in sh], self.w2)
         ps["b1"], ps["b2"] = b1, b2
         ps["mid"], ps["out"] = u8(b1["out_bytes"]), u8(b2["out_bytes"])
+        call = lambda b, out_store: _lib.PlanCall(b["kid"], b["d"].data_ptr(), C.cast(b["h"], C.c_void_p), b["inp"].data_ptr(), b["scale"].data_ptr(),  # noqa: E731
+                                                  out_store.data_ptr(), b["plan"].data_ptr())
+        ps["calls"] = (call(b1, ps["mid"]), call(b2, ps["out"]))
         ps["dst"] = torch.empty(r_cap, dtype=torch.int32, device=dev)
         ps["perm"] = torch.empty(r_cap, dtype=torch.int64, device=dev)
         ps["slot"] = torch.empty(r_cap, dtype=torch.int64, device=dev)
@@ -186,7 +189,7 @@ class MxMoELayer:
         framework's fused-MoE operator computes after routing (permute, quantise, gate_up, SiLU * up, down, un-permute + combine).
 
         Same kernels and results as `forward` + `combine`, but nothing here waits for the routing: the tables of both launches are
-        derived from the tokens-per-expert counts by a planning kernel on the device (`mxmoe_plan_block`), the stores and plan
+        derived from the tokens-per-expert counts by a planning kernel on the device (`mxmoe_plan_layer`: both blocks in one launch), the stores and plan
         buffers are allocated once per (tokens, top-k) for the worst case, and every launch argument is independent of the data.
         The call only enqueues nine kernels (no synchronisation, no allocation after the first call when `out` is given), so it can
         be captured into a HIP graph.  Intermediate buffers belong to the layer and are reused by the next call of the same shape."""
@@ -207,10 +210,7 @@ class MxMoELayer:
         ck = lambda rc: _lib.check(lib, rc)  # noqa: E731
         ck(lib.mxmoe_build_permutation(ids.data_ptr(), t, topk, e_cnt, ps["dst"].data_ptr(), ps["perm"].data_ptr(), ps["slot"].data_ptr(), ps["recv"].data_ptr(),
                                        ps["perm_ws"].data_ptr(), stream))
-        ck(lib.mxmoe_plan_block(b1["kid"], ps["recv"].data_ptr(), e_cnt, ps["shared_rows"], b1["d"].data_ptr(), b1["h"], b1["inp"].data_ptr(), b1["scale"].data_ptr(),
-                                ps["mid"].data_ptr(), b1["plan"].data_ptr(), stream))
-        ck(lib.mxmoe_plan_block(b2["kid"], ps["recv"].data_ptr(), e_cnt, ps["shared_rows"], b2["d"].data_ptr(), b2["h"], b2["inp"].data_ptr(), b2["scale"].data_ptr(),
-                                ps["out"].data_ptr(), b2["plan"].data_ptr(), stream))
+        ck(lib.mxmoe_plan_layer(C.byref(ps["calls"][0]), C.byref(ps["calls"][1]), ps["recv"].data_ptr(), e_cnt, ps["shared_rows"], stream))
         hk, hf, _sg, sgp = ps["had1"]
         ck(lib.mxmoe_quant_act_planned(hidden.data_ptr(), b1["inp"].data_ptr(), b1["scale"].data_ptr(), ps["dst"].data_ptr(), ps["perm"].data_ptr(), b1["plan"].data_ptr(),
                                        cfg.hidden, ps["r_cap"], t, e_cnt, has_shared, cfg.rotate, hk, hf, sgp, stream))
