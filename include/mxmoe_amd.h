@@ -107,6 +107,12 @@ size_t mxmoe_permute_workspace_bytes(int total_rows, int num_experts);
 int mxmoe_build_permutation(const int32_t* topk_ids, int num_tokens, int topk, int num_experts, int32_t* dst_exp_sorted, int64_t* perm_indices,
                             int64_t* src_slot, int64_t* recv_tokens_per_exp, void* workspace, void* stream);
 
+/* The same, and also the inverse map: row_of_slot[t * topk + k] = sorted row of token t's k-th expert, -1 where that expert id was out of
+ * range (int32 [num_tokens * topk]).  With it the combine needs no preparation pass (mxmoe_combine_planned).  No counterpart in the
+ * reference, whose un-permute op is an empty stub (ref_bind.cu:66). */
+int mxmoe_build_permutation_inv(const int32_t* topk_ids, int num_tokens, int topk, int num_experts, int32_t* dst_exp_sorted, int64_t* perm_indices,
+                                int64_t* src_slot, int64_t* recv_tokens_per_exp, int32_t* row_of_slot, void* workspace, void* stream);
+
 /* The same permutation for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc).  No counterpart in the reference.  The per-block histograms that the `workspace` argument
  * above brings in live in a static device array of mxmoe_static_scratch_bytes() bytes (1 MiB per GPU, held until the process
@@ -199,6 +205,11 @@ int mxmoe_silu_mul_quant_planned(const void* gate_up, const void* d_plan_gate_up
                                  const float* had_signs, void* stream);
 int mxmoe_unpermute_combine_planned(const void* down_out, const void* d_plan_down, int num_problems, const float* topk_weights, const int64_t* src_slot, int num_tokens,
                                     int topk, int K, void* out, void* workspace, void* stream);
+
+/* The combine of the planned forward when the permutation already delivered the inverse map (mxmoe_build_permutation_inv): one
+ * launch, no workspace. */
+int mxmoe_combine_planned(const void* down_out, const void* d_plan_down, int num_problems, const float* topk_weights, const int32_t* row_of_slot, int num_tokens,
+                          int topk, int K, void* out, void* stream);
 
 /* ---- diagnostic (no counterpart in the reference): the rate the int8 matrix pipes sustain on their own ----
  * One launch of a bare loop of v_mfma_i32_32x32x32_i8 (8 independent accumulators per wave, two waves per SIMD, no memory traffic in

@@ -82,7 +82,7 @@ __global__ void __launch_bounds__(64) perm_scan_kernel(int32_t* __restrict__ his
 
 __global__ void __launch_bounds__(64) perm_scatter_kernel(const int32_t* __restrict__ ids, int total, int E, int topk, int nbits, const int32_t* __restrict__ hist,
                                                           const int64_t* __restrict__ recv, int32_t* __restrict__ dst_exp_sorted, int64_t* __restrict__ perm,
-                                                          int64_t* __restrict__ src_slot) {
+                                                          int64_t* __restrict__ src_slot, int32_t* __restrict__ row_of_slot) {
   extern __shared__ int32_t run[];  // next free rank per expert for this block
   {  // first row of every expert = exclusive scan of the per-expert totals, plus this block's offset inside the expert
     int carry = 0;
@@ -114,6 +114,56 @@ __global__ void __launch_bounds__(64) perm_scatter_kernel(const int32_t* __restr
       if (src_slot) src_slot[pos] = idx;
       if (before == 0) run[e] = first + __popcll(same);
     }
+    // the inverse map (sorted row of every (token, slot); -1 where the expert id was out of range), for the combine
+    if (row_of_slot && ok) row_of_slot[idx] = e < E ? first + before : -1;
+    __syncthreads();
+  }
+}
+
+// The three kernels above in one, for at most kPermChunk (token, slot) entries (decode-sized batches): one single-wave workgroup
+// counts, scans the experts and scatters, where three launches would cost more than their work.
+__global__ void __launch_bounds__(64) perm_small_kernel(const int32_t* __restrict__ ids, int total, int E, int topk, int nbits, int64_t* __restrict__ recv,
+                                                        int32_t* __restrict__ dst_exp_sorted, int64_t* __restrict__ perm, int64_t* __restrict__ src_slot,
+                                                        int32_t* __restrict__ row_of_slot) {
+  extern __shared__ int32_t run[];  // [E] counts, then next free rank per expert
+  const int lane = threadIdx.x;
+  for (int e = lane; e < E; e += 64) run[e] = 0;
+  __syncthreads();
+  for (int idx = lane; idx < total; idx += 64) {
+    const int e = ids[idx];
+    if (e >= 0 && e < E) atomicAdd(&run[e], 1);
+  }
+  __syncthreads();
+  int carry = 0;
+  for (int e0 = 0; e0 < E; e0 += 64) {
+    const int e = e0 + lane;
+    const int v = e < E ? run[e] : 0;
+    const int inc = wave_inclusive_scan(v, lane);
+    if (e < E) {
+      recv[e] = v;
+      run[e] = carry + inc - v;
+    }
+    carry += __shfl(inc, 63);
+  }
+  __syncthreads();
+  for (int i = 0; i < total; i += 64) {  // sub-chunks in order keep the sort stable
+    const int idx = i + lane;
+    const bool ok = idx < total;
+    int e = ok ? ids[idx] : -1;
+    if (e < 0 || e >= E) e = E;
+    const uint64_t same = match_same(e, nbits);
+    const int before = __popcll(same & ((1ull << lane) - 1));
+    int first = 0;
+    if (e < E) first = run[e];
+    __syncthreads();
+    if (e < E) {
+      const int pos = first + before;
+      dst_exp_sorted[pos] = e;
+      perm[pos] = idx / topk;
+      if (src_slot) src_slot[pos] = idx;
+      if (before == 0) run[e] = first + __popcll(same);
+    }
+    if (row_of_slot && ok) row_of_slot[idx] = e < E ? first + before : -1;
     __syncthreads();
   }
 }
@@ -1481,16 +1531,21 @@ size_t mxmoe_permute_workspace_bytes(int total, int num_experts) {
 }
 
 static int build_permutation_impl(const int32_t* topk_ids, int num_tokens, int topk, int num_experts, int32_t* dst_exp_sorted, int64_t* perm_indices,
-                                  int64_t* src_slot, int64_t* recv_tokens_per_exp, int32_t* hist, hipStream_t s) {
+                                  int64_t* src_slot, int64_t* recv_tokens_per_exp, int32_t* hist, hipStream_t s, int32_t* row_of_slot = nullptr) {
   const int total = num_tokens * topk;
   const int blocks = (total + kPermChunk - 1) / kPermChunk;
   int nbits = 1;
   while ((1 << nbits) <= num_experts) ++nbits;  // ids 0..E (E = parked lanes)
   const size_t lds = (size_t)num_experts * sizeof(int32_t);
-  hipLaunchKernelGGL(perm_hist_kernel, dim3(blocks), dim3(64), lds, s, topk_ids, total, num_experts, hist);
-  hipLaunchKernelGGL(perm_scan_kernel, dim3(num_experts), dim3(64), 0, s, hist, blocks, num_experts, recv_tokens_per_exp);
-  hipLaunchKernelGGL(perm_scatter_kernel, dim3(blocks), dim3(64), lds, s, topk_ids, total, num_experts, topk, nbits, hist, recv_tokens_per_exp, dst_exp_sorted, perm_indices,
-                     src_slot);
+  if (blocks == 1) {
+    hipLaunchKernelGGL(perm_small_kernel, dim3(1), dim3(64), lds, s, topk_ids, total, num_experts, topk, nbits, recv_tokens_per_exp, dst_exp_sorted, perm_indices, src_slot,
+                       row_of_slot);
+  } else {
+    hipLaunchKernelGGL(perm_hist_kernel, dim3(blocks), dim3(64), lds, s, topk_ids, total, num_experts, hist);
+    hipLaunchKernelGGL(perm_scan_kernel, dim3(num_experts), dim3(64), 0, s, hist, blocks, num_experts, recv_tokens_per_exp);
+    hipLaunchKernelGGL(perm_scatter_kernel, dim3(blocks), dim3(64), lds, s, topk_ids, total, num_experts, topk, nbits, hist, recv_tokens_per_exp, dst_exp_sorted,
+                       perm_indices, src_slot, row_of_slot);
+  }
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     last_error() = std::string("kernel launch failed: ") + hipGetErrorString(e);
@@ -1521,6 +1576,17 @@ int mxmoe_build_permutation(const int32_t* topk_ids, int num_tokens, int topk, i
   }
   return build_permutation_impl(topk_ids, num_tokens, topk, num_experts, dst_exp_sorted, perm_indices, src_slot, recv_tokens_per_exp,
                                 reinterpret_cast<int32_t*>(workspace), (hipStream_t)stream);
+}
+
+int mxmoe_build_permutation_inv(const int32_t* topk_ids, int num_tokens, int topk, int num_experts, int32_t* dst_exp_sorted, int64_t* perm_indices,
+                                int64_t* src_slot, int64_t* recv_tokens_per_exp, int32_t* row_of_slot, void* workspace, void* stream) {
+  if (const int rc = check_permutation_args(topk_ids, num_tokens, topk, num_experts, dst_exp_sorted, perm_indices, src_slot, recv_tokens_per_exp)) return rc;
+  if (!workspace || !row_of_slot) {
+    last_error() = "null pointer";
+    return 5;
+  }
+  return build_permutation_impl(topk_ids, num_tokens, topk, num_experts, dst_exp_sorted, perm_indices, src_slot, recv_tokens_per_exp,
+                                reinterpret_cast<int32_t*>(workspace), (hipStream_t)stream, row_of_slot);
 }
 
 // ---- the permutation for callers that may not allocate: the per-block histograms live in a static device array ----
@@ -1729,6 +1795,27 @@ int mxmoe_unpermute_combine(const void* down_out, const void* shared_out, const 
   if (rows > 0) hipLaunchKernelGGL(combine_invert_kernel, dim3((rows + 255) / 256), dim3(256), 0, s, src_slot, rows, slots, row_of_slot, (const int64_t*)nullptr);
   hipLaunchKernelGGL(combine_kernel, dim3(num_tokens), dim3(256), 0, s, reinterpret_cast<const _Float16*>(down_out), reinterpret_cast<const _Float16*>(shared_out),
                      topk_weights, row_of_slot, topk, K, reinterpret_cast<_Float16*>(out), (const int64_t*)nullptr);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    last_error() = std::string("kernel launch failed: ") + hipGetErrorString(e);
+    return 4;
+  }
+  return 0;
+}
+
+int mxmoe_combine_planned(const void* down_out, const void* d_plan_down, int num_problems, const float* topk_weights, const int32_t* row_of_slot, int num_tokens,
+                          int topk, int K, void* out, void* stream) {
+  if (num_tokens <= 0 || topk <= 0 || K <= 0 || K % 8 || num_problems <= 0) {
+    last_error() = "bad combine size (K must be a multiple of 8)";
+    return 3;
+  }
+  if (!down_out || !d_plan_down || !topk_weights || !row_of_slot || !out) {
+    last_error() = "null pointer";
+    return 5;
+  }
+  const int64_t* misc = reinterpret_cast<const int64_t*>(reinterpret_cast<const uint8_t*>(d_plan_down) + mxmoe::PlanLayout(num_problems).misc);
+  hipLaunchKernelGGL(combine_kernel, dim3(num_tokens), dim3(256), 0, (hipStream_t)stream, reinterpret_cast<const _Float16*>(down_out), (const _Float16*)nullptr, topk_weights,
+                     row_of_slot, topk, K, reinterpret_cast<_Float16*>(out), misc + 1);
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     last_error() = std::string("kernel launch failed: ") + hipGetErrorString(e);

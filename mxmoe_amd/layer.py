@@ -168,6 +168,7 @@ class MxMoELayer:
         ps["dst"] = torch.empty(r_cap, dtype=torch.int32, device=dev)
         ps["perm"] = torch.empty(r_cap, dtype=torch.int64, device=dev)
         ps["slot"] = torch.empty(r_cap, dtype=torch.int64, device=dev)
+        ps["row_of_slot"] = torch.empty(r_cap, dtype=torch.int32, device=dev)
         ps["recv"] = torch.empty(e_cnt, dtype=torch.int64, device=dev)
         ps["perm_ws"] = u8(lib.mxmoe_permute_workspace_bytes(r_cap, e_cnt))
         ps["comb_ws"] = u8(lib.mxmoe_combine_workspace_bytes(t, topk))
@@ -191,7 +192,7 @@ class MxMoELayer:
         Same kernels and results as `forward` + `combine`, but nothing here waits for the routing: the tables of both launches are
         derived from the tokens-per-expert counts by a planning kernel on the device (`mxmoe_plan_layer`: both blocks in one launch), the stores and plan
         buffers are allocated once per (tokens, top-k) for the worst case, and every launch argument is independent of the data.
-        The call only enqueues nine kernels (no synchronisation, no allocation after the first call when `out` is given), so it can
+        The call only enqueues seven kernels (nine when more than 256 (token, slot) pairs are permuted; no synchronisation, no allocation after the first call when `out` is given), so it can
         be captured into a HIP graph.  Intermediate buffers belong to the layer and are reused by the next call of the same shape."""
         cfg, dev = self.cfg, self.device
         lib = _lib.load()
@@ -208,8 +209,8 @@ class MxMoELayer:
         final = out if out is not None else torch.empty((t, cfg.hidden), dtype=torch.float16, device=dev)
         assert final.shape == (t, cfg.hidden) and final.dtype == torch.float16 and final.is_contiguous()
         ck = lambda rc: _lib.check(lib, rc)  # noqa: E731
-        ck(lib.mxmoe_build_permutation(ids.data_ptr(), t, topk, e_cnt, ps["dst"].data_ptr(), ps["perm"].data_ptr(), ps["slot"].data_ptr(), ps["recv"].data_ptr(),
-                                       ps["perm_ws"].data_ptr(), stream))
+        ck(lib.mxmoe_build_permutation_inv(ids.data_ptr(), t, topk, e_cnt, ps["dst"].data_ptr(), ps["perm"].data_ptr(), ps["slot"].data_ptr(), ps["recv"].data_ptr(),
+                                           ps["row_of_slot"].data_ptr(), ps["perm_ws"].data_ptr(), stream))
         ck(lib.mxmoe_plan_layer(C.byref(ps["calls"][0]), C.byref(ps["calls"][1]), ps["recv"].data_ptr(), e_cnt, ps["shared_rows"], stream))
         hk, hf, _sg, sgp = ps["had1"]
         ck(lib.mxmoe_quant_act_planned(hidden.data_ptr(), b1["inp"].data_ptr(), b1["scale"].data_ptr(), ps["dst"].data_ptr(), ps["perm"].data_ptr(), b1["plan"].data_ptr(),
@@ -220,8 +221,8 @@ class MxMoELayer:
         ck(lib.mxmoe_silu_mul_quant_planned(ps["mid"].data_ptr(), b1["plan"].data_ptr(), b2["inp"].data_ptr(), b2["scale"].data_ptr(), ps["dst"].data_ptr(), b2["plan"].data_ptr(),
                                             cfg.inter, i_sh, ps["r_cap"], t, e_cnt, has_shared, cfg.rotate, hk, hf, sgp, stream))
         ck(lib.mxmoe_group_gemm_planned(b2["kid"], b2["plan"].data_ptr(), b2["grid"], stream))
-        ck(lib.mxmoe_unpermute_combine_planned(ps["out"].data_ptr(), b2["plan"].data_ptr(), ps["et"], w.data_ptr(), ps["slot"].data_ptr(), t, topk, cfg.hidden,
-                                               final.data_ptr(), ps["comb_ws"].data_ptr(), stream))
+        ck(lib.mxmoe_combine_planned(ps["out"].data_ptr(), b2["plan"].data_ptr(), ps["et"], w.data_ptr(), ps["row_of_slot"].data_ptr(), t, topk, cfg.hidden,
+                                     final.data_ptr(), stream))
         return final
 
     def call_with_host_tables(self, hidden: torch.Tensor, topk_ids: torch.Tensor, topk_weights: torch.Tensor) -> torch.Tensor:

@@ -355,6 +355,29 @@ def test_planned_forward_drops_out_of_range_experts_like_the_operators():
     assert torch.equal(got, want) and bool(torch.isfinite(got).all())
 
 
+def test_combine_entry_points_of_the_planned_forward_agree():
+    """mxmoe_combine_planned (inverse map from the permutation) against mxmoe_unpermute_combine_planned (inverse map built from
+    src_slot by two preparation launches) on the same plan and down output, with dropped ids."""
+    from mxmoe_amd import _lib
+
+    cfg, layer = _small_layer(num_shared=1)
+    from mxmoe_amd import synth
+
+    hidden = synth.make_hidden(cfg)
+    ids, w = synth.make_routing(cfg)
+    ids = torch.where(ids == 2, torch.full_like(ids, cfg.num_experts + 3), ids)
+    wd = w.to("cuda").contiguous()
+    want = layer(hidden, ids, wd).clone()
+    lib = _lib.load()
+    ps = layer._planned_setup(cfg.tokens, cfg.topk)
+    out = torch.zeros_like(want)
+    stream = torch.cuda.current_stream().cuda_stream
+    _lib.check(lib, lib.mxmoe_unpermute_combine_planned(ps["out"].data_ptr(), ps["b2"]["plan"].data_ptr(), ps["et"], wd.data_ptr(), ps["slot"].data_ptr(), cfg.tokens,
+                                                        cfg.topk, cfg.hidden, out.data_ptr(), ps["comb_ws"].data_ptr(), stream))
+    torch.cuda.synchronize()
+    assert torch.equal(out, want)
+
+
 def test_planned_forward_replays_from_a_graph():
     """The whole forward inside a HIP graph (nothing in it synchronises, allocates or depends on the routing): each replay, with new
     routing and new hidden states written into the captured input buffers and eager work in between, equals the eager forward."""

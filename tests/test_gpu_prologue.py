@@ -32,6 +32,47 @@ def test_permutation_matches_oracle_and_is_stable():
         assert np.array_equal(recv.cpu().numpy(), o_recv)
 
 
+def test_permutation_with_inverse_map_small_and_large_and_dropped_ids():
+    """mxmoe_build_permutation_inv: the reference's four outputs plus row_of_slot, the inverse map the combine reads; sizes on both
+    sides of the single-launch path (at most 256 entries), ids out of range dropped (-1 in the inverse map)."""
+    from mxmoe_amd import _lib
+
+    lib = _lib.load()
+    rng = np.random.default_rng(3)
+    stream = torch.cuda.current_stream().cuda_stream
+    for (t, e, k) in [(1, 4, 2), (32, 64, 6), (42, 7, 6), (43, 7, 6), (64, 4, 4), (65, 4, 4), (700, 60, 4)]:
+        ids = _ids(rng, t, e, k)
+        ids[rng.random(ids.shape) < 0.15] = e + 2                            # dropped entries
+        if t > 3:
+            ids[1, 0] = -1
+        total = t * k
+        d_ids = torch.from_numpy(ids).to(DEV)
+        dst = torch.full((total,), -7, dtype=torch.int32, device=DEV)
+        perm = torch.full((total,), -7, dtype=torch.int64, device=DEV)
+        slot = torch.full((total,), -7, dtype=torch.int64, device=DEV)
+        recv = torch.empty(e, dtype=torch.int64, device=DEV)
+        inv = torch.full((total,), -7, dtype=torch.int32, device=DEV)
+        ws = torch.empty(max(lib.mxmoe_permute_workspace_bytes(total, e), 16), dtype=torch.uint8, device=DEV)
+        for _ in range(2):                                                   # a second call over the same buffers gives the same result
+            _lib.check(lib, lib.mxmoe_build_permutation_inv(d_ids.data_ptr(), t, k, e, dst.data_ptr(), perm.data_ptr(), slot.data_ptr(), recv.data_ptr(),
+                                                            inv.data_ptr(), ws.data_ptr(), stream))
+        torch.cuda.synchronize()
+        flat = ids.reshape(-1).astype(np.int64)
+        keep = np.nonzero((flat >= 0) & (flat < e))[0]                      # the oracle's stable sort, over the entries that are routed
+        order = keep[np.argsort(flat[keep], kind="stable")]
+        o_dst, o_perm, o_slot, o_recv = flat[order].astype(np.int32), order // k, order, np.bincount(flat[keep], minlength=e)
+        if len(keep) == total:
+            for a, b in zip((o_dst, o_perm, o_slot, o_recv), O.permute_by_expert(ids, e)):
+                assert np.array_equal(a, b)
+        r = len(o_dst)
+        assert int(recv.sum()) == r
+        assert np.array_equal(dst.cpu().numpy()[:r], o_dst) and np.array_equal(perm.cpu().numpy()[:r], o_perm)
+        assert np.array_equal(slot.cpu().numpy()[:r], o_slot) and np.array_equal(recv.cpu().numpy(), o_recv)
+        want = np.full(total, -1, np.int32)
+        want[o_slot] = np.arange(r, dtype=np.int32)
+        assert np.array_equal(inv.cpu().numpy(), want)
+
+
 def _unpack(store_view, tag, n):
     raw = store_view.contiguous().view(torch.uint8).cpu().numpy().reshape(store_view.shape[0], -1)
     if tag == 1:
