@@ -218,19 +218,19 @@ __global__ void __launch_bounds__(kPlanThreads) plan_block_kernel(const PlanPair
     misc[0] = s_tot[0][0] + s_tot[0][1] - (p.Et > p.E ? (long)p.shared_rows : 0);
     if (p.Et == p.E) misc[1] = 0;
     int total = 0, wg = 0, np = 0, ne = 0, flat = 0;
+    int last_tile0 = 0, last_wg0 = 0;  // of the phase being filled (kept here: reading them back from the table would wait for the store)
     for (int r = 0; r < p.info.nb; ++r) {
       const int tile0 = total;
       total += s_til[r][0] + s_til[r][1];
       ne += s_cnt[r][0] + s_cnt[r][1];
       if (total == tile0) continue;
       if (np < kMaxPhases) {  // shapes beyond the phase table share the last phase
-        fa->phase_tile0[np] = tile0;
-        fa->phase_wg0[np] = wg;
+        fa->phase_tile0[np] = last_tile0 = tile0;
+        fa->phase_wg0[np] = last_wg0 = wg;
         if (p.info.b[p.info.order[r]].BM <= 16) flat |= 1 << np;
         ++np;
       }
-      const int p0 = fa->phase_tile0[np - 1];
-      wg = fa->phase_wg0[np - 1] + (total - p0 + kNumXcd - 1) / kNumXcd * kNumXcd;
+      wg = last_wg0 + (total - last_tile0 + kNumXcd - 1) / kNumXcd * kNumXcd;
     }
     fa->phase_tile0[np] = total;
     fa->phase_wg0[np] = wg;
