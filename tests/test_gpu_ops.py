@@ -201,3 +201,21 @@ def test_function_type_call_with_exactly_fifteen_arguments():
             assert np.array_equal(c.cpu().numpy().view(np.uint16), p["out"].view(np.uint16)), f"{name}: {p['size']} {p['q']}"
         ran += 1
     assert ran >= 4                                                         # wxax, all, seq_launch_all, ms_launch_all
+
+
+def test_bench_diagnostics_run():
+    """bench.py's two diagnostic modes (matrix-pipe probe, one problem on three kinds of operand codes) at toy sizes: they must keep
+    running against the library they ship with, and their figures must be sane (a clock between 0.5 and 3 GHz, rates below the peak)."""
+    import importlib.util
+    from pathlib import Path
+
+    spec = importlib.util.spec_from_file_location("bench_under_test", Path(__file__).resolve().parent.parent / "bench.py")
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    probe = bench.mfma_probe(iters=2000, workgroups=512, repeats=1)
+    assert len(probe["modes"]) == 6
+    for m in probe["modes"].values():
+        assert 0.0 < m["tops"] <= 1.05 * bench.PEAK["int8"] and 0.5 < m["shader_clock_ghz"] < 3.0
+    one = bench.one_problem("w4a4:2048x512x1024")
+    assert set(one["operands"]) == {"random codes", "constant codes", "zero codes"}
+    assert all(0.0 < o["tops"] < bench.PEAK["int8"] for o in one["operands"].values())
