@@ -355,6 +355,39 @@ def test_planned_forward_drops_out_of_range_experts_like_the_operators():
     assert torch.equal(got, want) and bool(torch.isfinite(got).all())
 
 
+def test_single_block_planning_writes_what_the_paired_launch_writes():
+    """mxmoe_plan_block (one block per launch) against mxmoe_plan_layer (both blocks of the layer in one launch): identical plan
+    buffers for the same counts."""
+    from mxmoe_amd import _lib, synth
+
+    cfg, layer = _small_layer(num_shared=1)
+    hidden = synth.make_hidden(cfg)
+    ids, w = synth.make_routing(cfg)
+    layer(hidden, ids, w)
+    torch.cuda.synchronize()
+    lib = _lib.load()
+    ps = layer._planned_setup(cfg.tokens, cfg.topk)
+    stream = torch.cuda.current_stream().cuda_stream
+    for key, out_store in (("b1", ps["mid"]), ("b2", ps["out"])):
+        b = ps[key]
+        fresh = torch.zeros_like(b["plan"])
+        _lib.check(lib, lib.mxmoe_plan_block(b["kid"], ps["recv"].data_ptr(), cfg.num_experts, ps["shared_rows"], b["d"].data_ptr(), b["h"], b["inp"].data_ptr(),
+                                             b["scale"].data_ptr(), out_store.data_ptr(), fresh.data_ptr(), stream))
+        torch.cuda.synchronize()
+        got, want = fresh.cpu().numpy().copy(), b["plan"].cpu().numpy().copy()
+        # the header holds pointers into its own plan buffer (As .. sizes): compare them relative to the buffer's address
+        g64, w64 = got[:56].view(np.int64).copy(), want[:56].view(np.int64).copy()
+        assert g64[5] == 0 and w64[5] == 0                                  # no accumulator dumps
+        g64[5], w64[5] = fresh.data_ptr(), b["plan"].data_ptr()
+        assert np.array_equal(g64 - fresh.data_ptr(), w64 - b["plan"].data_ptr())
+        gi, wi = got[56:].view(np.int32), want[56:].view(np.int32)          # offset, entries, tiles, phases; phase_tile0[9]; phase_wg0[9]; flat; entries
+        ne, nph = int(wi[1]), int(wi[3])
+        assert np.array_equal(gi[:4], wi[:4]) and np.array_equal(gi[4:5 + nph], wi[4:5 + nph]) and np.array_equal(gi[13:14 + nph], wi[13:14 + nph])
+        assert gi[22] == wi[22] and np.array_equal(gi[23:23 + 4 * ne], wi[23:23 + 4 * ne])
+        first, last = lib.mxmoe_plan_offset(1, ps["et"]), lib.mxmoe_plan_offset(4, ps["et"]) + 12 * ps["et"]
+        assert np.array_equal(got[first:last], want[first:last])             # table, pointer arrays, row counts, sizes (what follows is padding)
+
+
 def test_combine_entry_points_of_the_planned_forward_agree():
     """mxmoe_combine_planned (inverse map from the permutation) against mxmoe_unpermute_combine_planned (inverse map built from
     src_slot by two preparation launches) on the same plan and down output, with dropped ids."""
