@@ -250,11 +250,14 @@ struct SkinnyWoTile {
 template <int WBITS_, int BM_ = 128, int BN_ = 128>
 struct WoMfmaTile {
   static constexpr int WBITS = WBITS_, BM = BM_, BN = BN_;
-  static_assert(BM == 128 && BN == 128, "2 x 2 waves of 64 tokens x 64 channels");
+  static_assert(BM == 128 && (BN == 128 || BN == 256), "2 x 2 waves of 64 tokens x 64 channels, or 4 waves of 128 x 64 side by side");
+  static constexpr int WM = BN == 128 ? 2 : 1;  // waves along the tokens
+  static constexpr int TM = BM / WM;            // tokens per wave
+  static constexpr int MB = TM / 16;            // token blocks per wave
   using Sk = SkinnyWoTile<WBITS, 128>;
   static constexpr int kStageBytes = BM * 256;
   static constexpr int kLdsBytes = 2 * kStageBytes;
-  static constexpr int kAccRegs = 64;
+  static constexpr int kAccRegs = 16 * MB;
   static constexpr int kABits = 16, kWBits = WBITS;  // fp16 activations, packed weights
   static constexpr int kLaneBytes = Sk::kLaneBytes, kBlockBytes = Sk::kBlockBytes;
   static constexpr int kDma = kStageBytes / 1024 / kWaves;  // direct-to-LDS loads per wave per stage
@@ -263,7 +266,7 @@ struct WoMfmaTile {
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = WM == 2 ? wave >> 1 : 0, wn = WM == 2 ? wave & 1 : wave;
     const int M = t.M, N = t.N, K = t.K;
     const int m0 = t.row0 + t.tile_m * BM, n0 = t.tile_n * BN;
     const int KB = K / 128;
@@ -290,8 +293,8 @@ struct WoMfmaTile {
 #pragma unroll
       for (int i = 0; i < kDma; ++i) dma16_to_lds(rs_x, __builtin_amdgcn_readfirstlane(lds_base + stage * kStageBytes + dma_lds[i]), dma_voff[i], koff);
     };
-    // fragment reads: token row wm*64 + mb*16 + lm, chunk lg*4 + j
-    const int xrow = wm * 64 + lm;
+    // fragment reads: token row wm*TM + mb*16 + lm, chunk lg*4 + j
+    const int xrow = wm * TM + lm;
     auto lds_x = [&](int stage, int mb, int j) {
       const int row = xrow + mb * 16;
       return *reinterpret_cast<const v4i*>(smem + stage * kStageBytes + row * 256 + (((lg * 4 + j) ^ (row & 15)) << 4));
@@ -306,11 +309,11 @@ struct WoMfmaTile {
     typename Sk::WReg wr[8];
     int sr[8];
 
-    v4f acc[4][4];  // [channel block][token block]
+    v4f acc[4][MB];  // [channel block][token block]
 #pragma unroll
     for (int nb = 0; nb < 4; ++nb)
 #pragma unroll
-      for (int mb = 0; mb < 4; ++mb) acc[nb][mb] = v4f{0.f, 0.f, 0.f, 0.f};
+      for (int mb = 0; mb < MB; ++mb) acc[nb][mb] = v4f{0.f, 0.f, 0.f, 0.f};
 
     {
       // prologue: exactly 8 ring loads are younger than the loads of the first activation stage, as in every later iteration
@@ -336,27 +339,32 @@ struct WoMfmaTile {
         vm_wait<8>();
         __syncthreads();  // ... for every wave; and every wave holds the previous stage's fragments in registers by now
         if (kb + 1 < KB) dma_x(kb + 1, st ^ 1);
-        v8h xf[4][4];
+        constexpr int base = st * 4;
+        // k sub-block by k sub-block: its token fragments, then every channel block's 8 weights per lane against all of them
 #pragma unroll
-        for (int mb = 0; mb < 4; ++mb)
+        for (int j = 0; j < 4; ++j) {
+          v8h xf[MB];
 #pragma unroll
-          for (int j = 0; j < 4; ++j) xf[mb][j] = __builtin_bit_cast(v8h, lds_x(st, mb, j));
+          for (int mb = 0; mb < MB; ++mb) xf[mb] = __builtin_bit_cast(v8h, lds_x(st, mb, j));
+#pragma unroll
+          for (int nb = 0; nb < 4; ++nb) {
+            v8h wf[4];
+            Sk::unpack(wr[base + nb], wf);  // only wf[j] is used: the rest folds away
+            const v2h sz = __builtin_bit_cast(v2h, sr[base + nb]);
+            const v8h s8 = {sz[0], sz[0], sz[0], sz[0], sz[0], sz[0], sz[0], sz[0]};
+            const v8h z8 = {sz[1], sz[1], sz[1], sz[1], sz[1], sz[1], sz[1], sz[1]};
+            const v8h w8 = __builtin_elementwise_fma(wf[j] - bias, s8, z8);  // exact q, then fma(q, scale, zero) in fp16
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) acc[nb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w8, xf[mb], acc[nb][mb], 0, 0, 0);
+          }
+          // keeps the scheduler from starting the next sub-block's unpacking and fragment reads early: that costs no time (the
+          // other wave of the SIMD fills the gap) and without it the 3-bit tile runs out of registers
+          __builtin_amdgcn_sched_barrier(0);
+        }
 #pragma unroll
         for (int nb = 0; nb < 4; ++nb) {
-          constexpr int base = st * 4;
-          v8h wf[4];
-          Sk::unpack(wr[base + nb], wf);
-          const v2h sz = __builtin_bit_cast(v2h, sr[base + nb]);
           wr[base + nb] = w_of(nb, kb + 2);
           sr[base + nb] = s_of(nb, kb + 2);
-          const v8h s8 = {sz[0], sz[0], sz[0], sz[0], sz[0], sz[0], sz[0], sz[0]};
-          const v8h z8 = {sz[1], sz[1], sz[1], sz[1], sz[1], sz[1], sz[1], sz[1]};
-#pragma unroll
-          for (int j = 0; j < 4; ++j) wf[j] = __builtin_elementwise_fma(wf[j] - bias, s8, z8);  // exact q, then fma(q, scale, zero) in fp16
-#pragma unroll
-          for (int mb = 0; mb < 4; ++mb)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) acc[nb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf[j], xf[mb][j], acc[nb][mb], 0, 0, 0);
         }
       };
 #pragma unroll 1
@@ -368,35 +376,37 @@ struct WoMfmaTile {
     vm_wait<0>();
     __syncthreads();  // LDS is reused for the output patch
 
-    // epilogue: [token][channel] fp16 patch per wave (64 x 64, row pitch 136 B), then 16-byte row-contiguous stores
+    // epilogue, 64 tokens at a time: [token][channel] fp16 patch per wave (64 x 64, row pitch 136 B), then 16-byte
+    // row-contiguous stores
     constexpr int kPitch = 64 * 2 + 8;
     uint8_t* patch = smem + wave * (64 * kPitch);
+    const int pr = lane >> 3, pc = lane & 7;  // 8 lanes x 16 B per 64-channel row, 8 rows per pass
 #pragma unroll
-    for (int nb = 0; nb < 4; ++nb)
+    for (int h = 0; h < TM / 64; ++h) {
 #pragma unroll
-      for (int mb = 0; mb < 4; ++mb) {
-        v4h o;
+      for (int nb = 0; nb < 4; ++nb)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) o[e] = (_Float16)acc[nb][mb][e];
-        *reinterpret_cast<v4h*>(patch + (mb * 16 + lm) * kPitch + (nb * 16 + lg * 4) * 2) = o;
-        if (t.acc_dump) {
-          const int m = m0 + wm * 64 + mb * 16 + lm, n = n0 + wn * 64 + nb * 16 + lg * 4;
-          if (m < M && n < N) {
+        for (int mb = 0; mb < 4; ++mb) {
+          const v4f a = acc[nb][h * 4 + mb];
+          v4h o;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const float f = acc[nb][mb][e];
-              gstore<int>(t.acc_dump + (long)m * N + n + e, __float_as_int(f));
+          for (int e = 0; e < 4; ++e) o[e] = (_Float16)a[e];
+          *reinterpret_cast<v4h*>(patch + (mb * 16 + lm) * kPitch + (nb * 16 + lg * 4) * 2) = o;
+          if (t.acc_dump) {
+            const int m = m0 + wm * TM + h * 64 + mb * 16 + lm, n = n0 + wn * 64 + nb * 16 + lg * 4;
+            if (m < M && n < N) {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) gstore<int>(t.acc_dump + (long)m * N + n + e, __float_as_int(a[e]));
             }
           }
         }
-      }
-    const int pr = lane >> 3, pc = lane & 7;  // 8 lanes x 16 B per 64-channel row, 8 rows per pass
 #pragma unroll
-    for (int r0 = 0; r0 < 64; r0 += 8) {
-      const int ml = r0 + pr;
-      const int m = m0 + wm * 64 + ml, n = n0 + wn * 64 + pc * 8;
-      const v4i v = *reinterpret_cast<const v4i*>(patch + ml * kPitch + pc * 16);
-      if (m < M && n < N) gstore_stream<v4i>(t.C + (long)m * N + n, v);
+      for (int r0 = 0; r0 < 64; r0 += 8) {
+        const int ml = r0 + pr;
+        const int m = m0 + wm * TM + h * 64 + ml, n = n0 + wn * 64 + pc * 8;
+        const v4i v = *reinterpret_cast<const v4i*>(patch + ml * kPitch + pc * 16);
+        if (m < M && n < N) gstore_stream<v4i>(t.C + (long)m * N + n, v);
+      }
     }
   }
 };

@@ -198,8 +198,8 @@ class TileConfig:
         if self.num_warps != 4:
             raise ValueError(f"{self!r}: gfx950 tiles use 4 wavefronts per workgroup")
         if self.is_weight_only():
-            if self.BK != 128 or not ((self.BM == 16 and self.BN % 64 == 0 and (self.WM, self.WN) == (1, 4)) or (self.BM, self.BN, self.WM, self.WN) == (128, 128, 2, 2)):
-                raise ValueError(f"{self!r}: weight-only tiles are 16 x (64k) x 128 (1 x 4 waves) or 128 x 128 x 128 (2 x 2 waves)")
+            if self.BK != 128 or not ((self.BM == 16 and self.BN % 64 == 0 and (self.WM, self.WN) == (1, 4)) or (self.BM, self.BN, self.WM, self.WN) in ((128, 128, 2, 2), (128, 256, 1, 4))):
+                raise ValueError(f"{self!r}: weight-only tiles are 16 x (64k) x 128 (1 x 4 waves), 128 x 128 x 128 (2 x 2 waves) or 128 x 256 x 128 (1 x 4 waves)")
             return
         k_elems = {"MFMA_F32_32x32x16_F16": 32, "MFMA_I32_32x32x32_I8": 64, "MFMA_I32_32x32x32_I8_FROM_I4": 128}[self.MMA]
         if self.BK != k_elems or self.STAGE != 3 or self.WK != 1 or (self.BM // self.WM) % 32 or (self.BN // self.WN) % 32:
@@ -245,7 +245,8 @@ def get_possible_tile_list(arch: str, qcfg: str) -> list:
     mma = QCFG_TO_MMA[qcfg]
     if mma == "MFMA_F32_16x16x32_F16":
         skinny = [_with_q(TileConfig(BM=16, BN=bn, BK=128, WM=1, WN=4, WK=1, STAGE=2, MMA=mma), qcfg) for bn in (128, 64)]
-        return skinny + [_with_q(TileConfig(BM=128, BN=128, BK=128, WM=2, WN=2, WK=1, STAGE=2, MMA=mma), qcfg)]
+        big = [_with_q(TileConfig(BM=128, BN=bn, BK=128, WM=wm, WN=wn, WK=1, STAGE=2, MMA=mma), qcfg) for bn, wm, wn in ((128, 2, 2), (256, 1, 4))]
+        return skinny + big
     bk = {"MFMA_F32_32x32x16_F16": 32, "MFMA_I32_32x32x32_I8": 64, "MFMA_I32_32x32x32_I8_FROM_I4": 128}[mma]
     if mma == "MFMA_F32_32x32x16_F16":
         shapes = [(128, 256, 2, 2), (64, 256, 1, 4), (32, 256, 1, 4), (128, 128, 2, 2), (256, 128, 2, 2)]

@@ -178,7 +178,8 @@ def test_weight_only_skinny():
 
 
 def test_weight_only_many_tokens():
-    """Experts with many tokens run the 128 x 128 dequantise-to-fp16 MFMA tile (and the remainder rows the skinny one)."""
+    """Experts with many tokens run the 128 x 256 dequantise-to-fp16 MFMA tile (and the remainder rows the skinny one); channel
+    counts that leave one or two of its four waves without channels are among the cases."""
     import ctypes as C
 
     from mxmoe_amd import _lib
@@ -186,8 +187,8 @@ def test_weight_only_many_tokens():
 
     rng = np.random.default_rng(5)
     probs = []
-    for (m, n, k, bits, sym) in [(200, 256, 512, 4, False), (129, 384, 1408, 3, False), (64, 128, 128, 4, True), (300, 2816, 256, 3, True),
-                                 (128, 192, 256, 4, False), (7, 256, 256, 4, False), (150, 256, 1408, 2, False)]:
+    for (m, n, k, bits, sym) in [(200, 256, 512, 4, False), (129, 384, 1408, 3, False), (64, 256, 128, 4, True), (300, 2816, 256, 3, True),
+                                 (128, 192, 256, 4, False), (7, 256, 256, 4, False), (150, 256, 1408, 2, False), (200, 128, 256, 4, False)]:
         x = rng.standard_normal((m, k)).astype(F16)
         w = (rng.standard_normal((n, k)) * 0.02).astype(F16)
         pw = quantize_and_pack(torch.from_numpy(w), (16, bits, 128, sym))
@@ -202,7 +203,7 @@ def test_weight_only_many_tokens():
     for b in branches:
         assert lib.mxmoe_kernel_branch(kid, b, info) == 0
         bms.append(info[1])
-    assert bms[:5] == [128] * 5 and bms[5] == 16 and bms[6] == 128, bms
+    assert bms[:5] == [128] * 5 and bms[5] == 16 and bms[6:] == [128, 128], bms
     for p, out in zip(probs, outs):
         assert np.isfinite(out).all()
         assert _rel(out, p["ref"]) <= 1e-2, (p["size"], p["q"], _rel(out, p["ref"]))
