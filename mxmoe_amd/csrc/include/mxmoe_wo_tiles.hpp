@@ -238,15 +238,18 @@ struct SkinnyWoTile {
   }
 };
 
-// Weight-only tile for experts with many tokens (w4a16 / w3a16, group 128): 128 tokens x 128 channels per workgroup, 64 x 64 per
-// wave.  Counterpart of the reference's cta_gemm_multistage_qb_v2 with its larger tiles
+// Weight-only tile for experts with many tokens (w4a16 / w3a16 / w2a16, group 128): 128 tokens x 256 channels per workgroup as four
+// waves side by side, each with all 128 tokens against its own 64 channels (BN = 128: 2 x 2 waves of 64 x 64, the shape with
+// half the token reuse per unpacked weight).  Counterpart of the reference's cta_gemm_multistage_qb_v2 with its larger tiles
 // (mxmoe/kernels/src/include/cta_gemm.cuh:113-286) and of Converter::dequant_frag (quantize.cuh:134-214): every packed weight
 // becomes fp16 as fma(q, scale, zero) in fp16, one rounding, exactly like the reference's __hfma2, and the products are summed in
-// fp32 by the fp16 MFMA over the whole of K.
+// fp32 by the fp16 MFMA over the whole of K, in the same order for both shapes.
 // Same packed weight and (scale, zero) layouts as the skinny tile: a wave streams its 4 channel blocks of each 128-wide k block
-// straight from global memory through a register ring and reuses each dequantised block for 4 token blocks x 4 MFMAs, so the
-// unpack work is a fraction of the matrix work.  Activations go global -> LDS (direct loads, two stages of 128 rows x 256 B,
-// 16-byte chunks XOR-swizzled with the row so that the 16 rows a read touches hit 16 different bank groups).
+// straight from global memory through a register ring and reuses each dequantised 8-weight operand for all of its token blocks
+// (8, or 4 in the 2 x 2 shape): the unpack work per MFMA, about 3 vector instructions in the 2 x 2 shape, is what bounds the tile.
+// The k block is walked in four 32-wide sub-blocks so that only one sub-block's token fragments are live beside the accumulators.
+// Activations go global -> LDS (direct loads, two stages of 128 rows x 256 B, 16-byte chunks XOR-swizzled with the row so that
+// the 16 rows a read touches hit 16 different bank groups).
 template <int WBITS_, int BM_ = 128, int BN_ = 128>
 struct WoMfmaTile {
   static constexpr int WBITS = WBITS_, BM = BM_, BN = BN_;
