@@ -17,7 +17,7 @@ import os
 import sys
 import time
 
-PEAK = {"int8": 5000.0, "fp16": 2500.0, "hbm": 8000.0}  # MI355X: TOP/s dense int8 MFMA, TFLOP/s dense fp16 MFMA, GB/s HBM3E
+PEAK = {"int8": 5000.0, "fp16": 2500.0, "fp6": 10100.0, "hbm": 8000.0}  # MI355X: TOP/s dense int8 MFMA, TFLOP/s dense fp16 / fp6 MFMA, GB/s HBM3E
 
 # HBM bytes per launch of the dominant (gate_up) kernel, from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE runs scaled by the
 # same counters on a plain 256 MiB copy (summaries: profiles/fused_group_gemm_<workload>.txt, profiles/counter_calibration_copy_256MiB.txt)
@@ -238,8 +238,10 @@ def time_whole_layer(cfg, layer, reps: int = 7) -> dict:
 
 
 def mfma_probe(iters: int = 20000, workgroups: int = 512, repeats: int = 3):
-    """Rate and shader clock of a bare v_mfma_i32_32x32x32_i8 loop (512 workgroups = two per CU, 8 independent accumulators per wave) for
-    four operand patterns.  Each pattern runs `repeats` times back to back after a short warm-up launch; the last run is reported."""
+    """Rate and shader clock of a bare loop of matrix instructions (512 workgroups = two per CU, 8 independent accumulators per wave):
+    v_mfma_i32_32x32x32_i8 for six operand patterns, then v_mfma_scale_f32_32x32x64_f8f6f4 on bf6 operands that hold int4 values (the
+    path on which int4 x int4 products are exact at twice the int8 instruction's rate).  Each pattern runs `repeats` times back to
+    back after a short warm-up launch; the last run is reported."""
     import torch
 
     from mxmoe_amd import _lib
@@ -249,8 +251,12 @@ def mfma_probe(iters: int = 20000, workgroups: int = 512, repeats: int = 3):
     out = torch.zeros(workgroups * 256 + 4, dtype=torch.int32, device="cuda")
     stream = torch.cuda.current_stream().cuda_stream
     ops = 2 * 32 * 32 * 32 * 8 * iters * 4 * workgroups
-    res = {"probe": "bare v_mfma_i32_32x32x32_i8 loop", "workgroups": workgroups, "iters": iters, "ops_per_launch": ops, "peak_tops": PEAK["int8"], "modes": {}}
-    for mode, name in enumerate(["zero operands", "constant operands", "random 16*int4 operands", "random int8 operands", "random offset-binary int4 operands (0..15)", "random sign-extended int4 operands"]):
+    res = {"probe": "bare matrix-instruction loop", "workgroups": workgroups, "iters": iters, "ops_per_launch_int8": ops, "ops_per_launch_bf6": 2 * ops,
+           "peak_tops": PEAK["int8"], "peak_tops_bf6": PEAK["fp6"], "modes": {}}
+    names = ["zero operands", "constant operands", "random 16*int4 operands", "random int8 operands", "random offset-binary int4 operands (0..15)",
+             "random sign-extended int4 operands", "bf6 32x32x64: random int4 values", "bf6 32x32x64: zero operands"]
+    for mode, name in enumerate(names):
+        mode_ops, peak = (2 * ops, PEAK["fp6"]) if mode >= 6 else (ops, PEAK["int8"])
         _lib.check(lib, lib.mxmoe_mfma_probe(mode, 100, workgroups, src.data_ptr(), out.data_ptr(), stream))
         torch.cuda.synchronize()
         for _ in range(repeats):
@@ -261,7 +267,7 @@ def mfma_probe(iters: int = 20000, workgroups: int = 512, repeats: int = 3):
             torch.cuda.synchronize()
             ms = e0.elapsed_time(e1)
         rec = out[-4:].cpu().numpy().view("uint64")
-        res["modes"][name] = {"ms": round(ms, 3), "tops": round(ops / (ms * 1e-3) / 1e12, 1), "of_peak": round(ops / (ms * 1e-3) / 1e12 / PEAK["int8"], 3),
+        res["modes"][name] = {"ms": round(ms, 3), "tops": round(mode_ops / (ms * 1e-3) / 1e12, 1), "of_peak": round(mode_ops / (ms * 1e-3) / 1e12 / peak, 3),
                               "shader_clock_ghz": round(float(rec[0]) / (float(rec[1]) * 10.0), 3)}
     return res
 

@@ -211,14 +211,21 @@ int mxmoe_unpermute_combine_planned(const void* down_out, const void* d_plan_dow
 int mxmoe_combine_planned(const void* down_out, const void* d_plan_down, int num_problems, const float* topk_weights, const int32_t* row_of_slot, int num_tokens,
                           int topk, int K, void* out, void* stream);
 
-/* ---- diagnostic (no counterpart in the reference): the rate the int8 matrix pipes sustain on their own ----
- * One launch of a bare loop of v_mfma_i32_32x32x32_i8 (8 independent accumulators per wave, two waves per SIMD, no memory traffic in
- * the loop): `workgroups` x 256 threads, `iters` x 8 instructions per wave = 2*32*32*32 * 8 * iters * 4 * workgroups operations.
- * mode: 0 all-zero operands, 1 a constant byte pattern, 2 random bytes 16*v (widened int4 codes),  3 random int8 bytes,
- * 4 random bytes 0..15 (offset-binary int4), 5 random sign-extended int4 bytes.
+/* ---- diagnostics (no counterpart in the reference): the rate the matrix pipes sustain on their own ----
+ * One launch of a bare loop of matrix instructions (8 independent accumulators per wave, two waves per SIMD, no memory traffic in
+ * the loop): `workgroups` x 256 threads, `iters` x 8 instructions per wave.
+ * Modes 0 - 5 run v_mfma_i32_32x32x32_i8 (2*32*32*32 * 8 * iters * 4 * workgroups operations): 0 all-zero operands, 1 a constant
+ * byte pattern, 2 random bytes 16*v (widened int4 codes), 3 random int8 bytes, 4 random bytes 0..15 (offset-binary int4), 5 random
+ * sign-extended int4 bytes.  Modes 6 and 7 run v_mfma_scale_f32_32x32x64_f8f6f4 on bf6 (e3m2) operands with unit scales (twice
+ * the operations per instruction): 6 random integers -8 .. 7 as bf6 codes, 7 zeros.
  * d_src: 65536 bytes of random data; d_out: (workgroups * 256 + 4) * 4 bytes; its last 16 bytes receive the shader-clock cycles and
  * the 100 MHz real-time ticks of workgroup 0's loop (two uint64), which give the clock the chip ran at.  bench.py --mfma-probe. */
 int mxmoe_mfma_probe(int mode, int iters, int workgroups, const void* d_src, void* d_out, void* stream);
+
+/* D[32][32] (fp32) = A . B^T for A, B of 32 x 64 int8 values in -8 .. 8 (device pointers), by one v_mfma_scale_f32_32x32x64_f8f6f4
+ * of one wave on operands re-encoded as bf6: every such integer is a bf6 number and the fp32 sums of their products are exact, so
+ * the result equals the integer product (what an int4 x int4 tile on the 6-bit float path would rely on). */
+int mxmoe_bf6_dot_probe(const void* d_a, const void* d_b, void* d_out, void* stream);
 
 #ifdef __cplusplus
 }

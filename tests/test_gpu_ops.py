@@ -213,9 +213,34 @@ def test_bench_diagnostics_run():
     bench = importlib.util.module_from_spec(spec)
     spec.loader.exec_module(bench)
     probe = bench.mfma_probe(iters=2000, workgroups=512, repeats=1)
-    assert len(probe["modes"]) == 6
-    for m in probe["modes"].values():
-        assert 0.0 < m["tops"] <= 1.05 * bench.PEAK["int8"] and 0.5 < m["shader_clock_ghz"] < 3.0
+    assert len(probe["modes"]) == 8
+    for name, m in probe["modes"].items():
+        peak = bench.PEAK["fp6"] if name.startswith("bf6") else bench.PEAK["int8"]
+        assert 0.0 < m["tops"] <= 1.05 * peak and 0.5 < m["shader_clock_ghz"] < 3.0
     one = bench.one_problem("w4a4:2048x512x1024")
     assert set(one["operands"]) == {"random codes", "constant codes", "zero codes"}
     assert all(0.0 < o["tops"] < bench.PEAK["int8"] for o in one["operands"].values())
+
+
+def test_int4_products_are_exact_on_the_bf6_matrix_path():
+    """Integers -8 .. 8 are bf6 (e3m2) numbers and fp32 adds their products exactly, so one v_mfma_scale_f32_32x32x64_f8f6f4 on
+    operands re-encoded as bf6 must return the integer product A . B^T: random int4 matrices, the extreme -8 x -8 (4096 per entry),
+    +8 (outside int4 but a bf6 number; used by symmetric ranges) and a one-hot pattern that pins the lane-to-(row, k) map."""
+    from mxmoe_amd import _lib
+
+    lib = _lib.load()
+    rng = np.random.default_rng(21)
+    onehot_a, onehot_b = np.zeros((32, 64), np.int8), np.zeros((32, 64), np.int8)
+    for r in range(32):
+        onehot_a[r, (5 * r + 3) % 64] = (r % 15) - 7
+        onehot_b[r, (5 * r + 3) % 64] = 7 - (r % 13)
+    cases = [(rng.integers(-8, 8, (32, 64)).astype(np.int8), rng.integers(-8, 8, (32, 64)).astype(np.int8)) for _ in range(4)]
+    cases += [(np.full((32, 64), -8, np.int8), np.full((32, 64), -8, np.int8)), (np.full((32, 64), 8, np.int8), rng.integers(-8, 9, (32, 64)).astype(np.int8)),
+              (onehot_a, onehot_b), (onehot_a, rng.integers(-8, 8, (32, 64)).astype(np.int8))]
+    out = torch.empty(32, 32, dtype=torch.float32, device=DEV)
+    for a, b in cases:
+        ta, tb = torch.from_numpy(a).to(DEV), torch.from_numpy(b).to(DEV)
+        _lib.check(lib, lib.mxmoe_bf6_dot_probe(ta.data_ptr(), tb.data_ptr(), out.data_ptr(), torch.cuda.current_stream().cuda_stream))
+        torch.cuda.synchronize()
+        want = a.astype(np.int64) @ b.astype(np.int64).T
+        assert np.array_equal(out.cpu().numpy().astype(np.int64), want) and np.array_equal(out.cpu().numpy(), want.astype(np.float32))
