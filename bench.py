@@ -299,6 +299,49 @@ def one_problem(spec: str):
     return res
 
 
+def bf6_probe(dims: str):
+    """One int4 x int4 problem M x N x K on the 6-bit float matrix path (the diagnostic kernel mxmoe_bf6_gemm_probe: bf6 operand
+    fragments, exact accumulators) next to the same shape through the int4 tile of the default kernel: uniformly random values
+    -8 .. 7, bell-shaped ones (a rounded normal of deviation 2.5, what rotated activations quantise to), and zeros."""
+    import torch
+
+    from mxmoe_amd import _lib, bf6, harness
+
+    m, n, k = (int(x) for x in dims.lower().split("x"))
+    lib = _lib.load()
+    stream = torch.cuda.current_stream().cuda_stream
+    gen = torch.Generator("cuda").manual_seed(0)
+    ops = 2 * m * n * k
+    res = {"problem": dims, "ops": ops, "peak_tops_int8": PEAK["int8"], "peak_tops_fp6": PEAK["fp6"], "bf6_probe": {}, "int4_tile": {}}
+    sa = torch.full((m,), 0.01, dtype=torch.float16, device="cuda")
+    sb = torch.full((n,), 0.01, dtype=torch.float16, device="cuda")
+    c = torch.empty(m, n, dtype=torch.float16, device="cuda")
+
+    def values(kind, rows):
+        if kind == "uniform values":
+            return torch.randint(-8, 8, (rows, k), dtype=torch.int8, device="cuda", generator=gen)
+        if kind == "bell-shaped values":
+            return (torch.randn(rows, k, device="cuda", generator=gen) * 2.5).round().clamp(-8, 7).to(torch.int8)
+        return torch.zeros(rows, k, dtype=torch.int8, device="cuda")
+
+    prob = harness.make_problem({"shape": [m, n, k], "w_bits": 4, "a_bits": 4, "gsize": -1, "sym": True}, None)
+    launch = harness._launch_of([prob], lib, lib.mxmoe_find_kernel(b"groupgemm_hz_fused_wxax"))
+    from mxmoe_amd import pack
+
+    for kind in ("uniform values", "bell-shaped values", "zero values"):
+        a, b = values(kind, m), values(kind, n)
+        a6, b6 = bf6.pack_fragments(a), bf6.pack_fragments(b)
+        run = lambda: _lib.check(lib, lib.mxmoe_bf6_gemm_probe(a6.data_ptr(), b6.data_ptr(), sa.data_ptr(), sb.data_ptr(), c.data_ptr(), None, m, n, k, stream))
+        ms = harness.bench_func(run, warmup=20, iters=30)["median"]
+        res["bf6_probe"][kind] = {"us": round(ms * 1e3, 1), "tops": round(ops / ms / 1e9, 1), "of_fp6_peak": round(ops / ms / 1e9 / PEAK["fp6"], 3)}
+        prob["A"].copy_(pack.pack_int4_k(a))                                  # the same values through the integer tile
+        prob["B"].copy_(pack.pack_wxax_fragments(pack.pack_int4_k(b)))
+        ms = harness.bench_func(launch.run, warmup=20, iters=30)["median"]
+        res["int4_tile"][kind] = {"us": round(ms * 1e3, 1), "tops": round(ops / ms / 1e9, 1), "of_int8_peak": round(ops / ms / 1e9 / PEAK["int8"], 3)}
+        del a, b, a6, b6
+    return res
+
+
 def run_workload(name: str, steps: int, warmup: int, tokens=None, whole: bool = True):
     cfg, layer = build_layer(name, tokens)
     ms, up, dn = time_layer(layer, steps, warmup)
@@ -328,6 +371,9 @@ def main() -> int:
     ap.add_argument("--one-problem", default="", metavar="FMT:MxNxK",
                     help="instead of the benchmark, time one GroupGEMM problem (FMT w4a4 or w8a8, e.g. w4a4:32768x2048x4096) through the default "
                          "kernel with random, constant and all-zero operand codes: the same instruction stream at three levels of operand toggling")
+    ap.add_argument("--bf6-probe", default="", metavar="MxNxK",
+                    help="instead of the benchmark, time one int4 x int4 problem on the 6-bit float matrix path (diagnostic kernel) and through the int4 tile "
+                         "(M, N and K multiples of 256, e.g. 32768x2048x4096)")
     ap.add_argument("--mfma-probe", action="store_true",
                     help="instead of the benchmark, time a bare loop of int8 matrix instructions per operand pattern (the ceiling of the matrix pipes on this GPU)")
     args = ap.parse_args()
@@ -352,6 +398,9 @@ def main() -> int:
     if args.mfma_probe:
         print(json.dumps(mfma_probe()))
         return 0
+    if args.bf6_probe:
+        print(json.dumps(bf6_probe(args.bf6_probe)))
+        return
     if args.one_problem:
         print(json.dumps(one_problem(args.one_problem)))
         return 0
