@@ -312,7 +312,8 @@ def bf6_probe(dims: str):
     stream = torch.cuda.current_stream().cuda_stream
     gen = torch.Generator("cuda").manual_seed(0)
     ops = 2 * m * n * k
-    res = {"problem": dims, "ops": ops, "peak_tops_int8": PEAK["int8"], "peak_tops_fp6": PEAK["fp6"], "bf6_probe": {}, "int4_tile": {}}
+    shapes = {"bf6_probe_256x256_one_wave_per_simd": 0, "bf6_probe_128x256_two_workgroups_per_cu": 1}
+    res = {"problem": dims, "ops": ops, "peak_tops_int8": PEAK["int8"], "peak_tops_fp6": PEAK["fp6"], **{k_: {} for k_ in shapes}, "int4_tile": {}}
     sa = torch.full((m,), 0.01, dtype=torch.float16, device="cuda")
     sb = torch.full((n,), 0.01, dtype=torch.float16, device="cuda")
     c = torch.empty(m, n, dtype=torch.float16, device="cuda")
@@ -331,9 +332,10 @@ def bf6_probe(dims: str):
     for kind in ("uniform values", "bell-shaped values", "zero values"):
         a, b = values(kind, m), values(kind, n)
         a6, b6 = bf6.pack_fragments(a), bf6.pack_fragments(b)
-        run = lambda: _lib.check(lib, lib.mxmoe_bf6_gemm_probe(a6.data_ptr(), b6.data_ptr(), sa.data_ptr(), sb.data_ptr(), c.data_ptr(), None, m, n, k, stream))
-        ms = harness.bench_func(run, warmup=20, iters=30)["median"]
-        res["bf6_probe"][kind] = {"us": round(ms * 1e3, 1), "tops": round(ops / ms / 1e9, 1), "of_fp6_peak": round(ops / ms / 1e9 / PEAK["fp6"], 3)}
+        for name, shape in shapes.items():
+            run = lambda: _lib.check(lib, lib.mxmoe_bf6_gemm_probe(a6.data_ptr(), b6.data_ptr(), sa.data_ptr(), sb.data_ptr(), c.data_ptr(), None, m, n, k, shape, stream))
+            ms = harness.bench_func(run, warmup=20, iters=30)["median"]
+            res[name][kind] = {"us": round(ms * 1e3, 1), "tops": round(ops / ms / 1e9, 1), "of_fp6_peak": round(ops / ms / 1e9 / PEAK["fp6"], 3)}
         prob["A"].copy_(pack.pack_int4_k(a))                                  # the same values through the integer tile
         prob["B"].copy_(pack.pack_wxax_fragments(pack.pack_int4_k(b)))
         ms = harness.bench_func(launch.run, warmup=20, iters=30)["median"]

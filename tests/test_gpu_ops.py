@@ -247,15 +247,16 @@ def test_int4_products_are_exact_on_the_bf6_matrix_path():
 
 
 def test_int4_gemm_on_the_bf6_matrix_path_is_exact():
-    """The diagnostic GEMM on bf6 fragments: its accumulators equal the integer product and its fp16 outputs the epilogue formula
-    half(acc * (sa * sb)) evaluated in fp32, bit for bit - several workgroups per XCD range, K of 4 to 24 steps, the values
-    -8 and +8 included."""
+    """The diagnostic GEMM on bf6 fragments, both workgroup shapes: its accumulators equal the integer product and its fp16 outputs
+    the epilogue formula half(acc * (sa * sb)) evaluated in fp32, bit for bit - several workgroups per XCD range, K of 4 to 24 steps,
+    the values -8 and +8 included."""
     from mxmoe_amd import _lib, bf6
 
     lib = _lib.load()
     rng = np.random.default_rng(33)
     stream = torch.cuda.current_stream().cuda_stream
-    for (m, n, k) in [(256, 256, 256), (512, 768, 512), (256, 512, 1536), (2304, 256, 768)]:
+    for shape, (m, n, k) in [(0, (256, 256, 256)), (0, (512, 768, 512)), (0, (256, 512, 1536)), (0, (2304, 256, 768)),
+                             (1, (128, 256, 256)), (1, (384, 768, 512)), (1, (128, 512, 1536)), (1, (1152, 256, 768))]:
         a = rng.integers(-8, 9, (m, k)).astype(np.int8)
         b = rng.integers(-8, 8, (n, k)).astype(np.int8)
         sa = (rng.random(m) * 0.05 + 0.001).astype(F16)
@@ -264,14 +265,16 @@ def test_int4_gemm_on_the_bf6_matrix_path_is_exact():
         tsa, tsb = torch.from_numpy(sa).to(DEV), torch.from_numpy(sb).to(DEV)
         c = torch.full((m, n), float("nan"), dtype=torch.float16, device=DEV)
         ci = torch.full((m, n), -1, dtype=torch.int32, device=DEV)
-        _lib.check(lib, lib.mxmoe_bf6_gemm_probe(ta.data_ptr(), tb.data_ptr(), tsa.data_ptr(), tsb.data_ptr(), c.data_ptr(), ci.data_ptr(), m, n, k, stream))
+        _lib.check(lib, lib.mxmoe_bf6_gemm_probe(ta.data_ptr(), tb.data_ptr(), tsa.data_ptr(), tsb.data_ptr(), c.data_ptr(), ci.data_ptr(), m, n, k, shape, stream))
         torch.cuda.synchronize()
         acc = a.astype(np.int64) @ b.astype(np.int64).T
-        assert np.array_equal(ci.cpu().numpy().astype(np.int64), acc), (m, n, k)
+        assert np.array_equal(ci.cpu().numpy().astype(np.int64), acc), (shape, m, n, k)
         want = (acc.astype(np.float32) * (sa.astype(np.float32)[:, None] * sb.astype(np.float32)[None, :])).astype(F16)
-        assert np.array_equal(c.cpu().numpy().view(np.uint16), want.view(np.uint16)), (m, n, k)
+        assert np.array_equal(c.cpu().numpy().view(np.uint16), want.view(np.uint16)), (shape, m, n, k)
         c.fill_(float("nan"))   # the same without the accumulator dump
-        _lib.check(lib, lib.mxmoe_bf6_gemm_probe(ta.data_ptr(), tb.data_ptr(), tsa.data_ptr(), tsb.data_ptr(), c.data_ptr(), None, m, n, k, stream))
+        _lib.check(lib, lib.mxmoe_bf6_gemm_probe(ta.data_ptr(), tb.data_ptr(), tsa.data_ptr(), tsb.data_ptr(), c.data_ptr(), None, m, n, k, shape, stream))
         torch.cuda.synchronize()
-        assert np.array_equal(c.cpu().numpy().view(np.uint16), want.view(np.uint16)), (m, n, k)
-    assert lib.mxmoe_bf6_gemm_probe(ta.data_ptr(), tb.data_ptr(), tsa.data_ptr(), tsb.data_ptr(), c.data_ptr(), None, 250, 256, 256, stream) == 3
+        assert np.array_equal(c.cpu().numpy().view(np.uint16), want.view(np.uint16)), (shape, m, n, k)
+    assert lib.mxmoe_bf6_gemm_probe(ta.data_ptr(), tb.data_ptr(), tsa.data_ptr(), tsb.data_ptr(), c.data_ptr(), None, 250, 256, 256, 0, stream) == 3
+    assert lib.mxmoe_bf6_gemm_probe(ta.data_ptr(), tb.data_ptr(), tsa.data_ptr(), tsb.data_ptr(), c.data_ptr(), None, 128, 256, 256, 0, stream) == 3
+    assert lib.mxmoe_bf6_gemm_probe(ta.data_ptr(), tb.data_ptr(), tsa.data_ptr(), tsb.data_ptr(), c.data_ptr(), None, 256, 256, 256, 2, stream) == 3
