@@ -231,8 +231,8 @@ int mxmoe_bf6_dot_probe(const void* d_a, const void* d_b, void* d_out, void* str
  * C[M][N] (fp16) = half(acc * (float(sa[m]) * float(sb[n]))), acc = sum_k a[m][k] * b[n][k], and acc itself as int32 into d_cint
  * when that is not null.  d_a6 / d_b6: the int4 values of A [M][K] and B [N][K] as bf6 fragments (32 rows x 64 k per fragment of
  * 1536 bytes, k step major: mxmoe_amd/bf6.py: pack_fragments); sa [M], sb [N] fp16.  shape 0: workgroups of 256 x 256 as 2 x 2 waves
- * of 128 x 128, one wave per SIMD (M a multiple of 256); shape 1: workgroups of 128 x 256 as four waves of 128 x 64, two workgroups
- * per CU (M a multiple of 128).  N and K multiples of 256.  Returns 0, 3 for bad arguments, 4 for a launch error.
+ * of 128 x 128, one wave per SIMD (M and K multiples of 256); shape 1: workgroups of 128 x 256 as four waves of 128 x 64, two
+ * workgroups per CU (M and K multiples of 128, K >= 256).  N a multiple of 256.  Returns 0, 3 for bad arguments, 4 for a launch error.
  * bench.py --bf6-probe. */
 int mxmoe_bf6_gemm_probe(const void* d_a6, const void* d_b6, const void* d_sa, const void* d_sb, void* d_c, void* d_cint, int M, int N, int K, int shape,
                          void* stream);

@@ -67,7 +67,8 @@ __global__ void __launch_bounds__(256, CA == 4 ? 1 : 2) bf6_gemm_kernel(const ui
   constexpr int kStage = 4 * WROWS * kFrag; // the workgroup's token fragments of one k step
   constexpr int kDma = CA == 4 ? 3 : 2;     // direct-to-LDS loads per wave and stage (1 KB each)
   constexpr int kPieces = kStage / 1024;    // 12 or 6; with 6 pieces two of the eight loads bring a piece a second time
-  constexpr int kYounger = 2 * CA + 2 * (kDma + 2 * CA);  // loads younger than a step's stage when the step begins, see below
+  constexpr int RD = CA == 4 ? 4 : 2;       // steps the channel-fragment ring runs ahead (alone on its SIMD a wave needs the longer one)
+  constexpr int kYounger = RD == 4 ? 2 * CA + 2 * (kDma + 2 * CA) : kDma + 2 * CA;  // outstanding loads a step may begin with, see below
   __shared__ __align__(16) uint8_t smem[kStages * kStage];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -118,17 +119,28 @@ __global__ void __launch_bounds__(256, CA == 4 ? 1 : 2) bf6_gemm_kernel(const ui
       for (int r = 0; r < 16; ++r) acc[c][t][r] = 0.f;
 
   // Every vector-memory load of the loop is issued and awaited by hand.  Order within step ks: after the barrier the kDma
-  // direct-to-LDS loads of stage ks + 3, and after the matrix instructions the 2 CA ring loads of step ks + 4's channel fragments
-  // (with one wave per SIMD nothing else hides a load's latency, so the ring runs four steps ahead).  When step ks begins, the
-  // loads younger than its stage (issued in step ks - 3) are 2 CA + 2 (kDma + 2 CA) = 30 or 16, and its channel fragments
-  // (issued in step ks - 4) are older still: one wait for "at most that many outstanding" covers both.  The prologue issues its
-  // loads in the same pattern.
-  Frag br[4][CA];
+  // direct-to-LDS loads of stage ks + 3, and after the matrix instructions the 2 CA ring loads of step ks + RD's channel fragments.
+  // Ring four steps ahead (one wave per SIMD: nothing else hides a load's latency): when step ks begins, the loads younger than
+  // its stage (issued in step ks - 3) are 2 CA + 2 (kDma + 2 CA) = 30, and its channel fragments (issued in step ks - 4) are older
+  // still.  Ring two steps ahead: the loads younger than its channel fragments (issued in step ks - 2) are the kDma + 2 CA = 6 of
+  // step ks - 1, and its stage is older still.  One wait for "at most that many outstanding" covers both operands either way, and
+  // the prologue issues its loads in the order the steps before ks = 0 would have.
+  Frag br[RD][CA];
+  if constexpr (RD == 4) {
 #pragma unroll
-  for (int p = 0; p < 4; ++p) {
+    for (int p = 0; p < 4; ++p) {
 #pragma unroll
-    for (int j = 0; j < CA; ++j) br[p][j] = load_b(p, j);
-    if (p < 3) dma_a(p);
+      for (int j = 0; j < CA; ++j) br[p][j] = load_b(p, j);
+      if (p < 3) dma_a(p);
+    }
+  } else {
+    dma_a(0);
+    dma_a(1);
+#pragma unroll
+    for (int j = 0; j < CA; ++j) br[0][j] = load_b(0, j);
+    dma_a(2);
+#pragma unroll
+    for (int j = 0; j < CA; ++j) br[1][j] = load_b(1, j);
   }
 
   auto step = [&](auto parc, int ks) {
@@ -148,19 +160,19 @@ __global__ void __launch_bounds__(256, CA == 4 ? 1 : 2) bf6_gemm_kernel(const ui
     }
     __builtin_amdgcn_sched_barrier(0);  // the ring registers are free only after the last instruction that reads them
 #pragma unroll
-    for (int j = 0; j < CA; ++j) br[par][j] = load_b(ks + 4, j);
+    for (int j = 0; j < CA; ++j) br[par][j] = load_b(ks + RD, j);
   };
 #pragma unroll 1
-  for (int ks = 0; ks < KS; ks += 4) {  // K is a multiple of 256: whole groups of four steps
+  for (int ks = 0; ks < KS; ks += RD) {  // K is a multiple of 64 RD: whole rounds of the ring
     step(std::integral_constant<int, 0>{}, ks);
     step(std::integral_constant<int, 1>{}, ks + 1);
-    step(std::integral_constant<int, 2>{}, ks + 2);
-    step(std::integral_constant<int, 3>{}, ks + 3);
+    if constexpr (RD == 4) {
+      step(std::integral_constant<int, 2>{}, ks + 2);
+      step(std::integral_constant<int, 3>{}, ks + 3);
+    }
   }
-  wait_frags<0>(br[0]);  // everything has landed (vmcnt(0)), the loads past the end of K included
-  wait_frags<0>(br[1]);
-  wait_frags<0>(br[2]);
-  wait_frags<0>(br[3]);
+#pragma unroll
+  for (int p = 0; p < RD; ++p) wait_frags<0>(br[p]);  // everything has landed (vmcnt(0)), the loads past the end of K included
 
   // epilogue: lane l holds, of fragment pair (c, t), token l % 32 and channels 8*(r/4) + 4*(l/32) + r%4, r = 0..15.  32 tokens at a
   // time go through a [token][channel] patch in LDS and leave as 16-byte pieces of whole rows of the wave's channels: stores of
@@ -207,12 +219,12 @@ __global__ void __launch_bounds__(256, CA == 4 ? 1 : 2) bf6_gemm_kernel(const ui
 
 // C[M][N] (fp16) = half(acc * (float(sa[m]) * float(sb[n]))) with acc = sum_k a[m][k] * b[n][k] over int4 values stored as bf6
 // fragments (layout above; mxmoe_amd.bf6.pack_fragments), and the accumulators themselves as int32 into d_cint when it is given.
-// shape 0: workgroups of 256 x 256 (one wave per SIMD), M a multiple of 256; shape 1: workgroups of 128 x 256 (two per CU), M a
-// multiple of 128.  N and K multiples of 256.  Returns 0, 3 for bad arguments, 4 for a launch error.
+// shape 0: workgroups of 256 x 256 (one wave per SIMD), M and K multiples of 256; shape 1: workgroups of 128 x 256 (two per CU), M
+// and K multiples of 128 (K >= 256).  N a multiple of 256.  Returns 0, 3 for bad arguments, 4 for a launch error.
 extern "C" int mxmoe_bf6_gemm_probe(const void* d_a6, const void* d_b6, const void* d_sa, const void* d_sb, void* d_c, void* d_cint, int M, int N, int K,
                                     int shape, void* stream) {
-  const int tm = shape == 0 ? 256 : 128;
-  if (!d_a6 || !d_b6 || !d_sa || !d_sb || !d_c || shape < 0 || shape > 1 || M < tm || N < 256 || K < 256 || M % tm || N % 256 || K % 256) return 3;
+  const int tm = shape == 0 ? 256 : 128, km = shape == 0 ? 256 : 128;  // rows of a workgroup; k covered by one round of the ring
+  if (!d_a6 || !d_b6 || !d_sa || !d_sb || !d_c || shape < 0 || shape > 1 || M < tm || N < 256 || K < 256 || M % tm || N % 256 || K % km) return 3;
   if ((long)M * K / 64 * 48 >= (1L << 32) || (long)N * K / 64 * 48 >= (1L << 31)) return 3;  // operands addressed with 32-bit offsets
   const int ntiles = (M / tm) * (N / 256);
   const int grid = (ntiles + 7) / 8 * 8;

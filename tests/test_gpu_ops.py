@@ -256,7 +256,7 @@ def test_int4_gemm_on_the_bf6_matrix_path_is_exact():
     rng = np.random.default_rng(33)
     stream = torch.cuda.current_stream().cuda_stream
     for shape, (m, n, k) in [(0, (256, 256, 256)), (0, (512, 768, 512)), (0, (256, 512, 1536)), (0, (2304, 256, 768)),
-                             (1, (128, 256, 256)), (1, (384, 768, 512)), (1, (128, 512, 1536)), (1, (1152, 256, 768))]:
+                             (1, (128, 256, 256)), (1, (384, 768, 512)), (1, (128, 512, 1536)), (1, (1152, 256, 768)), (1, (256, 256, 1408))]:
         a = rng.integers(-8, 9, (m, k)).astype(np.int8)
         b = rng.integers(-8, 8, (n, k)).astype(np.int8)
         sa = (rng.random(m) * 0.05 + 0.001).astype(F16)
@@ -278,3 +278,4 @@ def test_int4_gemm_on_the_bf6_matrix_path_is_exact():
     assert lib.mxmoe_bf6_gemm_probe(ta.data_ptr(), tb.data_ptr(), tsa.data_ptr(), tsb.data_ptr(), c.data_ptr(), None, 250, 256, 256, 0, stream) == 3
     assert lib.mxmoe_bf6_gemm_probe(ta.data_ptr(), tb.data_ptr(), tsa.data_ptr(), tsb.data_ptr(), c.data_ptr(), None, 128, 256, 256, 0, stream) == 3
     assert lib.mxmoe_bf6_gemm_probe(ta.data_ptr(), tb.data_ptr(), tsa.data_ptr(), tsb.data_ptr(), c.data_ptr(), None, 256, 256, 256, 2, stream) == 3
+    assert lib.mxmoe_bf6_gemm_probe(ta.data_ptr(), tb.data_ptr(), tsa.data_ptr(), tsb.data_ptr(), c.data_ptr(), None, 256, 256, 1408, 0, stream) == 3
