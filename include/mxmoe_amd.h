@@ -39,8 +39,8 @@ int mxmoe_kernel_branch(int kernel_id, int branch, int32_t out[8]);
  *
  * One launch computes Cs[p][M,N] = As[p][M,K] * Bs[p][N,K]^T for every problem p in its own format.
  * As, Bs, scale_a, scale_b, Cs, Ds, d_sizes and d_q are DEVICE arrays of `problem_count` entries; h_sizes and h_q are
- * their HOST mirrors (as in the reference).  Ds must be the same array as Cs or NULL (anything else is error 3: results are written
- * to Cs only); lda/ldb/ldc/ldd and d_q are DEVICE arrays accepted for signature compatibility and never read (leading dimensions are
+ * their HOST mirrors (as in the reference).  Ds is accepted and never read: results are written to Cs only, as by the reference's kernels
+ * (hz_fused.cuh:89,110; its caller passes a second array with the same entries, test.cu:446-459); lda/ldb/ldc/ldd and d_q are DEVICE arrays accepted for signature compatibility and never read (leading dimensions are
  * K, K, N; the reference's kernels ignore them as well and its caller passes nullptr, ref_bind.cu:413).
  * A kernel registered with the sequential or the multi-stream policy (mxmoe_kernel_policy) runs the same problem list as one launch
  * per run of consecutive problems of equal format, on `stream` or on up to 4 library-owned side streams that fork from and join
@@ -62,7 +62,7 @@ int mxmoe_kernel_branch(int kernel_id, int branch, int32_t out[8]);
  * receive the raw accumulators (int32 for w8a8 / w4a4 per channel, fp32 bit patterns otherwise: for w4a4_g128 the fp32 sum over the
  * groups of float(group's int32 sum) * (scale_a * scale_b), groups in ascending order); used by the parity tests.
  * Errors: 1 "quant type not supported" (same text as the reference launcher, compose_kernel.py:433), 2 bad kernel id,
- * 3 unsupported shape (K not a multiple of the tile's K step, N not a multiple of 8) or Ds differs from Cs, 4 launch failure, 5 a required array is NULL
+ * 3 unsupported shape (K not a multiple of the tile's K step, N not a multiple of 8), 4 launch failure, 5 a required array is NULL
  * (the scale arrays are required as soon as one non-empty problem is quantised). */
 int mxmoe_group_gemm(int kernel_id, const void* const* As, const void* const* Bs, const void* const* scale_a, const void* const* scale_b,
                      void* const* Cs, void* const* Ds, const int64_t* lda, const int64_t* ldb, const int64_t* ldc, const int64_t* ldd,
@@ -95,6 +95,12 @@ int mxmoe_group_gemm_plan(int kernel_id, const mxmoe_dim3* h_sizes, const mxmoe_
  * {entries, tiles, phases, workgroups}, phase_tile0[9], phase_wg0[9], then per entry {first tile, first row, rows, problem | branch << 16}.
  * At most 120 problems; used by the tests that compare the device-side planner with the host launcher. */
 int mxmoe_group_gemm_plan_tables(int kernel_id, const mxmoe_dim3* h_sizes, const mxmoe_qparams* h_q, int problem_count, int32_t* out, int out_ints);
+
+/* The tile each workgroup of such a launch runs when the grid holds `grid` workgroups (host-only; the role of the block -> tile walk of
+ * mxmoe/kernels/src/include/tile_scheduler.cuh:25-49): tile_of_wg[w] = tile index, or -1 for a workgroup without a tile.  A planned
+ * launch is enqueued with a grid sized for the worst routing, so `grid` may exceed the workgroups the tables need; the function the
+ * kernels call to find their tile is the one evaluated here. */
+int mxmoe_group_gemm_plan_tile_map(int kernel_id, const mxmoe_dim3* h_sizes, const mxmoe_qparams* h_q, int problem_count, int grid, int32_t* tile_of_wg);
 
 /* ---- token permutation: replaces gg_permute_inp and the sort / bincount prologue of quant_inp_act
  *      (mxmoe/kernels/src/ref_bind.cu:47-64, 449-453) ----

@@ -68,6 +68,7 @@ SIGNATURES = {
     "mxmoe_silu_mul_quant_planned": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P]),
     "mxmoe_unpermute_combine_planned": (_I, [_P, _P, _I, _P, _P, _I, _I, _I, _P, _P, _P]),
     "mxmoe_group_gemm_plan_tables": (_I, [_I, C.POINTER(Dim3), C.POINTER(QParams), _I, C.POINTER(C.c_int32), _I]),
+    "mxmoe_group_gemm_plan_tile_map": (_I, [_I, C.POINTER(Dim3), C.POINTER(QParams), _I, _I, C.POINTER(C.c_int32)]),
     "mxmoe_combine_workspace_bytes": (C.c_size_t, [_I, _I]),
     "mxmoe_unpermute_combine": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P]),
 }
@@ -76,7 +77,7 @@ _cached = {}
 
 
 GEMM_ONLY = ("mxmoe_last_error", "mxmoe_num_kernels", "mxmoe_kernel_name", "mxmoe_find_kernel", "mxmoe_kernel_num_branches", "mxmoe_kernel_branch",
-             "mxmoe_group_gemm", "mxmoe_group_gemm_plan", "mxmoe_group_gemm_plan_tables", "mxmoe_kernel_func", "mxmoe_get_kernel", "mxmoe_kernel_policy", "mxmoe_set_stream", "mxmoe_get_stream",
+             "mxmoe_group_gemm", "mxmoe_group_gemm_plan", "mxmoe_group_gemm_plan_tables", "mxmoe_group_gemm_plan_tile_map", "mxmoe_kernel_func", "mxmoe_get_kernel", "mxmoe_kernel_policy", "mxmoe_set_stream", "mxmoe_get_stream",
              "mxmoe_last_status")
 
 # the reference's FuncType (registry.cuh:28-39): 15 arguments, no return value

@@ -124,4 +124,18 @@ int mxmoe_group_gemm_plan_tables(int kernel_id, const mxmoe_dim3* h_sizes, const
   return 0;
 }
 
+int mxmoe_group_gemm_plan_tile_map(int kernel_id, const mxmoe_dim3* h_sizes, const mxmoe_qparams* h_q, int problem_count, int grid, int32_t* tile_of_wg) {
+  auto& reg = registry();
+  if (problem_count <= 0 || problem_count > kMaxProblems || !h_sizes || !h_q || !tile_of_wg || grid < 0 || kernel_id < 0 || kernel_id >= (int)reg.size()) {
+    last_error() = "bad argument";
+    return 5;
+  }
+  FusedArgs a;
+  std::memset(&a, 0, sizeof a);
+  int planned = 0;
+  if (const int rc = build_fused_tables(reg[kernel_id], h_sizes, h_q, 0, problem_count, a, &planned)) return rc;
+  for (int wg = 0; wg < grid; ++wg) tile_of_wg[wg] = tile_of_workgroup(&a, wg);
+  return 0;
+}
+
 }  // extern "C"

@@ -234,6 +234,7 @@ __global__ void __launch_bounds__(kPlanThreads) plan_block_kernel(const PlanPair
     }
     fa->phase_tile0[np] = total;
     fa->phase_wg0[np] = wg;
+    if (np == 0) fa->phase_tile0[1] = fa->phase_wg0[1] = 0;  // a plan without tiles still holds one (empty) phase range
     fa->num_phases = np;
     fa->phase_flat = flat;
     fa->num_entries = ne;

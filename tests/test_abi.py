@@ -133,17 +133,49 @@ def test_missing_arrays_are_refused_before_any_launch(lib):
     assert lib.mxmoe_group_gemm_plan(-1, None, None, 1, None, None) == 5
 
 
-def test_ds_must_alias_cs(lib):
-    """Results are written to Cs only, so a caller handing over a different Ds array is refused instead of being left with
-    stale memory (the reference passes the same array twice, ref_bind.cu:413)."""
+def test_ds_is_accepted_and_ignored(lib):
+    """The reference's caller hands the kernels a second pointer array Ds with the same entries as Cs (test.cu:446-459) and its
+    kernels store through Cs only (hz_fused.cuh:89,110): a distinct Ds array is no error here either.  Host-only: the call
+    below passes every check up to the launch and is refused for its (missing) scale arrays, not for its Ds."""
     from mxmoe_amd import _lib
 
     sizes = (_lib.Dim3 * 1)(_lib.Dim3(8, 256, 128))
     q = (_lib.QParams * 1)(_lib.QParams(4, 4, -1, 1))
     one, other = (C.c_void_p * 1)(0), (C.c_void_p * 1)(0)
     a, b = C.addressof(one), C.addressof(other)
-    rc = lib.mxmoe_group_gemm(0, a, a, a, a, a, b, None, None, None, None, a, sizes, None, q, 1, None, None)
-    assert rc == 3 and b"Ds" in lib.mxmoe_last_error()
+    rc = lib.mxmoe_group_gemm(0, a, a, None, None, a, b, None, None, None, None, a, sizes, None, q, 1, None, None)
+    assert rc == 5 and b"scale arrays" in lib.mxmoe_last_error()
+    empty = (_lib.Dim3 * 1)(_lib.Dim3(0, 256, 128))                       # no rows: nothing to launch, every check passed
+    assert lib.mxmoe_group_gemm(0, a, a, a, a, a, b, None, None, None, None, a, empty, None, q, 1, None, None) == 0
+
+
+def test_every_tile_is_run_by_exactly_one_workgroup_of_an_oversized_grid(lib):
+    """A planned launch is enqueued with a grid sized for the worst routing.  The function the kernels call to find their tile,
+    evaluated on the host over such a grid: every tile of the launch exactly once, every surplus workgroup without a tile
+    (a surplus workgroup folded back into the last phase would run one of its tiles a second time)."""
+    import random
+
+    from mxmoe_amd import _lib
+
+    rnd = random.Random(5)
+    fmts = [((4, 4, -1, True), 128), ((8, 8, -1, True), 64), ((16, 4, 128, False), 128), ((16, 16, -1, True), 32)]
+    for trial in range(30):
+        pick = rnd.sample(fmts, rnd.choice([1, 2, 3]))
+        probs = []
+        for _ in range(rnd.choice([1, 5, 60, 120])):
+            q, kmul = rnd.choice(pick)
+            probs.append(((rnd.choice([0, 1, 31, 33, 100, 129, 546, 3000]), 16 * rnd.randint(1, 200), kmul * rnd.randint(1, 20)), q))
+        if trial == 0:
+            probs = [((0, 256, 128), (4, 4, -1, True))] * 3                # a launch without any tile
+        rc, _, tiles = _plan(lib, -1, probs)
+        assert rc >= 1000
+        sizes = (_lib.Dim3 * len(probs))(*[_lib.Dim3(*p[0]) for p in probs])
+        qs = (_lib.QParams * len(probs))(*[_lib.QParams(p[1][0], p[1][1], p[1][2], int(p[1][3])) for p in probs])
+        grid = tiles + 8 * 9 + rnd.choice([0, 8, 200, 1000])
+        out = (C.c_int32 * grid)()
+        assert lib.mxmoe_group_gemm_plan_tile_map(rc - 1000, sizes, qs, len(probs), grid, out) == 0, lib.mxmoe_last_error()
+        seen = sorted(t for t in out if t >= 0)
+        assert seen == list(range(tiles)), (trial, tiles, len(seen))
 
 
 def test_kernels_are_exported_with_the_reference_function_type(lib):

@@ -355,6 +355,26 @@ def test_planned_forward_drops_out_of_range_experts_like_the_operators():
     assert torch.equal(got, want) and bool(torch.isfinite(got).all())
 
 
+def test_planned_forward_without_any_tile_after_a_forward_with_tiles():
+    """Every routed id belongs to experts this GPU does not hold and there is no shared expert: both launches have no tile.  The
+    plan buffers still hold the previous forward's tables (they are reused between calls), and the launches run with their
+    worst-case grids; the result is all zeros, as the host-planned forward gives."""
+    from mxmoe_amd import synth
+
+    cfg, layer = _small_layer(0)
+    hidden = synth.make_hidden(cfg)
+    ids, w = synth.make_routing(cfg)
+    first = layer(hidden, ids, w).clone()                               # fills the plan buffers with a real plan
+    torch.cuda.synchronize()
+    assert bool((first != 0).any())
+    away = torch.full_like(ids, cfg.num_experts + 1)
+    got = layer(hidden, away, w)
+    torch.cuda.synchronize()
+    assert torch.equal(got, torch.zeros_like(got))
+    assert torch.equal(layer.call_with_host_tables(hidden, away, w), got)
+    assert torch.equal(layer(hidden, ids, w), first)                    # and the buffers serve the next real forward
+
+
 def test_single_block_planning_writes_what_the_paired_launch_writes():
     """mxmoe_plan_block (one block per launch) against mxmoe_plan_layer (both blocks of the layer in one launch): identical plan
     buffers for the same counts."""
