@@ -40,7 +40,7 @@ def check_no_spills(remarks: str) -> None:
             name = m.group(1)
             continue
         m = re.search(r"remark:\s+VGPRs Spill: (\d+)", line)
-        if m and name and "WxAxTile" in name and int(m.group(1)) > 0:
+        if m and name and ("WxAxTile" in name or "Bf6Tile" in name) and int(m.group(1)) > 0:
             raise RuntimeError(f"{name}: {m.group(1)} vector registers spilled in a kernel with hand-tracked loads; shrink the tile's "
                                f"register ring or lower its waves per SIMD")
 
@@ -215,7 +215,7 @@ def build_default(verbose: bool = False) -> Path:
     libmxmoe_amd.so."""
     from .kernels.compose_kernel import emit_default_library
 
-    sources = sorted(CSRC.glob("*.hip")) + [emit_default_library()]
+    sources = sorted(CSRC.glob("*.hip")) + emit_default_library()
     return hipcc_build(sources, LIB, verbose=verbose)
 
 

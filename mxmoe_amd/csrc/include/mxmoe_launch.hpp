@@ -22,6 +22,7 @@
 
 #include "mxmoe_tiles.hpp"
 #include "mxmoe_grp_tiles.hpp"
+#include "mxmoe_bf6_tiles.hpp"
 #include "mxmoe_wo_tiles.hpp"
 
 namespace mxmoe {
@@ -235,6 +236,7 @@ struct BranchInfo {
   int lds_bytes;
   int k_multiple;  // K must be a multiple of this
   int max_m;       // largest M this branch accepts (skinny weight-only tiles), or 0 = any
+  int k_min = 0;   // smallest K this branch accepts, or 0 = one k_multiple
 };
 
 template <class T>
@@ -259,6 +261,15 @@ struct BranchOf<WxAxTile<OP, BM, BN>> {
   static BranchInfo get() {
     using T = WxAxTile<OP, BM, BN>;
     return BranchInfo{OP == Op::I8 ? Fmt::W8A8 : Fmt::W4A4, BM, BN, T::BK, 1, 4, T::kLdsBytes, T::BK, 0};
+  }
+};
+template <int BM>
+struct BranchOf<Bf6Tile<BM>> {
+  // same format as the int4 tiles on the int8 instruction; what differs is the layout both operands are handed over in (6-bit
+  // fragments), so the two kinds never share a kernel: the kernel a caller picks says which layout its operands have
+  static BranchInfo get() {
+    using T = Bf6Tile<BM>;
+    return BranchInfo{Fmt::W4A4, BM, T::BN, T::BK, 1, 4, T::kLdsBytes, 128, 0, 256};
   }
 };
 template <int WBITS, int BN>
@@ -547,7 +558,7 @@ inline bool kernel_covers(const FusedKernel& k, const mxmoe_qparams* q, int coun
 // K a multiple of the tile's K step, N a multiple of 8 (16 for the weight-only layouts)
 inline bool shape_ok(const BranchInfo& bi, const mxmoe_dim3& sz) {
   const bool wo = bi.fmt == Fmt::W4A16 || bi.fmt == Fmt::W3A16 || bi.fmt == Fmt::W2A16;
-  return sz.z != 0 && sz.z % bi.k_multiple == 0 && sz.y % 8 == 0 && !(wo && sz.y % 16 != 0);
+  return sz.z != 0 && sz.z % bi.k_multiple == 0 && (int)sz.z >= bi.k_min && sz.y % 8 == 0 && !(wo && sz.y % 16 != 0);
 }
 
 // Tile tables of one launch over problems [base, base + n) (n <= kMaxProblems): entries, phases, totals of `a`; *grid receives the

@@ -25,7 +25,7 @@ from itertools import product
 from pathlib import Path
 
 from .. import build as _build
-from .kernel_sketch import ABI_TU, KERNEL_DECLARATION_TEMPLATE, KERNEL_DEFINITION_TEMPLATE
+from .kernel_sketch import ABI_TU, DEFAULT_ORDER_TEMPLATE, KERNEL_DECLARATION_TEMPLATE, KERNEL_DEFERRED_TEMPLATE, KERNEL_DEFINITION_TEMPLATE
 from .tile_config import QCFG_MAP, SUPPORTED_QCFG, TileConfig, get_gpu_info, get_info_from_qcfg_str, get_possible_tile_list  # noqa: F401
 
 
@@ -128,19 +128,20 @@ class TemplateGenerator:
         return _build.hipcc_build(self.files, out)
 
 
-def build_kernel_source(tile_cfg, kname: str, kernel_type: KernelType = KernelType.Fused):
-    """(declaration comment, translation unit) of one kernel; `tile_cfg` maps qcfg -> TileConfig or tuple of TileConfig."""
+def build_kernel_source(tile_cfg, kname: str, kernel_type: KernelType = KernelType.Fused, deferred: bool = False):
+    """(declaration comment, translation unit) of one kernel; `tile_cfg` maps qcfg -> TileConfig or tuple of TileConfig.
+    `deferred`: the unit defines `register_<kname>()` instead of registering from a static initialiser."""
     pairs = [(q, t) for q, item in tile_cfg.items() for t in _flat([item])]
     tiles = ", ".join(t.cpp_type() for _, t in pairs)
     comment = "; ".join(f"{q} if {BRANCH_CONDITION_MAP[q]} -> {t.to_str()}" for q, t in pairs)
-    defn = KERNEL_DEFINITION_TEMPLATE.substitute(KernelName=kname, Tiles=tiles, Comment=comment, Policy=POLICY[str(kernel_type)])
+    defn = (KERNEL_DEFERRED_TEMPLATE if deferred else KERNEL_DEFINITION_TEMPLATE).substitute(KernelName=kname, Tiles=tiles, Comment=comment, Policy=POLICY[str(kernel_type)])
     decl = f"//   {kname}: " + ", ".join(f"[{q}: ({t.BM},{t.BN},{t.BK}) ({t.WM},{t.WN},{t.WK}) {t.STAGE}]" for q, t in pairs)
     return decl, defn
 
 
-def _pick(arch: str, qcfg: str, *shapes):
-    """Candidate tiles of `qcfg` with the given (BM, BN) shapes, in that order."""
-    by_shape = {(t.BM, t.BN): t for t in get_possible_tile_list(arch, qcfg)}
+def _pick(arch: str, qcfg: str, *shapes, bf6: bool = False):
+    """Candidate tiles of `qcfg` with the given (BM, BN) shapes, in that order (`bf6`: the tiles on the 6-bit float path)."""
+    by_shape = {(t.BM, t.BN): t for t in get_possible_tile_list(arch, qcfg) if t.is_bf6() == bf6}
     return tuple(by_shape[s] for s in shapes)
 
 
@@ -152,6 +153,8 @@ def default_kernel_specs(arch: str = "gfx950"):
     wo_all = OrderedDict((q, wo[q] + wo_big[q]) for q in wo)
     everything = OrderedDict([(w4, _pick(arch, w4, (128, 256), (32, 256))), (w8, _pick(arch, w8, (128, 256), (32, 256))),
                               ("fp16", _pick(arch, "fp16", (128, 256), (32, 256))), *wo_all.items(), ("w4a4_g128_sym", _pick(arch, "w4a4_g128_sym", (64, 256)))])
+    everything_b6 = OrderedDict(everything)
+    everything_b6[w4] = _pick(arch, w4, (128, 256), (32, 256), bf6=True)
     return [
         ("groupgemm_hz_fused_wxax", KernelType.Fused, OrderedDict([(w4, _pick(arch, w4, (128, 256), (64, 256), (32, 256))), (w8, _pick(arch, w8, (128, 256), (64, 256), (32, 256)))])),
         ("groupgemm_hz_fused_fp16", KernelType.Fused, OrderedDict([("fp16", _pick(arch, "fp16", (128, 256), (64, 256), (32, 256)))])),
@@ -161,27 +164,43 @@ def default_kernel_specs(arch: str = "gfx950"):
         ("groupgemm_hz_fused_all", KernelType.Fused, everything),
         ("groupgemm_seq_launch_all", KernelType.Sequential, everything),
         ("groupgemm_ms_launch_all", KernelType.MultiStream, everything),
+        # the same two kernels with w4a4 on the 6-bit float path: both operands of a w4a4 problem are bf6 fragments (the quantisers'
+        # tag 4, pack.pack_bf6_fragments).  Registered last: a caller that does not ask for them by name never gets them.
+        ("groupgemm_hz_fused_wxax_b6", KernelType.Fused, OrderedDict([(w4, _pick(arch, w4, (128, 256), (64, 256), (32, 256), bf6=True)), (w8, _pick(arch, w8, (128, 256), (64, 256), (32, 256)))])),
+        ("groupgemm_hz_fused_all_b6", KernelType.Fused, everything_b6),
     ]
 
 
-def emit_default_library(out_dir: str | os.PathLike | None = None, arch: str = "gfx950") -> Path:
-    """Write the translation unit that registers the default kernels (one file: the seven registrations share their tile
-    instantiations) and return its path."""
+def emit_default_library(out_dir: str | os.PathLike | None = None, arch: str = "gfx950") -> list:
+    """Write the translation units that register the default kernels, one per kernel (they compile in parallel), and return
+    their paths in registry order.  Static initialisers of different translation units run in link order, which is the order of
+    this list, so every unit registers through one ordered table instead: unit i only fills slot i, and the last step of
+    library start-up (the unit written last) registers the slots in order."""
     out_dir = Path(out_dir) if out_dir else GEN_DIR
     out_dir.mkdir(parents=True, exist_ok=True)
-    body = []
-    for kname, ktype, tile_cfg in default_kernel_specs(arch):
+    specs = default_kernel_specs(arch)
+    paths, keep = [], set()
+    for kname, ktype, tile_cfg in specs:
         for t in _flat(tile_cfg.values()):
             t.validate()
         if not is_fusion_compatible(list(tile_cfg.values())):
             raise ValueError(f"{kname}: branches disagree on the wavefront count")
-        _decl, defn = build_kernel_source(tile_cfg, kname, ktype)
-        body.append(defn.replace('#include "mxmoe_launch.hpp"\n', ""))
-    path = out_dir / "default_kernels.hip"
-    text = '#include "mxmoe_launch.hpp"\n' + "".join(body)
-    if not path.exists() or path.read_text() != text:
-        path.write_text(text)
-    return path
+        _decl, defn = build_kernel_source(tile_cfg, kname, ktype, deferred=True)
+        path = out_dir / f"default_{kname}.hip"
+        if not path.exists() or path.read_text() != defn:
+            path.write_text(defn)
+        paths.append(path)
+        keep.add(path.name)
+    order = out_dir / "default_order.hip"
+    text = DEFAULT_ORDER_TEMPLATE.substitute(Decls="\n".join(f"int register_{k}();" for k, _t, _c in specs),
+                                             Calls="\n".join(f"    register_{k}();" for k, _t, _c in specs))
+    if not order.exists() or order.read_text() != text:
+        order.write_text(text)
+    keep.add(order.name)
+    for old in out_dir.glob("default_*.hip"):
+        if old.name not in keep:
+            old.unlink()
+    return paths + [order]
 
 
 def main(argv=None) -> int:

@@ -45,9 +45,15 @@ MMA_SHAPE = {
     "MFMA_I32_32x32x32_I8": (32, 32, 32),
     "MFMA_I32_32x32x32_I8_FROM_I4": (32, 32, 32),  # int4 operands widened to int8 (16*v) in registers
     "MFMA_F32_16x16x32_F16": (16, 16, 32),
+    # int4 values held as 6-bit floats (bf6, e3m2: every integer -8 .. 8 is one) on v_mfma_scale_f32_32x32x64_f8f6f4 with unit
+    # scales: the fp32 accumulators are the exact integer sums, at twice the int8 instruction's rate
+    "MFMA_F32_32x32x64_BF6_FROM_I4": (32, 32, 64),
 }
-MMA_TO_ACC_TYPE = {"MFMA_F32_32x32x16_F16": "float", "MFMA_I32_32x32x32_I8": "int32_t", "MFMA_I32_32x32x32_I8_FROM_I4": "int32_t", "MFMA_F32_16x16x32_F16": "float"}
-MMA_TO_INP_TYPE = {"MFMA_F32_32x32x16_F16": "half", "MFMA_I32_32x32x32_I8": "int8_t", "MFMA_I32_32x32x32_I8_FROM_I4": "int4_t", "MFMA_F32_16x16x32_F16": "half"}
+MMA_TO_ACC_TYPE = {"MFMA_F32_32x32x16_F16": "float", "MFMA_I32_32x32x32_I8": "int32_t", "MFMA_I32_32x32x32_I8_FROM_I4": "int32_t", "MFMA_F32_16x16x32_F16": "float",
+                   "MFMA_F32_32x32x64_BF6_FROM_I4": "float"}
+MMA_TO_INP_TYPE = {"MFMA_F32_32x32x16_F16": "half", "MFMA_I32_32x32x32_I8": "int8_t", "MFMA_I32_32x32x32_I8_FROM_I4": "int4_t", "MFMA_F32_16x16x32_F16": "half",
+                   "MFMA_F32_32x32x64_BF6_FROM_I4": "int4_t"}
+BF6_MMA = "MFMA_F32_32x32x64_BF6_FROM_I4"
 
 QCFG_TO_MMA = {
     "fp16": "MFMA_F32_32x32x16_F16",
@@ -162,6 +168,10 @@ class TileConfig:
     def is_skinny(self) -> bool:
         return self.is_weight_only() and self.BM == 16
 
+    def is_bf6(self) -> bool:
+        """int4 operands handed over as bf6 fragments (both activations and weights; the quantisers write them, tag 4)."""
+        return self.MMA == BF6_MMA
+
     def is_group_wa(self) -> bool:
         """Both operands int4 with a scale per 128-wide K group (w4a4_g128_sym)."""
         return self.MMA == "MFMA_I32_32x32x32_I8_FROM_I4" and getattr(self.QCFGA, "GSIZE", -1) == 128
@@ -177,6 +187,8 @@ class TileConfig:
             return 2 * self.BM * 256  # two stages of BM activation rows x one 128-wide k block
         if self.is_group_wa():
             return self.STAGE * self.BM * 64
+        if self.is_bf6():  # four stages of the tile's token fragments (1536 bytes per 32 rows, rounded up to 1 KB pieces), or the epilogue patch
+            return max(4 * (-(-(self.BM // 32 * 1536) // 1024) * 1024), 4 * 32 * (64 * 2 + 16))
         if self.MMA != "MFMA_F32_32x32x16_F16":  # activations only: 3 stages of BM x 64 B, or the epilogue patch if larger
             return max(self.STAGE * self.BM * 64, 4 * min(self.BM, 64) * (64 * 2 + 8))
         return self.STAGE * (self.BM + self.BN) * 64
@@ -187,6 +199,8 @@ class TileConfig:
             return f"SkinnyWoTile<{self.QCFGB.QBITS}, {self.BN}>"
         if self.is_weight_only():
             return f"WoMfmaTile<{self.QCFGB.QBITS}, {self.BM}, {self.BN}>"
+        if self.is_bf6():
+            return f"Bf6Tile<{self.BM}>"
         op = {"MFMA_F32_32x32x16_F16": "Op::F16", "MFMA_I32_32x32x32_I8": "Op::I8", "MFMA_I32_32x32x32_I8_FROM_I4": "Op::I4"}[self.MMA]
         if self.is_group_wa():
             return f"WxAxGTile<{self.BM}>"
@@ -200,6 +214,10 @@ class TileConfig:
         if self.is_weight_only():
             if self.BK != 128 or not ((self.BM == 16 and self.BN % 64 == 0 and (self.WM, self.WN) == (1, 4)) or (self.BM, self.BN, self.WM, self.WN) in ((128, 128, 2, 2), (128, 256, 1, 4))):
                 raise ValueError(f"{self!r}: weight-only tiles are 16 x (64k) x 128 (1 x 4 waves), 128 x 128 x 128 (2 x 2 waves) or 128 x 256 x 128 (1 x 4 waves)")
+            return
+        if self.is_bf6():
+            if (self.BN, self.BK, self.WM, self.WN, self.WK, self.STAGE) != (256, 64, 1, 4, 1, 4) or self.BM not in (32, 64, 128):
+                raise ValueError(f"{self!r}: bf6 tiles are BM x 256 x 64 with 1 x 4 waves and 4 stages, BM in 32 / 64 / 128")
             return
         k_elems = {"MFMA_F32_32x32x16_F16": 32, "MFMA_I32_32x32x32_I8": 64, "MFMA_I32_32x32x32_I8_FROM_I4": 128}[self.MMA]
         if self.BK != k_elems or self.STAGE != 3 or self.WK != 1 or (self.BM // self.WM) % 32 or (self.BN // self.WN) % 32:
@@ -254,7 +272,10 @@ def get_possible_tile_list(arch: str, qcfg: str) -> list:
         shapes = [(64, 256, 1, 4), (32, 256, 1, 4)]
     else:
         shapes = [(128, 256, 1, 4), (64, 256, 1, 4), (32, 256, 1, 4)]
-    return [_with_q(TileConfig(BM=bm, BN=bn, BK=bk, WM=wm, WN=wn, WK=1, STAGE=3, MMA=mma), qcfg) for bm, bn, wm, wn in shapes]
+    tiles = [_with_q(TileConfig(BM=bm, BN=bn, BK=bk, WM=wm, WN=wn, WK=1, STAGE=3, MMA=mma), qcfg) for bm, bn, wm, wn in shapes]
+    if qcfg == "w4a4_g-1_sym":  # the same shapes on the 6-bit float path (operands as bf6 fragments): never mixed with the tiles above in one kernel
+        tiles += [_with_q(TileConfig(BM=bm, BN=256, BK=64, WM=1, WN=4, WK=1, STAGE=4, MMA=BF6_MMA), qcfg) for bm in (128, 64, 32)]
+    return tiles
 
 
 _FIELD = re.compile(r"(BM|BN|BK|WM|WN|WK|STAGE|SPLITK)=(-?\d+)")

@@ -91,3 +91,55 @@ def pack_weight_only_scales(scale: torch.Tensor, zero: torch.Tensor) -> torch.Te
     assert n % 16 == 0
     sz = torch.stack([scale.to(torch.float16), zero.to(torch.float16)], dim=-1)  # [N, G, 2]
     return sz.reshape(n // 16, 16, g, 2).permute(0, 2, 1, 3).reshape(-1).contiguous()
+
+
+# ---- int4 values as 6-bit floats (bf6, e3m2): the operand format of the w4a4 tiles on v_mfma_scale_f32_32x32x64_f8f6f4 ----
+# Every integer -8 .. 8 is a bf6 number (sign, 3 exponent bits with bias 3, 2 mantissa bits); exponent | mantissa of 0 .. 8:
+_BF6_MAGNITUDE = (0, 12, 16, 18, 20, 21, 22, 23, 24)
+BF6_FRAGMENT_BYTES = 1536
+
+
+def bf6_encode(q: torch.Tensor) -> torch.Tensor:
+    """Integers -8 .. 8 -> 6-bit bf6 codes (uint8)."""
+    if q.numel() and (int(q.min()) < -8 or int(q.max()) > 8):
+        raise ValueError("bf6 holds the integers -8 .. 8 exactly, nothing beyond")
+    mag = torch.tensor(_BF6_MAGNITUDE, dtype=torch.uint8, device=q.device)
+    return mag[q.abs().long()] | ((q < 0).to(torch.uint8) << 5)
+
+
+def bf6_decode(code: torch.Tensor) -> torch.Tensor:
+    """6-bit bf6 codes -> their values as float32 (any code, not only those of integers)."""
+    c = code.to(torch.int32)
+    e, m = (c >> 2) & 7, c & 3
+    val = torch.where(e == 0, m.float() * 0.0625, (1.0 + m.float() * 0.25) * torch.pow(2.0, (e - 3).float()))
+    return torch.where((c & 32) != 0, -val, val)
+
+
+def pack_bf6_fragments(q: torch.Tensor) -> torch.Tensor:
+    """[R, K] integers -8 .. 8 (K a multiple of 64; rows are padded with zeros to a multiple of 32) -> uint8
+    [ceil(R/32), K/64, 1536] flattened: fragments of 32 rows x 64 k, row block major.  Lane l of a fragment (row l % 32,
+    k = 64 ks + 32 (l // 32) + i) holds its 32 codes as 192 bits, value i at bit 6 i; the first 16 bytes of that string lie at byte
+    16 l of the fragment, the last 8 at byte 1024 + 8 l.  Both operands of the bf6 tiles use this layout (weights: rows = channels;
+    activations: rows = the tokens of one expert, which is what the quantisers write for tag 4)."""
+    r, k = q.shape
+    if k % 64:
+        raise ValueError("K must be a multiple of 64")
+    rb = (r + 31) // 32
+    if rb * 32 != r:
+        q = torch.cat([q, torch.zeros((rb * 32 - r, k), dtype=q.dtype, device=q.device)])
+    c = bf6_encode(q).view(rb, 32, k // 64, 2, 32).permute(0, 2, 3, 1, 4).contiguous()      # [row block, k step, k half, row, value]
+    bits = (c.unsqueeze(-1) >> torch.arange(6, device=q.device, dtype=torch.uint8)) & 1      # value i -> bits 6 i .. 6 i + 5
+    bits = bits.reshape(rb, k // 64, 64, 24, 8)                                               # lane = row + 32 * k half; 192 bits = 24 bytes
+    by = (bits << torch.arange(8, device=q.device, dtype=torch.uint8)).sum(-1).to(torch.uint8)
+    return torch.cat([by[..., :16].reshape(rb, k // 64, 1024), by[..., 16:].reshape(rb, k // 64, 512)], dim=-1).reshape(-1).contiguous()
+
+
+def unpack_bf6_fragments(frag: torch.Tensor, r: int, k: int) -> torch.Tensor:
+    """Inverse of `pack_bf6_fragments` -> float32 [r, k] (the values the codes stand for)."""
+    rb = (r + 31) // 32
+    f = frag.view(torch.uint8).reshape(rb, k // 64, 1536)
+    by = torch.cat([f[..., :1024].reshape(rb, k // 64, 64, 16), f[..., 1024:].reshape(rb, k // 64, 64, 8)], dim=-1)   # [rb, ks, lane, 24]
+    bits = ((by.unsqueeze(-1) >> torch.arange(8, device=frag.device, dtype=torch.uint8)) & 1).reshape(rb, k // 64, 64, 32, 6)
+    code = (bits << torch.arange(6, device=frag.device, dtype=torch.uint8)).sum(-1).to(torch.uint8)                  # [rb, ks, lane, value]
+    vals = bf6_decode(code).reshape(rb, k // 64, 2, 32, 32).permute(0, 3, 1, 2, 4).reshape(rb * 32, k)
+    return vals[:r].contiguous()

@@ -23,11 +23,13 @@ class PackedWeight:
         return self.data.numel() * self.data.element_size() + (0 if self.scale is None else self.scale.numel() * self.scale.element_size())
 
 
-def quantize_and_pack(w: torch.Tensor, qparams, keep_codes: bool = False) -> PackedWeight:
+def quantize_and_pack(w: torch.Tensor, qparams, keep_codes: bool = False, bf6: bool = False) -> PackedWeight:
     """RTN-quantise `w` [N, K] fp16 for `(a_bits, w_bits, gsize, sym)` and pack it.
 
     fp16: kept as is.  w8a8 / w4a4: per-channel symmetric codes (int8 / packed nibbles, K contiguous) re-ordered into MFMA
     fragment blocks (`pack.pack_wxax_fragments`), fp16 scale [N].
+    With `bf6`, w4a4 weights become bf6 fragments (`pack.pack_bf6_fragments`) for the kernels whose w4a4 tiles run on the 6-bit
+    float matrix path; every other format is unaffected.
     w4a16 / w3a16 group-128: unsigned codes in the wave-interleaved layout with a (scale, zero) table; symmetric
     variants are stored offset-binary with zero = -2^(b-1) * scale (exact).
     """
@@ -36,10 +38,10 @@ def quantize_and_pack(w: torch.Tensor, qparams, keep_codes: bool = False) -> Pac
     if w_bits >= 16:
         return PackedWeight(w.contiguous(), None, tuple(qparams), n, k)
     q, scale, zp = quant_minmax(w, w_bits, gsize, sym)
-    return pack_codes(q, scale, zp, qparams, n, k, keep_codes)
+    return pack_codes(q, scale, zp, qparams, n, k, keep_codes, bf6)
 
 
-def pack_codes(q: torch.Tensor, scale: torch.Tensor, zp: torch.Tensor, qparams, n: int, k: int, keep_codes: bool = False) -> PackedWeight:
+def pack_codes(q: torch.Tensor, scale: torch.Tensor, zp: torch.Tensor, qparams, n: int, k: int, keep_codes: bool = False, bf6: bool = False) -> PackedWeight:
     """Pack integer codes `q` [N, K] with their fp16 `scale` / `zp` (one per channel, or per channel and group; value = q * scale + zp)
     into the kernels' layouts.  Symmetric codes are signed, asymmetric ones 0 .. 2^bits - 1."""
     a_bits, w_bits, gsize, sym = qparams
@@ -53,6 +55,8 @@ def pack_codes(q: torch.Tensor, scale: torch.Tensor, zp: torch.Tensor, qparams, 
     if a_bits < 16:
         assert gsize == -1 and sym, "w-a formats are per-channel symmetric"
         qi = q.to(torch.int8)
+        if bf6 and w_bits == 4:  # for the tiles on the 6-bit float path (kernels "..._b6"): the same codes as bf6 fragments
+            return PackedWeight(pack.pack_bf6_fragments(qi.reshape(n, k)), scale.reshape(n).contiguous(), tuple(qparams), n, k, qi if keep_codes else None)
         data = pack.pack_wxax_fragments(qi if w_bits == 8 else pack.pack_int4_k(qi))
         return PackedWeight(data, scale.reshape(n).contiguous(), tuple(qparams), n, k, qi if keep_codes else None)
     assert gsize == 128, "weight-only kernels implement group size 128"

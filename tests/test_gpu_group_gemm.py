@@ -16,7 +16,8 @@ def _rel(a, b):
     return np.abs(a - b).max() / max(np.abs(b).max(), 1e-6)
 
 
-def _wxax_problem(rng, m, n, k, bits, rotate=False):
+def _wxax_problem(rng, m, n, k, bits, rotate=False, bf6=False):
+    """`bf6`: int4 operands as bf6 fragments, the layout of the kernels whose w4a4 tiles run on the 6-bit float matrix path."""
     from mxmoe_amd import pack
 
     x = rng.standard_normal((m, k)).astype(F16)
@@ -24,10 +25,13 @@ def _wxax_problem(rng, m, n, k, bits, rotate=False):
     qa, sa, _ = O.quant_minmax(x, bits, -1, True)
     qb, sb, _ = O.quant_minmax(w, bits, -1, True)
     ta, tb = torch.from_numpy(qa.astype(np.int8)), torch.from_numpy(qb.astype(np.int8))
-    if bits == 4:
-        ta, tb = pack.pack_int4_k(ta), pack.pack_int4_k(tb)
     acc = O.int_gemm(qa, qb)
-    tb = pack.pack_wxax_fragments(tb)                      # weights travel in MFMA fragment order
+    if bits == 4 and bf6:
+        ta, tb = pack.pack_bf6_fragments(ta), pack.pack_bf6_fragments(tb)
+    else:
+        if bits == 4:
+            ta, tb = pack.pack_int4_k(ta), pack.pack_int4_k(tb)
+        tb = pack.pack_wxax_fragments(tb)                  # weights travel in MFMA fragment order
     return dict(A=ta.to(DEV), B=tb.to(DEV), sa=torch.from_numpy(sa.reshape(-1)).to(DEV), sb=torch.from_numpy(sb.reshape(-1)).to(DEV),
                 acc=acc, out=O.epilogue_wxax(acc, sa.reshape(-1), sb.reshape(-1)),
                 fq=O.gemm_fakequant(O.dequant(qa, sa, 0 * sa, -1), O.dequant(qb, sb, 0 * sb, -1)),
@@ -58,6 +62,46 @@ def test_wxax_mixed_launch_bit_exact_accumulators():
         assert np.array_equal(acc, p["acc"]), f"int32 accumulators differ for {p['size']} {p['q']}"
         assert np.array_equal(out.view(np.uint16), p["out"].view(np.uint16)), f"fp16 epilogue differs for {p['size']}"
         assert _rel(out, p["fq"]) <= 1e-2                                  # tolerance of the fake-quant comparison
+
+
+@pytest.mark.parametrize("kernel", ["groupgemm_hz_fused_wxax_b6", "groupgemm_hz_fused_all_b6"])
+def test_w4a4_on_the_bf6_matrix_path_bit_exact(kernel):
+    """The kernels whose w4a4 tiles run on v_mfma_scale_f32_32x32x64_f8f6f4 (int4 values as bf6 fragments on both sides), mixed
+    with w8a8 in one launch: the accumulators are the integer products and the fp16 outputs the integer tiles' epilogue, bit for
+    bit, for ragged row counts (every tile height, segments, rows past the last block), channel counts that are no multiple of a
+    tile or of a fragment, and K from the shortest the tile takes to Qwen's and Mixtral's."""
+    from mxmoe_amd import _lib
+
+    kid = _lib.load().mxmoe_find_kernel(kernel.encode())
+    assert kid >= 0
+    rng = np.random.default_rng(21)
+    shapes = [(1, 256, 256, 4), (31, 512, 256, 8), (33, 384, 1408, 4), (130, 256, 256, 8), (300, 768, 384, 4), (64, 2816, 2048, 4),
+              (129, 2048, 1408, 8), (17, 264, 256, 4), (546, 520, 512, 4), (97, 1024, 4096, 4), (32, 256, 128 * 5, 4)]
+    probs = [_wxax_problem(rng, m, n, k, b, bf6=True) for (m, n, k, b) in shapes]
+    for rep in range(3):
+        g, outs, accs = _launch(probs, kernel_id=kid)
+        for p, out, acc in zip(probs, outs, accs):
+            assert np.array_equal(acc, p["acc"]), f"launch {rep}: accumulators differ for {p['size']} {p['q']}"
+            assert np.array_equal(out.view(np.uint16), p["out"].view(np.uint16)), f"launch {rep}: fp16 epilogue differs for {p['size']}"
+            assert _rel(out, p["fq"]) <= 1e-2
+    # extreme codes: every product at its largest magnitude, K = 14336 (sums of 64 * K stay far below 2^24)
+    m, n, k = 40, 256, 14336
+    qa = np.where(rng.random((m, k)) < 0.5, -7, 7).astype(np.int8)
+    qb = np.where(rng.random((n, k)) < 0.5, -7, 7).astype(np.int8)
+    qb[::2] = 7
+    qa[1::2] = 7
+    from mxmoe_amd import pack
+
+    one = np.ones(max(m, n), F16)
+    p = dict(A=pack.pack_bf6_fragments(torch.from_numpy(qa)).to(DEV), B=pack.pack_bf6_fragments(torch.from_numpy(qb)).to(DEV), sa=torch.from_numpy(one[:m].copy()).to(DEV),
+             sb=torch.from_numpy(one[:n].copy()).to(DEV), size=(m, n, k), q=(4, 4, -1, True))
+    _, _, accs = _launch([p], kernel_id=kid)
+    assert np.array_equal(accs[0], O.int_gemm(qa, qb))
+    # shapes the tile does not take are refused on the host
+    bad = _wxax_problem(rng, 4, 256, 256, 4, bf6=True)
+    bad["size"] = (4, 256, 128)
+    with pytest.raises(RuntimeError, match="not supported by tile"):
+        _launch([bad], kernel_id=kid)
 
 
 def test_wxax_empty_and_single_row_problems():

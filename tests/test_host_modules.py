@@ -79,6 +79,9 @@ def test_gen_workload_follows_the_reference_rules(tmp_path):
 
 def test_template_generator_product_and_sources(tmp_path):
     tiles = {q: tile_config.get_possible_tile_list("gfx950", q)[:n] for q, n in (("w4a4_g-1_sym", 3), ("w8a8_g-1_sym", 2))}
+    # w4a4 also lists the tiles on the 6-bit float path (operands as bf6 fragments); they form kernels of their own
+    b6 = [t for t in tile_config.get_possible_tile_list("gfx950", "w4a4_g-1_sym") if t.is_bf6()]
+    assert [t.cpp_type() for t in b6] == ["Bf6Tile<128>", "Bf6Tile<64>", "Bf6Tile<32>"] and all(t.validate() is None for t in b6)
     g = TemplateGenerator("gfx950", ["w8a8_g-1_sym", "w4a4_g-1_sym"], KernelType.Fused, tiles, out_dir=tmp_path)
     assert g.qcfgs == ["w4a4_g-1_sym", "w8a8_g-1_sym"]                     # sorted, as compose_kernel.py:82
     files = g.generate_source_code()
@@ -108,7 +111,11 @@ def test_default_library_is_generator_output(tmp_path, lib):
     from mxmoe_amd.kernels import compose_kernel as ck
 
     specs = ck.default_kernel_specs()
-    src = ck.emit_default_library(tmp_path).read_text()
+    files = ck.emit_default_library(tmp_path)
+    assert len(files) == len(specs) + 1                                   # one unit per kernel, and the unit that registers them in order
+    src = "".join(f.read_text() for f in files)
+    order = files[-1].read_text()
+    assert [n for n in re.findall(r"    register_(\w+)\(\);", order)] == [name for name, _t, _c in specs]
     assert lib.mxmoe_num_kernels() == len(specs)
     policy = {ck.KernelType.Fused: 0, ck.KernelType.Sequential: 1, ck.KernelType.MultiStream: 2}
     import ctypes as C
