@@ -274,6 +274,55 @@ __device__ __forceinline__ float lane_xor(float v) {
   return __int_as_float(x);
 }
 
+// ---- tag 4: per-token int4 codes written as bf6 fragments, the operand layout of the w4a4 tiles on the 6-bit float matrix path
+// (mxmoe_bf6_tiles.hpp).  Scale and codes are those of tag 2; only the storage differs: an expert's region holds ceil(rows / 32) row
+// blocks of n / 64 fragments of 1536 bytes, row block major, and local row r of the expert is lane (r % 32) + 32 (k half) of its
+// block's fragments.  Every row kernel leaves the row's codes in LDS as fp16 integers in natural order; a thread then turns 32
+// consecutive codes into one lane's 192 bits with one conversion instruction and stores them as 16 + 8 bytes.
+typedef _Float16 v32h __attribute__((ext_vector_type(32)));
+typedef unsigned v6u __attribute__((ext_vector_type(6)));
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+typedef unsigned v2u __attribute__((ext_vector_type(2)));
+
+// the eight codes of a chunk: v / scale rounded to fp16, clamped to +-7, rounded to the nearest integer (ties to even)
+template <class Div>
+__device__ __forceinline__ v8h bf6_chunk_codes(const float (&v)[8], const Div& div) {
+  v8h o;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) o[j] = (_Float16)rintf(fminf(fmaxf(round_h(div(v[j])), -7.0f), 7.0f));
+  return o;
+}
+
+// Codes of one row in LDS (fp16; value k at byte (k / row_elems) * pitch + (k % row_elems) * 2) -> the row's place in its expert's
+// fragment region.  Thread t of nt takes the groups of 32 codes t, t + nt, ...
+__device__ __forceinline__ void bf6_emit_row(const uint8_t* codes, int row_elems, int pitch, int n, uint8_t* region, long lrow, int t, int nt) {
+  const int KS = n >> 6;
+  uint8_t* blk = region + (lrow >> 5) * (long)KS * kBf6Frag;
+  const int r = (int)(lrow & 31);
+  for (int hf = t; hf < (n >> 5); hf += nt) {
+    const int k0 = hf << 5;
+    const uint8_t* src = codes + (k0 / row_elems) * pitch + (k0 % row_elems) * 2;
+    v32h c;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const v8h part = *reinterpret_cast<const v8h*>(src + q * 16);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) c[q * 8 + j] = part[j];
+    }
+    const v6u w = __builtin_amdgcn_cvt_scalef32_pk32_bf6_f16(c, 1.0f);
+    uint8_t* frag = blk + (hf >> 1) * kBf6Frag;
+    const int l = ((hf & 1) << 5) | r;
+    gstore<v4u>(frag + 16 * l, v4u{w[0], w[1], w[2], w[3]});
+    gstore<v2u>(frag + 1024 + 8 * l, v2u{w[4], w[5]});
+  }
+}
+
+// Workgroup -> group of four rows for the kernels that run one row per wave: the eight workgroups that share an XCD (workgroup id
+// modulo 8) within a run of 64 take eight consecutive groups, i.e. 32 consecutive rows.  Rows of one 32-row block of a fragment
+// region share cache lines (16 or 8 bytes per row side by side); written through one L2 they leave it as whole lines.  Needs a grid
+// that is a multiple of 64.
+__device__ __forceinline__ int xcd_row_group(int wg) { return (wg & ~63) | ((wg & 7) << 3) | ((wg >> 3) & 7); }
+
 // NT threads per workgroup (256, or 192 when that wastes fewer lanes: a 1408-element row is 176 chunks of 8).
 template <int MAXC, bool SILU, int NT>
 __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
@@ -619,6 +668,17 @@ __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
     if (scale == 0.0f) scale = 1.0f;       // quantize.cuh:258
     const ScaleDiv div(scale);
     if (tid == 0) a.scale_store[scale_off + lrow] = (_Float16)scale;
+    if (tag == 4) {  // the row's codes as fp16 in LDS (in place of the row itself, which every thread is done reading), then fragments
+      uint8_t* codes = reinterpret_cast<uint8_t*>(x);
+#pragma unroll
+      for (int i = 0; i < MAXC; ++i) {
+        const int c = tid + i * NT;
+        if (c < nchunks) *reinterpret_cast<v8h*>(codes + c * 16) = bf6_chunk_codes(v[i], div);
+      }
+      __syncthreads();
+      bf6_emit_row(codes, n, 0, n, a.inp_store + 2 * inp_off, lrow, tid, NT);
+      continue;  // (the next row begins with a barrier before it touches LDS)
+    }
     uint8_t* out = a.inp_store + 2 * (inp_off + lrow * (tag == 1 ? n / 2 : n / 4));
 #pragma unroll
     for (int i = 0; i < MAXC; ++i) {
@@ -652,12 +712,13 @@ __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
 // 512 .. n/2 between a lane's own chunks (registers).  Four independent rows per workgroup, nothing shared between them.
 template <int NI, bool SILU>
 __global__ void __launch_bounds__(256) row_quant_wave_kernel(const RowArgs a) {
+  extern __shared__ __align__(16) uint8_t wave_codes[];  // [4 waves][n] fp16: a row's codes on their way to bf6 fragments (tag 4)
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int n = a.plan.n;  // == a.plan_shared.n == 512 * NI
   const int stride_rows = gridDim.x * 4;
   const _Float16* const src_shared = shared_src(a);
-  for (int row = blockIdx.x * 4 + wave; row < a.rows; row += stride_rows) {
+  for (int row = xcd_row_group(blockIdx.x) * 4 + wave; row < a.rows; row += stride_rows) {
     if (!row_exists(a, row)) continue;
     const bool shared_row = row >= a.R;
     const int e = shared_row ? a.E : a.dst_exp[row];
@@ -783,6 +844,17 @@ __global__ void __launch_bounds__(256) row_quant_wave_kernel(const RowArgs a) {
     if (scale == 0.0f) scale = 1.0f;       // quantize.cuh:258
     const ScaleDiv div(scale);
     if (lane == 0) a.scale_store[scale_off + lrow] = (_Float16)scale;
+    if (tag == 4) {
+      uint8_t* codes = wave_codes + wave * (n * 2);
+#pragma unroll
+      for (int i = 0; i < NI; ++i) *reinterpret_cast<v8h*>(codes + (lane + 64 * i) * 16) = bf6_chunk_codes(v[i], div);
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_wave_barrier();
+      bf6_emit_row(codes, n, 0, n, a.inp_store + 2 * inp_off, lrow, lane, 64);
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_wave_barrier();  // the next row's codes come after these reads
+      continue;
+    }
     uint8_t* out = a.inp_store + 2 * (inp_off + lrow * (tag == 1 ? n / 2 : n / 4));
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
@@ -883,7 +955,7 @@ __global__ void __launch_bounds__(256) row_quant_dense_kernel(const RowArgs a) {
   const int stride_rows = gridDim.x * 4;
   RowMeta next_meta;
   v8h next_g[MAXC], next_u[MAXC];
-  const int row0 = blockIdx.x * 4 + wave;
+  const int row0 = xcd_row_group(blockIdx.x) * 4 + wave;
   if (row0 < a.rows) {
     next_meta = load_meta(row0);
     load_data(next_meta, next_g, next_u);
@@ -1086,6 +1158,19 @@ __global__ void __launch_bounds__(256) row_quant_dense_kernel(const RowArgs a) {
     if (scale == 0.0f) scale = 1.0f;       // quantize.cuh:258
     const ScaleDiv div(scale);
     if (lane == 0) a.scale_store[scale_off + lrow] = (_Float16)scale;
+    if (tag == 4) {  // codes into the wave's row buffer (its reads of the rotated row are behind a wave barrier), then fragments
+#pragma unroll
+      for (int i = 0; i < MAXC; ++i) {
+        const int c = lane + 64 * i;
+        if (c < nchunks) *reinterpret_cast<v8h*>(yrow + c * 16) = bf6_chunk_codes(v[i], div);
+      }
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_wave_barrier();
+      bf6_emit_row(yrow, n, 0, n, a.inp_store + 2 * inp_off, lrow, lane, 64);
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_wave_barrier();  // the next row's writes come after these reads
+      continue;
+    }
     uint8_t* out = a.inp_store + 2 * (inp_off + lrow * (tag == 1 ? n / 2 : n / 4));
 #pragma unroll
     for (int i = 0; i < MAXC; ++i) {
@@ -1332,6 +1417,18 @@ __global__ void __launch_bounds__(512) row_quant_wide_kernel(const RowArgs a) {
     if (scale == 0.0f) scale = 1.0f;       // quantize.cuh:258
     const ScaleDiv div(scale);
     if (tid == 0) a.scale_store[scale_off + lrow] = (_Float16)scale;
+    if (tag == 4) {  // codes into the rotated row's buffer, each wave over its own k rows, then fragments by the whole workgroup
+      __syncthreads();  // (a row that was not rotated did not pass the barriers that order the previous row's readers of this buffer)
+#pragma unroll
+      for (int i = 0; i < MAXC; ++i) {
+        const int kr = wave + 8 * i;
+        if (kr < kb) *reinterpret_cast<v8h*>(yrow + kr * kWidePitch + lane * 16) = bf6_chunk_codes(v[i], div);
+      }
+      __syncthreads();
+      bf6_emit_row(yrow, 512, kWidePitch, n, a.inp_store + 2 * inp_off, lrow, tid, 512);
+      __syncthreads();
+      continue;
+    }
     uint8_t* out = a.inp_store + 2 * (inp_off + lrow * (tag == 1 ? n / 2 : n / 4));
 #pragma unroll
     for (int i = 0; i < MAXC; ++i) {
@@ -1390,12 +1487,14 @@ static int launch_rows(const RowArgs& a, int lds_bytes, hipStream_t s) {
   // pure power-of-two rows (no table-driven Hadamard factor): one row per wave
   const int n = a.plan.n;
   if (a.plan.kb == 1 && a.plan_shared.kb == 1 && a.plan_shared.n == n && n % 512 == 0 && n <= 4096 && (n & (n - 1)) == 0) {
-    const int wgrid = (a.rows + 3) / 4 < cus * 8 ? (a.rows + 3) / 4 : cus * 8;
+    // (a multiple of 64 workgroups: xcd_row_group permutes within runs of 64)
+    const int wgrid = ((a.rows + 3) / 4 < cus * 8 ? (a.rows + 3) / 4 : cus * 8) + 63 & ~63;
+    const int wlds = 4 * n * 2;  // the waves' code rows (tag 4)
     switch (n / 512) {
-      case 1: hipLaunchKernelGGL((row_quant_wave_kernel<1, SILU>), dim3(wgrid), dim3(256), 0, s, a); break;
-      case 2: hipLaunchKernelGGL((row_quant_wave_kernel<2, SILU>), dim3(wgrid), dim3(256), 0, s, a); break;
-      case 4: hipLaunchKernelGGL((row_quant_wave_kernel<4, SILU>), dim3(wgrid), dim3(256), 0, s, a); break;
-      default: hipLaunchKernelGGL((row_quant_wave_kernel<8, SILU>), dim3(wgrid), dim3(256), 0, s, a); break;
+      case 1: hipLaunchKernelGGL((row_quant_wave_kernel<1, SILU>), dim3(wgrid), dim3(256), wlds, s, a); break;
+      case 2: hipLaunchKernelGGL((row_quant_wave_kernel<2, SILU>), dim3(wgrid), dim3(256), wlds, s, a); break;
+      case 4: hipLaunchKernelGGL((row_quant_wave_kernel<4, SILU>), dim3(wgrid), dim3(256), wlds, s, a); break;
+      default: hipLaunchKernelGGL((row_quant_wave_kernel<8, SILU>), dim3(wgrid), dim3(256), wlds, s, a); break;
     }
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
@@ -1406,7 +1505,7 @@ static int launch_rows(const RowArgs& a, int lds_bytes, hipStream_t s) {
   }
   // table-driven factor times H_8, one size of row: one row per wave, dense stage on the matrix cores
   if (a.plan.kb > 1 && a.plan.m == 8 && a.plan.f <= 4 && a.plan.kb <= 64 && n <= 2048 && a.plan_shared.n == n && a.plan_shared.kb == a.plan.kb && a.rotate != 0) {
-    const int wgrid = (a.rows + 3) / 4 < cus * 4 ? (a.rows + 3) / 4 : cus * 4;
+    const int wgrid = ((a.rows + 3) / 4 < cus * 4 ? (a.rows + 3) / 4 : cus * 4) + 63 & ~63;
     const int dlds = 4 * kDenseWaveLds;
     switch ((n / 8 + 63) / 64) {
       case 1: hipLaunchKernelGGL((row_quant_dense_kernel<1, SILU>), dim3(wgrid), dim3(256), dlds, s, a); break;

@@ -545,7 +545,15 @@ int register_fused(const char* fn_name, Policy policy = Policy::Fused) {
   return id;
 }
 
-// A kernel can run a problem list when it has a branch for every format in it.
+// Whether the kernel's w4a4 tiles run on the 6-bit float matrix path, i.e. take both operands as bf6 fragments.
+inline bool kernel_takes_bf6(const FusedKernel& k) {
+  for (const BranchInfo& b : k.branches)
+    if (b.fmt == Fmt::W4A4 && b.BK == 64) return true;
+  return false;
+}
+
+// A kernel can run a problem list when it has a branch for every format in it.  The automatic choice (kernel_id = -1) never
+// falls on a kernel that takes bf6 fragments: QParams do not say how the operands are laid out, so those kernels are asked for by id.
 inline bool kernel_covers(const FusedKernel& k, const mxmoe_qparams* q, int count) {
   for (int i = 0; i < count; ++i) {
     const Fmt f = classify(q[i]);
@@ -683,7 +691,7 @@ inline int group_gemm(int kernel_id, const void* const* As, const void* const* B
   auto& reg = registry();
   if (kernel_id < 0) {
     for (int i = 0; i < (int)reg.size() && kernel_id < 0; ++i)
-      if (reg[i].policy == Policy::Fused && kernel_covers(reg[i], h_q, count)) kernel_id = i;
+      if (reg[i].policy == Policy::Fused && !kernel_takes_bf6(reg[i]) && kernel_covers(reg[i], h_q, count)) kernel_id = i;
     if (kernel_id < 0) {
       last_error() = "quant type not supported";  // same message as the reference launcher (compose_kernel.py:433)
       return 1;

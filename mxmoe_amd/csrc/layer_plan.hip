@@ -14,9 +14,14 @@
 
 namespace mxmoe {
 
+// A block descriptor (not the QParams arrays of the launcher, whose padding bytes belong to the caller) may ask for the int4 codes of
+// per-token activations as bf6 fragments, the operand layout of the kernels whose w4a4 tiles run on the 6-bit float matrix path.
+__host__ __device__ inline bool wants_bf6(const mxmoe_qparams& q) { return q._pad[0] == 1 && q.a_bits == 4 && q.w_bits == 4 && q.gsize == -1; }
+
 __host__ __device__ inline int act_tag_of(const mxmoe_qparams& q) {  // ref_bind.cu:461-473
   if (q.a_bits >= 16) return 0;
   if (q.a_bits == 8 && q.gsize == -1) return 1;
+  if (wants_bf6(q)) return 4;
   if (q.a_bits == 4 && q.gsize == -1) return 2;
   if (q.a_bits == 4 && q.gsize == 128) return 3;
   return -1;
@@ -88,14 +93,16 @@ __global__ void __launch_bounds__(kPlanThreads) plan_block_kernel(const PlanPair
     fmt = fmt_of(d.q);
     N = (int)d.N;
     K = (int)d.K;
-    qld = tag == 0 ? K : (tag == 1 ? K / 2 : K / 4);  // fp16 elements per packed activation row (ref_bind.cu:491)
+    qld = tag == 0 ? K : (tag == 1 ? K / 2 : K / 4);  // fp16 elements per packed activation row (ref_bind.cu:491); unused for tag 4
     sld = tag == 0 ? 0 : (tag == 3 ? K / 128 : 1);   // scales per row (ref_bind.cu:492)
     out_ld = N;
   }
   // exclusive sums over the experts before this one
   long tot[4], routed_tot;
   long first_row = wave_excl_scan(rows, lane, &tot[0]);
-  long inp_off = wave_excl_scan(qld * rows, lane, &tot[1]);
+  // packed activations of the expert, in fp16 elements: rows of qld elements, or (tag 4) whole blocks of 32 rows of K / 64 fragments
+  const long inp_elems = tag == 4 ? ((rows + 31) >> 5) * (long)(K >> 6) * (kBf6Frag / 2) : qld * rows;
+  long inp_off = wave_excl_scan(inp_elems, lane, &tot[1]);
   long sc_off = wave_excl_scan(sld * rows, lane, &tot[2]);
   long out_off = wave_excl_scan(out_ld * rows, lane, &tot[3]);
   wave_excl_scan(e < p.E ? rows : 0, lane, &routed_tot);
@@ -259,6 +266,8 @@ static int resolve_kernel(int kernel_id, const mxmoe_block_desc* h_desc, int et)
       Segment sg[2];
       const int f = fmt_of(h_desc[i].q);
       if (f == (int)Fmt::UNSUPPORTED || plan_segments(plan_of(k), f, 1, 256, sg) < 0) return false;
+      // a kernel's w4a4 tiles take packed int4 rows or bf6 fragments, never both: the descriptor says which the block will get
+      if (f == (int)Fmt::W4A4 && kernel_takes_bf6(k) != wants_bf6(h_desc[i].q)) return false;
     }
     return true;
   };

@@ -18,10 +18,14 @@ from .weights import quantize_and_pack
 
 
 class MxMoELayer:
-    def __init__(self, cfg: MoEConfig, device="cuda", formats=None, weights=None, keep_codes: bool = False, packed=None):
+    def __init__(self, cfg: MoEConfig, device="cuda", formats=None, weights=None, keep_codes: bool = False, packed=None, bf6: bool = False):
         """weights: [(W13, W2)] fp16 per expert (default: the configuration's seeded synthetic weights); packed: ([PackedWeight] for
-        gate_up, [PackedWeight] for down) already quantised and packed, e.g. from `checkpoint.load_layer` (formats are taken from them)."""
+        gate_up, [PackedWeight] for down) already quantised and packed, e.g. from `checkpoint.load_layer` (formats are taken from them).
+        bf6: run the w4a4 blocks on the 6-bit float matrix path: their weights are packed as bf6 fragments, the quantisers write their
+        activations as bf6 fragments (tag 4) and both launches use a kernel whose w4a4 tiles take that layout.  Same integer codes, same
+        accumulators and outputs, bit for bit; the operands occupy 0.75 instead of 0.5 bytes per value."""
         self.cfg = cfg
+        self.bf6 = bool(bf6)
         self.device = torch.device(device)
         self.n_exp_total = cfg.num_experts + (1 if cfg.num_shared else 0)
         if packed is not None:
@@ -37,10 +41,12 @@ class MxMoELayer:
         for e in range(self.n_exp_total if packed is None else 0):
             w13, w2 = weights[e] if weights is not None else expert_weights(cfg, e)
             gu, dn = self.formats[e]
-            self.w13.append(quantize_and_pack(w13.to(self.device), gu, keep_codes))
-            self.w2.append(quantize_and_pack(w2.to(self.device), dn, keep_codes))
+            self.w13.append(quantize_and_pack(w13.to(self.device), gu, keep_codes, bf6=self.bf6))
+            self.w2.append(quantize_and_pack(w2.to(self.device), dn, keep_codes, bf6=self.bf6))
         self.qp_gate_up = [f[0] for f in self.formats]
         self.qp_down = [f[1] for f in self.formats]
+        self.kid_gate_up = ops.select_kernel(self.qp_gate_up, self.bf6)
+        self.kid_down = ops.select_kernel(self.qp_down, self.bf6)
         self.state = None
         self._static = None
 
@@ -56,11 +62,11 @@ class MxMoELayer:
         topk_ids = topk_ids.to(self.device)
         st = {}
         (st["inp"], st["sa"], st["mid"], st["inp_store"], st["sa_store"], st["mid_store"], st["recv"], st["perm"], st["dst"]) = ops.quant_inp_act(
-            hidden, topk_ids, cfg.num_experts, cfg.inter, cfg.num_shared, self.qp_gate_up, rotate=cfg.rotate)
+            hidden, topk_ids, cfg.num_experts, cfg.inter, cfg.num_shared, self.qp_gate_up, rotate=cfg.rotate, bf6=self.bf6)
         i_sh = cfg.inter * max(cfg.num_shared, 1)
         acc1 = [torch.zeros(m.shape, dtype=torch.int32, device=self.device) for m in st["mid"]] if dump_acc else None
         st["gg1"] = ops.prepare_gg(st["inp"], [w.data for w in self.w13], st["sa"], [w.scale for w in self.w13], st["mid"], 2 * cfg.inter, cfg.hidden,
-                                   2 * i_sh, cfg.hidden, self.qp_gate_up, st["recv"], acc_dump=acc1)
+                                   2 * i_sh, cfg.hidden, self.qp_gate_up, st["recv"], kernel_id=self.kid_gate_up, acc_dump=acc1)
         st["acc1"] = acc1
         st["dump_acc"] = dump_acc
         st["hidden"], st["topk_ids"] = hidden, topk_ids
@@ -74,11 +80,11 @@ class MxMoELayer:
         cfg, st = self.cfg, self.state
         (st["inp2"], st["sa2"], st["out"], st["inp2_store"], st["sa2_store"], st["out_store"]) = ops.silu_mul_then_quant(
             st["mid_store"], len(st["mid"]), cfg.num_experts, cfg.hidden, cfg.inter, cfg.num_shared, cfg.tokens, cfg.topk, st["dst"], st["recv"],
-            self.qp_down, rotate=cfg.rotate)
+            self.qp_down, rotate=cfg.rotate, bf6=self.bf6)
         i_sh = cfg.inter * max(cfg.num_shared, 1)
         acc2 = [torch.zeros(o.shape, dtype=torch.int32, device=self.device) for o in st["out"]] if st["dump_acc"] else None
         st["gg2"] = ops.prepare_gg(st["inp2"], [w.data for w in self.w2], st["sa2"], [w.scale for w in self.w2], st["out"], cfg.hidden, cfg.inter,
-                                   cfg.hidden, i_sh, self.qp_down, st["recv"], acc_dump=acc2)
+                                   cfg.hidden, i_sh, self.qp_down, st["recv"], kernel_id=self.kid_down, acc_dump=acc2)
         st["acc2"] = acc2
 
     def down(self):
@@ -112,7 +118,7 @@ class MxMoELayer:
             def ptrs(ws):
                 return [w.data.data_ptr() for w in ws], [0 if w.scale is None else w.scale.data_ptr() for w in ws]
 
-            self._static = (LT.static_block(self.qp_gate_up, gu_w, gu_n, *ptrs(self.w13)), LT.static_block(self.qp_down, dn_w, dn_n, *ptrs(self.w2)))
+            self._static = (LT.static_block(self.qp_gate_up, gu_w, gu_n, *ptrs(self.w13), bf6=self.bf6), LT.static_block(self.qp_down, dn_w, dn_n, *ptrs(self.w2), bf6=self.bf6))
         return self._static
 
     # ---- the forward that never waits for its routing ---------------------------------------------------------
@@ -138,7 +144,8 @@ class MxMoELayer:
             h = (_lib.BlockDesc * et)()
             for e in range(et):
                 a, w, g, sym = qps[e]
-                h[e] = _lib.BlockDesc(int(a), int(w), int(g), 1 if sym else 0, (C.c_uint8 * 3)(), int(ns[e]), int(ks[e]), ws[e].data.data_ptr(),
+                layout = (C.c_uint8 * 3)(1 if self.bf6 and (int(a), int(w), int(g)) == (4, 4, -1) else 0, 0, 0)  # 1: activations as bf6 fragments
+                h[e] = _lib.BlockDesc(int(a), int(w), int(g), 1 if sym else 0, layout, int(ns[e]), int(ks[e]), ws[e].data.data_ptr(),
                                       0 if ws[e].scale is None else ws[e].scale.data_ptr())
             d = torch.frombuffer(bytearray(bytes(h)), dtype=torch.uint8).to(dev)
             kid = lib.mxmoe_plan_select_kernel(-1, h, et)
@@ -148,11 +155,13 @@ class MxMoELayer:
             if grid < 0:
                 raise RuntimeError(lib.mxmoe_last_error().decode())
             # worst-case stores: every routed row as wide as the widest routed expert's packed row
-            tags = [ops.act_tag(int(q[0]), int(q[2])) for q in qps]
-            qld = [k if tg == 0 else (k // 2 if tg == 1 else k // 4) for tg, k in zip(tags, ks)]
+            tags = [ops.act_tag(int(q[0]), int(q[2]), self.bf6 and int(q[1]) == 4) for q in qps]
+            # fp16 elements per row; bf6 fragments (tag 4) take 3/8 of an element per value and whole blocks of 32 rows per expert
+            qld = [k * 3 // 8 if tg == 4 else (k if tg == 0 else (k // 2 if tg == 1 else k // 4)) for tg, k in zip(tags, ks)]
             sld = [0 if tg == 0 else (k // 128 if tg == 3 else 1) for tg, k in zip(tags, ks)]
             sh = [e_cnt] if has_shared else []
-            inp = 2 * (max(qld[:e_cnt]) * r_cap + sum(qld[e] * shared_rows for e in sh))
+            pad = 32 * e_cnt if 4 in tags else 0
+            inp = 2 * (max(qld[:e_cnt]) * (r_cap + pad) + sum(qld[e] * (shared_rows + 31) // 32 * 32 for e in sh))
             sc = 2 * (max(sld[:e_cnt]) * r_cap + sum(sld[e] * shared_rows for e in sh))
             out = 2 * (max(ns[:e_cnt]) * r_cap + sum(ns[e] * shared_rows for e in sh))
             return {"h": h, "d": d, "kid": kid, "grid": grid, "plan": u8(lib.mxmoe_plan_bytes(et)), "inp": u8(inp), "scale": u8(sc), "out_bytes": out}
@@ -273,20 +282,20 @@ class MxMoELayer:
                 raise RuntimeError("routed and shared intermediate sizes need the same Hadamard order")
             return hk, hf, None if sg is None else sg.data_ptr()
 
-        def launch(ptr_off, sizes_off, h_sizes, h_q):
+        def launch(ptr_off, sizes_off, h_sizes, h_q, kid):
             row = lambda i: base + ptr_off + i * count * 8  # noqa: E731
-            _lib.check(lib, lib.mxmoe_group_gemm(-1, row(0), row(1), row(2), row(3), row(4), row(4), None, None, None, None, base + sizes_off,
+            _lib.check(lib, lib.mxmoe_group_gemm(kid, row(0), row(1), row(2), row(3), row(4), row(4), None, None, None, None, base + sizes_off,
                                                  h_sizes.ctypes.data_as(C.POINTER(_lib.Dim3)), None, h_q.ctypes.data_as(C.POINTER(_lib.QParams)), count, None, stream))
 
         hk, hf, sg = signs(cfg.hidden, cfg.hidden)
         _lib.check(lib, lib.mxmoe_quant_act(hidden.data_ptr(), inp1.data_ptr(), sa1.data_ptr(), dst.data_ptr(), perm.data_ptr(), base + off[0],
                                             cfg.hidden, routed, t, e_cnt, int(has_shared), cfg.rotate, hk, hf, sg, stream))
-        launch(off[2], off[4], s1, q1)
+        launch(off[2], off[4], s1, q1, self.kid_gate_up)
         i_sh = cfg.inter * max(cfg.num_shared, 1)
         hk, hf, sg = signs(cfg.inter, i_sh)
         _lib.check(lib, lib.mxmoe_silu_mul_quant(mid.data_ptr(), mid.data_ptr() + routed * 2 * cfg.inter * 2, inp2.data_ptr(), sa2.data_ptr(), dst.data_ptr(), base + off[1],
                                                  cfg.inter, i_sh, routed, t, e_cnt, int(has_shared), cfg.rotate, hk, hf, sg, stream))
-        launch(off[3], off[5], s2, q2)
+        launch(off[3], off[5], s2, q2, self.kid_down)
         ws = torch.empty(lib.mxmoe_combine_workspace_bytes(t, topk), dtype=torch.uint8, device=dev)
         shared_ptr = out.data_ptr() + routed * cfg.hidden * 2 if has_shared else None
         _lib.check(lib, lib.mxmoe_unpermute_combine(out.data_ptr(), shared_ptr, w.data_ptr(), slot.data_ptr(), routed, t, topk, cfg.hidden, final.data_ptr(), ws.data_ptr(), stream))

@@ -21,14 +21,14 @@ def _oracle_block(x, w, qp, rotate_mode):
     return O.linear_block(x, w, qp, rot) if qp[0] < 16 else O.linear_block(O.online_hadamard(x) if rot else x, w, qp, False)
 
 
-def _run(cfg, formats):
+def _run(cfg, formats, bf6=False):
     from mxmoe_amd import synth
     from mxmoe_amd.layer import MxMoELayer
 
     hidden = synth.make_hidden(cfg)
     ids, _ = synth.make_routing(cfg)
     weights = [synth.expert_weights(cfg, e) for e in range(cfg.num_experts + (1 if cfg.num_shared else 0))]
-    layer = MxMoELayer(cfg, formats=formats, weights=weights)
+    layer = MxMoELayer(cfg, formats=formats, weights=weights, bf6=bf6)
     outs = layer.forward(hidden, ids, dump_acc=True)
     torch.cuda.synchronize()
     st = layer.state
@@ -56,12 +56,14 @@ def _run(cfg, formats):
     return results
 
 
-def test_wxax_layer_is_bit_exact_end_to_end():
+@pytest.mark.parametrize("bf6", [False, True])
+def test_wxax_layer_is_bit_exact_end_to_end(bf6):
+    """bf6: the w4a4 blocks on the 6-bit float matrix path (weights and activations as bf6 fragments): the same bits."""
     from mxmoe_amd import synth
 
-    cfg = synth.MoEConfig("t", "test", 5, 2, 256, 1408, 40, num_shared=0, rotate=1)
+    cfg = synth.MoEConfig("t", "test", 5, 2, 256, 1408, 40 if not bf6 else 150, num_shared=0, rotate=1)
     fm = [(synth.W4A4, synth.W8A8), (synth.W8A8, synth.W4A4), (synth.W4A4, synth.W4A4), (synth.W8A8, synth.W8A8), (synth.W4A4, synth.W8A8)]
-    for r in _run(cfg, fm):
+    for r in _run(cfg, fm, bf6):
         assert np.array_equal(r["g_acc1"], r["acc1"]), f"gate_up accumulators, expert {r['e']}"
         assert np.array_equal(r["g_mid"].view(np.uint16), r["mid"].view(np.uint16)), f"gate_up fp16, expert {r['e']}"
         assert np.array_equal(r["g_acc2"], r["acc2"]), f"down accumulators, expert {r['e']}"
@@ -247,7 +249,7 @@ def test_layer_from_fake_quantised_weights_is_their_function(tmp_path):
     assert err2 > 3 * err, (err, err2)
 
 
-def _small_layer(num_shared=1, rotate=1):
+def _small_layer(num_shared=1, rotate=1, bf6=False):
     from mxmoe_amd import synth
     from mxmoe_amd.layer import MxMoELayer
 
@@ -255,7 +257,7 @@ def _small_layer(num_shared=1, rotate=1):
     g = synth.W4A4G128
     fm = [(synth.W4A4, synth.W8A8), (synth.W8A8, synth.W4A4), (g, g), (synth.W4A16, synth.W3A16), (synth.FP16, synth.FP16), (synth.W4A4, synth.W4A4),
           (synth.W8A8, synth.W8A8)][: 6 + (1 if num_shared else 0)]
-    return cfg, MxMoELayer(cfg, formats=fm)
+    return cfg, MxMoELayer(cfg, formats=fm, bf6=bf6)
 
 
 @pytest.mark.parametrize("num_shared", [0, 1])
@@ -373,6 +375,29 @@ def test_planned_forward_without_any_tile_after_a_forward_with_tiles():
     assert torch.equal(got, torch.zeros_like(got))
     assert torch.equal(layer.call_with_host_tables(hidden, away, w), got)
     assert torch.equal(layer(hidden, ids, w), first)                    # and the buffers serve the next real forward
+
+
+@pytest.mark.parametrize("num_shared", [0, 1])
+def test_layer_on_the_bf6_matrix_path_gives_the_same_bits_in_every_form(num_shared):
+    """A layer whose w4a4 blocks run on the 6-bit float matrix path (every format in one layer, so the mixed kernel): stepwise
+    operators, host-planned forward, device-planned forward and the layer without bf6 all return identical outputs."""
+    from mxmoe_amd import synth
+
+    cfg, plain = _small_layer(num_shared)
+    _, layer = _small_layer(num_shared, bf6=True)
+    assert layer.kid_gate_up >= 0 and layer.kid_down >= 0 and plain.kid_gate_up == -1
+    hidden = synth.make_hidden(cfg)
+    ids, w = synth.make_routing(cfg)
+    ids[5:40, 0] = 5                                                    # a w4a4 expert with more than one block of rows
+    plain.forward(hidden, ids)
+    want = plain.combine(w).clone()
+    layer.forward(hidden, ids)
+    assert torch.equal(layer.combine(w), want)
+    assert torch.equal(layer.call_with_host_tables(hidden, ids, w), want)
+    assert torch.equal(layer(hidden, ids, w), want)
+    ids2 = torch.where(ids == 0, torch.full_like(ids, 1), ids)          # another routing through the same buffers
+    plain.forward(hidden, ids2)
+    assert torch.equal(layer(hidden, ids2, w), plain.combine(w))
 
 
 def test_single_block_planning_writes_what_the_paired_launch_writes():

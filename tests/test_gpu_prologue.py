@@ -170,6 +170,91 @@ def test_silu_mul_then_quant_bit_exact(n, n_sh, rotate):
         p += 1
 
 
+def _bf6_rows(view, m, k):
+    """Codes of the m rows of an expert whose activations were written as bf6 fragments (tag 4)."""
+    from mxmoe_amd import pack
+
+    return pack.unpack_bf6_fragments(view.contiguous().view(torch.uint8).reshape(-1), m, k).cpu().numpy().astype(np.int8)
+
+
+@pytest.mark.parametrize("k,rotate", [(2048, 1), (4096, 1), (256, 0), (1408, 1), (14336, 1), (2816, 2), (512, 2), (8192, 1)])
+def test_quant_inp_act_writes_int4_codes_as_bf6_fragments(k, rotate):
+    """With bf6=True the per-token int4 experts get their codes as bf6 fragments (the operand layout of the tiles on the 6-bit float
+    matrix path): same scales and the same codes as the packed rows, value for value, in every row kernel (one row per wave with and
+    without the dense stage, wide rows, the general kernel); rows per expert straddle the 32-row blocks; other formats are untouched."""
+    from mxmoe_amd import ops
+
+    rng = np.random.default_rng(k + rotate)
+    t, e, topk, n_sh = 70, 5, 2, 1
+    x = rng.standard_normal((t, k)).astype(F16)
+    x[3] = 0
+    ids = _ids(rng, t, e, topk)
+    qp = [(4, 4, -1, True), (8, 8, -1, True), (4, 4, -1, True), (16, 16, -1, True), (4, 4, -1, True), (4, 4, -1, True)]
+    res = ops.quant_inp_act(torch.from_numpy(x).to(DEV), torch.from_numpy(ids).to(DEV), e, 1408, n_sh, qp, rotate=rotate, bf6=True)
+    inp_list, scale_list = res[:2]
+    torch.cuda.synchronize()
+    _, o_perm, _, o_recv = O.permute_by_expert(ids, e)
+    p = st = 0
+    for ex in range(e + 1):
+        m = t if ex == e else int(o_recv[ex])
+        if m == 0:
+            continue
+        rows = x if ex == e else x[o_perm[st:st + m]]
+        if ex < e:
+            st += m
+        a_bits = qp[ex][0]
+        tag = O.act_tag(a_bits, qp[ex][2])
+        xr = O.online_hadamard(rows) if rotate == 2 or (rotate == 1 and tag != 0) else rows
+        got = inp_list[p]
+        if tag == 0:
+            assert np.array_equal(got.cpu().numpy().view(np.uint16), xr.view(np.uint16))
+        else:
+            q, s, _ = O.quant_minmax(xr, a_bits, -1, True)
+            assert np.array_equal(scale_list[p].cpu().numpy().view(np.uint16), s.reshape(-1).view(np.uint16)), f"expert {ex} scales"
+            if a_bits == 4:
+                assert got.shape == (-(-m // 32) * 32, k * 3 // 8)
+                assert np.array_equal(_bf6_rows(got, m, k), q.astype(np.int8)), f"expert {ex} codes"
+            else:
+                assert np.array_equal(_unpack(got, tag, k), q.astype(np.int8)), f"expert {ex} codes"
+        p += 1
+    assert p == len(inp_list)
+
+
+@pytest.mark.parametrize("n,n_sh,rotate", [(1408, 2, 1), (2048, 0, 1), (14336, 0, 1), (512, 1, 0)])
+def test_silu_mul_then_quant_writes_bf6_fragments(n, n_sh, rotate):
+    from mxmoe_amd import ops
+
+    rng = np.random.default_rng(n + 7)
+    t, e, topk = 40, 4, 2
+    ids = _ids(rng, t, e, topk)
+    o_dst, _, _, o_recv = O.permute_by_expert(ids, e)
+    gu = (rng.standard_normal((t * topk, 2 * n)) * 2).astype(F16)
+    gu_sh = (rng.standard_normal((t, 2 * n * max(n_sh, 1))) * 2).astype(F16)
+    flat = np.concatenate([gu.reshape(-1), gu_sh.reshape(-1)]) if n_sh else gu.reshape(-1)
+    qp = [(4, 4, -1, True), (8, 8, -1, True), (4, 4, -1, True), (4, 4, -1, True), (4, 4, -1, True)]
+    res = ops.silu_mul_then_quant(torch.from_numpy(flat).to(DEV), int((o_recv != 0).sum()), e, 2048, n, n_sh, t, topk,
+                                  torch.from_numpy(o_dst).to(DEV), torch.from_numpy(o_recv), qp, rotate=rotate, bf6=True)
+    inp_list, scale_list = res[:2]
+    torch.cuda.synchronize()
+    p = st = 0
+    for ex in range(e + (1 if n_sh else 0)):
+        m = t if ex == e else int(o_recv[ex])
+        if m == 0:
+            continue
+        src = gu_sh if ex == e else gu[st:st + m]
+        if ex < e:
+            st += m
+        y = O.silu_mul(src)
+        if rotate:
+            y = O.online_hadamard(y)
+        q, s, _ = O.quant_minmax(y, qp[ex][0], -1, True)
+        assert np.array_equal(scale_list[p].cpu().numpy().view(np.uint16), s.reshape(-1).view(np.uint16)), f"expert {ex} scales"
+        got = inp_list[p]
+        codes = _bf6_rows(got, m, y.shape[1]) if qp[ex][0] == 4 else _unpack(got, 1, y.shape[1])
+        assert np.array_equal(codes, q.astype(np.int8)), f"expert {ex} codes"
+        p += 1
+
+
 def test_unsupported_activation_format():
     from mxmoe_amd import ops
 
