@@ -24,7 +24,7 @@ PEAK = {"int8": 5000.0, "fp16": 2500.0, "fp6": 10100.0, "hbm": 8000.0}  # MI355X
 TRAFFIC = {"c1": 727583767, "c2": 557234807, "c3": 685202780, "c4": 202350701, "c5": 5812150537}
 
 
-def build_layer(name: str, tokens: int | None):
+def build_layer(name: str, tokens: int | None, bf6=False):
     import torch
 
     from mxmoe_amd import synth
@@ -33,7 +33,7 @@ def build_layer(name: str, tokens: int | None):
     cfg = synth.get_config(name, tokens)
     hidden = synth.make_hidden(cfg)
     ids, _ = synth.make_routing(cfg)
-    layer = MxMoELayer(cfg)
+    layer = MxMoELayer(cfg, bf6=bf6)
     layer.prepare(hidden, ids)
     layer.gate_up()
     layer.act()
@@ -346,8 +346,8 @@ def bf6_probe(dims: str):
     return res
 
 
-def run_workload(name: str, steps: int, warmup: int, tokens=None, whole: bool = True):
-    cfg, layer = build_layer(name, tokens)
+def run_workload(name: str, steps: int, warmup: int, tokens=None, whole: bool = True, bf6=False):
+    cfg, layer = build_layer(name, tokens, bf6)
     ms, up, dn = time_layer(layer, steps, warmup)
     ops = layer.gemm_ops()
     st = layer.state
@@ -368,6 +368,9 @@ def main() -> int:
     ap.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c4", "c5"])
     ap.add_argument("--also", default="c2,c4", help="comma-separated extra workloads reported under 'also' (empty to skip)")
     ap.add_argument("--tokens", type=int, default=None)
+    ap.add_argument("--w4a4-path", default="int8", choices=["bf6", "int8", "bf6-down"],
+                    help="matrix instruction of the w4a4 blocks: int8 = v_mfma_i32_32x32x32_i8 on codes widened in registers, bf6 = "
+                         "v_mfma_scale_f32_32x32x64_f8f6f4 on int4 values held as 6-bit floats (exact), bf6-down = bf6 for the down blocks only")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-whole-layer", action="store_true", help="skip the wall-clock timing of the whole forward (profiling runs: the trace then ends with the launches the roofline entry is measured on)")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="BYTES",
@@ -410,16 +413,26 @@ def main() -> int:
         return 0
     from mxmoe_amd import synth
 
-    cfg, layer, main_res = run_workload(args.workload, args.steps, args.warmup, args.tokens, not args.no_whole_layer)
+    bf6 = {"int8": False, "bf6": True, "bf6-down": (False, True)}[args.w4a4_path]
+    cfg, layer, main_res = run_workload(args.workload, args.steps, args.warmup, args.tokens, not args.no_whole_layer, bf6)
     also = {}
     del layer
     torch.cuda.empty_cache()
     for extra in [w for w in args.also.split(",") if w and w != args.workload]:
-        _, lay, res = run_workload(extra, max(10, args.steps // 2), max(5, args.warmup // 2), whole=not args.no_whole_layer)
+        _, lay, res = run_workload(extra, max(10, args.steps // 2), max(5, args.warmup // 2), whole=not args.no_whole_layer, bf6=bf6)
         also[extra] = res
         del lay
         torch.cuda.empty_cache()
 
+    # the same workload with its w4a4 blocks on the other matrix instruction (same codes, same results bit for bit), for comparison
+    alt = None
+    if any(tuple(q) == synth.W4A4 for f in synth.draw_formats(cfg) for q in f) and args.tokens is None:
+        other = "int8" if args.w4a4_path != "int8" else "bf6"
+        _, lay, res = run_workload(args.workload, max(10, args.steps // 2), max(5, args.warmup // 2), whole=False, bf6=other == "bf6")
+        alt = {"w4a4_path": other, **{k: res[k] for k in ("tops", "ms_per_step", "gate_up_us", "down_us")},
+               "gate_up_launch_us": res["roofline"]["launch_us"], "down_launch_us": res["roofline_other_launch"]["launch_us"]}
+        del lay
+        torch.cuda.empty_cache()
     fm = sorted({synth.qcfg_str(q) for f in synth.draw_formats(cfg) for q in f})
     out = {
         "metric": "GroupGEMM TOPS, Qwen1.5-MoE layer bs=8192" if args.workload in ("c2", "c3") else f"GroupGEMM TOPS, {cfg.description}",
@@ -437,7 +450,8 @@ def main() -> int:
         "config": {"workload": f"{args.workload}: {cfg.description}", "experts": cfg.num_experts, "topk": cfg.topk, "hidden": cfg.hidden,
                    "intermediate": cfg.inter, "tokens": cfg.tokens, "formats": fm, "step": "gate_up GroupGEMM launch + down GroupGEMM launch"},
         "roofline": main_res["roofline"],
-        "detail": {k: main_res[k] for k in ("gate_up_us", "down_us", "gate_up_tops", "down_tops", "ops", "whole_layer", "roofline_other_launch")},
+        "detail": {**{k: main_res[k] for k in ("gate_up_us", "down_us", "gate_up_tops", "down_tops", "ops", "whole_layer", "roofline_other_launch")},
+                   "w4a4_path": args.w4a4_path, "other_w4a4_path": alt},
         "also": also,
     }
     if not args.no_cpu_baseline:

@@ -22,10 +22,11 @@ class MxMoELayer:
         """weights: [(W13, W2)] fp16 per expert (default: the configuration's seeded synthetic weights); packed: ([PackedWeight] for
         gate_up, [PackedWeight] for down) already quantised and packed, e.g. from `checkpoint.load_layer` (formats are taken from them).
         bf6: run the w4a4 blocks on the 6-bit float matrix path: their weights are packed as bf6 fragments, the quantisers write their
-        activations as bf6 fragments (tag 4) and both launches use a kernel whose w4a4 tiles take that layout.  Same integer codes, same
-        accumulators and outputs, bit for bit; the operands occupy 0.75 instead of 0.5 bytes per value."""
+        activations as bf6 fragments (tag 4) and the launch uses a kernel whose w4a4 tiles take that layout.  Same integer codes, same
+        accumulators and outputs, bit for bit; the operands occupy 0.75 instead of 0.5 bytes per value.  One flag for both linear
+        blocks, or a pair (gate_up, down)."""
         self.cfg = cfg
-        self.bf6 = bool(bf6)
+        self.bf6_gate_up, self.bf6_down = (bool(bf6[0]), bool(bf6[1])) if isinstance(bf6, (tuple, list)) else (bool(bf6), bool(bf6))
         self.device = torch.device(device)
         self.n_exp_total = cfg.num_experts + (1 if cfg.num_shared else 0)
         if packed is not None:
@@ -41,12 +42,12 @@ class MxMoELayer:
         for e in range(self.n_exp_total if packed is None else 0):
             w13, w2 = weights[e] if weights is not None else expert_weights(cfg, e)
             gu, dn = self.formats[e]
-            self.w13.append(quantize_and_pack(w13.to(self.device), gu, keep_codes, bf6=self.bf6))
-            self.w2.append(quantize_and_pack(w2.to(self.device), dn, keep_codes, bf6=self.bf6))
+            self.w13.append(quantize_and_pack(w13.to(self.device), gu, keep_codes, bf6=self.bf6_gate_up))
+            self.w2.append(quantize_and_pack(w2.to(self.device), dn, keep_codes, bf6=self.bf6_down))
         self.qp_gate_up = [f[0] for f in self.formats]
         self.qp_down = [f[1] for f in self.formats]
-        self.kid_gate_up = ops.select_kernel(self.qp_gate_up, self.bf6)
-        self.kid_down = ops.select_kernel(self.qp_down, self.bf6)
+        self.kid_gate_up = ops.select_kernel(self.qp_gate_up, self.bf6_gate_up)
+        self.kid_down = ops.select_kernel(self.qp_down, self.bf6_down)
         self.state = None
         self._static = None
 
@@ -62,7 +63,7 @@ class MxMoELayer:
         topk_ids = topk_ids.to(self.device)
         st = {}
         (st["inp"], st["sa"], st["mid"], st["inp_store"], st["sa_store"], st["mid_store"], st["recv"], st["perm"], st["dst"]) = ops.quant_inp_act(
-            hidden, topk_ids, cfg.num_experts, cfg.inter, cfg.num_shared, self.qp_gate_up, rotate=cfg.rotate, bf6=self.bf6)
+            hidden, topk_ids, cfg.num_experts, cfg.inter, cfg.num_shared, self.qp_gate_up, rotate=cfg.rotate, bf6=self.bf6_gate_up)
         i_sh = cfg.inter * max(cfg.num_shared, 1)
         acc1 = [torch.zeros(m.shape, dtype=torch.int32, device=self.device) for m in st["mid"]] if dump_acc else None
         st["gg1"] = ops.prepare_gg(st["inp"], [w.data for w in self.w13], st["sa"], [w.scale for w in self.w13], st["mid"], 2 * cfg.inter, cfg.hidden,
@@ -80,7 +81,7 @@ class MxMoELayer:
         cfg, st = self.cfg, self.state
         (st["inp2"], st["sa2"], st["out"], st["inp2_store"], st["sa2_store"], st["out_store"]) = ops.silu_mul_then_quant(
             st["mid_store"], len(st["mid"]), cfg.num_experts, cfg.hidden, cfg.inter, cfg.num_shared, cfg.tokens, cfg.topk, st["dst"], st["recv"],
-            self.qp_down, rotate=cfg.rotate, bf6=self.bf6)
+            self.qp_down, rotate=cfg.rotate, bf6=self.bf6_down)
         i_sh = cfg.inter * max(cfg.num_shared, 1)
         acc2 = [torch.zeros(o.shape, dtype=torch.int32, device=self.device) for o in st["out"]] if st["dump_acc"] else None
         st["gg2"] = ops.prepare_gg(st["inp2"], [w.data for w in self.w2], st["sa2"], [w.scale for w in self.w2], st["out"], cfg.hidden, cfg.inter,
@@ -118,7 +119,8 @@ class MxMoELayer:
             def ptrs(ws):
                 return [w.data.data_ptr() for w in ws], [0 if w.scale is None else w.scale.data_ptr() for w in ws]
 
-            self._static = (LT.static_block(self.qp_gate_up, gu_w, gu_n, *ptrs(self.w13), bf6=self.bf6), LT.static_block(self.qp_down, dn_w, dn_n, *ptrs(self.w2), bf6=self.bf6))
+            self._static = (LT.static_block(self.qp_gate_up, gu_w, gu_n, *ptrs(self.w13), bf6=self.bf6_gate_up),
+                            LT.static_block(self.qp_down, dn_w, dn_n, *ptrs(self.w2), bf6=self.bf6_down))
         return self._static
 
     # ---- the forward that never waits for its routing ---------------------------------------------------------
@@ -140,11 +142,11 @@ class MxMoELayer:
         def u8(n):
             return torch.empty(max(int(n), 16), dtype=torch.uint8, device=dev)
 
-        def block(qps, ns, ks, ws):
+        def block(qps, ns, ks, ws, bf6):
             h = (_lib.BlockDesc * et)()
             for e in range(et):
                 a, w, g, sym = qps[e]
-                layout = (C.c_uint8 * 3)(1 if self.bf6 and (int(a), int(w), int(g)) == (4, 4, -1) else 0, 0, 0)  # 1: activations as bf6 fragments
+                layout = (C.c_uint8 * 3)(1 if bf6 and (int(a), int(w), int(g)) == (4, 4, -1) else 0, 0, 0)  # 1: activations as bf6 fragments
                 h[e] = _lib.BlockDesc(int(a), int(w), int(g), 1 if sym else 0, layout, int(ns[e]), int(ks[e]), ws[e].data.data_ptr(),
                                       0 if ws[e].scale is None else ws[e].scale.data_ptr())
             d = torch.frombuffer(bytearray(bytes(h)), dtype=torch.uint8).to(dev)
@@ -155,7 +157,7 @@ class MxMoELayer:
             if grid < 0:
                 raise RuntimeError(lib.mxmoe_last_error().decode())
             # worst-case stores: every routed row as wide as the widest routed expert's packed row
-            tags = [ops.act_tag(int(q[0]), int(q[2]), self.bf6 and int(q[1]) == 4) for q in qps]
+            tags = [ops.act_tag(int(q[0]), int(q[2]), bf6 and int(q[1]) == 4) for q in qps]
             # fp16 elements per row; bf6 fragments (tag 4) take 3/8 of an element per value and whole blocks of 32 rows per expert
             qld = [k * 3 // 8 if tg == 4 else (k if tg == 0 else (k // 2 if tg == 1 else k // 4)) for tg, k in zip(tags, ks)]
             sld = [0 if tg == 0 else (k // 128 if tg == 3 else 1) for tg, k in zip(tags, ks)]
@@ -167,8 +169,8 @@ class MxMoELayer:
             return {"h": h, "d": d, "kid": kid, "grid": grid, "plan": u8(lib.mxmoe_plan_bytes(et)), "inp": u8(inp), "scale": u8(sc), "out_bytes": out}
 
         sh = [1] if has_shared else []
-        b1 = block(self.qp_gate_up, [2 * cfg.inter] * e_cnt + [2 * i_sh for _ in sh], [cfg.hidden] * et, self.w13)
-        b2 = block(self.qp_down, [cfg.hidden] * et, [cfg.inter] * e_cnt + [i_sh for _ in sh], self.w2)
+        b1 = block(self.qp_gate_up, [2 * cfg.inter] * e_cnt + [2 * i_sh for _ in sh], [cfg.hidden] * et, self.w13, self.bf6_gate_up)
+        b2 = block(self.qp_down, [cfg.hidden] * et, [cfg.inter] * e_cnt + [i_sh for _ in sh], self.w2, self.bf6_down)
         ps["b1"], ps["b2"] = b1, b2
         ps["mid"], ps["out"] = u8(b1["out_bytes"]), u8(b2["out_bytes"])
         call = lambda b, out_store: _lib.PlanCall(b["kid"], b["d"].data_ptr(), C.cast(b["h"], C.c_void_p), b["inp"].data_ptr(), b["scale"].data_ptr(),  # noqa: E731
@@ -308,15 +310,27 @@ class MxMoELayer:
 
     def algorithmic_bytes(self) -> dict:
         """Bytes every launch must move at least once: packed weights + scales of touched experts, packed activations
-        + their scales, fp16 outputs."""
+        + their scales, fp16 outputs.  Codes count at their format's width (int4: half a byte) whatever layout carries them: the bf6
+        fragments of the 6-bit float path occupy 0.75 bytes per value, which shows in measured traffic, not here."""
         st = self.state
         recv = st["recv"]
         cfg = self.cfg
-        touched = [e for e in range(self.n_exp_total) if e == cfg.num_experts or int(recv[e]) > 0]
         out = {}
-        for name, ws, a_list, s_list, c_list in (("gate_up", self.w13, st["inp"], st["sa"], st["mid"]), ("down", self.w2, st["inp2"], st["sa2"], st["out"])):
-            w = sum(ws[e].nbytes for e in touched)
-            a = sum(t.numel() * t.element_size() for t in a_list) + sum(t.numel() * t.element_size() for t in s_list)
-            c = sum(t.numel() * t.element_size() for t in c_list)
+        for name, qps, ws in (("gate_up", self.qp_gate_up, self.w13), ("down", self.qp_down, self.w2)):
+            w = a = c = 0
+            for e in range(self.n_exp_total):
+                m = cfg.tokens if e == cfg.num_experts else int(recv[e])
+                if m == 0:
+                    continue
+                a_bits, w_bits, gsize, _sym = (int(v) for v in qps[e])
+                n, k = ws[e].n, ws[e].k
+                if w_bits >= 16:
+                    w += 2 * n * k
+                elif a_bits >= 16:                      # weight-only: codes + (scale, zero) per group
+                    w += n * k * w_bits // 8 + 4 * n * (k // gsize if gsize > 0 else 1)
+                else:                                   # codes + one scale per channel (and group)
+                    w += n * k * w_bits // 8 + 2 * n * (k // gsize if gsize > 0 else 1)
+                a += m * k * min(a_bits, 16) // 8 + (0 if a_bits >= 16 else 2 * m * (k // gsize if gsize > 0 else 1))
+                c += 2 * m * n
             out[name] = {"weights": w, "activations": a, "outputs": c, "total": w + a + c}
         return out
