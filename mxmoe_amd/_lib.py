@@ -88,16 +88,16 @@ def load(path: str | Path | None = None) -> C.CDLL:
     """Load the library and attach the C-ABI signatures.  A generated library (`path` given) carries the GroupGEMM entry
     points only; the default library must export everything the header declares."""
     p = Path(path) if path is not None else LIB_PATH
-    if p.exists():  # a library rebuilt under the same name (a generated one, per format set) is a different library
-        st = p.stat()
-        key = (str(p), st.st_mtime_ns, st.st_ino)
-        if key in _cached:
-            return _cached[key]
     if not p.exists():
         raise RuntimeError(
             f"{p} is missing: build it with `python -m mxmoe_amd.build` (hipcc, gfx950). "
             "mxmoe_amd has no CPU fallback for its kernels."
         )
+    # one handle per file name: the system loader caches shared libraries by name too (generated libraries carry a digest of
+    # their kernel set in their name, so a different set is a different file)
+    key = str(p.resolve())
+    if key in _cached:
+        return _cached[key]
     lib = C.CDLL(str(p))
     for name, (res, args) in SIGNATURES.items():
         if path is not None and name not in GEMM_ONLY and not hasattr(lib, name):

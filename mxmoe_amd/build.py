@@ -226,7 +226,7 @@ def sample_generator():
     from .kernels.compose_kernel import GEN_DIR, KernelType, TemplateGenerator
     from .kernels.tile_config import get_possible_tile_list
 
-    tiles = {q: [t for t in get_possible_tile_list("gfx950", q) if t.BM in (128, 32)] for q in ("w4a4_g-1_sym", "w8a8_g-1_sym")}
+    tiles = {q: [t for t in get_possible_tile_list("gfx950", q) if t.BM in (128, 32) and not t.is_bf6()] for q in ("w4a4_g-1_sym", "w8a8_g-1_sym")}
     for q in tiles:
         tiles[q] = tiles[q] + [tuple(tiles[q])]
     gen = TemplateGenerator("gfx950", list(tiles), KernelType.Fused, tiles, out_dir=GEN_DIR / "sample_w4a4_w8a8")

@@ -92,6 +92,12 @@ int mxmoe_group_gemm_plan(int kernel_id, const mxmoe_dim3* h_sizes, const mxmoe_
     if (branch_out) branch_out[i] = ns ? sg[0].branch : pick_branch(plan_of(k), (int)f, 1, (int)h_sizes[i].y);
     for (int j = 0; j < ns; ++j) {
       const BranchInfo& bi = k.branches[sg[j].branch];
+      if (!shape_ok(bi, h_sizes[i])) {  // what the launch itself would refuse
+        char buf[200];
+        snprintf(buf, sizeof buf, "problem %d: shape [%u,%u,%u] not supported by tile %s (K %% %d, N %% 8)", i, h_sizes[i].x, h_sizes[i].y, h_sizes[i].z, fmt_name(bi.fmt, true), bi.k_multiple);
+        last_error() = buf;
+        return 3;
+      }
       total += ((sg[j].rows + bi.BM - 1) / bi.BM) * (int)((h_sizes[i].y + bi.BN - 1) / bi.BN);
     }
   }

@@ -5,7 +5,7 @@ bench_input_file :870-946; timing protocol mxmoe/kernels/src/test_utils.h:97-191
 Per (layer, "gate_up" | "down") problem list: fp16 operands ~ U(-1, 1) (seed 42), operands quantised + packed per problem,
 every registered fused kernel that covers the formats is timed (<= 30 warm-up, <= 50 timed launches, HIP events, median)
 and reported as `kernel_name, avg_time (ms), TFLOPS, speedup` against the best fp16 grouped GEMM of the same shapes (the
-reference's CUTLASS baseline; here the fp16 MFMA kernel), written to `<output>-<layer>-<gate_up|down>.csv`.
+reference's CUTLASS baseline; here the fp16 MFMA kernel), written to `<output>-layer-<i>-<gate_up|down>.csv`.
 Sequential and multi-stream launches (one launch per contiguous run of equal-format problems, on one stream or dealt to
 side streams — the reference's ablation launchers, kernel_sketch.py:148-406, here policies of the C++ host launcher) are
 timed next to the fused launch.
@@ -23,11 +23,44 @@ from .quant import quant_minmax
 from .weights import quantize_and_pack
 
 
-def parse_input_file(path: str) -> dict:
-    """{layer name: {"gate_up": [...], "down": [...]}} with entries {"shape": [M, N, K], "w_bits", "a_bits", "gsize", "sym"}."""
+def parse_json_input(path: str) -> dict:
+    """test.cu:652-674: {case name: {"gate_up": [...], "down": [...]}} with entries {"shape": [M, N, K], "w_bits", "a_bits", "gsize",
+    "sym"}; every top-level key except "num_tokens" is a case (the workload generator writes "layer-<i>")."""
     with open(path) as f:
         data = json.load(f)
-    return {k: v for k, v in data.items() if k.startswith("layer-")}
+    return {k: v for k, v in data.items() if k != "num_tokens"}
+
+
+def parse_legacy_input(path: str) -> dict:
+    """test.cu:611-650: a text file with one problem per line, `a_bits-w_bits-gsize-{sym|asym} MxNxK` (any single character between the
+    numbers), all of them one problem list `{"test_case": {"gate_up": [...]}}`.  Weight bits 16 / 8 / 4 / 2 and activation bits
+    16 / 8 / 4, as there."""
+    import re
+
+    shapes = []
+    with open(path) as f:
+        for line in f:
+            if not line.strip():
+                continue
+            m = re.match(r"\s*(\d+)\D(\d+)\D(-?\d+)\D(sym|asym)\s+(\d+)\D(\d+)\D(\d+)\s*$", line)
+            if not m:
+                raise ValueError(f"cannot parse `{line.rstrip()}`: expected `a_bits-w_bits-gsize-sym MxNxK`")
+            a_bits, w_bits, gsize = int(m.group(1)), int(m.group(2)), int(m.group(3))
+            if w_bits not in (16, 8, 4, 2):
+                raise ValueError(f"Ava w bits: [16, 8, 4, 2]. Got {w_bits}")
+            if a_bits not in (16, 8, 4):
+                raise ValueError(f"Ava a bits: [16, 8, 4]. Got {a_bits}")
+            shapes.append({"shape": [int(m.group(5)), int(m.group(6)), int(m.group(7))], "w_bits": w_bits, "a_bits": a_bits, "gsize": gsize, "sym": m.group(4) == "sym"})
+    return {"test_case": {"gate_up": shapes}}
+
+
+def parse_input_file(path: str) -> dict:
+    """test.cu:676-691: a `.json` workload file or a legacy text file."""
+    import os
+
+    if not os.path.exists(path):
+        raise FileNotFoundError(f"input file: `{path}` not found")
+    return parse_json_input(path) if str(path).endswith(".json") else parse_legacy_input(path)
 
 
 def bench_func(fn, warmup: int = 20, iters: int = 50, max_warm_s: float = 10.0) -> dict:
@@ -50,8 +83,9 @@ def bench_func(fn, warmup: int = 20, iters: int = 50, max_warm_s: float = 10.0) 
     return {"min": ts[0], "max": ts[-1], "mean": sum(trim) / len(trim), "median": ts[len(ts) // 2]}
 
 
-def make_problem(entry: dict, gen: torch.Generator, device="cuda", keep_ref: bool = False) -> dict:
-    """Random fp16 operands for one workload entry, quantised and packed for its format (QInput::from_fp16)."""
+def make_problem(entry: dict, gen: torch.Generator, device="cuda", keep_ref: bool = False, bf6: bool = False) -> dict:
+    """Random fp16 operands for one workload entry, quantised and packed for its format (QInput::from_fp16).  `bf6`: w4a4 operands as
+    bf6 fragments, the layout of the kernels whose w4a4 tiles run on the 6-bit float matrix path (`kernel_takes_bf6`)."""
     m, n, k = entry["shape"]
     qp = (entry["a_bits"], entry["w_bits"], entry["gsize"], bool(entry["sym"]))
     if gen is None:  # values drawn on the device (timing-only problems)
@@ -60,19 +94,31 @@ def make_problem(entry: dict, gen: torch.Generator, device="cuda", keep_ref: boo
     else:
         a = (torch.rand(m, k, generator=gen, dtype=torch.float32) * 2 - 1).to(torch.float16).to(device)
         b = (torch.rand(n, k, generator=gen, dtype=torch.float32) * 2 - 1).to(torch.float16).to(device)
-    pw = quantize_and_pack(b, qp)
+    pw = quantize_and_pack(b, qp, bf6=bf6)
     prob = {"size": (m, n, k), "q": qp, "B": pw.data, "sb": pw.scale, "C": torch.zeros(m, n, dtype=torch.float16, device=device)}
     if qp[0] < 16:
         ag = qp[2] if qp[2] > 0 else -1                      # group-quantised activations (w4a4_g128_sym): scales [M, K / 128]
         qa, sa, _ = quant_minmax(a, qp[0], ag, True) if m else (a, a[:, :1], None)
         qi = qa.reshape(m, k).to(torch.int8)
-        prob["A"] = qi.contiguous() if qp[0] == 8 else pack.pack_int4_k(qi)
+        prob["A"] = qi.contiguous() if qp[0] == 8 else (pack.pack_bf6_fragments(qi) if bf6 and qp[2] == -1 and qp[1] == 4 else pack.pack_int4_k(qi))
         prob["sa"] = sa.reshape(-1).contiguous()
     else:
         prob["A"], prob["sa"] = a, None
     if keep_ref:
         prob["a16"], prob["b16"] = a, b
     return prob
+
+
+def kernel_takes_bf6(lib, kid: int) -> bool:
+    """Whether kernel `kid` has w4a4 tiles on the 6-bit float matrix path (64-wide K steps): its w4a4 operands are bf6 fragments."""
+    import ctypes as C
+
+    out = (C.c_int32 * 8)()
+    for b in range(lib.mxmoe_kernel_num_branches(kid)):
+        lib.mxmoe_kernel_branch(kid, b, out)
+        if out[0] == 2 and out[3] == 64:
+            return True
+    return False
 
 
 def _launch_of(probs, lib, kernel_id=-1) -> GroupGemmLaunch:
@@ -124,6 +170,7 @@ def bench_one_case(entries, lib=None, mode: str = "bench", filters=(), out_file:
     gen.manual_seed(42)
     probs = [make_problem(e, gen, keep_ref=(mode == "check")) for e in entries]
     probs = [p for p in probs if p["size"][0] > 0]
+    probs_b6 = None  # the same problems with their w4a4 operands as bf6 fragments, made when a kernel asks for them
 
     # fp16 baseline on the same shapes (role of the CUTLASS grouped GEMM, test.cu:774-781)
     gen2 = torch.Generator(device="cpu")
@@ -138,15 +185,21 @@ def bench_one_case(entries, lib=None, mode: str = "bench", filters=(), out_file:
         name = lib.mxmoe_kernel_name(kid).decode()
         if filters and not any(f in name for f in filters):
             continue
-        g = _launch_of(probs, lib, kid)
+        mine = probs
+        if kernel_takes_bf6(lib, kid) and any(p["q"][:3] == (4, 4, -1) for p in probs):
+            if probs_b6 is None:
+                gen.manual_seed(42)
+                probs_b6 = [make_problem(e, gen, keep_ref=(mode == "check"), bf6=True) for e in entries if e["shape"][0] > 0]
+            mine = probs_b6
+        g = _launch_of(mine, lib, kid)
         try:
             g.plan()
         except RuntimeError:
-            continue  # this kernel has no tile for one of the formats
+            continue  # this kernel has no tile for one of the formats (or does not take one of the shapes)
         if mode == "check":
             g.run()
             torch.cuda.synchronize()
-            for p in probs:
+            for p in mine:
                 ref = (p["a16"].float() @ p["b16"].float().T)
                 err = (p["C"].float() - ref).abs().max().item() if p["size"][0] else 0.0
                 tol = 1.0 if p["q"][1] >= 16 else float("inf")  # test_utils.h:71 — meaningful for fp16 only, as in the reference
@@ -183,12 +236,14 @@ def bench_one_case(entries, lib=None, mode: str = "bench", filters=(), out_file:
 
 
 def bench_input_file(input_path: str, output_prefix: str | None = None, lib=None, mode: str = "bench", filters=(), verbose: bool = False) -> dict:
-    """test.cu:870-946: every layer of the workload file, gate_up then down; CSV per (layer, GEMM)."""
+    """test.cu:870-946: every case of the input file (the layers of a workload file, gate_up then down; the one list of a legacy
+    file), one CSV per problem list named `<output>-<case>-<gate_up|down>.csv` (test.cu:942)."""
     out = {}
-    for layer, shapes in parse_input_file(input_path).items():
-        idx = layer.split("-")[1]
+    for case, lists in parse_input_file(input_path).items():
         for which in ("gate_up", "down"):
-            csv = f"{output_prefix}-{idx}-{which}.csv" if output_prefix else None
-            print(f"== {layer} {which}: {len(shapes[which])} problems")
-            out[(layer, which)] = bench_one_case(shapes[which], lib=lib, mode=mode, filters=filters, out_file=csv, verbose=verbose)
+            if which not in lists:
+                continue
+            csv = f"{output_prefix}-{case}-{which}.csv" if output_prefix else None
+            print(f"== {case} {which}: {len(lists[which])} problems")
+            out[(case, which)] = bench_one_case(lists[which], lib=lib, mode=mode, filters=filters, out_file=csv, verbose=verbose)
     return out

@@ -122,10 +122,24 @@ class TemplateGenerator:
         print(f"Generated {len(combos)} kernels for `{self.kernel_type}` {self.qcfgs}")
         return files
 
+    def library_path(self) -> Path:
+        """Where `build()` puts the library of this generator's kernels: the file name carries a digest of the kernel set, so two
+        format or tile sets never share a name (a process that loads both would otherwise get the first one back from the loader
+        the second time: shared libraries are cached by name)."""
+        import hashlib
+
+        text = ";".join(f"{self.kernel_type}_{i}:" + ",".join(f"{q}={t.to_str()}" for q, item in combo.items() for t in _flat([item]))
+                        for i, combo in enumerate(self.get_tile_configs()))
+        return self.out_dir / f"libmxmoe_{self.kernel_type}_{hashlib.sha1(text.encode()).hexdigest()[:10]}.so"
+
     def build(self, out: str | os.PathLike | None = None) -> Path:
         """hipcc the generated translation units into one shared library exporting the C-ABI."""
-        out = Path(out) if out else self.out_dir / f"libmxmoe_{self.kernel_type}.so"
-        return _build.hipcc_build(self.files, out)
+        if out is None:
+            out = self.library_path()
+            for old in self.out_dir.glob(f"libmxmoe_{self.kernel_type}*.so"):  # libraries of earlier kernel sets in this directory
+                if old != out:
+                    old.unlink()
+        return _build.hipcc_build(self.files, Path(out))
 
 
 def build_kernel_source(tile_cfg, kname: str, kernel_type: KernelType = KernelType.Fused, deferred: bool = False):

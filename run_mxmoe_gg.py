@@ -7,7 +7,7 @@ reference entry point (run_mxmoe_gg.py:32-121):
 
 Steps: qcfg set of the qconfig -> workload JSON from the expert-frequency trace (`out/workloads/...`) -> generate the fused
 kernels for that qcfg set -> hipcc them into one library (replaces cmake + ninja) -> time every kernel per layer
-(`out/bench/{model}-{dataset}-{bs}{suffix}-{layer}-{gate_up|down}.csv`, in-process instead of `./build/test bench`).
+(`out/bench/{model}-{dataset}-{bs}{suffix}-layer-{i}-{gate_up|down}.csv`, in-process instead of `./build/test bench`).
 
 The reference's traces come from real checkpoints (`calib/gate/{model}/{dataset}/4096/moe-gate.json`).  Without them,
 `--synthetic {c1..c5}` writes the trace and qconfig of a seeded synthetic configuration under `out/synthetic/` and uses
@@ -69,6 +69,7 @@ def main(argv=None) -> int:
     p.add_argument("--trace", type=str, default=None, help="expert-frequency trace file (moe-gate.json)")
     p.add_argument("--mode", type=str, default="bench", choices=["bench", "check"])
     p.add_argument("--max-kernels", type=int, default=0, help="generate at most this many tile combinations (0 = all)")
+    p.add_argument("--no-bench", action="store_true", help="stop after the workload file, the generated sources and the library (no GPU needed)")
     args = p.parse_args(argv)
 
     model_id, dataset, bs, layer = args.model, args.dataset, args.bs, args.layer
@@ -116,6 +117,11 @@ def main(argv=None) -> int:
 
     from mxmoe_amd import _lib
 
+    if args.no_bench:
+        for lyr in layers:
+            generate_workload_from_gate_trace(trace, bs, lyr, workload_path, args.qconfig, args.qstr if args.qconfig is None else None, exact_counts=exact)
+        print(f"workload: {workload_path}\nlibrary: {lib_path}")
+        return 0
     lib = _lib.load(lib_path)
     os.makedirs(f"{CUR_DIR}/out/bench", exist_ok=True)
     bench_save = f"{CUR_DIR}/out/bench/{model_id}-{dataset}-{bs}{workload_suffix.replace('.json', '')}"

@@ -118,7 +118,7 @@ def test_generated_library_mixed_launch_is_bit_exact():
 
     gen = build.sample_generator()
     gen.kernel_names = [f"groupgemm_{gen.kernel_type}_{i}" for i in range(len(gen.get_tile_configs()))]
-    lib = _lib.load(gen.out_dir / f"libmxmoe_{gen.kernel_type}.so")          # raises when the build did not produce it
+    lib = _lib.load(gen.library_path())                                      # raises when the build did not produce it
     assert lib.mxmoe_num_kernels() == len(gen.kernel_names) == 5
     probs = _mixed_problems(np.random.default_rng(21))
     for kid in range(lib.mxmoe_num_kernels()):
@@ -186,7 +186,7 @@ def test_function_type_call_with_exactly_fifteen_arguments():
     ran = 0
     for kid in range(lib.mxmoe_num_kernels()):
         name = lib.mxmoe_kernel_name(kid).decode()
-        if "w4a4_g-1_sym" not in name or "w8a8_g-1_sym" not in name:
+        if "w4a4_g-1_sym" not in name or "w8a8_g-1_sym" not in name or name.endswith("_b6"):   # (the _b6 kernels take w4a4 operands as bf6 fragments)
             continue
         fn = _lib.FUNC_TYPE(lib.mxmoe_kernel_func(kid))
         for c in Cs:
@@ -279,3 +279,42 @@ def test_int4_gemm_on_the_bf6_matrix_path_is_exact():
     assert lib.mxmoe_bf6_gemm_probe(ta.data_ptr(), tb.data_ptr(), tsa.data_ptr(), tsb.data_ptr(), c.data_ptr(), None, 128, 256, 256, 0, stream) == 3
     assert lib.mxmoe_bf6_gemm_probe(ta.data_ptr(), tb.data_ptr(), tsa.data_ptr(), tsb.data_ptr(), c.data_ptr(), None, 256, 256, 256, 2, stream) == 3
     assert lib.mxmoe_bf6_gemm_probe(ta.data_ptr(), tb.data_ptr(), tsa.data_ptr(), tsb.data_ptr(), c.data_ptr(), None, 256, 256, 1408, 0, stream) == 3
+
+
+def test_bench_harness_on_a_workload_file_and_a_legacy_file(tmp_path, capsys):
+    """The program the CLI ends in (test.cu:693-946): a synthetic DeepSeek-V2-Lite-shaped trace and qconfig -> workload file ->
+    `check`, then `bench` with the default library: one CSV per problem list, named `<output>-<case>-<gate_up|down>.csv`
+    (test.cu:942) with the header `kernel_name,avg_time,TFLOPS,speedup` (test.cu:858) and one line per kernel that covers the
+    formats; the same through a legacy text input."""
+    import json
+
+    from mxmoe_amd import _lib, harness, synth
+    from mxmoe_amd.kernels import gen_workload
+
+    cfg = synth.get_config("c4")
+    trace, qcfg, wl = tmp_path / "moe-gate.json", tmp_path / "q-wbits4.json", tmp_path / "w.json"
+    trace.write_text(json.dumps(synth.trace_dict(cfg)))
+    qcfg.write_text(json.dumps(synth.qconfig_dict(cfg)))
+    gen_workload.generate_workload_from_gate_trace(str(trace), cfg.tokens, 0, str(wl), str(qcfg), exact_counts=True)
+    lib = _lib.load()
+    harness.bench_input_file(str(wl), None, lib=lib, mode="check", filters=("groupgemm_hz_fused_wo",))
+    assert "max abs err vs fp16 reference" in capsys.readouterr().out
+    prefix = str(tmp_path / "bench" / "ds2-synthetic-32")
+    (tmp_path / "bench").mkdir()
+    res = harness.bench_input_file(str(wl), prefix, lib=lib, mode="bench")
+    assert set(res) == {("layer-0", "gate_up"), ("layer-0", "down")}
+    for which in ("gate_up", "down"):
+        lines = (tmp_path / "bench" / f"ds2-synthetic-32-layer-0-{which}.csv").read_text().splitlines()
+        assert lines[0] == "kernel_name,avg_time,TFLOPS,speedup"
+        names = [ln.split('",')[0].strip('"') for ln in lines[1:]]
+        assert any(n.endswith("groupgemm_hz_fused_wo") for n in names) and any(n.endswith("groupgemm_hz_fused_all") for n in names)
+        for ln in lines[1:]:
+            ms, tf, sp = (float(x) for x in ln.rsplit('",', 1)[1].split(","))
+            assert ms > 0 and tf > 0 and sp > 0
+        r = res[("layer-0", which)]
+        assert {"fp16-baseline", "mxmoe-hz", "mxmoe-seq", "mxmoe-ms"} <= set(r) and abs(r["mxmoe-hz"][0] - min(float(ln.rsplit('",', 1)[1].split(",")[0]) for ln in lines[1:])) < 1e-4
+    legacy = tmp_path / "cases.txt"
+    legacy.write_text("4-4--1-sym 300x512x256\n8-8--1-sym 64x256x128\n")
+    res = harness.bench_input_file(str(legacy), str(tmp_path / "bench" / "legacy"), lib=lib, mode="bench", filters=("groupgemm_hz_fused_wxax",))
+    assert list(res) == [("test_case", "gate_up")]
+    assert (tmp_path / "bench" / "legacy-test_case-gate_up.csv").read_text().splitlines()[0] == "kernel_name,avg_time,TFLOPS,speedup"

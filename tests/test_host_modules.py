@@ -337,3 +337,52 @@ def test_bench_refuses_more_than_one_gpu():
     root = Path(__file__).resolve().parent.parent
     res = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
     assert res.returncode == 2 and "one GPU" in res.stderr and res.stdout.strip() == ""
+
+
+def test_harness_input_parsers(tmp_path):
+    """test.cu:611-691: workload JSON files (every key but "num_tokens" is a case) and the legacy text form
+    `a_bits-w_bits-gsize-sym MxNxK`, one problem per line."""
+    from mxmoe_amd import harness
+
+    cfg = synth.get_config("c4")
+    trace, qcfg = tmp_path / "moe-gate.json", tmp_path / "q-wbits4.json"
+    trace.write_text(json.dumps(synth.trace_dict(cfg)))
+    qcfg.write_text(json.dumps(synth.qconfig_dict(cfg)))
+    w = tmp_path / "w.json"
+    gen_workload.generate_workload_from_gate_trace(str(trace), cfg.tokens, 0, str(w), str(qcfg))
+    cases = harness.parse_input_file(str(w))
+    assert list(cases) == ["layer-0"] and len(cases["layer-0"]["gate_up"]) == 65 and set(cases["layer-0"]["down"][0]) >= {"shape", "w_bits", "a_bits", "gsize", "sym"}
+    legacy = tmp_path / "cases.txt"
+    legacy.write_text("4-4--1-sym 512x2816x2048\n16-4-128-asym 32x2048x1408\n\n8x8x-1xsym 7,256,128\n")
+    got = harness.parse_input_file(str(legacy))
+    assert list(got) == ["test_case"] and list(got["test_case"]) == ["gate_up"]
+    assert got["test_case"]["gate_up"] == [
+        {"shape": [512, 2816, 2048], "w_bits": 4, "a_bits": 4, "gsize": -1, "sym": True},
+        {"shape": [32, 2048, 1408], "w_bits": 4, "a_bits": 16, "gsize": 128, "sym": False},
+        {"shape": [7, 256, 128], "w_bits": 8, "a_bits": 8, "gsize": -1, "sym": True}]
+    legacy.write_text("4-3-128-asym 1x256x128\n")
+    with pytest.raises(ValueError, match="Ava w bits"):                      # test.cu:633-636 lists 16 / 8 / 4 / 2
+        harness.parse_input_file(str(legacy))
+    with pytest.raises(FileNotFoundError):
+        harness.parse_input_file(str(tmp_path / "none.json"))
+
+
+def test_run_mxmoe_gg_up_to_the_library(tmp_path, monkeypatch):
+    """The CLI end to end without a GPU: synthetic trace and qconfig -> qcfg set -> workload JSON -> generated sources -> hipcc
+    -> a library that loads and registers the generated kernel (run_mxmoe_gg.py:34-111 up to the bench subprocess)."""
+    import run_mxmoe_gg as r
+    from mxmoe_amd import _lib
+    from mxmoe_amd.kernels import compose_kernel as ck
+
+    monkeypatch.setattr(r, "CUR_DIR", str(tmp_path))
+    monkeypatch.setattr(ck, "GEN_DIR", tmp_path / "generated")
+    assert r.main(["--synthetic", "c4", "--max-kernels", "1", "--no-bench"]) == 0
+    wl = json.loads((tmp_path / "out" / "workloads" / "ds2-synthetic-32--c4.json").read_text())
+    assert wl["num_tokens"] == 32 and len(wl["layer-0"]["gate_up"]) == 65
+    assert {(e["w_bits"], e["a_bits"], e["gsize"]) for e in wl["layer-0"]["down"]} == {(4, 16, 128), (3, 16, 128)}
+    libs = list((tmp_path / "generated").glob("libmxmoe_hz_fused_*.so"))
+    assert len(libs) == 1
+    lib = _lib.load(libs[0])
+    assert lib.mxmoe_num_kernels() == 1
+    name = lib.mxmoe_kernel_name(0).decode()
+    assert name.endswith("groupgemm_hz_fused_0") and "w4a16_g128_asym" in name and "w3a16_g128_asym" in name
