@@ -204,24 +204,31 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd<Tiles...>) fused_group
 
 // ------------------------------------------------------------------ host side ------------------------------------------------------------------
 
-enum class Fmt { FP16, W8A8, W4A4, W4A16, W3A16, W2A16, W4A4G128, UNSUPPORTED };
+enum class Fmt { FP16, W8A8, W4A4, W4A16, W3A16, W2A16, W4A4G128, W8A16, UNSUPPORTED };
 
-inline Fmt classify(const mxmoe_qparams& q) {
+// Format of a problem from its QParams.  Weight-only formats come with one (scale, zero) pair per channel and 128-wide K group or
+// per channel (group size -1): the tiles are the same, the packer repeats a per-channel pair for every group.
+__host__ __device__ inline Fmt classify(const mxmoe_qparams& q) {
   if (q.a_bits >= 16 && q.w_bits >= 16) return Fmt::FP16;
   if (q.a_bits == 8 && q.w_bits == 8 && q.gsize == -1 && q.sym) return Fmt::W8A8;
   if (q.a_bits == 4 && q.w_bits == 4 && q.gsize == -1 && q.sym) return Fmt::W4A4;
   if (q.a_bits == 4 && q.w_bits == 4 && q.gsize == 128 && q.sym) return Fmt::W4A4G128;
-  if (q.a_bits >= 16 && q.w_bits == 4 && q.gsize == 128) return Fmt::W4A16;
-  if (q.a_bits >= 16 && q.w_bits == 3 && q.gsize == 128) return Fmt::W3A16;
-  if (q.a_bits >= 16 && q.w_bits == 2 && q.gsize == 128) return Fmt::W2A16;
+  if (q.a_bits >= 16 && (q.gsize == 128 || q.gsize == -1)) {
+    if (q.w_bits == 8) return Fmt::W8A16;
+    if (q.w_bits == 4) return Fmt::W4A16;
+    if (q.w_bits == 3) return Fmt::W3A16;
+    if (q.w_bits == 2) return Fmt::W2A16;
+  }
   return Fmt::UNSUPPORTED;
 }
+__host__ __device__ inline bool is_weight_only(Fmt f) { return f == Fmt::W8A16 || f == Fmt::W4A16 || f == Fmt::W3A16 || f == Fmt::W2A16; }
 
 inline const char* fmt_name(Fmt f, bool sym) {
   switch (f) {
     case Fmt::FP16: return "fp16";
     case Fmt::W8A8: return "w8a8_g-1_sym";
     case Fmt::W4A4: return "w4a4_g-1_sym";
+    case Fmt::W8A16: return sym ? "w8a16_g128_sym" : "w8a16_g128_asym";
     case Fmt::W4A16: return sym ? "w4a16_g128_sym" : "w4a16_g128_asym";
     case Fmt::W3A16: return sym ? "w3a16_g128_sym" : "w3a16_g128_asym";
     case Fmt::W2A16: return sym ? "w2a16_g128_sym" : "w2a16_g128_asym";
@@ -276,7 +283,7 @@ template <int WBITS, int BN>
 struct BranchOf<SkinnyWoTile<WBITS, BN>> {
   static BranchInfo get() {
     using T = SkinnyWoTile<WBITS, BN>;
-    return BranchInfo{WBITS == 4 ? Fmt::W4A16 : WBITS == 3 ? Fmt::W3A16 : Fmt::W2A16, T::BM, BN, 128, 1, 4, T::kLdsBytes, 128, 0};
+    return BranchInfo{WBITS == 8 ? Fmt::W8A16 : WBITS == 4 ? Fmt::W4A16 : WBITS == 3 ? Fmt::W3A16 : Fmt::W2A16, T::BM, BN, 128, 1, 4, T::kLdsBytes, 128, 0};
   }
 };
 
@@ -315,7 +322,7 @@ template <int WBITS, int BM, int BN>
 struct BranchOf<WoMfmaTile<WBITS, BM, BN>> {
   static BranchInfo get() {
     using T = WoMfmaTile<WBITS, BM, BN>;
-    return BranchInfo{WBITS == 4 ? Fmt::W4A16 : WBITS == 3 ? Fmt::W3A16 : Fmt::W2A16, BM, BN, 128, T::WM, 4 / T::WM, T::kLdsBytes, 128, 0};
+    return BranchInfo{WBITS == 8 ? Fmt::W8A16 : WBITS == 4 ? Fmt::W4A16 : WBITS == 3 ? Fmt::W3A16 : Fmt::W2A16, BM, BN, 128, T::WM, 4 / T::WM, T::kLdsBytes, 128, 0};
   }
 };
 
@@ -334,6 +341,7 @@ inline double tile_cost(const BranchInfo& b) {
       {Fmt::W4A16, 16, 128, 0.37}, {Fmt::W4A16, 16, 64, 0.20}, {Fmt::W4A16, 128, 128, 1.00}, {Fmt::W4A16, 128, 256, 1.50},
       {Fmt::W3A16, 16, 128, 0.31}, {Fmt::W3A16, 16, 64, 0.20}, {Fmt::W3A16, 128, 128, 1.00}, {Fmt::W3A16, 128, 256, 1.50},
       {Fmt::W2A16, 16, 128, 0.25}, {Fmt::W2A16, 16, 64, 0.20}, {Fmt::W2A16, 128, 128, 1.00}, {Fmt::W2A16, 128, 256, 1.50},
+      {Fmt::W8A16, 16, 128, 0.60}, {Fmt::W8A16, 16, 64, 0.35}, {Fmt::W8A16, 128, 128, 1.00},
       {Fmt::W4A4G128, 64, 256, 1.00}, {Fmt::W4A4G128, 32, 256, 0.60},
   };
   for (const Row& r : table)
@@ -344,7 +352,7 @@ inline double tile_cost(const BranchInfo& b) {
 // Rough run time of one tile across formats, used only to order the tile list (expensive shapes first): the matrix pipe runs
 // fp16 at half the int8 rate, and int4 operands are widened to int8.
 inline double branch_cost(const BranchInfo& b) {
-  const double per_k = b.fmt == Fmt::FP16 ? 2.0 : (b.fmt == Fmt::W4A16 || b.fmt == Fmt::W3A16 || b.fmt == Fmt::W2A16) ? 1.2 : (b.fmt == Fmt::W8A8 ? 1.25 : 1.0);
+  const double per_k = b.fmt == Fmt::FP16 ? 2.0 : is_weight_only(b.fmt) ? 1.2 : (b.fmt == Fmt::W8A8 ? 1.25 : 1.0);
   return tile_cost(b) * per_k;
 }
 
@@ -565,7 +573,7 @@ inline bool kernel_covers(const FusedKernel& k, const mxmoe_qparams* q, int coun
 
 // K a multiple of the tile's K step, N a multiple of 8 (16 for the weight-only layouts)
 inline bool shape_ok(const BranchInfo& bi, const mxmoe_dim3& sz) {
-  const bool wo = bi.fmt == Fmt::W4A16 || bi.fmt == Fmt::W3A16 || bi.fmt == Fmt::W2A16;
+  const bool wo = is_weight_only(bi.fmt);
   return sz.z != 0 && sz.z % bi.k_multiple == 0 && (int)sz.z >= bi.k_min && sz.y % 8 == 0 && !(wo && sz.y % 16 != 0);
 }
 
@@ -705,7 +713,7 @@ inline int group_gemm(int kernel_id, const void* const* As, const void* const* B
   for (int i = 0; i < count; ++i) {  // the tiles read the scales unconditionally: refuse a launch whose scale arrays are missing
     const Fmt f = classify(h_q[i]);
     const bool wa = f == Fmt::W8A8 || f == Fmt::W4A4 || f == Fmt::W4A4G128;
-    const bool wo = f == Fmt::W4A16 || f == Fmt::W3A16 || f == Fmt::W2A16;
+    const bool wo = is_weight_only(f);
     if (h_sizes[i].x != 0 && ((wa && (!sa || !sb)) || (wo && !sb))) {
       last_error() = "scale arrays are required for quantised formats";
       return 5;

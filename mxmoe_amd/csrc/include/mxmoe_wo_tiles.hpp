@@ -1,4 +1,6 @@
-// Skinny weight-only tiles (w4a16 / w3a16, group 128) for experts that receive a handful of tokens.
+// Skinny weight-only tiles (w8a16 / w4a16 / w3a16 / w2a16, one (scale, zero) pair per channel and 128-wide K group) for experts that
+// receive a handful of tokens.  Per-channel formats (group size -1, the reference's cta_gemm_multistage_qb_v2 with GSIZE = -1,
+// mxmoe/kernels/src/include/cta_gemm.cuh:113-286) use the same tiles: their packer repeats the channel's pair for every group.
 //
 // These problems are HBM-bound: every packed weight is read exactly once and the work is arranged around that
 // stream.  A workgroup owns 16 tokens x BN channels; its 4 waves split K into contiguous quarters, keep their quarter of the
@@ -13,6 +15,7 @@
 // lets two masks and one shift produce four fp16 pairs in k order (magic-number conversion, no per-element shifts).
 // w3 stores 24 values in the low 3 bits of the 24 nibbles of three dwords; the 24 spare top bits hold values 24..31.
 // w2 stores values 16d..16d+7 in the low two bits of the nibbles of dword d and values 16d+8..16d+15 in the high two.
+// w8 stores one byte per value in k order (8 dwords per lane).
 //
 // The group scale is applied to the fp32 partial sum of each 128-wide group instead of to every weight:
 //   sum_k x[k]*(q[k]*s + z) = s * sum_k x[k]*q[k] + z * sum_k x[k]
@@ -32,7 +35,7 @@ namespace mxmoe {
 template <int WBITS_, int BN_>
 struct SkinnyWoTile {
   static constexpr int WBITS = WBITS_, BM = 16, BN = BN_;
-  static_assert(WBITS == 4 || WBITS == 3 || WBITS == 2, "w4 / w3 / w2 only");
+  static_assert(WBITS == 8 || WBITS == 4 || WBITS == 3 || WBITS == 2, "w8 / w4 / w3 / w2");
   static_assert(BN % 64 == 0, "the final reduction deals 16-channel blocks to 4 waves");
   static constexpr int NB = BN / 16;                 // 16-channel blocks per tile
   static constexpr int KP = 4;                       // k blocks (128 wide) per pass of a wave: their activations live in registers
@@ -43,7 +46,7 @@ struct SkinnyWoTile {
   static constexpr int kABits = 16, kWBits = WBITS;  // fp16 activations, packed weights
   static constexpr int kLaneBytes = WBITS * 4;       // packed bytes per lane per (channel block, k block)
   static constexpr int kBlockBytes = 64 * kLaneBytes;
-  static constexpr int kRing = 12;                   // packed blocks in flight per wave
+  static constexpr int kRing = WBITS == 8 ? 6 : 12;  // packed blocks in flight per wave (12 KB either way)
 
   struct WReg {
     int d[WBITS];
@@ -51,7 +54,11 @@ struct SkinnyWoTile {
 
   __device__ static __forceinline__ WReg load_w(const uint8_t* p) {
     WReg w;
-    if constexpr (WBITS == 4) {
+    if constexpr (WBITS == 8) {
+      const v4i a = gload<v4i>(p), b = gload<v4i>(p + 16);
+      w.d[0] = a[0]; w.d[1] = a[1]; w.d[2] = a[2]; w.d[3] = a[3];
+      w.d[4] = b[0]; w.d[5] = b[1]; w.d[6] = b[2]; w.d[7] = b[3];
+    } else if constexpr (WBITS == 4) {
       const v4i v = gload<v4i>(p);
       w.d[0] = v[0]; w.d[1] = v[1]; w.d[2] = v[2]; w.d[3] = v[3];
     } else if constexpr (WBITS == 3) {
@@ -80,9 +87,28 @@ struct SkinnyWoTile {
     return __builtin_bit_cast(v8h, o);
   }
 
+  // The bias each of the 8 values of an operand still carries after unpack(): 1024 for values placed by the 0x6400 constant, 64 for
+  // those placed by 0x5400 (8-bit codes are all placed by the first).
+  __device__ static __forceinline__ v8h bias8() {
+    constexpr float hi = WBITS == 8 ? 1024.0f : 64.0f;
+    return v8h{(_Float16)1024.0f, (_Float16)1024.0f, (_Float16)hi, (_Float16)hi, (_Float16)1024.0f, (_Float16)1024.0f, (_Float16)hi, (_Float16)hi};
+  }
+
   // The four 8-value MFMA operands (k sub-blocks j = 0..3) of one lane's 32 weights.
   __device__ static __forceinline__ void unpack(const WReg& w, v8h out[4]) {
-    if constexpr (WBITS == 4) {
+    if constexpr (WBITS == 8) {
+      // one byte per value, k order: byte b of a dword next to the constant byte 0x64 is the fp16 number 1024 + b
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        v4i o;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          o[2 * h] = (int)__builtin_amdgcn_perm(0x64646464u, (unsigned)w.d[2 * j + h], 0x04010400u);
+          o[2 * h + 1] = (int)__builtin_amdgcn_perm(0x64646464u, (unsigned)w.d[2 * j + h], 0x04030402u);
+        }
+        out[j] = __builtin_bit_cast(v8h, o);
+      }
+    } else if constexpr (WBITS == 4) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) out[j] = cvt8<0x000F000F, 0x00F000F0>(w.d[j]);
     } else if constexpr (WBITS == 3) {
@@ -110,7 +136,7 @@ struct SkinnyWoTile {
     const int K = t.K, KB = K / 128;
     const int lm = lane & 15, lg = lane >> 4;
     const v8h ones = {(_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f};
-    const v8h bias = {(_Float16)1024.0f, (_Float16)1024.0f, (_Float16)64.0f, (_Float16)64.0f, (_Float16)1024.0f, (_Float16)1024.0f, (_Float16)64.0f, (_Float16)64.0f};
+    const v8h bias = bias8();
     constexpr int Q = NB * NKB;  // blocks of this pass, channel block major
 
     // Everything the pass needs from memory is requested before anything is waited for, the weight ring first: the first blocks of
@@ -333,7 +359,7 @@ struct WoMfmaTile {
         sr[q] = s_of(q - 4, 1);
       }
       asm volatile("" ::: "memory");
-      const v8h bias = {(_Float16)1024.0f, (_Float16)1024.0f, (_Float16)64.0f, (_Float16)64.0f, (_Float16)1024.0f, (_Float16)1024.0f, (_Float16)64.0f, (_Float16)64.0f};
+      const v8h bias = Sk::bias8();
       // one k block; PAR = parity of kb, a compile-time constant so that the ring slots are fixed registers
       auto step = [&](auto parc, int kb) {
         constexpr int st = decltype(parc)::value;

@@ -27,16 +27,7 @@ __host__ __device__ inline int act_tag_of(const mxmoe_qparams& q) {  // ref_bind
   return -1;
 }
 
-__host__ __device__ inline int fmt_of(const mxmoe_qparams& q) {  // Fmt as an int (classify)
-  if (q.a_bits >= 16 && q.w_bits >= 16) return (int)Fmt::FP16;
-  if (q.a_bits == 8 && q.w_bits == 8 && q.gsize == -1 && q.sym) return (int)Fmt::W8A8;
-  if (q.a_bits == 4 && q.w_bits == 4 && q.gsize == -1 && q.sym) return (int)Fmt::W4A4;
-  if (q.a_bits == 4 && q.w_bits == 4 && q.gsize == 128 && q.sym) return (int)Fmt::W4A4G128;
-  if (q.a_bits >= 16 && q.w_bits == 4 && q.gsize == 128) return (int)Fmt::W4A16;
-  if (q.a_bits >= 16 && q.w_bits == 3 && q.gsize == 128) return (int)Fmt::W3A16;
-  if (q.a_bits >= 16 && q.w_bits == 2 && q.gsize == 128) return (int)Fmt::W2A16;
-  return (int)Fmt::UNSUPPORTED;
-}
+__host__ __device__ inline int fmt_of(const mxmoe_qparams& q) { return (int)classify(q); }
 
 struct PlanParams {
   const int64_t* recv;

@@ -180,6 +180,9 @@ def default_kernel_specs(arch: str = "gfx950"):
         ("groupgemm_ms_launch_all", KernelType.MultiStream, everything),
         # the same two kernels with w4a4 on the 6-bit float path: both operands of a w4a4 problem are bf6 fragments (the quantisers'
         # tag 4, pack.pack_bf6_fragments).  Registered last: a caller that does not ask for them by name never gets them.
+        # 8-bit weight-only formats in a kernel of their own (their tiles hold twice the packed registers of the 4-bit ones; a kernel
+        # runs at the occupancy of its largest branch)
+        ("groupgemm_hz_fused_wo8", KernelType.Fused, OrderedDict([("w8a16_g128_asym", _pick(arch, "w8a16_g128_asym", (16, 128), (128, 128)))])),
         ("groupgemm_hz_fused_wxax_b6", KernelType.Fused, OrderedDict([(w4, _pick(arch, w4, (128, 256), (64, 256), (32, 256), bf6=True)), (w8, _pick(arch, w8, (128, 256), (64, 256), (32, 256)))])),
         ("groupgemm_hz_fused_all_b6", KernelType.Fused, everything_b6),
     ]

@@ -29,14 +29,19 @@ TYPE_TO_BITS = {
     **dict.fromkeys(["int8_t", "uint8_t"], 8),
     **dict.fromkeys(["int4_t", "uint4_t"], 4),
     **dict.fromkeys(["int3_t", "uint3_t"], 3),
+    **dict.fromkeys(["int2_t", "uint2_t"], 2),
 }
+
+# weight-only formats: bits x group size (128, or -1 = one scale per channel) x symmetric / asymmetric (tile_config.py:40-59 lists
+# 8 / 4 / 2 bits with both group sizes; 3 bits is this library's addition)
+WEIGHT_ONLY_QCFG = [f"w{w}a16_g{g}_{s}" for w in (8, 4, 3, 2) for g in (128, -1) for s in ("sym", "asym")]
 
 SUPPORTED_QCFG = [
     "fp16",
     "w8a8_g-1_sym",
     "w4a4_g-1_sym",
     "w4a4_g128_sym",
-    *[f"w{w}a16_g128_{s}" for w in (4, 3, 2) for s in ("sym", "asym")],
+    *WEIGHT_ONLY_QCFG,
 ]
 
 # (M, N, K) of one MFMA instruction
@@ -60,7 +65,7 @@ QCFG_TO_MMA = {
     "w8a8_g-1_sym": "MFMA_I32_32x32x32_I8",
     "w4a4_g-1_sym": "MFMA_I32_32x32x32_I8_FROM_I4",
     "w4a4_g128_sym": "MFMA_I32_32x32x32_I8_FROM_I4",
-    **{f"w{w}a16_g128_{s}": "MFMA_F32_16x16x32_F16" for w in (4, 3, 2) for s in ("sym", "asym")},
+    **{q: "MFMA_F32_16x16x32_F16" for q in WEIGHT_ONLY_QCFG},
 }
 
 
@@ -248,7 +253,7 @@ QCFG_MAP = {
     "w8a8_g-1_sym": TileConfig(QCFGA=QCFG_W8A8, QCFGB=QCFG_W8A8),
     "w4a4_g-1_sym": TileConfig(QCFGA=QCFG_W4A4, QCFGB=QCFG_W4A4),
     "w4a4_g128_sym": TileConfig(QCFGA=QCFG_W4A4_G128, QCFGB=QCFG_W4A4_G128),
-    **{k: TileConfig(QCFGB=build_qcfgb_from_str(k)) for k in [f"w{w}a16_g128_{s}" for w in (4, 3, 2) for s in ("sym", "asym")]},
+    **{k: TileConfig(QCFGB=build_qcfgb_from_str(k)) for k in WEIGHT_ONLY_QCFG},
 }
 
 
@@ -263,7 +268,9 @@ def get_possible_tile_list(arch: str, qcfg: str) -> list:
     mma = QCFG_TO_MMA[qcfg]
     if mma == "MFMA_F32_16x16x32_F16":
         skinny = [_with_q(TileConfig(BM=16, BN=bn, BK=128, WM=1, WN=4, WK=1, STAGE=2, MMA=mma), qcfg) for bn in (128, 64)]
-        big = [_with_q(TileConfig(BM=128, BN=bn, BK=128, WM=wm, WN=wn, WK=1, STAGE=2, MMA=mma), qcfg) for bn, wm, wn in ((128, 2, 2), (256, 1, 4))]
+        # (8-bit weights: the ring of packed blocks is twice as large, which leaves room for the 2 x 2 shape's accumulators only)
+        shapes = ((128, 2, 2),) if QCFG_MAP[qcfg].QCFGB.QBITS == 8 else ((128, 2, 2), (256, 1, 4))
+        big = [_with_q(TileConfig(BM=128, BN=bn, BK=128, WM=wm, WN=wn, WK=1, STAGE=2, MMA=mma), qcfg) for bn, wm, wn in shapes]
         return skinny + big
     bk = {"MFMA_F32_32x32x16_F16": 32, "MFMA_I32_32x32x32_I8": 64, "MFMA_I32_32x32x32_I8_FROM_I4": 128}[mma]
     if mma == "MFMA_F32_32x32x16_F16":

@@ -62,12 +62,15 @@ def pack_weight_only(q: torch.Tensor, bits: int) -> torch.Tensor:
     bits == 3: dwords 0..2 hold values 0..23 in the low three bits of their nibbles; bit 3 of nibble p of
     dword d holds bit d of value 24 + e(p).
     bits == 2: dword d holds values 16d..16d+7 in the low two bits of its nibbles and values 16d+8..16d+15 in the high two.
+    bits == 8: one byte per value in k order, dword j = values 4j .. 4j+3 (8 dwords per lane).
     """
-    assert bits in (2, 3, 4)
+    assert bits in (2, 3, 4, 8)
     n, k = q.shape
     assert n % 16 == 0 and k % 128 == 0
     v = q.to(torch.int64).reshape(n // 16, 16, k // 128, 4, 32)       # [nb, row, kb, g, e32]
     v = v.permute(0, 2, 3, 1, 4).reshape(n // 16, k // 128, 64, 32)    # lane = g*16 + row
+    if bits == 8:
+        return v.to(torch.uint8).contiguous().view(torch.int32).reshape(-1).contiguous()
     shifts = torch.tensor([4 * p for p in _NIBBLE_OF_ELEM], dtype=torch.int64, device=q.device)
     if bits == 2:
         pairs = v.reshape(*v.shape[:-1], 2, 2, 8)                      # [.., dword, low / high half of the nibbles, e]

@@ -30,7 +30,7 @@ def quantize_and_pack(w: torch.Tensor, qparams, keep_codes: bool = False, bf6: b
     fragment blocks (`pack.pack_wxax_fragments`), fp16 scale [N].
     With `bf6`, w4a4 weights become bf6 fragments (`pack.pack_bf6_fragments`) for the kernels whose w4a4 tiles run on the 6-bit
     float matrix path; every other format is unaffected.
-    w4a16 / w3a16 group-128: unsigned codes in the wave-interleaved layout with a (scale, zero) table; symmetric
+    w8a16 / w4a16 / w3a16 / w2a16, group 128 or per channel (-1): unsigned codes in the wave-interleaved layout with a (scale, zero) table; symmetric
     variants are stored offset-binary with zero = -2^(b-1) * scale (exact).
     """
     a_bits, w_bits, gsize, sym = qparams
@@ -59,15 +59,17 @@ def pack_codes(q: torch.Tensor, scale: torch.Tensor, zp: torch.Tensor, qparams, 
             return PackedWeight(pack.pack_bf6_fragments(qi.reshape(n, k)), scale.reshape(n).contiguous(), tuple(qparams), n, k, qi if keep_codes else None)
         data = pack.pack_wxax_fragments(qi if w_bits == 8 else pack.pack_int4_k(qi))
         return PackedWeight(data, scale.reshape(n).contiguous(), tuple(qparams), n, k, qi if keep_codes else None)
-    assert gsize == 128, "weight-only kernels implement group size 128"
-    g = k // gsize
-    scale = scale.reshape(n, g)
-    zp = zp.reshape(n, g)
+    # weight-only: one (scale, zero) pair per channel and 128-wide K group.  Per-channel formats (group size -1) repeat the channel's
+    # pair for every group: the tiles apply the pair group by group either way.
+    assert gsize in (128, -1) and k % 128 == 0, "weight-only kernels take group size 128 or -1 (per channel), K a multiple of 128"
+    g = k // 128
+    scale = scale.reshape(n, -1).expand(n, g) if gsize == -1 else scale.reshape(n, g)
+    zp = zp.reshape(n, -1).expand(n, g) if gsize == -1 else zp.reshape(n, g)
     codes = q.reshape(n, k)
     if sym:
         off = 1 << (w_bits - 1)
         codes = codes + off
         zp = (-off * scale).to(scale.dtype)
     codes = codes.to(torch.uint8)
-    return PackedWeight(pack.pack_weight_only(codes, w_bits), pack.pack_weight_only_scales(scale, zp), tuple(qparams), n, k,
+    return PackedWeight(pack.pack_weight_only(codes, w_bits), pack.pack_weight_only_scales(scale.contiguous(), zp.contiguous()), tuple(qparams), n, k,
                         codes if keep_codes else None)

@@ -253,6 +253,33 @@ def test_weight_only_many_tokens():
         assert _rel(out, p["ref"]) <= 1e-2, (p["size"], p["q"], _rel(out, p["ref"]))
 
 
+def test_per_channel_and_eight_bit_weight_only_formats():
+    """The weight-only formats of the reference's generator beyond group 128 (mxmoe/kernels/tile_config.py:40-59; the kernel its
+    operator wires in is w4a16 per channel, asymmetric: mxmoe/kernels/src/ref_bind.cu:412-424, hz_fused.cuh:428-434): one scale per
+    channel (group size -1) for 4 / 3 / 2 bits, and 8-bit weights with either group size; few-token and many-token tiles, symmetric
+    and asymmetric, mixed in one launch per kernel.  Outputs within 1e-2 of the fake-quant path."""
+    from mxmoe_amd.weights import quantize_and_pack
+
+    rng = np.random.default_rng(31)
+    cases = [(3, 2816, 2048, 4, -1, False), (200, 256, 512, 4, -1, False), (16, 128, 1408, 3, -1, False), (150, 384, 1408, 2, -1, True), (5, 2048, 1408, 4, -1, True),
+             (3, 2816, 2048, 8, 128, False), (1, 256, 128, 8, -1, False), (200, 256, 512, 8, 128, True), (129, 384, 1408, 8, -1, True), (16, 160, 384, 8, 128, False),
+             (300, 2048, 1408, 8, -1, False)]
+    probs = []
+    for (m, n, k, bits, g, sym) in cases:
+        x = rng.standard_normal((m, k)).astype(F16)
+        w = (rng.standard_normal((n, k)) * 0.02).astype(F16)
+        pw = quantize_and_pack(torch.from_numpy(w), (16, bits, g, sym), keep_codes=True)
+        q, s, z = O.quant_minmax(w, bits, g, sym)
+        codes = q.reshape(n, k) + ((1 << (bits - 1)) if sym else 0)
+        assert np.array_equal(pw.q.numpy(), codes.astype(np.uint8))        # torch quantiser == oracle quantiser
+        probs.append(dict(A=torch.from_numpy(x).to(DEV), B=pw.data.to(DEV), sb=pw.scale.to(DEV), ref=O.gemm_fakequant(x, O.dequant(q, s, z, g)),
+                          size=(m, n, k), q=(16, bits, g, sym)))
+    for group in ([p for p in probs if p["q"][1] != 8], [p for p in probs if p["q"][1] == 8]):
+        g_, outs, _ = _launch(group, dump=False)
+        for p, out in zip(group, outs):
+            assert np.isfinite(out).all() and _rel(out, p["ref"]) <= 1e-2, (p["size"], p["q"], _rel(out, p["ref"]))
+
+
 def _any_problem(rng, fmt, m, n, k):
     from mxmoe_amd.weights import quantize_and_pack
 

@@ -103,7 +103,7 @@ def test_template_generator_product_and_sources(tmp_path):
     assert ('register_fused<WxAxTile<Op::I4, 128, 256>, WxAxTile<Op::I4, 64, 256>, WxAxTile<Op::I4, 32, 256>, WxAxTile<Op::I8, 128, 256>, '
             'WxAxTile<Op::I8, 64, 256>>("groupgemm_ms_launch_0", Policy::MultiStream)') in (tmp_path / "sets" / "ms_launch_0.hip").read_text()
     with pytest.raises(ValueError, match="Unsupported qcfg"):
-        TemplateGenerator("gfx950", ["w2a16_g-1_sym"])
+        TemplateGenerator("gfx950", ["w1a16_g128_sym"])
 
 
 def test_default_library_is_generator_output(tmp_path, lib):
