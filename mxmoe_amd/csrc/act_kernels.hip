@@ -293,6 +293,22 @@ __device__ __forceinline__ v8h bf6_chunk_codes(const float (&v)[8], const Div& d
   return o;
 }
 
+// ---- tag 5: per-token fp8 (OCP e4m3) codes for the kernels whose w8a8 tiles run the fp8 matrix instruction.  scale = max|x| / 448
+// (the largest e4m3 number) in fp16 like the integer scales; code = e4m3(clamp(fp16(x / scale), +-448)), round to nearest even; rows
+// are stored like int8 rows, one byte per value.
+template <class Div>
+__device__ __forceinline__ uint2 fp8_chunk_codes(const float (&v)[8], const Div& div) {
+  float r[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) r[j] = fminf(fmaxf(round_h(div(v[j])), -448.0f), 448.0f);
+  int lo = 0, hi = 0;
+  lo = __builtin_amdgcn_cvt_pk_fp8_f32(r[0], r[1], lo, false);
+  lo = __builtin_amdgcn_cvt_pk_fp8_f32(r[2], r[3], lo, true);
+  hi = __builtin_amdgcn_cvt_pk_fp8_f32(r[4], r[5], hi, false);
+  hi = __builtin_amdgcn_cvt_pk_fp8_f32(r[6], r[7], hi, true);
+  return make_uint2((unsigned)lo, (unsigned)hi);
+}
+
 // Codes of one row in LDS (fp16; value k at byte (k / row_elems) * pitch + (k % row_elems) * 2) -> the row's place in its expert's
 // fragment region.  Thread t of nt takes the groups of 32 codes t, t + nt, ...
 __device__ __forceinline__ void bf6_emit_row(const uint8_t* codes, int row_elems, int pitch, int n, uint8_t* region, long lrow, int t, int nt) {
@@ -663,7 +679,7 @@ __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
     amax = red[0];
 #pragma unroll
     for (int w = 1; w < NT / 64; ++w) amax = fmaxf(amax, red[w]);
-    const float upper = tag == 1 ? 127.0f : 7.0f;
+    const float upper = tag == 1 ? 127.0f : (tag == 5 ? 448.0f : 7.0f);
     float scale = round_h(amax / upper);   // fp16 division: fp32 quotient of two fp16 values, rounded to fp16
     if (scale == 0.0f) scale = 1.0f;       // quantize.cuh:258
     const ScaleDiv div(scale);
@@ -679,11 +695,15 @@ __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
       bf6_emit_row(codes, n, 0, n, a.inp_store + 2 * inp_off, lrow, tid, NT);
       continue;  // (the next row begins with a barrier before it touches LDS)
     }
-    uint8_t* out = a.inp_store + 2 * (inp_off + lrow * (tag == 1 ? n / 2 : n / 4));
+    uint8_t* out = a.inp_store + 2 * (inp_off + lrow * (tag == 1 || tag == 5 ? n / 2 : n / 4));
 #pragma unroll
     for (int i = 0; i < MAXC; ++i) {
       const int c = tid + i * NT;
       if (c < nchunks) {
+        if (tag == 5) {
+          *reinterpret_cast<uint2*>(out + c * 8) = fp8_chunk_codes(v[i], div);
+          continue;
+        }
         int q[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
@@ -839,7 +859,7 @@ __global__ void __launch_bounds__(256) row_quant_wave_kernel(const RowArgs a) {
       for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[i][j]));
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
-    const float upper = tag == 1 ? 127.0f : 7.0f;
+    const float upper = tag == 1 ? 127.0f : (tag == 5 ? 448.0f : 7.0f);
     float scale = round_h(amax / upper);   // fp16 division: fp32 quotient of two fp16 values, rounded to fp16
     if (scale == 0.0f) scale = 1.0f;       // quantize.cuh:258
     const ScaleDiv div(scale);
@@ -855,10 +875,14 @@ __global__ void __launch_bounds__(256) row_quant_wave_kernel(const RowArgs a) {
       __builtin_amdgcn_wave_barrier();  // the next row's codes come after these reads
       continue;
     }
-    uint8_t* out = a.inp_store + 2 * (inp_off + lrow * (tag == 1 ? n / 2 : n / 4));
+    uint8_t* out = a.inp_store + 2 * (inp_off + lrow * (tag == 1 || tag == 5 ? n / 2 : n / 4));
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
       const int c = lane + 64 * i;
+      if (tag == 5) {
+        *reinterpret_cast<uint2*>(out + c * 8) = fp8_chunk_codes(v[i], div);
+        continue;
+      }
       int q[8];
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
@@ -1153,7 +1177,7 @@ __global__ void __launch_bounds__(256) row_quant_dense_kernel(const RowArgs a) {
       for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[i][j]));  // chunks past the row hold zeros
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
-    const float upper = tag == 1 ? 127.0f : 7.0f;
+    const float upper = tag == 1 ? 127.0f : (tag == 5 ? 448.0f : 7.0f);
     float scale = round_h(amax / upper);   // fp16 division: fp32 quotient of two fp16 values, rounded to fp16
     if (scale == 0.0f) scale = 1.0f;       // quantize.cuh:258
     const ScaleDiv div(scale);
@@ -1171,11 +1195,15 @@ __global__ void __launch_bounds__(256) row_quant_dense_kernel(const RowArgs a) {
       __builtin_amdgcn_wave_barrier();  // the next row's writes come after these reads
       continue;
     }
-    uint8_t* out = a.inp_store + 2 * (inp_off + lrow * (tag == 1 ? n / 2 : n / 4));
+    uint8_t* out = a.inp_store + 2 * (inp_off + lrow * (tag == 1 || tag == 5 ? n / 2 : n / 4));
 #pragma unroll
     for (int i = 0; i < MAXC; ++i) {
       const int c = lane + 64 * i;
       if (c < nchunks) {
+        if (tag == 5) {
+          *reinterpret_cast<uint2*>(out + c * 8) = fp8_chunk_codes(v[i], div);
+          continue;
+        }
         int q[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
@@ -1412,7 +1440,7 @@ __global__ void __launch_bounds__(512) row_quant_wide_kernel(const RowArgs a) {
     amax = red[8];
 #pragma unroll
     for (int w = 1; w < 8; ++w) amax = fmaxf(amax, red[8 + w]);
-    const float upper = tag == 1 ? 127.0f : 7.0f;
+    const float upper = tag == 1 ? 127.0f : (tag == 5 ? 448.0f : 7.0f);
     float scale = round_h(amax / upper);   // fp16 division: fp32 quotient of two fp16 values, rounded to fp16
     if (scale == 0.0f) scale = 1.0f;       // quantize.cuh:258
     const ScaleDiv div(scale);
@@ -1429,12 +1457,16 @@ __global__ void __launch_bounds__(512) row_quant_wide_kernel(const RowArgs a) {
       __syncthreads();
       continue;
     }
-    uint8_t* out = a.inp_store + 2 * (inp_off + lrow * (tag == 1 ? n / 2 : n / 4));
+    uint8_t* out = a.inp_store + 2 * (inp_off + lrow * (tag == 1 || tag == 5 ? n / 2 : n / 4));
 #pragma unroll
     for (int i = 0; i < MAXC; ++i) {
       const int kr = wave + 8 * i;
       if (kr < kb) {
         const int c = kr * 64 + lane;
+        if (tag == 5) {
+          *reinterpret_cast<uint2*>(out + c * 8) = fp8_chunk_codes(v[i], div);
+          continue;
+        }
         int q[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) {

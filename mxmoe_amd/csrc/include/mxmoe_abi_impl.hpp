@@ -36,7 +36,7 @@ int mxmoe_kernel_branch(int kernel_id, int branch, int32_t out[8]) {
   const auto& k = registry()[kernel_id];
   if (branch < 0 || branch >= (int)k.branches.size()) { last_error() = "branch out of range"; return 2; }
   const BranchInfo& b = k.branches[branch];
-  out[0] = (int)b.fmt; out[1] = b.BM; out[2] = b.BN; out[3] = b.BK; out[4] = b.WGM; out[5] = b.WGN; out[6] = b.lds_bytes; out[7] = b.k_multiple;
+  out[0] = (int)b.fmt + 256 * b.variant; out[1] = b.BM; out[2] = b.BN; out[3] = b.BK; out[4] = b.WGM; out[5] = b.WGN; out[6] = b.lds_bytes; out[7] = b.k_multiple;
   return 0;
 }
 
@@ -78,7 +78,7 @@ int mxmoe_group_gemm_plan(int kernel_id, const mxmoe_dim3* h_sizes, const mxmoe_
   }
   if (kernel_id < 0) {
     for (int i = 0; i < (int)reg.size() && kernel_id < 0; ++i)
-      if (reg[i].policy == Policy::Fused && !kernel_takes_bf6(reg[i]) && kernel_covers(reg[i], h_q, problem_count)) kernel_id = i;
+      if (reg[i].policy == Policy::Fused && !kernel_has_variants(reg[i]) && kernel_covers(reg[i], h_q, problem_count)) kernel_id = i;
     if (kernel_id < 0) { last_error() = "quant type not supported"; return 1; }
   }
   if (kernel_id >= (int)reg.size()) { last_error() = "kernel id out of range"; return 2; }

@@ -244,7 +244,13 @@ struct BranchInfo {
   int k_multiple;  // K must be a multiple of this
   int max_m;       // largest M this branch accepts (skinny weight-only tiles), or 0 = any
   int k_min = 0;   // smallest K this branch accepts, or 0 = one k_multiple
+  // What QParams cannot say about the operands a branch takes: 0 as the format's table in the header says; 1 both operands of w4a4 as
+  // bf6 fragments (the tiles on the 6-bit float matrix path); 2 both operands of w8a8 as fp8 e4m3 codes with fp32 accumulation
+  // (w8a8_g-1_sym_E4M3, mxmoe/kernels/tile_config.py:45: QParams (8, 8, -1, sym) there as well).  A kernel with such a branch is
+  // never chosen automatically: the caller names it, because only the caller knows what its operands hold.
+  int variant = 0;
 };
+constexpr int kVariantBf6 = 1, kVariantFp8 = 2;
 
 template <class T>
 struct BranchOf;
@@ -267,7 +273,7 @@ template <Op OP, int BM, int BN>
 struct BranchOf<WxAxTile<OP, BM, BN>> {
   static BranchInfo get() {
     using T = WxAxTile<OP, BM, BN>;
-    return BranchInfo{OP == Op::I8 ? Fmt::W8A8 : Fmt::W4A4, BM, BN, T::BK, 1, 4, T::kLdsBytes, T::BK, 0};
+    return BranchInfo{OP == Op::I4 ? Fmt::W4A4 : Fmt::W8A8, BM, BN, T::BK, 1, 4, T::kLdsBytes, T::BK, 0, 0, OP == Op::F8 ? kVariantFp8 : 0};
   }
 };
 template <int BM>
@@ -276,7 +282,7 @@ struct BranchOf<Bf6Tile<BM>> {
   // fragments), so the two kinds never share a kernel: the kernel a caller picks says which layout its operands have
   static BranchInfo get() {
     using T = Bf6Tile<BM>;
-    return BranchInfo{Fmt::W4A4, BM, T::BN, T::BK, 1, 4, T::kLdsBytes, 128, 0, 256};
+    return BranchInfo{Fmt::W4A4, BM, T::BN, T::BK, 1, 4, T::kLdsBytes, 128, 0, 256, kVariantBf6};
   }
 };
 template <int WBITS, int BN>
@@ -534,7 +540,8 @@ int register_fused(const char* fn_name, Policy policy = Policy::Fused) {
   std::string n;
   for (const auto& b : k.branches) {
     char buf[160];
-    snprintf(buf, sizeof buf, "[%s: (%d,%d,%d) (%d,%d,1) 2], ", fmt_name(b.fmt, b.fmt == Fmt::W8A8 || b.fmt == Fmt::W4A4), b.BM, b.BN, b.BK, b.WGM, b.WGN);
+    snprintf(buf, sizeof buf, "[%s%s: (%d,%d,%d) (%d,%d,1) 2], ", fmt_name(b.fmt, b.fmt == Fmt::W8A8 || b.fmt == Fmt::W4A4), b.variant == kVariantFp8 ? "_E4M3" : "", b.BM, b.BN,
+             b.BK, b.WGM, b.WGN);
     n += buf;
     k.lds_bytes = std::max(k.lds_bytes, b.lds_bytes);
   }
@@ -553,15 +560,22 @@ int register_fused(const char* fn_name, Policy policy = Policy::Fused) {
   return id;
 }
 
-// Whether the kernel's w4a4 tiles run on the 6-bit float matrix path, i.e. take both operands as bf6 fragments.
-inline bool kernel_takes_bf6(const FusedKernel& k) {
+// Operand variant (BranchInfo::variant) of the kernel's tiles for format `f`, 0 when it has none or the plain ones.
+inline int kernel_variant(const FusedKernel& k, Fmt f) {
   for (const BranchInfo& b : k.branches)
-    if (b.fmt == Fmt::W4A4 && b.BK == 64) return true;
+    if (b.fmt == f && b.variant) return b.variant;
+  return 0;
+}
+inline bool kernel_takes_bf6(const FusedKernel& k) { return kernel_variant(k, Fmt::W4A4) == kVariantBf6; }
+inline bool kernel_has_variants(const FusedKernel& k) {
+  for (const BranchInfo& b : k.branches)
+    if (b.variant) return true;
   return false;
 }
 
 // A kernel can run a problem list when it has a branch for every format in it.  The automatic choice (kernel_id = -1) never
-// falls on a kernel that takes bf6 fragments: QParams do not say how the operands are laid out, so those kernels are asked for by id.
+// falls on a kernel with operand variants (bf6 fragments, fp8 codes): QParams do not say what the operands hold, so those kernels
+// are asked for by id.
 inline bool kernel_covers(const FusedKernel& k, const mxmoe_qparams* q, int count) {
   for (int i = 0; i < count; ++i) {
     const Fmt f = classify(q[i]);
@@ -699,7 +713,7 @@ inline int group_gemm(int kernel_id, const void* const* As, const void* const* B
   auto& reg = registry();
   if (kernel_id < 0) {
     for (int i = 0; i < (int)reg.size() && kernel_id < 0; ++i)
-      if (reg[i].policy == Policy::Fused && !kernel_takes_bf6(reg[i]) && kernel_covers(reg[i], h_q, count)) kernel_id = i;
+      if (reg[i].policy == Policy::Fused && !kernel_has_variants(reg[i]) && kernel_covers(reg[i], h_q, count)) kernel_id = i;
     if (kernel_id < 0) {
       last_error() = "quant type not supported";  // same message as the reference launcher (compose_kernel.py:433)
       return 1;

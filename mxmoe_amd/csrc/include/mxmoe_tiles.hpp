@@ -38,7 +38,7 @@ constexpr int kThreads = 256;  // workgroup size shared by every fused branch
 constexpr int kWaves = 4;
 constexpr int kRowBytes = 64;  // bytes of one operand row held in LDS per pipeline stage
 
-enum class Op { I8, I4, F16 };
+enum class Op { I8, I4, F16, F8 };  // F8: OCP e4m3 codes on the fp8 matrix instruction, fp32 accumulators
 
 // What one problem looks like to a tile.
 struct TileArgs {
@@ -158,6 +158,11 @@ template <>
 struct OpTraits<Op::F16> {
   using Acc = v16f;
   static constexpr int kBitsPerElem = 16;
+};
+template <>
+struct OpTraits<Op::F8> {
+  using Acc = v16f;
+  static constexpr int kBitsPerElem = 8;
 };
 
 // A BM x BN output tile computed by WGM x WGN waves with 32x32 MFMA blocks.
@@ -475,7 +480,7 @@ struct MfmaTile {
 // only the loads issued after this wave's activation loads of slice kt+1 are outstanding (a fixed count, see kYounger).
 template <Op OP, int BM_, int BN_>
 struct WxAxTile {
-  static_assert(OP == Op::I4 || OP == Op::I8, "integer formats only");
+  static_assert(OP == Op::I4 || OP == Op::I8 || OP == Op::F8, "one byte or half a byte per value");
   static constexpr Op kOp = OP;
   static constexpr int BM = BM_, BN = BN_, WGM = 1, WGN = 4;
   static constexpr int TM = BM, TN = BN / 4;
@@ -505,7 +510,22 @@ struct WxAxTile {
   static constexpr int kYounger = (U - (kDma - 1)) + (kDma < 2 ? kDma : 2) + 2;
   // K slices of weight fragments in flight per wave: int8 slices are half as long in time, so they are fetched further ahead
   static constexpr int kDepth = OP == Op::I4 ? 2 : 4;
-  using Acc = v16i;
+  using Acc = typename OpTraits<OP>::Acc;
+
+  // One 16-byte fragment pair of the byte formats.  int8: one instruction over the 32 k of the pair.  fp8 (e4m3): two instructions of
+  // 16 k, the first on the low 8 bytes of both lanes' fragments, the second on the high 8; which k a byte stands for is the same on
+  // both sides, and the sum runs over all of them either way (w8a8_g-1_sym_E4M3 of the reference: MMA_E4M3_K32,
+  // mxmoe/kernels/src/include/mm_tile.cuh:696-697).
+  __device__ static __forceinline__ void mma_bytes(Acc& c, const v4i& w, const v4i& a) {
+    if constexpr (OP == Op::F8) {
+      typedef long v2l __attribute__((ext_vector_type(2)));
+      const v2l wl = __builtin_bit_cast(v2l, w), al = __builtin_bit_cast(v2l, a);
+      c = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(wl[0], al[0], c, 0, 0, 0);
+      c = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(wl[1], al[1], c, 0, 0, 0);
+    } else {
+      c = __builtin_amdgcn_mfma_i32_32x32x32_i8(w, a, c, 0, 0, 0);
+    }
+  }
 
   // Vector-memory loads a wave issues in units a..b of one iteration: one weight fragment per unit, plus one activation load in
   // each of the first nd units (before the fragment).
@@ -590,8 +610,8 @@ struct WxAxTile {
     v4i pa[FM];              // int4: packed activation fragments of the next k-step
 
     auto mma = [&](Acc& c, const v4i* a, const v4i* b) {
-      c = __builtin_amdgcn_mfma_i32_32x32x32_i8(b[0], a[0], c, 0, 0, 0);
-      if constexpr (OP == Op::I4) c = __builtin_amdgcn_mfma_i32_32x32x32_i8(b[1], a[1], c, 0, 0, 0);
+      mma_bytes(c, b[0], a[0]);
+      if constexpr (OP == Op::I4) mma_bytes(c, b[1], a[1]);
     };
 
     // ---- prologue: slices 0 .. kDepth-2 complete, then the load pattern of one (virtual) iteration for slice kDepth-1, so that
@@ -681,7 +701,7 @@ struct WxAxTile {
             sched_mfma_valu<12 + (j == FN - 1 ? 12 * FM : 0), 2 * FM, 0>();
           } else {
 #pragma unroll
-            for (int i = 0; i < FM; ++i) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(pbq[P][j][step], aop[step][i][0], acc[i][j], 0, 0, 0);
+            for (int i = 0; i < FM; ++i) mma_bytes(acc[i][j], pbq[P][j][step], aop[step][i][0]);
           }
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -734,7 +754,9 @@ struct WxAxTile {
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
             const int m = m0 + i * 32 + lrow, n = n0 + wave * TN + j * 32 + (r / 4) * 8 + nq + (r & 3);
-            int a = (int)acc[i][j][r];
+            const auto v = acc[i][j][r];
+            int a;
+            if constexpr (OP == Op::F8) a = __builtin_bit_cast(int, (float)v); else a = (int)v;  // fp8: the fp32 sum's bit pattern
             if constexpr (OP == Op::I4) a >>= 8;  // exact
             if (m < M && n < N) gstore<int>(t.acc_dump + (long)m * N + n, a);
           }

@@ -14,12 +14,15 @@
 
 namespace mxmoe {
 
-// A block descriptor (not the QParams arrays of the launcher, whose padding bytes belong to the caller) may ask for the int4 codes of
-// per-token activations as bf6 fragments, the operand layout of the kernels whose w4a4 tiles run on the 6-bit float matrix path.
+// A block descriptor (not the QParams arrays of the launcher, whose padding bytes belong to the caller) may name an operand variant
+// in q._pad[0]: 1 = the int4 codes of per-token activations as bf6 fragments (for the kernels whose w4a4 tiles run on the 6-bit float
+// matrix path), 2 = per-token fp8 e4m3 codes instead of int8 ones (for the kernels whose w8a8 tiles run the fp8 instruction).
 __host__ __device__ inline bool wants_bf6(const mxmoe_qparams& q) { return q._pad[0] == 1 && q.a_bits == 4 && q.w_bits == 4 && q.gsize == -1; }
+__host__ __device__ inline bool wants_fp8(const mxmoe_qparams& q) { return q._pad[0] == 2 && q.a_bits == 8 && q.w_bits == 8 && q.gsize == -1; }
 
 __host__ __device__ inline int act_tag_of(const mxmoe_qparams& q) {  // ref_bind.cu:461-473
   if (q.a_bits >= 16) return 0;
+  if (wants_fp8(q)) return 5;
   if (q.a_bits == 8 && q.gsize == -1) return 1;
   if (wants_bf6(q)) return 4;
   if (q.a_bits == 4 && q.gsize == -1) return 2;
@@ -84,7 +87,7 @@ __global__ void __launch_bounds__(kPlanThreads) plan_block_kernel(const PlanPair
     fmt = fmt_of(d.q);
     N = (int)d.N;
     K = (int)d.K;
-    qld = tag == 0 ? K : (tag == 1 ? K / 2 : K / 4);  // fp16 elements per packed activation row (ref_bind.cu:491); unused for tag 4
+    qld = tag == 0 ? K : (tag == 1 || tag == 5 ? K / 2 : K / 4);  // fp16 elements per packed activation row (ref_bind.cu:491); unused for tag 4
     sld = tag == 0 ? 0 : (tag == 3 ? K / 128 : 1);   // scales per row (ref_bind.cu:492)
     out_ld = N;
   }
@@ -259,6 +262,7 @@ static int resolve_kernel(int kernel_id, const mxmoe_block_desc* h_desc, int et)
       if (f == (int)Fmt::UNSUPPORTED || plan_segments(plan_of(k), f, 1, 256, sg) < 0) return false;
       // a kernel's w4a4 tiles take packed int4 rows or bf6 fragments, never both: the descriptor says which the block will get
       if (f == (int)Fmt::W4A4 && kernel_takes_bf6(k) != wants_bf6(h_desc[i].q)) return false;
+      if (f == (int)Fmt::W8A8 && (kernel_variant(k, Fmt::W8A8) == kVariantFp8) != wants_fp8(h_desc[i].q)) return false;
     }
     return true;
   };

@@ -83,7 +83,7 @@ def bench_func(fn, warmup: int = 20, iters: int = 50, max_warm_s: float = 10.0) 
     return {"min": ts[0], "max": ts[-1], "mean": sum(trim) / len(trim), "median": ts[len(ts) // 2]}
 
 
-def make_problem(entry: dict, gen: torch.Generator, device="cuda", keep_ref: bool = False, bf6: bool = False) -> dict:
+def make_problem(entry: dict, gen: torch.Generator, device="cuda", keep_ref: bool = False, bf6: bool = False, fp8: bool = False) -> dict:
     """Random fp16 operands for one workload entry, quantised and packed for its format (QInput::from_fp16).  `bf6`: w4a4 operands as
     bf6 fragments, the layout of the kernels whose w4a4 tiles run on the 6-bit float matrix path (`kernel_takes_bf6`)."""
     m, n, k = entry["shape"]
@@ -94,12 +94,19 @@ def make_problem(entry: dict, gen: torch.Generator, device="cuda", keep_ref: boo
     else:
         a = (torch.rand(m, k, generator=gen, dtype=torch.float32) * 2 - 1).to(torch.float16).to(device)
         b = (torch.rand(n, k, generator=gen, dtype=torch.float32) * 2 - 1).to(torch.float16).to(device)
-    pw = quantize_and_pack(b, qp, bf6=bf6)
+    fp8 = fp8 and qp[:3] == (8, 8, -1)
+    pw = quantize_and_pack(b, qp, bf6=bf6, fp8=fp8)
     prob = {"size": (m, n, k), "q": qp, "B": pw.data, "sb": pw.scale, "C": torch.zeros(m, n, dtype=torch.float16, device=device)}
     if qp[0] < 16:
         ag = qp[2] if qp[2] > 0 else -1                      # group-quantised activations (w4a4_g128_sym): scales [M, K / 128]
-        qa, sa, _ = quant_minmax(a, qp[0], ag, True) if m else (a, a[:, :1], None)
-        qi = qa.reshape(m, k).to(torch.int8)
+        if fp8:
+            from .quant import quant_e4m3
+
+            qa, sa = quant_e4m3(a) if m else (a.view(torch.uint8)[:, :k], a[:, :1])
+            qi = qa.reshape(m, k).view(torch.int8)
+        else:
+            qa, sa, _ = quant_minmax(a, qp[0], ag, True) if m else (a, a[:, :1], None)
+            qi = qa.reshape(m, k).to(torch.int8)
         prob["A"] = qi.contiguous() if qp[0] == 8 else (pack.pack_bf6_fragments(qi) if bf6 and qp[2] == -1 and qp[1] == 4 else pack.pack_int4_k(qi))
         prob["sa"] = sa.reshape(-1).contiguous()
     else:
@@ -110,15 +117,17 @@ def make_problem(entry: dict, gen: torch.Generator, device="cuda", keep_ref: boo
 
 
 def kernel_takes_bf6(lib, kid: int) -> bool:
-    """Whether kernel `kid` has w4a4 tiles on the 6-bit float matrix path (64-wide K steps): its w4a4 operands are bf6 fragments."""
-    import ctypes as C
+    """Whether kernel `kid` has w4a4 tiles on the 6-bit float matrix path: its w4a4 operands are bf6 fragments."""
+    from .ops import kernel_variants
 
-    out = (C.c_int32 * 8)()
-    for b in range(lib.mxmoe_kernel_num_branches(kid)):
-        lib.mxmoe_kernel_branch(kid, b, out)
-        if out[0] == 2 and out[3] == 64:
-            return True
-    return False
+    return kernel_variants(lib, kid).get(2) == 1
+
+
+def kernel_takes_fp8(lib, kid: int) -> bool:
+    """Whether kernel `kid` runs its w8a8 problems on the fp8 instruction: their operands are e4m3 codes, not int8 ones."""
+    from .ops import kernel_variants
+
+    return kernel_variants(lib, kid).get(1) == 2
 
 
 def _launch_of(probs, lib, kernel_id=-1) -> GroupGemmLaunch:
@@ -170,7 +179,7 @@ def bench_one_case(entries, lib=None, mode: str = "bench", filters=(), out_file:
     gen.manual_seed(42)
     probs = [make_problem(e, gen, keep_ref=(mode == "check")) for e in entries]
     probs = [p for p in probs if p["size"][0] > 0]
-    probs_b6 = None  # the same problems with their w4a4 operands as bf6 fragments, made when a kernel asks for them
+    variants = {}    # the same problems with operand variants (w4a4 as bf6 fragments, w8a8 as fp8 codes), made when a kernel asks for them
 
     # fp16 baseline on the same shapes (role of the CUTLASS grouped GEMM, test.cu:774-781)
     gen2 = torch.Generator(device="cpu")
@@ -186,11 +195,12 @@ def bench_one_case(entries, lib=None, mode: str = "bench", filters=(), out_file:
         if filters and not any(f in name for f in filters):
             continue
         mine = probs
-        if kernel_takes_bf6(lib, kid) and any(p["q"][:3] == (4, 4, -1) for p in probs):
-            if probs_b6 is None:
+        want = (kernel_takes_bf6(lib, kid) and any(p["q"][:3] == (4, 4, -1) for p in probs), kernel_takes_fp8(lib, kid) and any(p["q"][:3] == (8, 8, -1) for p in probs))
+        if any(want):
+            if want not in variants:
                 gen.manual_seed(42)
-                probs_b6 = [make_problem(e, gen, keep_ref=(mode == "check"), bf6=True) for e in entries if e["shape"][0] > 0]
-            mine = probs_b6
+                variants[want] = [make_problem(e, gen, keep_ref=(mode == "check"), bf6=want[0], fp8=want[1]) for e in entries if e["shape"][0] > 0]
+            mine = variants[want]
         g = _launch_of(mine, lib, kid)
         try:
             g.plan()

@@ -183,6 +183,9 @@ def default_kernel_specs(arch: str = "gfx950"):
         # 8-bit weight-only formats in a kernel of their own (their tiles hold twice the packed registers of the 4-bit ones; a kernel
         # runs at the occupancy of its largest branch)
         ("groupgemm_hz_fused_wo8", KernelType.Fused, OrderedDict([("w8a16_g128_asym", _pick(arch, "w8a16_g128_asym", (16, 128), (128, 128)))])),
+        # w8a8 in fp8 (e4m3 codes on both sides), next to w4a4
+        ("groupgemm_hz_fused_wxax_e4m3", KernelType.Fused, OrderedDict([(w4, _pick(arch, w4, (128, 256), (64, 256), (32, 256))),
+                                                                         ("w8a8_g-1_sym_E4M3", _pick(arch, "w8a8_g-1_sym_E4M3", (128, 256), (64, 256), (32, 256)))])),
         ("groupgemm_hz_fused_wxax_b6", KernelType.Fused, OrderedDict([(w4, _pick(arch, w4, (128, 256), (64, 256), (32, 256), bf6=True)), (w8, _pick(arch, w8, (128, 256), (64, 256), (32, 256)))])),
         ("groupgemm_hz_fused_all_b6", KernelType.Fused, everything_b6),
     ]

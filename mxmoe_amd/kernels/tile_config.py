@@ -39,6 +39,7 @@ WEIGHT_ONLY_QCFG = [f"w{w}a16_g{g}_{s}" for w in (8, 4, 3, 2) for g in (128, -1)
 SUPPORTED_QCFG = [
     "fp16",
     "w8a8_g-1_sym",
+    "w8a8_g-1_sym_E4M3",  # fp8 (OCP e4m3) codes on both sides, fp32 accumulation (tile_config.py:45)
     "w4a4_g-1_sym",
     "w4a4_g128_sym",
     *WEIGHT_ONLY_QCFG,
@@ -53,16 +54,18 @@ MMA_SHAPE = {
     # int4 values held as 6-bit floats (bf6, e3m2: every integer -8 .. 8 is one) on v_mfma_scale_f32_32x32x64_f8f6f4 with unit
     # scales: the fp32 accumulators are the exact integer sums, at twice the int8 instruction's rate
     "MFMA_F32_32x32x64_BF6_FROM_I4": (32, 32, 64),
+    "MFMA_F32_32x32x16_FP8": (32, 32, 16),
 }
 MMA_TO_ACC_TYPE = {"MFMA_F32_32x32x16_F16": "float", "MFMA_I32_32x32x32_I8": "int32_t", "MFMA_I32_32x32x32_I8_FROM_I4": "int32_t", "MFMA_F32_16x16x32_F16": "float",
-                   "MFMA_F32_32x32x64_BF6_FROM_I4": "float"}
+                   "MFMA_F32_32x32x64_BF6_FROM_I4": "float", "MFMA_F32_32x32x16_FP8": "float"}
 MMA_TO_INP_TYPE = {"MFMA_F32_32x32x16_F16": "half", "MFMA_I32_32x32x32_I8": "int8_t", "MFMA_I32_32x32x32_I8_FROM_I4": "int4_t", "MFMA_F32_16x16x32_F16": "half",
-                   "MFMA_F32_32x32x64_BF6_FROM_I4": "int4_t"}
+                   "MFMA_F32_32x32x64_BF6_FROM_I4": "int4_t", "MFMA_F32_32x32x16_FP8": "fp8e4m3"}
 BF6_MMA = "MFMA_F32_32x32x64_BF6_FROM_I4"
 
 QCFG_TO_MMA = {
     "fp16": "MFMA_F32_32x32x16_F16",
     "w8a8_g-1_sym": "MFMA_I32_32x32x32_I8",
+    "w8a8_g-1_sym_E4M3": "MFMA_F32_32x32x16_FP8",
     "w4a4_g-1_sym": "MFMA_I32_32x32x32_I8_FROM_I4",
     "w4a4_g128_sym": "MFMA_I32_32x32x32_I8_FROM_I4",
     **{q: "MFMA_F32_16x16x32_F16" for q in WEIGHT_ONLY_QCFG},
@@ -110,6 +113,7 @@ class QConfig(QConfigBase):
 
 
 QCFG_W8A8 = QConfig(QBITS=8, GSIZE=-1, SYM=True, PACK_DIM="PackDim::K")
+QCFG_W8A8_E4M3 = QConfig(QBITS=8, GSIZE=-1, SYM=True, PACK_DIM="PackDim::K", USE_FP=True)
 QCFG_W4A4 = QConfig(QBITS=4, GSIZE=-1, SYM=True, PACK_DIM="PackDim::K")
 QCFG_W4A4_G128 = QConfig(QBITS=4, GSIZE=128, SYM=True, PACK_DIM="PackDim::K")
 
@@ -206,7 +210,7 @@ class TileConfig:
             return f"WoMfmaTile<{self.QCFGB.QBITS}, {self.BM}, {self.BN}>"
         if self.is_bf6():
             return f"Bf6Tile<{self.BM}>"
-        op = {"MFMA_F32_32x32x16_F16": "Op::F16", "MFMA_I32_32x32x32_I8": "Op::I8", "MFMA_I32_32x32x32_I8_FROM_I4": "Op::I4"}[self.MMA]
+        op = {"MFMA_F32_32x32x16_F16": "Op::F16", "MFMA_I32_32x32x32_I8": "Op::I8", "MFMA_I32_32x32x32_I8_FROM_I4": "Op::I4", "MFMA_F32_32x32x16_FP8": "Op::F8"}[self.MMA]
         if self.is_group_wa():
             return f"WxAxGTile<{self.BM}>"
         if op != "Op::F16":
@@ -224,7 +228,7 @@ class TileConfig:
             if (self.BN, self.BK, self.WM, self.WN, self.WK, self.STAGE) != (256, 64, 1, 4, 1, 4) or self.BM not in (32, 64, 128):
                 raise ValueError(f"{self!r}: bf6 tiles are BM x 256 x 64 with 1 x 4 waves and 4 stages, BM in 32 / 64 / 128")
             return
-        k_elems = {"MFMA_F32_32x32x16_F16": 32, "MFMA_I32_32x32x32_I8": 64, "MFMA_I32_32x32x32_I8_FROM_I4": 128}[self.MMA]
+        k_elems = {"MFMA_F32_32x32x16_F16": 32, "MFMA_I32_32x32x32_I8": 64, "MFMA_I32_32x32x32_I8_FROM_I4": 128, "MFMA_F32_32x32x16_FP8": 64}[self.MMA]
         if self.BK != k_elems or self.STAGE != 3 or self.WK != 1 or (self.BM // self.WM) % 32 or (self.BN // self.WN) % 32:
             raise ValueError(f"{self!r}: unsupported shape for {self.MMA} (BK must be {k_elems}, STAGE 3, wave tile a multiple of 32x32)")
         if self.is_group_wa() and self.BM not in (32, 64):
@@ -251,6 +255,7 @@ def build_qcfgb_from_str(qcfg: str) -> QConfig:
 QCFG_MAP = {
     "fp16": TileConfig(),
     "w8a8_g-1_sym": TileConfig(QCFGA=QCFG_W8A8, QCFGB=QCFG_W8A8),
+    "w8a8_g-1_sym_E4M3": TileConfig(QCFGA=QCFG_W8A8_E4M3, QCFGB=QCFG_W8A8_E4M3),
     "w4a4_g-1_sym": TileConfig(QCFGA=QCFG_W4A4, QCFGB=QCFG_W4A4),
     "w4a4_g128_sym": TileConfig(QCFGA=QCFG_W4A4_G128, QCFGB=QCFG_W4A4_G128),
     **{k: TileConfig(QCFGB=build_qcfgb_from_str(k)) for k in WEIGHT_ONLY_QCFG},
@@ -272,7 +277,7 @@ def get_possible_tile_list(arch: str, qcfg: str) -> list:
         shapes = ((128, 2, 2),) if QCFG_MAP[qcfg].QCFGB.QBITS == 8 else ((128, 2, 2), (256, 1, 4))
         big = [_with_q(TileConfig(BM=128, BN=bn, BK=128, WM=wm, WN=wn, WK=1, STAGE=2, MMA=mma), qcfg) for bn, wm, wn in shapes]
         return skinny + big
-    bk = {"MFMA_F32_32x32x16_F16": 32, "MFMA_I32_32x32x32_I8": 64, "MFMA_I32_32x32x32_I8_FROM_I4": 128}[mma]
+    bk = {"MFMA_F32_32x32x16_F16": 32, "MFMA_I32_32x32x32_I8": 64, "MFMA_I32_32x32x32_I8_FROM_I4": 128, "MFMA_F32_32x32x16_FP8": 64}[mma]
     if mma == "MFMA_F32_32x32x16_F16":
         shapes = [(128, 256, 2, 2), (64, 256, 1, 4), (32, 256, 1, 4), (128, 128, 2, 2), (256, 128, 2, 2)]
     elif qcfg == "w4a4_g128_sym":

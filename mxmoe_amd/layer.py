@@ -18,14 +18,17 @@ from .weights import quantize_and_pack
 
 
 class MxMoELayer:
-    def __init__(self, cfg: MoEConfig, device="cuda", formats=None, weights=None, keep_codes: bool = False, packed=None, bf6: bool = False):
+    def __init__(self, cfg: MoEConfig, device="cuda", formats=None, weights=None, keep_codes: bool = False, packed=None, bf6: bool = False, fp8: bool = False):
         """weights: [(W13, W2)] fp16 per expert (default: the configuration's seeded synthetic weights); packed: ([PackedWeight] for
         gate_up, [PackedWeight] for down) already quantised and packed, e.g. from `checkpoint.load_layer` (formats are taken from them).
         bf6: run the w4a4 blocks on the 6-bit float matrix path: their weights are packed as bf6 fragments, the quantisers write their
         activations as bf6 fragments (tag 4) and the launch uses a kernel whose w4a4 tiles take that layout.  Same integer codes, same
         accumulators and outputs, bit for bit; the operands occupy 0.75 instead of 0.5 bytes per value.  One flag for both linear
-        blocks, or a pair (gate_up, down)."""
+        blocks, or a pair (gate_up, down).
+        fp8: run the w8a8 blocks in fp8 (OCP e4m3 codes for weights and activations, fp32 accumulation on the fp8 matrix instruction;
+        the reference's w8a8_g-1_sym_E4M3) instead of int8.  A different number format: results differ from the int8 layer's."""
         self.cfg = cfg
+        self.fp8 = bool(fp8)
         self.bf6_gate_up, self.bf6_down = (bool(bf6[0]), bool(bf6[1])) if isinstance(bf6, (tuple, list)) else (bool(bf6), bool(bf6))
         self.device = torch.device(device)
         self.n_exp_total = cfg.num_experts + (1 if cfg.num_shared else 0)
@@ -42,12 +45,12 @@ class MxMoELayer:
         for e in range(self.n_exp_total if packed is None else 0):
             w13, w2 = weights[e] if weights is not None else expert_weights(cfg, e)
             gu, dn = self.formats[e]
-            self.w13.append(quantize_and_pack(w13.to(self.device), gu, keep_codes, bf6=self.bf6_gate_up))
-            self.w2.append(quantize_and_pack(w2.to(self.device), dn, keep_codes, bf6=self.bf6_down))
+            self.w13.append(quantize_and_pack(w13.to(self.device), gu, keep_codes, bf6=self.bf6_gate_up, fp8=self.fp8))
+            self.w2.append(quantize_and_pack(w2.to(self.device), dn, keep_codes, bf6=self.bf6_down, fp8=self.fp8))
         self.qp_gate_up = [f[0] for f in self.formats]
         self.qp_down = [f[1] for f in self.formats]
-        self.kid_gate_up = ops.select_kernel(self.qp_gate_up, self.bf6_gate_up)
-        self.kid_down = ops.select_kernel(self.qp_down, self.bf6_down)
+        self.kid_gate_up = ops.select_kernel(self.qp_gate_up, self.bf6_gate_up, self.fp8)
+        self.kid_down = ops.select_kernel(self.qp_down, self.bf6_down, self.fp8)
         self.state = None
         self._static = None
 
@@ -63,7 +66,7 @@ class MxMoELayer:
         topk_ids = topk_ids.to(self.device)
         st = {}
         (st["inp"], st["sa"], st["mid"], st["inp_store"], st["sa_store"], st["mid_store"], st["recv"], st["perm"], st["dst"]) = ops.quant_inp_act(
-            hidden, topk_ids, cfg.num_experts, cfg.inter, cfg.num_shared, self.qp_gate_up, rotate=cfg.rotate, bf6=self.bf6_gate_up)
+            hidden, topk_ids, cfg.num_experts, cfg.inter, cfg.num_shared, self.qp_gate_up, rotate=cfg.rotate, bf6=self.bf6_gate_up, fp8=self.fp8)
         i_sh = cfg.inter * max(cfg.num_shared, 1)
         acc1 = [torch.zeros(m.shape, dtype=torch.int32, device=self.device) for m in st["mid"]] if dump_acc else None
         st["gg1"] = ops.prepare_gg(st["inp"], [w.data for w in self.w13], st["sa"], [w.scale for w in self.w13], st["mid"], 2 * cfg.inter, cfg.hidden,
@@ -81,7 +84,7 @@ class MxMoELayer:
         cfg, st = self.cfg, self.state
         (st["inp2"], st["sa2"], st["out"], st["inp2_store"], st["sa2_store"], st["out_store"]) = ops.silu_mul_then_quant(
             st["mid_store"], len(st["mid"]), cfg.num_experts, cfg.hidden, cfg.inter, cfg.num_shared, cfg.tokens, cfg.topk, st["dst"], st["recv"],
-            self.qp_down, rotate=cfg.rotate, bf6=self.bf6_down)
+            self.qp_down, rotate=cfg.rotate, bf6=self.bf6_down, fp8=self.fp8)
         i_sh = cfg.inter * max(cfg.num_shared, 1)
         acc2 = [torch.zeros(o.shape, dtype=torch.int32, device=self.device) for o in st["out"]] if st["dump_acc"] else None
         st["gg2"] = ops.prepare_gg(st["inp2"], [w.data for w in self.w2], st["sa2"], [w.scale for w in self.w2], st["out"], cfg.hidden, cfg.inter,
@@ -119,8 +122,8 @@ class MxMoELayer:
             def ptrs(ws):
                 return [w.data.data_ptr() for w in ws], [0 if w.scale is None else w.scale.data_ptr() for w in ws]
 
-            self._static = (LT.static_block(self.qp_gate_up, gu_w, gu_n, *ptrs(self.w13), bf6=self.bf6_gate_up),
-                            LT.static_block(self.qp_down, dn_w, dn_n, *ptrs(self.w2), bf6=self.bf6_down))
+            self._static = (LT.static_block(self.qp_gate_up, gu_w, gu_n, *ptrs(self.w13), bf6=self.bf6_gate_up, fp8=self.fp8),
+                            LT.static_block(self.qp_down, dn_w, dn_n, *ptrs(self.w2), bf6=self.bf6_down, fp8=self.fp8))
         return self._static
 
     # ---- the forward that never waits for its routing ---------------------------------------------------------
@@ -146,7 +149,8 @@ class MxMoELayer:
             h = (_lib.BlockDesc * et)()
             for e in range(et):
                 a, w, g, sym = qps[e]
-                layout = (C.c_uint8 * 3)(1 if bf6 and (int(a), int(w), int(g)) == (4, 4, -1) else 0, 0, 0)  # 1: activations as bf6 fragments
+                variant = 1 if bf6 and (int(a), int(w), int(g)) == (4, 4, -1) else (2 if self.fp8 and (int(a), int(w), int(g)) == (8, 8, -1) else 0)
+                layout = (C.c_uint8 * 3)(variant, 0, 0)  # operand variant: 1 activations as bf6 fragments, 2 fp8 e4m3 codes
                 h[e] = _lib.BlockDesc(int(a), int(w), int(g), 1 if sym else 0, layout, int(ns[e]), int(ks[e]), ws[e].data.data_ptr(),
                                       0 if ws[e].scale is None else ws[e].scale.data_ptr())
             d = torch.frombuffer(bytearray(bytes(h)), dtype=torch.uint8).to(dev)
@@ -157,9 +161,9 @@ class MxMoELayer:
             if grid < 0:
                 raise RuntimeError(lib.mxmoe_last_error().decode())
             # worst-case stores: every routed row as wide as the widest routed expert's packed row
-            tags = [ops.act_tag(int(q[0]), int(q[2]), bf6 and int(q[1]) == 4) for q in qps]
+            tags = [ops.act_tag(int(q[0]), int(q[2]), bf6 and int(q[1]) == 4, self.fp8 and int(q[1]) == 8) for q in qps]
             # fp16 elements per row; bf6 fragments (tag 4) take 3/8 of an element per value and whole blocks of 32 rows per expert
-            qld = [k * 3 // 8 if tg == 4 else (k if tg == 0 else (k // 2 if tg == 1 else k // 4)) for tg, k in zip(tags, ks)]
+            qld = [k * 3 // 8 if tg == 4 else (k if tg == 0 else (k // 2 if tg in (1, 5) else k // 4)) for tg, k in zip(tags, ks)]
             sld = [0 if tg == 0 else (k // 128 if tg == 3 else 1) for tg, k in zip(tags, ks)]
             sh = [e_cnt] if has_shared else []
             pad = 32 * e_cnt if 4 in tags else 0

@@ -29,22 +29,22 @@ class BlockStatic:
     q: np.ndarray        # int32 [Et, 4] (a_bits, w_bits, gsize, sym) in the 16-byte QParams layout
 
 
-def static_block(qparams, widths, ns, b_ptrs, sb_ptrs, bf6: bool = False) -> BlockStatic:
+def static_block(qparams, widths, ns, b_ptrs, sb_ptrs, bf6: bool = False, fp8: bool = False) -> BlockStatic:
     """`qparams[e]`, input width `widths[e]`, output channels `ns[e]`, weight and scale addresses per expert; `bf6`: per-token int4
-    activations are bf6 fragments (tag 4)."""
+    activations are bf6 fragments (tag 4); `fp8`: per-token 8-bit activations are fp8 e4m3 codes (tag 5)."""
     et = len(qparams)
     tag = np.empty(et, np.int64)
     qld = np.empty(et, np.int64)
     sld = np.empty(et, np.int64)
     for e, (a_bits, w_bits, g, _s) in enumerate(qparams):
-        t = act_tag(int(a_bits), int(g), bf6 and int(w_bits) == 4)
+        t = act_tag(int(a_bits), int(g), bf6 and int(w_bits) == 4, fp8 and int(w_bits) == 8)
         if t < 0:
             raise RuntimeError("quant type not supported")
         w = int(widths[e])
         if t == 3 and w % 128:
             raise RuntimeError(f"group-128 activations need a row length that is a multiple of 128, got {w}")
         tag[e] = t
-        qld[e] = w if t == 0 else (w // 2 if t == 1 else w // 4)     # (tag 4: unused, see block_tables)
+        qld[e] = w if t == 0 else (w // 2 if t in (1, 5) else w // 4)     # (tag 4: unused, see block_tables)
         sld[e] = 0 if t == 0 else (w // 128 if t == 3 else 1)
     q = np.array([[int(a), int(w), int(g), 1 if s else 0] for (a, w, g, s) in qparams], dtype=np.int32).reshape(et, 4)
     n = np.asarray(ns, dtype=np.int64)

@@ -21,13 +21,15 @@ def _stream():
     return torch.cuda.current_stream().cuda_stream
 
 
-def act_tag(a_bits: int, gsize: int, bf6: bool = False) -> int:
-    """ref_bind.cu:461-473; with `bf6`, per-token int4 codes are written as bf6 fragments (tag 4: the operand layout of the kernels
-    whose w4a4 tiles run on the 6-bit float matrix path, `select_kernel(..., bf6=True)`)."""
+def act_tag(a_bits: int, gsize: int, bf6: bool = False, fp8: bool = False) -> int:
+    """ref_bind.cu:461-473, plus two tags for operand variants that QParams cannot name: with `bf6`, per-token int4 codes are written
+    as bf6 fragments (tag 4: the operand layout of the kernels whose w4a4 tiles run on the 6-bit float matrix path); with `fp8`,
+    per-token 8-bit codes are fp8 e4m3 numbers instead of int8 ones (tag 5: for the kernels whose w8a8 tiles run the fp8 instruction,
+    the reference's w8a8_g-1_sym_E4M3).  `select_kernel(..., bf6=, fp8=)` finds the matching kernel."""
     if a_bits >= 16:
         return 0
     if a_bits == 8 and gsize == -1:
-        return 1
+        return 5 if fp8 else 1
     if a_bits == 4 and gsize == -1:
         return 4 if bf6 else 2
     if a_bits == 4 and gsize == 128:
@@ -42,29 +44,43 @@ def packed_elems(tag: int, rows: int, width: int) -> int:
     """fp16 elements that `rows` packed activation rows of `width` values occupy (ref_bind.cu:491; tag 4: whole blocks of 32 rows)."""
     if tag == 4:
         return -(-rows // 32) * (width // 64) * BF6_FRAGMENT_HALVES
-    return rows * (width if tag == 0 else (width // 2 if tag == 1 else width // 4))
+    return rows * (width if tag == 0 else (width // 2 if tag in (1, 5) else width // 4))
 
 
-def select_kernel(qparams, bf6: bool = False, lib=None) -> int:
-    """Registry index of the first fused kernel with a tile for every format in `qparams`; with `bf6`, of the first one whose w4a4
-    tiles take bf6 fragments (such kernels are never chosen automatically by the launcher, which cannot see the operand layout)."""
+def kernel_variants(lib, kid: int) -> dict:
+    """{format id: operand variant} of kernel `kid`'s branches that take a variant (1 bf6 fragments, 2 fp8 e4m3 codes)."""
     import ctypes as C
 
+    out, res = (C.c_int32 * 8)(), {}
+    for b in range(lib.mxmoe_kernel_num_branches(kid)):
+        lib.mxmoe_kernel_branch(kid, b, out)
+        if out[0] >> 8:
+            res[out[0] & 255] = out[0] >> 8
+    return res
+
+
+def select_kernel(qparams, bf6: bool = False, fp8: bool = False, lib=None) -> int:
+    """Registry index of the first fused kernel with a tile for every format in `qparams` whose operand variants are exactly the ones
+    asked for: w4a4 operands as bf6 fragments (`bf6`), w8a8 operands as fp8 e4m3 codes (`fp8`).  -1 (the launcher's own choice) when
+    none is asked for; kernels with variants are never chosen automatically, since the launcher cannot see what the operands hold."""
     lib = lib or _lib.load()
-    if not bf6:
-        return -1
     qs = sorted({tuple(int(v) for v in q) for q in qparams})
+    want = {}
+    if bf6 and (4, 4, -1, 1) in qs:
+        want[2] = 1
+    if fp8 and (8, 8, -1, 1) in qs:
+        want[1] = 2
+    if not want:
+        return -1
     sizes = (_lib.Dim3 * len(qs))(*[_lib.Dim3(1, 256, 256) for _ in qs])
     hq = (_lib.QParams * len(qs))(*[_lib.QParams(a, w, g, 1 if s else 0) for (a, w, g, s) in qs])
-    out = (C.c_int32 * 8)()
+    fmt_ids = {(4, 4, -1): 2, (8, 8, -1): 1}
+    mine = {fmt_ids[q[:3]] for q in qs if q[:3] in fmt_ids}
     for kid in range(lib.mxmoe_num_kernels()):
         if lib.mxmoe_kernel_policy(kid) != 0:
             continue
-        takes_bf6 = False
-        for b in range(lib.mxmoe_kernel_num_branches(kid)):
-            lib.mxmoe_kernel_branch(kid, b, out)
-            takes_bf6 |= out[0] == 2 and out[3] == 64
-        if takes_bf6 and lib.mxmoe_group_gemm_plan(kid, sizes, hq, len(qs), None, None) == 1000 + kid:
+        have = {f: v for f, v in kernel_variants(lib, kid).items() if f in mine}
+        if have == want and lib.mxmoe_group_gemm_plan(kid, sizes, hq, len(qs), None, None) == 1000 + kid:
             return kid
     raise RuntimeError("quant type not supported")
 
@@ -94,7 +110,7 @@ def build_permutation(topk_ids: torch.Tensor, num_experts: int):
     return dst, perm, slot, recv
 
 
-def _offsets(recv_cpu, num_tokens: int, num_experts: int, has_shared: bool, qparams_per_exp, ld: int, ld_shared: int, bf6: bool = False):
+def _offsets(recv_cpu, num_tokens: int, num_experts: int, has_shared: bool, qparams_per_exp, ld: int, ld_shared: int, bf6: bool = False, fp8: bool = False):
     """Host offset builder of ref_bind.cu:475-505 / 635-671 (units: fp16 elements)."""
     et = num_experts + (1 if has_shared else 0)
     if len(qparams_per_exp) < et:
@@ -105,15 +121,15 @@ def _offsets(recv_cpu, num_tokens: int, num_experts: int, has_shared: bool, qpar
     acc = io = so = 0
     for e in range(et):
         a_bits, _w, g, _s = qparams_per_exp[e]
-        tag = act_tag(int(a_bits), int(g), bf6 and int(_w) == 4)
-        if tag not in (0, 1, 2, 3, 4):
+        tag = act_tag(int(a_bits), int(g), bf6 and int(_w) == 4, fp8 and int(_w) == 8)
+        if tag not in (0, 1, 2, 3, 4, 5):
             raise RuntimeError("quant type not supported")
         width = ld_shared if e == num_experts else ld
         if tag == 3 and width % 128:
             raise RuntimeError(f"group-128 activations need a row length that is a multiple of 128, got {width}")
         if tag == 4 and (width % 128 or width < 256):
             raise RuntimeError(f"bf6 fragments need a row length that is a multiple of 128 and at least 256, got {width}")
-        qld = width * 3 // 8 if tag == 4 else (width if tag == 0 else (width // 2 if tag == 1 else width // 4))
+        qld = width * 3 // 8 if tag == 4 else (width if tag == 0 else (width // 2 if tag in (1, 5) else width // 4))
         sld = 0 if tag == 0 else (width // 128 if tag == 3 else 1)    # scales per row (ref_bind.cu:492)
         n = num_tokens if e == num_experts else int(recv_list[e])
         for c, v in zip(cols, (tag, acc, io, so)):
@@ -141,7 +157,7 @@ def _views(store, scale_store, table, rows, inp_sizes, scale_sizes, lds):
     return inp_list, scale_list
 
 
-def quant_inp_act(hidden, topk_ids, num_experts: int, N: int, num_shared_experts: int, qparams_per_exp, verbose: bool = False, rotate: int = 0, bf6: bool = False):
+def quant_inp_act(hidden, topk_ids, num_experts: int, N: int, num_shared_experts: int, qparams_per_exp, verbose: bool = False, rotate: int = 0, bf6: bool = False, fp8: bool = False):
     """ref_bind.cu:434-592.  Returns (inp_list, scale_list, out_list, inp_store, scale_store, out_store,
     recv_tokens_per_exp (int64 CPU), perm_indices, dst_exp_sorted).  The lists are views into the stores, one per
     non-empty problem (shared expert last); out_list[p] is the [M_p, 2N] (shared: [T, 2N * num_shared]) gate_up output buffer."""
@@ -153,7 +169,7 @@ def quant_inp_act(hidden, topk_ids, num_experts: int, N: int, num_shared_experts
     has_shared = num_shared_experts > 0
     dst, perm, _slot, recv = build_permutation(topk_ids, num_experts)
     recv_cpu = recv.cpu()                                   # one small D2H copy, as ref_bind.cu:451
-    table, rows, inp_sizes, scale_sizes, lds, io, so = _offsets(recv_cpu, t, num_experts, has_shared, qparams_per_exp, k, k, bf6)
+    table, rows, inp_sizes, scale_sizes, lds, io, so = _offsets(recv_cpu, t, num_experts, has_shared, qparams_per_exp, k, k, bf6, fp8)
     dev = hidden.device
     inp_store = torch.empty(io, dtype=torch.float16, device=dev)
     scale_store = torch.empty(so, dtype=torch.float16, device=dev)
@@ -178,7 +194,7 @@ def quant_inp_act(hidden, topk_ids, num_experts: int, N: int, num_shared_experts
 
 
 def silu_mul_then_quant(inp, num_problems: int, num_experts: int, K: int, N: int, num_shared_experts: int, num_tokens: int, topk: int,
-                        values_sorted, recv_tokens_per_exp, qparams_per_exp, rotate: int = 0, bf6: bool = False):
+                        values_sorted, recv_tokens_per_exp, qparams_per_exp, rotate: int = 0, bf6: bool = False, fp8: bool = False):
     """ref_bind.cu:595-757.  `inp` is the flat gate_up output store ([R, 2N] routed rows then [T, 2N*num_shared] shared rows),
     `values_sorted` the sorted expert ids.  Returns (inp_list, scale_list, out_list, inp_store, scale_store, out_store) where
     out_list[p] is the [M_p, K] buffer of the down projection."""
@@ -187,7 +203,7 @@ def silu_mul_then_quant(inp, num_problems: int, num_experts: int, K: int, N: int
     dev = inp.device
     recv_cpu = recv_tokens_per_exp.cpu()
     r = int(recv_cpu.sum())                                 # routed rows in the store (ids out of range were dropped by the permutation)
-    table, rows, inp_sizes, scale_sizes, lds, io, so = _offsets(recv_cpu, num_tokens, num_experts, has_shared, qparams_per_exp, N, N * max(num_shared_experts, 1), bf6)
+    table, rows, inp_sizes, scale_sizes, lds, io, so = _offsets(recv_cpu, num_tokens, num_experts, has_shared, qparams_per_exp, N, N * max(num_shared_experts, 1), bf6, fp8)
     inp_store = torch.empty(io, dtype=torch.float16, device=dev)
     scale_store = torch.empty(so, dtype=torch.float16, device=dev)
     out_store = torch.empty((1 + topk) * num_tokens * K, dtype=torch.float16, device=dev)

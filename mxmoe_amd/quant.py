@@ -30,6 +30,21 @@ def quant_minmax(t: torch.Tensor, bits: int, gsize: int, sym: bool, clip=(1.0, 1
     return q.reshape(t.shape), scale, zp
 
 
+E4M3_MAX = 448.0
+
+
+def quant_e4m3(t: torch.Tensor):
+    """Per-row fp8 (OCP e4m3) quantisation with the arithmetic of the symmetric integer formats: scale = max|row| / 448 in the
+    tensor's dtype (a zero row gets 1), codes = e4m3(clamp(row / scale, +-448)) rounded to nearest even.  Returns (codes uint8 of
+    t's shape, scale [rows, 1]).  The format of the reference's w8a8_g-1_sym_E4M3 tiles (mxmoe/kernels/tile_config.py:45,192), whose
+    repository holds no quantiser for it."""
+    r = t.reshape(-1, t.shape[-1])
+    scale = r.abs().amax(dim=-1, keepdim=True) / E4M3_MAX
+    scale = torch.where(scale == 0, torch.ones_like(scale), scale)
+    q = r.div(scale).clamp(-E4M3_MAX, E4M3_MAX).to(torch.float32).to(torch.float8_e4m3fn)
+    return q.view(torch.uint8).reshape(t.shape), scale
+
+
 class Quantizer:
     """mxmoe/quant/quant.py:87-109."""
 

@@ -23,11 +23,12 @@ class PackedWeight:
         return self.data.numel() * self.data.element_size() + (0 if self.scale is None else self.scale.numel() * self.scale.element_size())
 
 
-def quantize_and_pack(w: torch.Tensor, qparams, keep_codes: bool = False, bf6: bool = False) -> PackedWeight:
+def quantize_and_pack(w: torch.Tensor, qparams, keep_codes: bool = False, bf6: bool = False, fp8: bool = False) -> PackedWeight:
     """RTN-quantise `w` [N, K] fp16 for `(a_bits, w_bits, gsize, sym)` and pack it.
 
     fp16: kept as is.  w8a8 / w4a4: per-channel symmetric codes (int8 / packed nibbles, K contiguous) re-ordered into MFMA
     fragment blocks (`pack.pack_wxax_fragments`), fp16 scale [N].
+    With `fp8`, w8a8 weights are fp8 e4m3 codes (same layout as int8) for the kernels whose w8a8 tiles run the fp8 instruction.
     With `bf6`, w4a4 weights become bf6 fragments (`pack.pack_bf6_fragments`) for the kernels whose w4a4 tiles run on the 6-bit
     float matrix path; every other format is unaffected.
     w8a16 / w4a16 / w3a16 / w2a16, group 128 or per channel (-1): unsigned codes in the wave-interleaved layout with a (scale, zero) table; symmetric
@@ -37,6 +38,12 @@ def quantize_and_pack(w: torch.Tensor, qparams, keep_codes: bool = False, bf6: b
     n, k = w.shape
     if w_bits >= 16:
         return PackedWeight(w.contiguous(), None, tuple(qparams), n, k)
+    if fp8 and (a_bits, w_bits, gsize) == (8, 8, -1):
+        # w8a8 on the fp8 instruction (the reference's w8a8_g-1_sym_E4M3): per-channel e4m3 codes in the int8 tiles' fragment order
+        from .quant import quant_e4m3
+
+        codes, scale = quant_e4m3(w)
+        return PackedWeight(pack.pack_wxax_fragments(codes), scale.reshape(n).contiguous(), tuple(qparams), n, k, codes if keep_codes else None)
     q, scale, zp = quant_minmax(w, w_bits, gsize, sym)
     return pack_codes(q, scale, zp, qparams, n, k, keep_codes, bf6)
 

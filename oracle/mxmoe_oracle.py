@@ -36,6 +36,11 @@ is this build's own deterministic definition; agreement with the reference at th
 ``silu_mul`` (the reference's kernel source for it, act_kernel.cuh, is absent; torch's fp16
 ``act_fn(g) * u`` rounds the activation to fp16 before the multiply, here silu(g) stays in fp32
 and the product is rounded once), at most one fp16 ulp of the product apart.
+* ``e4m3_encode`` / ``e4m3_decode`` / ``quant_e4m3`` / ``fp8_gemm`` — all 256 codes round-trip, hand-computed ties
+  (to even) at normal, subnormal and top-of-range spacings, every fp16 value against an independent
+  library cast (torch.float8_e4m3fn), absmax -> +-448; the fp8 format of the reference's w8a8_g-1_sym_E4M3 tiles
+  has no quantiser in the reference (only the matrix instruction, mm_tile.cuh:696-697), so its scale rule
+  (max / 448) is this build's definition: parity unpinned beyond "per-row scale, e4m3 codes, fp32 sums".
 * ``dense_grid`` / the exact dense stage of ``online_hadamard`` — python-int sums in shuffled
   orders give the same bits; grid edges (zero rows, subnormal and largest fp16 values).
 * ``fma_f32`` / ``exp_f32_fixed`` — one correct rounding against exact rational arithmetic.
@@ -447,6 +452,71 @@ def act_offsets(recv: np.ndarray, num_tokens: int, qparams_per_exp, k_dim: int, 
         io += ld * n
         so += sld * n
     return out
+
+
+# --------------------------------------------------------------------------------------------
+# fp8 (OCP e4m3) — the operand format of the reference's w8a8_g-1_sym_E4M3 tiles (mxmoe/kernels/tile_config.py:45,192,
+# mma.sync ... e4m3.e4m3.f32, mxmoe/kernels/src/include/cuda_utils.cuh:385-410)
+# --------------------------------------------------------------------------------------------
+E4M3_MAX = 448.0
+
+
+def e4m3_decode(code: np.ndarray) -> np.ndarray:
+    """uint8 e4m3 codes -> float32: sign, 4 exponent bits (bias 7), 3 mantissa bits; exponent 0 is subnormal (m / 8 * 2^-6);
+    0x7F / 0xFF are NaN (the format has no infinities)."""
+    c = np.asarray(code).astype(np.int32)
+    e, m = (c >> 3) & 15, c & 7
+    mag = np.where(e == 0, m / 8.0 * 2.0 ** -6, (1.0 + m / 8.0) * np.exp2(e - 7.0))
+    mag = np.where((e == 15) & (m == 7), np.nan, mag)
+    return np.where(c & 128, -mag, mag).astype(F32)
+
+
+def e4m3_encode(x: np.ndarray) -> np.ndarray:
+    """float values with |x| <= 448 -> uint8 e4m3 codes, round to nearest, ties to even (on the 3-bit mantissa, or on the
+    subnormal grid of 2^-9 below 2^-6)."""
+    x = np.asarray(x, dtype=np.float64)
+    if x.size and np.abs(x).max() > E4M3_MAX:
+        raise ValueError("clamp to +-448 first")
+    a = np.abs(x)
+    _, ex = np.frexp(np.where(a > 0, a, 1.0))                  # a = f * 2^ex, 0.5 <= f < 1  ->  floor(log2 a) = ex - 1
+    e = np.maximum(ex - 1, -6)                                  # below 2^-6 the spacing stays that of the smallest normal binade
+    q = np.rint(a / np.exp2(e - 3.0))                           # multiples of the spacing 2^(e-3); np.rint rounds ties to even
+    carry = q >= 16                                             # rounded up into the next binade
+    e = np.where(carry, e + 1, e)
+    q = np.where(carry, 8, q).astype(np.int64)
+    code = np.where(q < 8, q, ((e + 7) << 3) | (q - 8)).astype(np.int64)   # q < 8: subnormal (exponent field 0)
+    return (code | np.where(np.signbit(x), 128, 0)).astype(np.uint8)
+
+
+def quant_e4m3(t: np.ndarray):
+    """Per-row fp8 quantisation in the dtype of ``t`` (fp16 on the path), the symmetric integer rule with 448 for the upper code:
+    ``scale = max|row| / 448`` (zero rows: 1), ``codes = e4m3(clamp(row / scale, +-448))``.  Returns (codes uint8, scale [rows, 1])."""
+    dt = t.dtype
+    r = t.reshape(-1, t.shape[-1])
+    scale = (np.abs(r).max(axis=-1, keepdims=True) / dt.type(E4M3_MAX)).astype(dt)
+    scale = np.where(scale == 0, dt.type(1), scale).astype(dt)
+    q = np.clip((r / scale).astype(dt), dt.type(-E4M3_MAX), dt.type(E4M3_MAX))
+    return e4m3_encode(q.astype(np.float64)).reshape(t.shape), scale
+
+
+def fp8_gemm(ca: np.ndarray, cb: np.ndarray) -> np.ndarray:
+    """``acc[m, n] = sum_k value(ca[m, k]) * value(cb[n, k])`` for e4m3 codes, as float32.  Every product is exact in fp32; the
+    matrix instruction adds the products of a step in an order and an alignment of its own (measured: about 2^-16 of the largest sum
+    away from this float64 sum rounded once), so comparisons with it carry a tolerance."""
+    return (e4m3_decode(ca).astype(np.float64) @ e4m3_decode(cb).astype(np.float64).T).astype(F32)
+
+
+def linear_block_fp8(x: np.ndarray, w: np.ndarray, rotate: bool):
+    """One w8a8 block in fp8: activations optionally rotated, per-token e4m3; weights per-channel e4m3; fp32 sums; the w-a epilogue.
+    Returns (out fp16, out of the fake-quant path fp16: dequantised operands multiplied in float64)."""
+    xr = online_hadamard(x) if rotate else x
+    ca, sa = quant_e4m3(xr)
+    cb, sb = quant_e4m3(w)
+    acc = fp8_gemm(ca, cb)
+    out = (acc * (sa.reshape(-1, 1).astype(F32) * sb.reshape(1, -1).astype(F32))).astype(F32).astype(F16)
+    xq = (e4m3_decode(ca).astype(F16) * sa.astype(F16)).astype(F16)
+    wq = (e4m3_decode(cb).astype(F16) * sb.astype(F16)).astype(F16)
+    return out, gemm_fakequant(xq, wq)
 
 
 # --------------------------------------------------------------------------------------------

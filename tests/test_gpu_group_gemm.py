@@ -104,6 +104,38 @@ def test_w4a4_on_the_bf6_matrix_path_bit_exact(kernel):
         _launch([bad], kernel_id=kid)
 
 
+def test_w8a8_in_fp8_e4m3_next_to_w4a4():
+    """The kernel whose w8a8 tiles run the fp8 matrix instruction (the reference's w8a8_g-1_sym_E4M3, tile_config.py:45): e4m3
+    codes on both sides, fp32 sums.  The instruction adds the products of a step in an order and an alignment of its own (sums
+    come out about 2^-16 of the largest sum away from the float64 sum), so the fp32 sums are compared within 2e-4 of the largest,
+    the fp16 outputs within 1e-3 of the oracle's and 1e-2 of the fake-quant path; the w4a4 problems of the same launch stay bit-exact."""
+    from mxmoe_amd import _lib, pack
+
+    lib = _lib.load()
+    kid = lib.mxmoe_find_kernel(b"groupgemm_hz_fused_wxax_e4m3")
+    assert kid >= 0 and "w8a8_g-1_sym_E4M3" in lib.mxmoe_kernel_name(kid).decode()
+    rng = np.random.default_rng(41)
+    probs = []
+    for (m, n, k) in [(1, 256, 64), (31, 512, 256), (129, 2048, 1408), (300, 264, 384), (64, 2816, 2048)]:
+        x = rng.standard_normal((m, k)).astype(F16)
+        w = (rng.standard_normal((n, k)) * 0.02).astype(F16)
+        ca, sa = O.quant_e4m3(x)
+        cb, sb = O.quant_e4m3(w)
+        acc = O.fp8_gemm(ca, cb)
+        out, fq = O.linear_block_fp8(x, w, False)
+        probs.append(dict(A=torch.from_numpy(ca).to(DEV), B=pack.pack_wxax_fragments(torch.from_numpy(cb)).to(DEV), sa=torch.from_numpy(sa.reshape(-1)).to(DEV),
+                          sb=torch.from_numpy(sb.reshape(-1)).to(DEV), acc32=acc, out=out, fq=fq, size=(m, n, k), q=(8, 8, -1, True)))
+    probs.insert(2, _wxax_problem(rng, 70, 512, 256, 4))
+    _, outs, accs = _launch(probs, kernel_id=kid)
+    for p, out, acc in zip(probs, outs, accs):
+        if "acc32" in p:
+            got = acc.view(np.float32)
+            assert np.abs(got - p["acc32"]).max() <= 2e-4 * np.abs(p["acc32"]).max() + 1e-6, p["size"]
+            assert np.isfinite(out).all() and _rel(out, p["out"]) <= 1e-3 and _rel(out, p["fq"]) <= 1e-2, (p["size"], _rel(out, p["out"]))
+        else:
+            assert np.array_equal(acc, p["acc"]) and np.array_equal(out.view(np.uint16), p["out"].view(np.uint16))
+
+
 def test_wxax_empty_and_single_row_problems():
     rng = np.random.default_rng(1)
     probs = [_wxax_problem(rng, m, 256, 128, b) for (m, b) in [(5, 8), (1, 4)]]

@@ -400,6 +400,45 @@ def test_layer_on_the_bf6_matrix_path_gives_the_same_bits_in_every_form(num_shar
     assert torch.equal(layer(hidden, ids2, w), plain.combine(w))
 
 
+def test_layer_with_w8a8_blocks_in_fp8():
+    """MxMoELayer(fp8=True): the w8a8 blocks of a mixed w4a4 / w8a8 layer in e4m3 (weights, activations, fp8 matrix instruction).
+    Stepwise operators, host-planned and device-planned forwards agree bit for bit with each other (same kernels, same order of
+    additions), and each block of every expert is within 1e-3 of the oracle's block in that format on the same input."""
+    from mxmoe_amd import synth
+    from mxmoe_amd.layer import MxMoELayer
+
+    cfg = synth.MoEConfig("t", "test", 4, 2, 256, 1408, 60, num_shared=0, rotate=1)
+    fm = [(synth.W8A8, synth.W8A8), (synth.W4A4, synth.W8A8), (synth.W8A8, synth.W4A4), (synth.W4A4, synth.W4A4)]
+    weights = [synth.expert_weights(cfg, e) for e in range(4)]
+    layer = MxMoELayer(cfg, formats=fm, weights=weights, fp8=True)
+    assert layer.kid_gate_up >= 0
+    hidden = synth.make_hidden(cfg)
+    ids, w = synth.make_routing(cfg)
+    outs = [o.cpu().numpy() for o in layer.forward(hidden, ids)]
+    want = layer.combine(w).clone()
+    assert torch.equal(layer(hidden, ids, w), want) and torch.equal(layer.call_with_host_tables(hidden, ids, w), want)
+    _, perm, _, recv = O.permute_by_expert(ids.numpy(), cfg.num_experts)
+    row = p = 0
+    for e in range(4):
+        m = int(recv[e])
+        if m == 0:
+            continue
+        x = hidden.numpy()[perm[row:row + m]]
+        row += m
+
+        def block(inp, wt, qp):
+            return O.linear_block_fp8(inp, wt, True)[0] if qp == synth.W8A8 else O.linear_block(inp, wt, qp, True)[0]
+
+        # block by block, the second one on the intermediate the GPU produced: a last-bit difference in the first block's fp32 sums can
+        # move an e4m3 code of the second block's input by a whole step of that coarse format, which is no error of either block
+        mid = block(x, weights[e][0].numpy(), fm[e][0])
+        g_mid = layer.state["mid"][p].cpu().numpy()
+        assert _rel(g_mid, mid) <= 1e-3, (e, _rel(g_mid, mid))
+        ref = block(O.silu_mul(g_mid), weights[e][1].numpy(), fm[e][1])
+        assert np.isfinite(outs[p]).all() and _rel(outs[p], ref) <= 1e-3, (e, _rel(outs[p], ref))
+        p += 1
+
+
 def test_single_block_planning_writes_what_the_paired_launch_writes():
     """mxmoe_plan_block (one block per launch) against mxmoe_plan_layer (both blocks of the layer in one launch): identical plan
     buffers for the same counts."""

@@ -255,6 +255,43 @@ def test_silu_mul_then_quant_writes_bf6_fragments(n, n_sh, rotate):
         p += 1
 
 
+@pytest.mark.parametrize("k,rotate", [(2048, 1), (1408, 1), (14336, 1), (2816, 0)])
+def test_quant_inp_act_writes_fp8_codes(k, rotate):
+    """With fp8=True the per-token 8-bit experts get e4m3 codes and scales max / 448, bit for bit the oracle's, in every row kernel;
+    the other formats are untouched."""
+    from mxmoe_amd import ops
+
+    rng = np.random.default_rng(k + 11)
+    t, e, topk = 40, 4, 2
+    x = (rng.standard_normal((t, k)) * rng.uniform(0.01, 20, (t, 1))).astype(F16)
+    x[3] = 0
+    ids = _ids(rng, t, e, topk)
+    qp = [(8, 8, -1, True), (4, 4, -1, True), (8, 8, -1, True), (16, 16, -1, True), (8, 8, -1, True)]
+    res = ops.quant_inp_act(torch.from_numpy(x).to(DEV), torch.from_numpy(ids).to(DEV), e, 1408, 1, qp, rotate=rotate, fp8=True)
+    inp_list, scale_list = res[:2]
+    torch.cuda.synchronize()
+    _, o_perm, _, o_recv = O.permute_by_expert(ids, e)
+    p = st = 0
+    for ex in range(e + 1):
+        m = t if ex == e else int(o_recv[ex])
+        if m == 0:
+            continue
+        rows = x if ex == e else x[o_perm[st:st + m]]
+        if ex < e:
+            st += m
+        tag = O.act_tag(qp[ex][0], qp[ex][2])
+        xr = O.online_hadamard(rows) if rotate and tag != 0 else rows
+        got = inp_list[p]
+        if tag == 1:
+            c, s_ = O.quant_e4m3(xr)
+            assert np.array_equal(scale_list[p].cpu().numpy().view(np.uint16), s_.reshape(-1).view(np.uint16)), f"expert {ex} scales"
+            assert np.array_equal(got.contiguous().view(torch.uint8).cpu().numpy().reshape(m, -1), c), f"expert {ex} codes"
+        elif tag == 2:
+            q, s_, _ = O.quant_minmax(xr, 4, -1, True)
+            assert np.array_equal(_unpack(got, 2, k), q.astype(np.int8))
+        p += 1
+
+
 def test_unsupported_activation_format():
     from mxmoe_amd import ops
 

@@ -289,3 +289,56 @@ def test_shared_reciprocal_division_is_exact_for_all_fp16_pairs():
     assert same.all(), (a[~same][:5], b[~same][:5])
     plain = (m0 == mt) & ((e0 - 34) == et)
     assert 0.05 < (~plain).mean() < 0.6
+
+
+def test_e4m3_codes_known_answers_and_round_trip():
+    """fp8 (OCP e4m3): all 254 number codes decode and re-encode to themselves; hand-computed values and ties (to even) at the
+    spacings of the normal range (1 + m/8), of the top binade (256 .. 448, spacing 32) and of the subnormals (multiples of 2^-9)."""
+    from oracle import mxmoe_oracle as O
+
+    codes = np.arange(256, dtype=np.uint8)
+    vals = O.e4m3_decode(codes)
+    num = ~np.isnan(vals)
+    assert num.sum() == 254 and np.isnan(vals[0x7F]) and np.isnan(vals[0xFF])
+    assert np.array_equal(O.e4m3_encode(vals[num]), codes[num])
+    assert vals[0x7E] == 448.0 and vals[0xFE] == -448.0 and vals[0x38] == 1.0 and vals[0x01] == 2.0 ** -9 and vals[0x08] == 2.0 ** -6 and vals[0x3C] == 1.5
+    # ties: halfway between 1.0 (mantissa 000, even) and 1.125 (001) -> 1.0; between 1.125 and 1.25 (010, even) -> 1.25
+    assert list(O.e4m3_encode(np.array([1.0625, 1.1875, 1.0626, -1.1874]))) == [0x38, 0x3A, 0x39, 0xB9]
+    # top binade: 416 (m 101) .. 448 (m 110, even): 432 -> 448; 400 is between 384 (100) and 416 (101) -> 384
+    assert list(O.e4m3_encode(np.array([432.0, 400.0, 447.9, 240.0]))) == [0x7E, 0x7C, 0x7E, 0x77]
+    # carry into the next binade: 1.97 -> 2.0; subnormals: 1.5 * 2^-9 -> 2 * 2^-9 (even), 0.5 * 2^-9 -> 0 (even), largest subnormal + half -> smallest normal
+    assert list(O.e4m3_encode(np.array([1.97, 1.5 * 2.0 ** -9, 0.5 * 2.0 ** -9, 7.5 * 2.0 ** -9, 0.0, -0.0]))) == [0x40, 0x02, 0x00, 0x08, 0x00, 0x80]
+    with pytest.raises(ValueError):
+        O.e4m3_encode(np.array([449.0]))
+
+
+def test_e4m3_against_an_independent_cast_and_the_quantiser_rule():
+    """Every finite fp16 value up to 448 in magnitude: the oracle's codes equal a library cast to float8_e4m3fn (torch, used here as
+    an independent implementation of the same standard format).  quant_e4m3: the row's largest magnitude lands on +-448, no code
+    is NaN, a zero row has scale 1, and dequantised values are within half a spacing (2^-4 relative) of the scaled input."""
+    import torch
+
+    from oracle import mxmoe_oracle as O
+
+    x = torch.arange(0, 65536, dtype=torch.int32).to(torch.int16).view(torch.float16)
+    x = x[torch.isfinite(x) & (x.abs() <= 448)]
+    want = x.float().to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    assert np.array_equal(O.e4m3_encode(x.float().numpy()), want)
+    rng = np.random.default_rng(3)
+    t = (rng.standard_normal((64, 512)) * rng.uniform(1e-3, 30, (64, 1))).astype(F16)
+    t[5] = 0
+    c, s = O.quant_e4m3(t)
+    v = O.e4m3_decode(c)
+    assert not np.isnan(v).any() and s[5, 0] == 1 and (v[5] == 0).all()
+    live = np.abs(t).max(axis=1) > 0
+    assert np.all(np.abs(v[live]).max(axis=1) == 448.0)
+    ratio = (t[live].astype(np.float64) / s[live].astype(np.float64))
+    assert np.all(np.abs(v[live] - ratio) <= np.maximum(np.abs(ratio) * 2.0 ** -4, 2.0 ** -10) * 1.01 + np.abs(ratio) * 2.0 ** -10)
+    # the torch mirror used to pack weights gives the same codes and scales
+    from mxmoe_amd.quant import quant_e4m3
+
+    tc, ts = quant_e4m3(torch.from_numpy(t))
+    assert np.array_equal(tc.numpy(), c) and np.array_equal(ts.numpy().view(np.uint16), s.view(np.uint16))
+    # and fp8_gemm on one-hot / unit operands returns the operand values themselves
+    a = O.e4m3_encode(np.eye(8)[:, :8] * 1.0)
+    assert np.array_equal(O.fp8_gemm(c[:3, :8], a), v[:3, :8])
