@@ -237,115 +237,6 @@ def time_whole_layer(cfg, layer, reps: int = 7) -> dict:
     return out
 
 
-def mfma_probe(iters: int = 20000, workgroups: int = 512, repeats: int = 3):
-    """Rate and shader clock of a bare loop of matrix instructions (512 workgroups = two per CU, 8 independent accumulators per wave):
-    v_mfma_i32_32x32x32_i8 for six operand patterns, then v_mfma_scale_f32_32x32x64_f8f6f4 on bf6 operands that hold int4 values (the
-    path on which int4 x int4 products are exact at twice the int8 instruction's rate).  Each pattern runs `repeats` times back to
-    back after a short warm-up launch; the last run is reported."""
-    import torch
-
-    from mxmoe_amd import _lib
-
-    lib = _lib.load()
-    src = torch.randint(0, 256, (65536,), dtype=torch.uint8, device="cuda", generator=torch.Generator("cuda").manual_seed(0))
-    out = torch.zeros(workgroups * 256 + 4, dtype=torch.int32, device="cuda")
-    stream = torch.cuda.current_stream().cuda_stream
-    ops = 2 * 32 * 32 * 32 * 8 * iters * 4 * workgroups
-    res = {"probe": "bare matrix-instruction loop", "workgroups": workgroups, "iters": iters, "ops_per_launch_int8": ops, "ops_per_launch_bf6": 2 * ops,
-           "peak_tops": PEAK["int8"], "peak_tops_bf6": PEAK["fp6"], "modes": {}}
-    names = ["zero operands", "constant operands", "random 16*int4 operands", "random int8 operands", "random offset-binary int4 operands (0..15)",
-             "random sign-extended int4 operands", "bf6 32x32x64: random int4 values", "bf6 32x32x64: zero operands"]
-    for mode, name in enumerate(names):
-        mode_ops, peak = (2 * ops, PEAK["fp6"]) if mode >= 6 else (ops, PEAK["int8"])
-        _lib.check(lib, lib.mxmoe_mfma_probe(mode, 100, workgroups, src.data_ptr(), out.data_ptr(), stream))
-        torch.cuda.synchronize()
-        for _ in range(repeats):
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            _lib.check(lib, lib.mxmoe_mfma_probe(mode, iters, workgroups, src.data_ptr(), out.data_ptr(), stream))
-            e1.record()
-            torch.cuda.synchronize()
-            ms = e0.elapsed_time(e1)
-        rec = out[-4:].cpu().numpy().view("uint64")
-        res["modes"][name] = {"ms": round(ms, 3), "tops": round(mode_ops / (ms * 1e-3) / 1e12, 1), "of_peak": round(mode_ops / (ms * 1e-3) / 1e12 / peak, 3),
-                              "shader_clock_ghz": round(float(rec[0]) / (float(rec[1]) * 10.0), 3)}
-    return res
-
-
-def one_problem(spec: str):
-    """One problem of one format through the default integer kernel, timed with its quantised random operands, then with every code
-    byte set to one constant, then with all codes zero.  The launches are identical instruction for instruction; what differs is how
-    many operand bits toggle in the matrix pipes, and with it the clock the GPU sustains."""
-    import torch
-
-    from mxmoe_amd import _lib, harness
-
-    fmt, dims = spec.split(":")
-    m, n, k = (int(x) for x in dims.lower().split("x"))
-    bits = {"w4a4": 4, "w8a8": 8}[fmt]
-    lib = _lib.load()
-    prob = harness.make_problem({"shape": [m, n, k], "w_bits": bits, "a_bits": bits, "gsize": -1, "sym": True}, None)
-    launch = harness._launch_of([prob], lib, lib.mxmoe_find_kernel(b"groupgemm_hz_fused_wxax"))
-    res = {"problem": spec, "kernel": "groupgemm_hz_fused_wxax", "ops": 2 * m * n * k, "peak_tops": PEAK["int8"], "operands": {}}
-    for name in ("random codes", "constant codes", "zero codes"):
-        if name == "constant codes":
-            prob["A"].fill_(0x37)
-            prob["B"].fill_(0x5A)
-        elif name == "zero codes":
-            prob["A"].zero_()
-            prob["B"].zero_()
-        ms = harness.bench_func(launch.run, warmup=20, iters=30)["median"]
-        res["operands"][name] = {"us": round(ms * 1e3, 1), "tops": round(2 * m * n * k / ms / 1e9, 1), "of_peak": round(2 * m * n * k / ms / 1e9 / PEAK["int8"], 3)}
-    return res
-
-
-def bf6_probe(dims: str):
-    """One int4 x int4 problem M x N x K on the 6-bit float matrix path (the diagnostic kernel mxmoe_bf6_gemm_probe: bf6 operand
-    fragments, exact accumulators) next to the same shape through the int4 tile of the default kernel: uniformly random values
-    -8 .. 7, bell-shaped ones (a rounded normal of deviation 2.5, what rotated activations quantise to), and zeros."""
-    import torch
-
-    from mxmoe_amd import _lib, bf6, harness
-
-    m, n, k = (int(x) for x in dims.lower().split("x"))
-    lib = _lib.load()
-    stream = torch.cuda.current_stream().cuda_stream
-    gen = torch.Generator("cuda").manual_seed(0)
-    ops = 2 * m * n * k
-    shapes = {"bf6_probe_256x256_one_wave_per_simd": 0, "bf6_probe_128x256_two_workgroups_per_cu": 1}
-    res = {"problem": dims, "ops": ops, "peak_tops_int8": PEAK["int8"], "peak_tops_fp6": PEAK["fp6"], **{k_: {} for k_ in shapes}, "int4_tile": {}}
-    sa = torch.full((m,), 0.01, dtype=torch.float16, device="cuda")
-    sb = torch.full((n,), 0.01, dtype=torch.float16, device="cuda")
-    c = torch.empty(m, n, dtype=torch.float16, device="cuda")
-
-    def values(kind, rows):
-        if kind == "uniform values":
-            return torch.randint(-8, 8, (rows, k), dtype=torch.int8, device="cuda", generator=gen)
-        if kind == "bell-shaped values":
-            return (torch.randn(rows, k, device="cuda", generator=gen) * 2.5).round().clamp(-8, 7).to(torch.int8)
-        return torch.zeros(rows, k, dtype=torch.int8, device="cuda")
-
-    prob = harness.make_problem({"shape": [m, n, k], "w_bits": 4, "a_bits": 4, "gsize": -1, "sym": True}, None)
-    launch = harness._launch_of([prob], lib, lib.mxmoe_find_kernel(b"groupgemm_hz_fused_wxax"))
-    from mxmoe_amd import pack
-
-    for kind in ("uniform values", "bell-shaped values", "zero values"):
-        a, b = values(kind, m), values(kind, n)
-        a6, b6 = bf6.pack_fragments(a), bf6.pack_fragments(b)
-        for name, shape in shapes.items():
-            if shape == 0 and (m % 256 or k % 256):  # that shape's workgroups and ring need multiples of 256
-                continue
-            run = lambda: _lib.check(lib, lib.mxmoe_bf6_gemm_probe(a6.data_ptr(), b6.data_ptr(), sa.data_ptr(), sb.data_ptr(), c.data_ptr(), None, m, n, k, shape, stream))
-            ms = harness.bench_func(run, warmup=20, iters=30)["median"]
-            res[name][kind] = {"us": round(ms * 1e3, 1), "tops": round(ops / ms / 1e9, 1), "of_fp6_peak": round(ops / ms / 1e9 / PEAK["fp6"], 3)}
-        prob["A"].copy_(pack.pack_int4_k(a))                                  # the same values through the integer tile
-        prob["B"].copy_(pack.pack_wxax_fragments(pack.pack_int4_k(b)))
-        ms = harness.bench_func(launch.run, warmup=20, iters=30)["median"]
-        res["int4_tile"][kind] = {"us": round(ms * 1e3, 1), "tops": round(ops / ms / 1e9, 1), "of_int8_peak": round(ops / ms / 1e9 / PEAK["int8"], 3)}
-        del a, b, a6, b6
-    return res
-
-
 def run_workload(name: str, steps: int, warmup: int, tokens=None, whole: bool = True, bf6=False):
     cfg, layer = build_layer(name, tokens, bf6)
     ms, up, dn = time_layer(layer, steps, warmup)
@@ -375,14 +266,6 @@ def main() -> int:
     ap.add_argument("--no-whole-layer", action="store_true", help="skip the wall-clock timing of the whole forward (profiling runs: the trace then ends with the launches the roofline entry is measured on)")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="BYTES",
                     help="instead of the benchmark, run a plain device copy of BYTES bytes 5 times (reference point for the FETCH_SIZE / WRITE_SIZE counters)")
-    ap.add_argument("--one-problem", default="", metavar="FMT:MxNxK",
-                    help="instead of the benchmark, time one GroupGEMM problem (FMT w4a4 or w8a8, e.g. w4a4:32768x2048x4096) through the default "
-                         "kernel with random, constant and all-zero operand codes: the same instruction stream at three levels of operand toggling")
-    ap.add_argument("--bf6-probe", default="", metavar="MxNxK",
-                    help="instead of the benchmark, time one int4 x int4 problem on the 6-bit float matrix path (diagnostic kernel) and through the int4 tile "
-                         "(N a multiple of 256, M and K of 128, e.g. 32768x2048x4096)")
-    ap.add_argument("--mfma-probe", action="store_true",
-                    help="instead of the benchmark, time a bare loop of int8 matrix instructions per operand pattern (the ceiling of the matrix pipes on this GPU)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (the layer would shard by expert, one all-to-all of rows either side of the launches). Use --gpus 1.", file=sys.stderr)
@@ -401,15 +284,6 @@ def main() -> int:
             dst.copy_(src)
         torch.cuda.synchronize()
         print(json.dumps({"copy_bytes": args.copy_calibration, "copies": 5}))
-        return 0
-    if args.mfma_probe:
-        print(json.dumps(mfma_probe()))
-        return 0
-    if args.bf6_probe:
-        print(json.dumps(bf6_probe(args.bf6_probe)))
-        return
-    if args.one_problem:
-        print(json.dumps(one_problem(args.one_problem)))
         return 0
     from mxmoe_amd import synth
 

@@ -172,7 +172,9 @@ int mxmoe_unpermute_combine(const void* down_out, const void* shared_out, const 
  * fused launch) into a plan buffer; the *_planned entry points read their tables from it.  Same kernels, same results.
  *
  * A block is described per expert by mxmoe_block_desc {QParams, N, K, packed weights, weight scales} (d_desc in device memory, h_desc
- * its host mirror; the shared expert, when shared_rows > 0, is entry num_experts and has shared_rows rows).  At most 120 problems.
+ * its host mirror; the shared expert, when shared_rows > 0, is entry num_experts and has shared_rows rows).  At most 4096 problems; a
+ * block of more than 120 is planned and run as launches of 120 consecutive experts each (one FusedArgs per launch at the head of
+ * the plan buffer).
  * Stores are laid out as the host path lays them out (experts in order, rows packed), so they must be sized for the worst case:
  * capacity rows x the widest row of any expert.
  *
@@ -189,7 +191,8 @@ int mxmoe_unpermute_combine(const void* down_out, const void* shared_out, const 
  *                                  their scales that the block reads, out_store: where its output rows go);
  *   mxmoe_plan_layer               the same for the two blocks of a layer (gate_up, down) in one launch: both plans depend on nothing
  *                                  but the tokens-per-expert counts, and a forward of a few dozen microseconds feels every launch;
- *   mxmoe_group_gemm_planned       the fused launch, grid from mxmoe_plan_grid_bound (workgroups past the planned tiles exit at once);
+ *   mxmoe_group_gemm_planned       the fused launch(es) of a block of num_problems experts, grid from mxmoe_plan_grid_bound (workgroups past
+ *                                  the planned tiles exit at once);
  *   mxmoe_quant_act_planned, mxmoe_silu_mul_quant_planned, mxmoe_unpermute_combine_planned
  *                                  as their namesakes, with d_plan in place of exp_table / row counts / shared-expert pointers;
  *                                  rows_capacity = tokens x top-k (rows that were not routed because their expert id was out of
@@ -202,7 +205,7 @@ int mxmoe_plan_grid_bound(int kernel_id, const mxmoe_block_desc* h_desc, int num
 int mxmoe_plan_block(int kernel_id, const int64_t* d_recv_tokens_per_exp, int num_experts, int shared_rows, const mxmoe_block_desc* d_desc,
                      const mxmoe_block_desc* h_desc, const void* inp_store, const void* scale_store, void* out_store, void* d_plan, void* stream);
 int mxmoe_plan_layer(const mxmoe_plan_call* gate_up, const mxmoe_plan_call* down, const int64_t* d_recv_tokens_per_exp, int num_experts, int shared_rows, void* stream);
-int mxmoe_group_gemm_planned(int kernel_id, const void* d_plan, int grid, void* stream);
+int mxmoe_group_gemm_planned(int kernel_id, const void* d_plan, int num_problems, int grid, void* stream);
 int mxmoe_quant_act_planned(const void* hidden, void* inp_store, void* scale_store, const int32_t* dst_exp_sorted, const int64_t* perm_indices, const void* d_plan,
                             int K, int rows_capacity, int num_tokens, int num_experts, int has_shared, int rotate, int had_k, int had_f, const float* had_signs,
                             void* stream);
@@ -216,32 +219,6 @@ int mxmoe_unpermute_combine_planned(const void* down_out, const void* d_plan_dow
  * launch, no workspace. */
 int mxmoe_combine_planned(const void* down_out, const void* d_plan_down, int num_problems, const float* topk_weights, const int32_t* row_of_slot, int num_tokens,
                           int topk, int K, void* out, void* stream);
-
-/* ---- diagnostics (no counterpart in the reference): the rate the matrix pipes sustain on their own ----
- * One launch of a bare loop of matrix instructions (8 independent accumulators per wave, two waves per SIMD, no memory traffic in
- * the loop): `workgroups` x 256 threads, `iters` x 8 instructions per wave.
- * Modes 0 - 5 run v_mfma_i32_32x32x32_i8 (2*32*32*32 * 8 * iters * 4 * workgroups operations): 0 all-zero operands, 1 a constant
- * byte pattern, 2 random bytes 16*v (widened int4 codes), 3 random int8 bytes, 4 random bytes 0..15 (offset-binary int4), 5 random
- * sign-extended int4 bytes.  Modes 6 and 7 run v_mfma_scale_f32_32x32x64_f8f6f4 on bf6 (e3m2) operands with unit scales (twice
- * the operations per instruction): 6 random integers -8 .. 7 as bf6 codes, 7 zeros.
- * d_src: 65536 bytes of random data; d_out: (workgroups * 256 + 4) * 4 bytes; its last 16 bytes receive the shader-clock cycles and
- * the 100 MHz real-time ticks of workgroup 0's loop (two uint64), which give the clock the chip ran at.  bench.py --mfma-probe. */
-int mxmoe_mfma_probe(int mode, int iters, int workgroups, const void* d_src, void* d_out, void* stream);
-
-/* D[32][32] (fp32) = A . B^T for A, B of 32 x 64 int8 values in -8 .. 8 (device pointers), by one v_mfma_scale_f32_32x32x64_f8f6f4
- * of one wave on operands re-encoded as bf6: every such integer is a bf6 number and the fp32 sums of their products are exact, so
- * the result equals the integer product (what an int4 x int4 tile on the 6-bit float path would rely on). */
-int mxmoe_bf6_dot_probe(const void* d_a, const void* d_b, void* d_out, void* stream);
-
-/* One int4 x int4 GEMM on that path, as a tile with its operands coming from memory would run it (not part of the fused GroupGEMM):
- * C[M][N] (fp16) = half(acc * (float(sa[m]) * float(sb[n]))), acc = sum_k a[m][k] * b[n][k], and acc itself as int32 into d_cint
- * when that is not null.  d_a6 / d_b6: the int4 values of A [M][K] and B [N][K] as bf6 fragments (32 rows x 64 k per fragment of
- * 1536 bytes, k step major: mxmoe_amd/bf6.py: pack_fragments); sa [M], sb [N] fp16.  shape 0: workgroups of 256 x 256 as 2 x 2 waves
- * of 128 x 128, one wave per SIMD (M and K multiples of 256); shape 1: workgroups of 128 x 256 as four waves of 128 x 64, two
- * workgroups per CU (M and K multiples of 128, K >= 256).  N a multiple of 256.  Returns 0, 3 for bad arguments, 4 for a launch error.
- * bench.py --bf6-probe. */
-int mxmoe_bf6_gemm_probe(const void* d_a6, const void* d_b6, const void* d_sa, const void* d_sb, void* d_c, void* d_cint, int M, int N, int K, int shape,
-                         void* stream);
 
 #ifdef __cplusplus
 }

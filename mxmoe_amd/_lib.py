@@ -48,9 +48,6 @@ SIGNATURES = {
     "mxmoe_quant_act": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P]),
     "mxmoe_silu_mul_quant": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P]),
     "mxmoe_group_gemm_plan": (_I, [_I, C.POINTER(Dim3), C.POINTER(QParams), _I, C.POINTER(C.c_int32), C.POINTER(C.c_int32)]),
-    "mxmoe_mfma_probe": (_I, [_I, _I, _I, _P, _P, _P]),
-    "mxmoe_bf6_dot_probe": (_I, [_P, _P, _P, _P]),
-    "mxmoe_bf6_gemm_probe": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
     "mxmoe_kernel_func": (_P, [_I]),
     "mxmoe_get_kernel": (_P, [C.c_char_p]),
     "mxmoe_kernel_policy": (_I, [_I]),
@@ -63,7 +60,7 @@ SIGNATURES = {
     "mxmoe_plan_grid_bound": (_I, [_I, _P, _I, _I, _I]),
     "mxmoe_plan_block": (_I, [_I, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P]),
     "mxmoe_plan_layer": (_I, [_P, _P, _P, _I, _I, _P]),
-    "mxmoe_group_gemm_planned": (_I, [_I, _P, _I, _P]),
+    "mxmoe_group_gemm_planned": (_I, [_I, _P, _I, _I, _P]),
     "mxmoe_quant_act_planned": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P]),
     "mxmoe_silu_mul_quant_planned": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P]),
     "mxmoe_unpermute_combine_planned": (_I, [_P, _P, _I, _P, _P, _I, _I, _I, _P, _P, _P]),

@@ -44,6 +44,7 @@ struct PlanParams {
 };
 
 constexpr int kPlanThreads = 128;
+constexpr int kMaxPlannedProblems = 4096;  // experts of a planned block (run as launches of kMaxProblems experts each)
 static_assert(kMaxProblems <= kPlanThreads, "one thread per problem");
 
 __device__ __forceinline__ long wave_excl_scan(long v, int lane, long* total) {
@@ -57,66 +58,105 @@ __device__ __forceinline__ long wave_excl_scan(long v, int lane, long* total) {
   return inc - v;
 }
 
-// One workgroup of two waves, thread e = expert e (the shared expert, if any, is expert E with `shared_rows` rows).  Everything the
-// host launcher computes (launch_range), with the same functions and in the same order, so the two produce identical tables;
-// prefix sums over experts are wave scans, and an entry finds its place from per-branch counts instead of a sequential walk.
+// One workgroup of two waves per launch, thread e = expert e0 + e of the launch's chunk of experts [e0, e0 + kMaxProblems) (the shared
+// expert, if any, is expert E with `shared_rows` rows).  Everything the host launcher computes (launch_range), with the same
+// functions and in the same order, so the two produce identical tables; prefix sums over experts are wave scans (a later chunk
+// first sums what the experts before it occupy), and an entry finds its place from per-branch counts instead of a sequential walk.
 struct PlanPair {
   PlanParams p[2];
+  int chunks;  // launches per block
 };
 
 __global__ void __launch_bounds__(kPlanThreads) plan_block_kernel(const PlanPair pair) {
-  const PlanParams& p = pair.p[blockIdx.x];  // one workgroup per block of the layer (gate_up, down): both only read the counts
+  const PlanParams& p = pair.p[blockIdx.x / pair.chunks];  // one workgroup per launch of each block of the layer (gate_up, down): all only read the counts
+  const int chunk = blockIdx.x % pair.chunks;
+  const int e0 = chunk * kMaxProblems;                       // first expert of this launch
+  const int ecnt = min(kMaxProblems, p.Et - e0);             // experts of this launch
   __shared__ long s_tot[4][2];                       // per wave: rows, packed input, scales, output elements
+  __shared__ long s_base[5][2];                      // the same four, and the routed rows, summed over the experts before this launch
   __shared__ int s_cnt[kMaxBranches][2], s_til[kMaxBranches][2];  // per run-order rank and wave: entries, tiles
   __shared__ int s_cnt_long[kMaxBranches][2], s_til_long[kMaxBranches][2];  // ... of which belong to long-K problems
   const int e = threadIdx.x, lane = e & 63, wave = e >> 6;
+  const int ge = e0 + e;                             // this thread's expert
+  const bool mine = e < ecnt;
   const PlanLayout lay(p.Et);
-  FusedArgs* fa = reinterpret_cast<FusedArgs*>(p.plan);
+  FusedArgs* fa = reinterpret_cast<FusedArgs*>(p.plan + chunk * kFusedArgsStride);
   int64_t* table = reinterpret_cast<int64_t*>(p.plan + lay.table);
   const void** ptrs = reinterpret_cast<const void**>(p.plan + lay.ptrs);
   int64_t* misc = reinterpret_cast<int64_t*>(p.plan + lay.misc);
   mxmoe_dim3* sizes = reinterpret_cast<mxmoe_dim3*>(p.plan + lay.sizes);
 
-  long rows = 0, qld = 0, sld = 0, out_ld = 0;
+  // what one expert occupies: rows, packed activation elements, scales, output elements (all in fp16 elements but the rows)
+  auto footprint = [&](int x, long (&f)[4], int* tag_out, mxmoe_block_desc* d_out) {
+    const mxmoe_block_desc d = p.desc[x];
+    const long rows = x < p.E ? (long)p.recv[x] : (long)p.shared_rows;
+    const int tag = act_tag_of(d.q), K = (int)d.K;
+    const long qld = tag == 0 ? K : (tag == 1 || tag == 5 ? K / 2 : K / 4);  // fp16 elements per packed activation row (ref_bind.cu:491)
+    const long sld = tag == 0 ? 0 : (tag == 3 ? K / 128 : 1);                // scales per row (ref_bind.cu:492)
+    f[0] = rows;
+    // packed activations: rows of qld elements, or (tag 4) whole blocks of 32 rows of K / 64 fragments
+    f[1] = tag == 4 ? ((rows + 31) >> 5) * (long)(K >> 6) * (kBf6Frag / 2) : qld * rows;
+    f[2] = sld * rows;
+    f[3] = (long)d.N * rows;
+    if (tag_out) *tag_out = tag;
+    if (d_out) *d_out = d;
+  };
+  // experts before this launch
+  long base[5] = {0, 0, 0, 0, 0};
+  for (int x = e; x < e0; x += kPlanThreads) {
+    long f[4];
+    footprint(x, f, nullptr, nullptr);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) base[i] += f[i];
+    if (x < p.E) base[4] += f[0];
+  }
+#pragma unroll
+  for (int i = 0; i < 5; ++i) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) base[i] += __shfl_xor(base[i], o);
+    if (lane == 0) s_base[i][wave] = base[i];
+  }
+
+  long rows = 0, sld = 0;
+  long foot[4] = {0, 0, 0, 0};
   int tag = 0, fmt = 0, N = 0, K = 0;
   mxmoe_block_desc d{};
-  if (e < p.Et) {
-    d = p.desc[e];
-    rows = e < p.E ? (long)p.recv[e] : (long)p.shared_rows;
-    tag = act_tag_of(d.q);
+  if (mine) {
+    footprint(ge, foot, &tag, &d);
+    rows = foot[0];
     fmt = fmt_of(d.q);
     N = (int)d.N;
     K = (int)d.K;
-    qld = tag == 0 ? K : (tag == 1 || tag == 5 ? K / 2 : K / 4);  // fp16 elements per packed activation row (ref_bind.cu:491); unused for tag 4
-    sld = tag == 0 ? 0 : (tag == 3 ? K / 128 : 1);   // scales per row (ref_bind.cu:492)
-    out_ld = N;
+    sld = tag == 0 ? 0 : (tag == 3 ? K / 128 : 1);
   }
-  // exclusive sums over the experts before this one
+  // exclusive sums over the experts of this launch before this one
   long tot[4], routed_tot;
-  long first_row = wave_excl_scan(rows, lane, &tot[0]);
-  // packed activations of the expert, in fp16 elements: rows of qld elements, or (tag 4) whole blocks of 32 rows of K / 64 fragments
-  const long inp_elems = tag == 4 ? ((rows + 31) >> 5) * (long)(K >> 6) * (kBf6Frag / 2) : qld * rows;
-  long inp_off = wave_excl_scan(inp_elems, lane, &tot[1]);
-  long sc_off = wave_excl_scan(sld * rows, lane, &tot[2]);
-  long out_off = wave_excl_scan(out_ld * rows, lane, &tot[3]);
-  wave_excl_scan(e < p.E ? rows : 0, lane, &routed_tot);
+  long first_row = wave_excl_scan(foot[0], lane, &tot[0]);
+  long inp_off = wave_excl_scan(foot[1], lane, &tot[1]);
+  long sc_off = wave_excl_scan(foot[2], lane, &tot[2]);
+  long out_off = wave_excl_scan(foot[3], lane, &tot[3]);
+  wave_excl_scan(mine && ge < p.E ? rows : 0, lane, &routed_tot);
   if (lane == 0) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) s_tot[i][wave] = tot[i];
   }
   // smallest K of the launch: problems above it run first inside their branch (see launch_range)
   __shared__ int s_kmin[2];
+  __shared__ long s_routed[2];
   {
-    int km = e < p.Et ? K : 0x7fffffff;
+    int km = mine ? K : 0x7fffffff;
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) km = min(km, __shfl_xor(km, o));
-    if (lane == 0) s_kmin[wave] = km;
+    if (lane == 0) {
+      s_kmin[wave] = km;
+      s_routed[wave] = routed_tot;
+    }
   }
   __syncthreads();
-  const bool long_k = e < p.Et && K > min(s_kmin[0], s_kmin[1]);
+  const bool long_k = mine && K > min(s_kmin[0], s_kmin[1]);
   // segments of this problem and, per branch in run order, this wave's entries and tiles
   Segment sg[2];
-  const int ns = e < p.Et ? plan_segments(p.info, fmt, (int)rows, N, sg) : 0;
+  const int ns = mine ? plan_segments(p.info, fmt, (int)rows, N, sg) : 0;
   int seg_tiles[2], seg_rank[2], seg_pos[2], seg_first[2];
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
@@ -126,11 +166,11 @@ __global__ void __launch_bounds__(kPlanThreads) plan_block_kernel(const PlanPair
   }
   for (int r = 0; r < p.info.nb; ++r) {
     const int b = p.info.order[r];
-    int mine = 0, which = -1;
+    int mine_tiles = 0, which = -1;
 #pragma unroll
     for (int j = 0; j < 2; ++j)
       if (j < ns && sg[j].branch == b && seg_tiles[j] > 0) {
-        mine = seg_tiles[j];
+        mine_tiles = seg_tiles[j];
         which = j;
       }
     // entries of this branch in this wave, long-K problems first: position = matching lanes that run earlier, first tile = their tiles
@@ -140,7 +180,7 @@ __global__ void __launch_bounds__(kPlanThreads) plan_block_kernel(const PlanPair
       const uint64_t has_long = __ballot(which >= 0 && long_k);
       tc = __popcll(has);
       tc_long = __popcll(has_long);
-      int inc_long = long_k ? mine : 0, inc_rest = long_k ? 0 : mine;
+      int inc_long = long_k ? mine_tiles : 0, inc_rest = long_k ? 0 : mine_tiles;
 #pragma unroll
       for (int o = 1; o < 64; o <<= 1) {
         const int t0 = __shfl_up(inc_long, o), t1 = __shfl_up(inc_rest, o);
@@ -158,7 +198,7 @@ __global__ void __launch_bounds__(kPlanThreads) plan_block_kernel(const PlanPair
           seg_rank[j] = r;
           // position / first tile inside this wave's entries of its own class; the other wave's and the other class's are added below
           seg_pos[j] = long_k ? __popcll(has_long & before) : __popcll(has & ~has_long & before);
-          seg_first[j] = long_k ? inc_long - mine : inc_rest - mine;
+          seg_first[j] = long_k ? inc_long - mine_tiles : inc_rest - mine_tiles;
         }
     }
     if (lane == 0) {
@@ -175,18 +215,22 @@ __global__ void __launch_bounds__(kPlanThreads) plan_block_kernel(const PlanPair
     sc_off += s_tot[2][0];
     out_off += s_tot[3][0];
   }
-  if (e < p.Et) {
-    table[e] = tag;
-    table[p.Et + e] = first_row;
-    table[2 * p.Et + e] = inp_off;
-    table[3 * p.Et + e] = sc_off;
-    ptrs[e] = p.inp + 2 * inp_off;
-    ptrs[p.Et + e] = d.B;
-    ptrs[2 * p.Et + e] = sld > 0 ? p.scale + 2 * sc_off : nullptr;
-    ptrs[3 * p.Et + e] = d.scale_b;
-    ptrs[4 * p.Et + e] = p.out + 2 * out_off;
-    sizes[e] = mxmoe_dim3{(uint32_t)rows, (uint32_t)N, (uint32_t)K};
-    if (e == p.E) misc[1] = (int64_t)(p.out + 2 * out_off);
+  first_row += s_base[0][0] + s_base[0][1];
+  inp_off += s_base[1][0] + s_base[1][1];
+  sc_off += s_base[2][0] + s_base[2][1];
+  out_off += s_base[3][0] + s_base[3][1];
+  if (mine) {
+    table[ge] = tag;
+    table[p.Et + ge] = first_row;
+    table[2 * p.Et + ge] = inp_off;
+    table[3 * p.Et + ge] = sc_off;
+    ptrs[ge] = p.inp + 2 * inp_off;
+    ptrs[p.Et + ge] = d.B;
+    ptrs[2 * p.Et + ge] = sld > 0 ? p.scale + 2 * sc_off : nullptr;
+    ptrs[3 * p.Et + ge] = d.scale_b;
+    ptrs[4 * p.Et + ge] = p.out + 2 * out_off;
+    sizes[ge] = mxmoe_dim3{(uint32_t)rows, (uint32_t)N, (uint32_t)K};
+    if (ge == p.E) misc[1] = (int64_t)(p.out + 2 * out_off);
   }
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
@@ -211,13 +255,13 @@ __global__ void __launch_bounds__(kPlanThreads) plan_block_kernel(const PlanPair
           first += s_til[r][0] - s_til_long[r][0];
         }
       }
-      fa->entry[pos] = FusedArgs::Entry{first, sg[j].row0, sg[j].rows, e | (sg[j].branch << 16)};
+      fa->entry[pos] = FusedArgs::Entry{first, sg[j].row0, sg[j].rows, e | (sg[j].branch << 16)};  // problem index relative to the launch's first
     }
   }
   if (e == 0) {
-    // rows routed = sum over the routed experts: wave 0's part is in routed_tot, wave 1 holds experts 64.. (all routed or shared)
-    misc[0] = s_tot[0][0] + s_tot[0][1] - (p.Et > p.E ? (long)p.shared_rows : 0);
-    if (p.Et == p.E) misc[1] = 0;
+    // rows routed = sum over the routed experts of every launch: the last launch knows them all
+    if (chunk == pair.chunks - 1) misc[0] = s_base[4][0] + s_base[4][1] + s_routed[0] + s_routed[1];
+    if (chunk == 0 && p.Et == p.E) misc[1] = 0;
     int total = 0, wg = 0, np = 0, ne = 0, flat = 0;
     int last_tile0 = 0, last_wg0 = 0;  // of the phase being filled (kept here: reading them back from the table would wait for the store)
     for (int r = 0; r < p.info.nb; ++r) {
@@ -240,7 +284,7 @@ __global__ void __launch_bounds__(kPlanThreads) plan_block_kernel(const PlanPair
     fa->phase_flat = flat;
     fa->num_entries = ne;
     fa->total_tiles = total;
-    fa->problem_offset = 0;
+    fa->problem_offset = e0;
     fa->As = reinterpret_cast<const uint8_t* const*>(ptrs);
     fa->Bs = reinterpret_cast<const uint8_t* const*>(ptrs + p.Et);
     fa->sa = reinterpret_cast<const _Float16* const*>(ptrs + 2 * p.Et);
@@ -249,7 +293,6 @@ __global__ void __launch_bounds__(kPlanThreads) plan_block_kernel(const PlanPair
     fa->acc = nullptr;
     fa->sizes = sizes;
   }
-  (void)routed_tot;
 }
 
 // Kernel for the formats of `h_desc`, checked once on the host: every problem's format has a branch and its shape fits it.
@@ -322,8 +365,8 @@ size_t mxmoe_plan_offset(int which, int num_problems) {
 }
 
 int mxmoe_plan_select_kernel(int kernel_id, const mxmoe_block_desc* h_desc, int num_problems) {
-  if (!h_desc || num_problems <= 0 || num_problems > kMaxProblems) {
-    last_error() = "a planned launch holds 1 to 120 problems";
+  if (!h_desc || num_problems <= 0 || num_problems > kMaxPlannedProblems) {
+    last_error() = "a planned block holds 1 to 4096 problems";
     return -3;
   }
   return resolve_kernel(kernel_id, h_desc, num_problems);
@@ -417,8 +460,9 @@ static int fill_plan_params(PlanParams& p, int kernel_id, const int64_t* d_recv,
   return 0;
 }
 
-static int launch_plan(const PlanPair& pair, int blocks, void* stream) {
-  hipLaunchKernelGGL(plan_block_kernel, dim3(blocks), dim3(kPlanThreads), 0, (hipStream_t)stream, pair);
+static int launch_plan(PlanPair& pair, int blocks, void* stream) {
+  pair.chunks = PlanLayout(pair.p[0].Et).chunks;
+  hipLaunchKernelGGL(plan_block_kernel, dim3(blocks * pair.chunks), dim3(kPlanThreads), 0, (hipStream_t)stream, pair);
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     last_error() = std::string("kernel launch failed: ") + hipGetErrorString(e);
@@ -451,21 +495,25 @@ int mxmoe_plan_layer(const mxmoe_plan_call* gate_up, const mxmoe_plan_call* down
   return launch_plan(pair, 2, stream);
 }
 
-int mxmoe_group_gemm_planned(int kernel_id, const void* d_plan, int grid, void* stream) {
+int mxmoe_group_gemm_planned(int kernel_id, const void* d_plan, int num_problems, int grid, void* stream) {
   auto& reg = registry();
   if (kernel_id < 0 || kernel_id >= (int)reg.size()) {
     last_error() = "kernel id out of range";
     return 2;
   }
-  if (!d_plan || grid <= 0) {
-    last_error() = "null plan or empty grid";
+  if (!d_plan || grid <= 0 || num_problems <= 0 || num_problems > kMaxPlannedProblems) {
+    last_error() = "null plan, empty grid or bad problem count";
     return 5;
   }
   const FusedKernel& k = reg[kernel_id];
-  const hipError_t e = k.launch_planned(reinterpret_cast<const FusedArgs*>(d_plan), grid, k.lds_bytes, (hipStream_t)stream);
-  if (e != hipSuccess) {
-    last_error() = std::string("kernel launch failed: ") + hipGetErrorString(e);
-    return 4;
+  // one launch per chunk of kMaxProblems experts, each reading its own tables (workgroups past a launch's tiles leave at once)
+  const int chunks = PlanLayout(num_problems).chunks;
+  for (int c = 0; c < chunks; ++c) {
+    const hipError_t e = k.launch_planned(reinterpret_cast<const FusedArgs*>(reinterpret_cast<const uint8_t*>(d_plan) + c * kFusedArgsStride), grid, k.lds_bytes, (hipStream_t)stream);
+    if (e != hipSuccess) {
+      last_error() = std::string("kernel launch failed: ") + hipGetErrorString(e);
+      return 4;
+    }
   }
   return 0;
 }

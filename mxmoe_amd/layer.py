@@ -230,12 +230,12 @@ class MxMoELayer:
         hk, hf, _sg, sgp = ps["had1"]
         ck(lib.mxmoe_quant_act_planned(hidden.data_ptr(), b1["inp"].data_ptr(), b1["scale"].data_ptr(), ps["dst"].data_ptr(), ps["perm"].data_ptr(), b1["plan"].data_ptr(),
                                        cfg.hidden, ps["r_cap"], t, e_cnt, has_shared, cfg.rotate, hk, hf, sgp, stream))
-        ck(lib.mxmoe_group_gemm_planned(b1["kid"], b1["plan"].data_ptr(), b1["grid"], stream))
+        ck(lib.mxmoe_group_gemm_planned(b1["kid"], b1["plan"].data_ptr(), ps["et"], b1["grid"], stream))
         i_sh = cfg.inter * max(cfg.num_shared, 1)
         hk, hf, _sg, sgp = ps["had2"]
         ck(lib.mxmoe_silu_mul_quant_planned(ps["mid"].data_ptr(), b1["plan"].data_ptr(), b2["inp"].data_ptr(), b2["scale"].data_ptr(), ps["dst"].data_ptr(), b2["plan"].data_ptr(),
                                             cfg.inter, i_sh, ps["r_cap"], t, e_cnt, has_shared, cfg.rotate, hk, hf, sgp, stream))
-        ck(lib.mxmoe_group_gemm_planned(b2["kid"], b2["plan"].data_ptr(), b2["grid"], stream))
+        ck(lib.mxmoe_group_gemm_planned(b2["kid"], b2["plan"].data_ptr(), ps["et"], b2["grid"], stream))
         ck(lib.mxmoe_combine_planned(ps["out"].data_ptr(), b2["plan"].data_ptr(), ps["et"], w.data_ptr(), ps["row_of_slot"].data_ptr(), t, topk, cfg.hidden,
                                      final.data_ptr(), stream))
         return final

@@ -266,5 +266,6 @@ def test_planned_grid_bound_covers_every_routing(lib):
         assert bound <= 2.5 * worst + 600, (fmts, worst, bound)
     bad = (_lib.BlockDesc * 1)(_lib.BlockDesc(8, 4, -1, 1, (C.c_uint8 * 3)(), 256, 128, 0, 0))
     assert lib.mxmoe_plan_select_kernel(-1, bad, 1) < 0 and lib.mxmoe_last_error() == b"quant type not supported"
-    assert lib.mxmoe_plan_select_kernel(-1, desc, 121) < 0
+    assert lib.mxmoe_plan_select_kernel(-1, desc, 4097) < 0               # checked before any entry is read
+    assert lib.mxmoe_plan_bytes(130) >= 2 * 4096 + 130 * (32 + 40 + 12)   # a block of more than 120 experts: one table header per launch
     assert lib.mxmoe_plan_bytes(60) >= 4096 + 60 * (32 + 40 + 12)

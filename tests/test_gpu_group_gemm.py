@@ -97,6 +97,17 @@ def test_w4a4_on_the_bf6_matrix_path_bit_exact(kernel):
              sb=torch.from_numpy(one[:n].copy()).to(DEV), size=(m, n, k), q=(4, 4, -1, True))
     _, _, accs = _launch([p], kernel_id=kid)
     assert np.array_equal(accs[0], O.int_gemm(qa, qb))
+    # values the quantiser never emits but the format holds (-8, +8), and one-hot operands that pin which (row, k) a lane's bits stand for
+    m, n, k = 96, 256, 512
+    qa, qb = rng.integers(-8, 9, (m, k)).astype(np.int8), rng.integers(-8, 9, (n, k)).astype(np.int8)
+    ha, hb = np.zeros((m, k), np.int8), rng.integers(-8, 9, (n, k)).astype(np.int8)
+    for r in range(m):
+        ha[r, (37 * r + 11) % k] = (r % 15) - 7
+    for a_, b_ in ((qa, qb), (ha, hb)):
+        p = dict(A=pack.pack_bf6_fragments(torch.from_numpy(a_)).to(DEV), B=pack.pack_bf6_fragments(torch.from_numpy(b_)).to(DEV), sa=torch.from_numpy(one[:m].copy()).to(DEV),
+                 sb=torch.from_numpy(one[:n].copy()).to(DEV), size=(m, n, k), q=(4, 4, -1, True))
+        _, _, accs = _launch([p], kernel_id=kid)
+        assert np.array_equal(accs[0], O.int_gemm(a_, b_))
     # shapes the tile does not take are refused on the host
     bad = _wxax_problem(rng, 4, 256, 256, 4, bf6=True)
     bad["size"] = (4, 256, 128)

@@ -439,6 +439,29 @@ def test_layer_with_w8a8_blocks_in_fp8():
         p += 1
 
 
+def test_planned_forward_of_more_experts_than_one_launch_holds():
+    """130 routed experts and a shared one: each block runs as two launches (experts 0 .. 119, then the rest), planned on the device
+    chunk by chunk; the result equals the stepwise operators' (whose host launcher splits long problem lists the same way) and the
+    host-planned forward's, also with experts left empty and with dropped ids."""
+    from mxmoe_amd import synth
+    from mxmoe_amd.layer import MxMoELayer
+
+    cfg = synth.MoEConfig("t", "test", 130, 3, 256, 512, 120, num_shared=1, rotate=1, formats=(synth.W4A4, synth.W8A8, synth.FP16), format_probs=(0.4, 0.4, 0.2))
+    layer = MxMoELayer(cfg)
+    hidden = synth.make_hidden(cfg)
+    ids, w = synth.make_routing(cfg)
+    ids = torch.where(ids == 125, torch.full_like(ids, 7), ids)         # an expert of the second launch receives nothing
+    for trial in range(2):
+        layer.forward(hidden, ids)
+        want = layer.combine(w).clone()
+        got = layer(hidden, ids, w)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), trial
+        assert torch.equal(layer.call_with_host_tables(hidden, ids, w), want)
+        ids = ids.clone()
+        ids[::5, 1] = cfg.num_experts + 3                                # second round: some slots belong to experts held elsewhere
+
+
 def test_single_block_planning_writes_what_the_paired_launch_writes():
     """mxmoe_plan_block (one block per launch) against mxmoe_plan_layer (both blocks of the layer in one launch): identical plan
     buffers for the same counts."""

@@ -169,7 +169,7 @@ def test_function_type_call_with_exactly_fifteen_arguments():
     mxmoe_set_stream; outputs equal the oracle's bit for bit."""
     import ctypes as C
 
-    from mxmoe_amd import _lib
+    from mxmoe_amd import _lib, ops
 
     lib = _lib.load()
     probs = _mixed_problems(np.random.default_rng(23))
@@ -186,7 +186,7 @@ def test_function_type_call_with_exactly_fifteen_arguments():
     ran = 0
     for kid in range(lib.mxmoe_num_kernels()):
         name = lib.mxmoe_kernel_name(kid).decode()
-        if "w4a4_g-1_sym" not in name or "w8a8_g-1_sym" not in name or name.endswith("_b6"):   # (the _b6 kernels take w4a4 operands as bf6 fragments)
+        if "w4a4_g-1_sym" not in name or "w8a8_g-1_sym" not in name or ops.kernel_variants(lib, kid):   # (kernels with operand variants take bf6 fragments / fp8 codes)
             continue
         fn = _lib.FUNC_TYPE(lib.mxmoe_kernel_func(kid))
         for c in Cs:
@@ -201,84 +201,6 @@ def test_function_type_call_with_exactly_fifteen_arguments():
             assert np.array_equal(c.cpu().numpy().view(np.uint16), p["out"].view(np.uint16)), f"{name}: {p['size']} {p['q']}"
         ran += 1
     assert ran >= 4                                                         # wxax, all, seq_launch_all, ms_launch_all
-
-
-def test_bench_diagnostics_run():
-    """bench.py's two diagnostic modes (matrix-pipe probe, one problem on three kinds of operand codes) at toy sizes: they must keep
-    running against the library they ship with, and their figures must be sane (a clock between 0.5 and 3 GHz, rates below the peak)."""
-    import importlib.util
-    from pathlib import Path
-
-    spec = importlib.util.spec_from_file_location("bench_under_test", Path(__file__).resolve().parent.parent / "bench.py")
-    bench = importlib.util.module_from_spec(spec)
-    spec.loader.exec_module(bench)
-    probe = bench.mfma_probe(iters=2000, workgroups=512, repeats=1)
-    assert len(probe["modes"]) == 8
-    for name, m in probe["modes"].items():
-        peak = bench.PEAK["fp6"] if name.startswith("bf6") else bench.PEAK["int8"]
-        assert 0.0 < m["tops"] <= 1.05 * peak and 0.5 < m["shader_clock_ghz"] < 3.0
-    one = bench.one_problem("w4a4:2048x512x1024")
-    assert set(one["operands"]) == {"random codes", "constant codes", "zero codes"}
-    assert all(0.0 < o["tops"] < bench.PEAK["int8"] for o in one["operands"].values())
-
-
-def test_int4_products_are_exact_on_the_bf6_matrix_path():
-    """Integers -8 .. 8 are bf6 (e3m2) numbers and fp32 adds their products exactly, so one v_mfma_scale_f32_32x32x64_f8f6f4 on
-    operands re-encoded as bf6 must return the integer product A . B^T: random int4 matrices, the extreme -8 x -8 (4096 per entry),
-    +8 (outside int4 but a bf6 number; used by symmetric ranges) and a one-hot pattern that pins the lane-to-(row, k) map."""
-    from mxmoe_amd import _lib
-
-    lib = _lib.load()
-    rng = np.random.default_rng(21)
-    onehot_a, onehot_b = np.zeros((32, 64), np.int8), np.zeros((32, 64), np.int8)
-    for r in range(32):
-        onehot_a[r, (5 * r + 3) % 64] = (r % 15) - 7
-        onehot_b[r, (5 * r + 3) % 64] = 7 - (r % 13)
-    cases = [(rng.integers(-8, 8, (32, 64)).astype(np.int8), rng.integers(-8, 8, (32, 64)).astype(np.int8)) for _ in range(4)]
-    cases += [(np.full((32, 64), -8, np.int8), np.full((32, 64), -8, np.int8)), (np.full((32, 64), 8, np.int8), rng.integers(-8, 9, (32, 64)).astype(np.int8)),
-              (onehot_a, onehot_b), (onehot_a, rng.integers(-8, 8, (32, 64)).astype(np.int8))]
-    out = torch.empty(32, 32, dtype=torch.float32, device=DEV)
-    for a, b in cases:
-        ta, tb = torch.from_numpy(a).to(DEV), torch.from_numpy(b).to(DEV)
-        _lib.check(lib, lib.mxmoe_bf6_dot_probe(ta.data_ptr(), tb.data_ptr(), out.data_ptr(), torch.cuda.current_stream().cuda_stream))
-        torch.cuda.synchronize()
-        want = a.astype(np.int64) @ b.astype(np.int64).T
-        assert np.array_equal(out.cpu().numpy().astype(np.int64), want) and np.array_equal(out.cpu().numpy(), want.astype(np.float32))
-
-
-def test_int4_gemm_on_the_bf6_matrix_path_is_exact():
-    """The diagnostic GEMM on bf6 fragments, both workgroup shapes: its accumulators equal the integer product and its fp16 outputs
-    the epilogue formula half(acc * (sa * sb)) evaluated in fp32, bit for bit - several workgroups per XCD range, K of 4 to 24 steps,
-    the values -8 and +8 included."""
-    from mxmoe_amd import _lib, bf6
-
-    lib = _lib.load()
-    rng = np.random.default_rng(33)
-    stream = torch.cuda.current_stream().cuda_stream
-    for shape, (m, n, k) in [(0, (256, 256, 256)), (0, (512, 768, 512)), (0, (256, 512, 1536)), (0, (2304, 256, 768)),
-                             (1, (128, 256, 256)), (1, (384, 768, 512)), (1, (128, 512, 1536)), (1, (1152, 256, 768)), (1, (256, 256, 1408))]:
-        a = rng.integers(-8, 9, (m, k)).astype(np.int8)
-        b = rng.integers(-8, 8, (n, k)).astype(np.int8)
-        sa = (rng.random(m) * 0.05 + 0.001).astype(F16)
-        sb = (rng.random(n) * 0.05 + 0.001).astype(F16)
-        ta, tb = bf6.pack_fragments(torch.from_numpy(a).to(DEV)), bf6.pack_fragments(torch.from_numpy(b).to(DEV))
-        tsa, tsb = torch.from_numpy(sa).to(DEV), torch.from_numpy(sb).to(DEV)
-        c = torch.full((m, n), float("nan"), dtype=torch.float16, device=DEV)
-        ci = torch.full((m, n), -1, dtype=torch.int32, device=DEV)
-        _lib.check(lib, lib.mxmoe_bf6_gemm_probe(ta.data_ptr(), tb.data_ptr(), tsa.data_ptr(), tsb.data_ptr(), c.data_ptr(), ci.data_ptr(), m, n, k, shape, stream))
-        torch.cuda.synchronize()
-        acc = a.astype(np.int64) @ b.astype(np.int64).T
-        assert np.array_equal(ci.cpu().numpy().astype(np.int64), acc), (shape, m, n, k)
-        want = (acc.astype(np.float32) * (sa.astype(np.float32)[:, None] * sb.astype(np.float32)[None, :])).astype(F16)
-        assert np.array_equal(c.cpu().numpy().view(np.uint16), want.view(np.uint16)), (shape, m, n, k)
-        c.fill_(float("nan"))   # the same without the accumulator dump
-        _lib.check(lib, lib.mxmoe_bf6_gemm_probe(ta.data_ptr(), tb.data_ptr(), tsa.data_ptr(), tsb.data_ptr(), c.data_ptr(), None, m, n, k, shape, stream))
-        torch.cuda.synchronize()
-        assert np.array_equal(c.cpu().numpy().view(np.uint16), want.view(np.uint16)), (shape, m, n, k)
-    assert lib.mxmoe_bf6_gemm_probe(ta.data_ptr(), tb.data_ptr(), tsa.data_ptr(), tsb.data_ptr(), c.data_ptr(), None, 250, 256, 256, 0, stream) == 3
-    assert lib.mxmoe_bf6_gemm_probe(ta.data_ptr(), tb.data_ptr(), tsa.data_ptr(), tsb.data_ptr(), c.data_ptr(), None, 128, 256, 256, 0, stream) == 3
-    assert lib.mxmoe_bf6_gemm_probe(ta.data_ptr(), tb.data_ptr(), tsa.data_ptr(), tsb.data_ptr(), c.data_ptr(), None, 256, 256, 256, 2, stream) == 3
-    assert lib.mxmoe_bf6_gemm_probe(ta.data_ptr(), tb.data_ptr(), tsa.data_ptr(), tsb.data_ptr(), c.data_ptr(), None, 256, 256, 1408, 0, stream) == 3
 
 
 def test_bench_harness_on_a_workload_file_and_a_legacy_file(tmp_path, capsys):

@@ -85,29 +85,32 @@ def test_wxax_fragment_order_round_trip_and_lane_map():
 
 def test_bf6_codes_and_fragment_layout():
     """bf6 (e3m2, bias 3) codes of the integers -8 .. 8 decode to themselves, and the fragment buffer holds, for lane l of fragment
-    (k step, row block), row l % 32 and k = 64 * step + 32 * (l // 32) + i as value i at bit 6 i of 24 bytes split 16 + 8."""
+    (row block, k step), row l % 32 and k = 64 * step + 32 * (l // 32) + i as value i at bit 6 i of 24 bytes split 16 + 8; rows are
+    padded to whole blocks of 32; unpacking returns the values."""
     import torch
 
-    from mxmoe_amd import bf6
+    from mxmoe_amd import pack
 
     q = torch.arange(-8, 9, dtype=torch.int8)
-    codes = bf6.encode(q)
+    codes = pack.bf6_encode(q)
     assert codes.tolist() == [56, 55, 54, 53, 52, 50, 48, 44, 0, 12, 16, 18, 20, 21, 22, 23, 24]
-    assert bf6.decode(codes).tolist() == [float(v) for v in range(-8, 9)]
-    assert bf6.decode(torch.tensor([1, 2, 3, 4, 63], dtype=torch.uint8)).tolist() == [0.0625, 0.125, 0.1875, 0.25, -28.0]  # subnormals, largest
-    x = torch.randint(-8, 9, (64, 192), dtype=torch.int8, generator=torch.Generator().manual_seed(4))
-    f = bf6.pack_fragments(x).numpy().reshape(3, 2, bf6.FRAGMENT_BYTES)
-    for ks in range(3):
-        for rb in range(2):
-            for lane in (0, 1, 31, 32, 47, 63):
-                raw = bytes(f[ks, rb, 16 * lane:16 * lane + 16]) + bytes(f[ks, rb, 1024 + 8 * lane:1024 + 8 * lane + 8])
+    assert pack.bf6_decode(codes).tolist() == [float(v) for v in range(-8, 9)]
+    assert pack.bf6_decode(torch.tensor([1, 2, 3, 4, 63], dtype=torch.uint8)).tolist() == [0.0625, 0.125, 0.1875, 0.25, -28.0]  # subnormals, largest
+    x = torch.randint(-8, 9, (50, 192), dtype=torch.int8, generator=torch.Generator().manual_seed(4))
+    buf = pack.pack_bf6_fragments(x)
+    f = buf.numpy().reshape(2, 3, pack.BF6_FRAGMENT_BYTES)
+    for rb in range(2):
+        for ks in range(3):
+            for lane in (0, 1, 17, 31, 32, 47, 63):
+                raw = bytes(f[rb, ks, 16 * lane:16 * lane + 16]) + bytes(f[rb, ks, 1024 + 8 * lane:1024 + 8 * lane + 8])
                 v = int.from_bytes(raw, "little")
-                vals = bf6.decode(torch.tensor([(v >> (6 * i)) & 63 for i in range(32)], dtype=torch.uint8)).to(torch.int8)
-                k0 = 64 * ks + 32 * (lane // 32)
-                assert torch.equal(vals, x[32 * rb + lane % 32, k0:k0 + 32])
+                vals = pack.bf6_decode(torch.tensor([(v >> (6 * i)) & 63 for i in range(32)], dtype=torch.uint8)).to(torch.int8)
+                row, k0 = 32 * rb + lane % 32, 64 * ks + 32 * (lane // 32)
+                assert torch.equal(vals, x[row, k0:k0 + 32] if row < 50 else torch.zeros(32, dtype=torch.int8))
+    assert torch.equal(pack.unpack_bf6_fragments(buf, 50, 192), x.float())
     import pytest
 
     with pytest.raises(ValueError):
-        bf6.encode(torch.tensor([9], dtype=torch.int8))
+        pack.bf6_encode(torch.tensor([9], dtype=torch.int8))
     with pytest.raises(ValueError):
-        bf6.pack_fragments(torch.zeros(33, 64, dtype=torch.int8))
+        pack.pack_bf6_fragments(torch.zeros(32, 96, dtype=torch.int8))
