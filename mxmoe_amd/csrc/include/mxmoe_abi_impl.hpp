@@ -77,8 +77,7 @@ int mxmoe_group_gemm_plan(int kernel_id, const mxmoe_dim3* h_sizes, const mxmoe_
     return 5;
   }
   if (kernel_id < 0) {
-    for (int i = 0; i < (int)reg.size() && kernel_id < 0; ++i)
-      if (reg[i].policy == Policy::Fused && !kernel_has_variants(reg[i]) && kernel_covers(reg[i], h_q, problem_count)) kernel_id = i;
+    kernel_id = auto_kernel(h_sizes, h_q, problem_count);
     if (kernel_id < 0) { last_error() = "quant type not supported"; return 1; }
   }
   if (kernel_id >= (int)reg.size()) { last_error() = "kernel id out of range"; return 2; }

@@ -72,6 +72,7 @@ struct Bf6Tile {
   static constexpr int kPatchBytes = kWaves * 32 * kPitch;
   static constexpr int kLdsBytes = kStages * kStage > kPatchBytes ? kStages * kStage : kPatchBytes;
   static constexpr int kAccRegs = TF * CA * 16;
+  static constexpr int kWavesWanted = 2;  // waves per SIMD a kernel of such tiles is compiled for
   static constexpr int kABits = 6, kWBits = 6;       // bits per activation / weight element as stored
 
   __device__ static __forceinline__ void run(const TileArgs& t, uint8_t* __restrict__ smem) {

@@ -27,6 +27,7 @@ struct WxAxGTile {
   static constexpr int kStageBytes = BM * kRowBytes, kStages = 3;
   static constexpr int kLdsBytes = kStages * kStageBytes;
   static constexpr int kAccRegs = 2 * FM * FN * 16;
+  static constexpr int kWavesWanted = 2;  // waves per SIMD a kernel of such tiles is compiled for
   static constexpr int kABits = 4, kWBits = 4;  // bits per activation / weight element
   static constexpr int kPieces = BM / 16;                       // 1 KB pieces (16 rows) of one activation slice
   static constexpr int kQ = (kPieces + kWaves - 1) / kWaves;    // pieces a wave copies per slice

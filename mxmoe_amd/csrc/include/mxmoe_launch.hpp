@@ -112,8 +112,13 @@ struct Dispatch<I, T, Rest...> {
 
 // Waves per SIMD the register allocator should aim for: 2 (two co-resident workgroups per CU, 256 registers per lane) unless a
 // tile keeps more than 128 accumulator registers per lane, which needs the full 512-register budget of a lone wave.
+// A kernel made only of tiles that ask for more waves (the few-token weight-only tiles: latency-bound streams that gain from every
+// further workgroup in flight) is compiled for the smallest number any of its tiles asks for.
+constexpr int min_of(int a) { return a; }
+template <class... R>
+constexpr int min_of(int a, R... r) { return a < min_of(r...) ? a : min_of(r...); }
 template <class... Tiles>
-constexpr int kWavesPerSimd = ((Tiles::kAccRegs > 128) || ...) ? 1 : 2;
+constexpr int kWavesPerSimd = ((Tiles::kAccRegs > 128) || ...) ? 1 : min_of(Tiles::kWavesWanted...);
 
 // Tables are read through the constant address space: what a workgroup reads from them is the same for all lanes and is not
 // written while the kernel runs (a planned launch's tables were written by the planning kernel before it), so every read is a
@@ -285,10 +290,10 @@ struct BranchOf<Bf6Tile<BM>> {
     return BranchInfo{Fmt::W4A4, BM, T::BN, T::BK, 1, 4, T::kLdsBytes, 128, 0, 256, kVariantBf6};
   }
 };
-template <int WBITS, int BN>
-struct BranchOf<SkinnyWoTile<WBITS, BN>> {
+template <int WBITS, int BN, int KP, int RING, int WAVES>
+struct BranchOf<SkinnyWoTile<WBITS, BN, KP, RING, WAVES>> {
   static BranchInfo get() {
-    using T = SkinnyWoTile<WBITS, BN>;
+    using T = SkinnyWoTile<WBITS, BN, KP, RING, WAVES>;
     return BranchInfo{WBITS == 8 ? Fmt::W8A16 : WBITS == 4 ? Fmt::W4A16 : WBITS == 3 ? Fmt::W3A16 : Fmt::W2A16, T::BM, BN, 128, 1, 4, T::kLdsBytes, 128, 0};
   }
 };
@@ -312,6 +317,9 @@ struct FusedKernel {
   mxmoe_func_t func;  // the kernel as a function of the reference's FuncType (registry.cuh:28-39)
   LaunchPlannedFn launch_planned;  // the same kernel reading its tables from device memory (device-side planning)
   int plan_index;                  // index into plan_infos()
+  // Largest row count per problem this kernel is meant for, 0 = any.  A kernel with a limit is preferred by the automatic choice when
+  // every problem of the list stays within it (the few-token kernels: same results, more workgroups per CU).
+  int max_rows_hint;
 };
 
 inline std::vector<FusedKernel>& registry() {
@@ -531,10 +539,11 @@ struct FuncThunk {
 };
 
 template <class... Tiles>
-int register_fused(const char* fn_name, Policy policy = Policy::Fused) {
+int register_fused(const char* fn_name, Policy policy = Policy::Fused, int max_rows_hint = 0) {
   static_assert(sizeof...(Tiles) <= kMaxBranches, "the planners' branch table holds kMaxBranches tile shapes per kernel");
   FusedKernel k;
   k.policy = policy;
+  k.max_rows_hint = max_rows_hint;
   k.branches = {BranchOf<Tiles>::get()...};
   k.lds_bytes = 0;
   std::string n;
@@ -583,6 +592,27 @@ inline bool kernel_covers(const FusedKernel& k, const mxmoe_qparams* q, int coun
     if (f == Fmt::UNSUPPORTED || plan_segments(plan_of(k), (int)f, 1, 256, sg) < 0) return false;
   }
   return true;
+}
+
+// The kernel the launcher picks when the caller names none: the first fused kernel without operand variants that has a tile for every
+// format; a kernel made for few rows per problem wins when no problem has more (`max_rows` < 0: row counts unknown, none of those).
+inline int auto_kernel_for(const mxmoe_qparams* h_q, int count, long max_rows) {
+  auto& reg = registry();
+  int plain = -1;
+  for (int i = 0; i < (int)reg.size(); ++i) {
+    if (reg[i].policy != Policy::Fused || kernel_has_variants(reg[i]) || !kernel_covers(reg[i], h_q, count)) continue;
+    if (reg[i].max_rows_hint > 0) {
+      if (max_rows >= 0 && max_rows <= reg[i].max_rows_hint) return i;
+    } else if (plain < 0) {
+      plain = i;
+    }
+  }
+  return plain;
+}
+inline int auto_kernel(const mxmoe_dim3* h_sizes, const mxmoe_qparams* h_q, int count) {
+  long max_rows = 0;
+  for (int i = 0; i < count; ++i) max_rows = std::max(max_rows, (long)h_sizes[i].x);
+  return auto_kernel_for(h_q, count, max_rows);
 }
 
 // K a multiple of the tile's K step, N a multiple of 8 (16 for the weight-only layouts)
@@ -712,8 +742,7 @@ inline int group_gemm(int kernel_id, const void* const* As, const void* const* B
   if (count <= 0) return 0;
   auto& reg = registry();
   if (kernel_id < 0) {
-    for (int i = 0; i < (int)reg.size() && kernel_id < 0; ++i)
-      if (reg[i].policy == Policy::Fused && !kernel_has_variants(reg[i]) && kernel_covers(reg[i], h_q, count)) kernel_id = i;
+    kernel_id = auto_kernel(h_sizes, h_q, count);
     if (kernel_id < 0) {
       last_error() = "quant type not supported";  // same message as the reference launcher (compose_kernel.py:433)
       return 1;

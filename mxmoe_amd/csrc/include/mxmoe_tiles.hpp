@@ -180,6 +180,7 @@ struct MfmaTile {
   static constexpr int kStages = 3;
   static constexpr int kLdsBytes = kStages * kStageBytes;
   static constexpr int kAccRegs = FM * FN * 16;
+  static constexpr int kWavesWanted = 2;  // waves per SIMD a kernel of such tiles is compiled for
   static constexpr int kABits = OpTraits<OP>::kBitsPerElem, kWBits = kABits;  // bits per activation / weight element
   static constexpr int A_CHUNKS = BM * 4, B_CHUNKS = BN * 4;
   static constexpr int A_IT = (A_CHUNKS + kThreads - 1) / kThreads, B_IT = (B_CHUNKS + kThreads - 1) / kThreads;
@@ -495,6 +496,7 @@ struct WxAxTile {
   static constexpr int kPatchBytes = kWaves * FI * 32 * kPitch;
   static constexpr int kLdsBytes = kStages * kStageBytes > kPatchBytes ? kStages * kStageBytes : kPatchBytes;
   static constexpr int kAccRegs = FM * FN * 16;
+  static constexpr int kWavesWanted = 2;  // waves per SIMD a kernel of such tiles is compiled for
   static constexpr int kABits = OpTraits<OP>::kBitsPerElem, kWBits = kABits;  // bits per activation / weight element
   static constexpr int kOps = OP == Op::I4 ? 2 : 1;
   static constexpr int U = 4;                                    // units per K slice

@@ -32,21 +32,24 @@
 
 namespace mxmoe {
 
-template <int WBITS_, int BN_>
+// KP: k blocks (128 wide) per pass of a wave, whose activations live in registers; RING: packed weight blocks in flight per wave;
+// WAVES: waves per SIMD a kernel made of such tiles alone is compiled for (fewer registers per wave, more workgroups per CU).
+template <int WBITS_, int BN_, int KP_ = 4, int RING_ = (WBITS_ == 8 ? 6 : 12), int WAVES_ = 2>
 struct SkinnyWoTile {
   static constexpr int WBITS = WBITS_, BM = 16, BN = BN_;
   static_assert(WBITS == 8 || WBITS == 4 || WBITS == 3 || WBITS == 2, "w8 / w4 / w3 / w2");
   static_assert(BN % 64 == 0, "the final reduction deals 16-channel blocks to 4 waves");
   static constexpr int NB = BN / 16;                 // 16-channel blocks per tile
-  static constexpr int KP = 4;                       // k blocks (128 wide) per pass of a wave: their activations live in registers
+  static constexpr int KP = KP_;                     // k blocks (128 wide) per pass of a wave: their activations live in registers
   static constexpr int kRedBytes = kWaves * NB * 64 * 16;  // per-wave partial sums for the final reduction
   static constexpr int kScaleBytes = NB * KP * 64;         // per-wave patch of (scale, zero) pairs of one pass
   static constexpr int kLdsBytes = kRedBytes + kWaves * kScaleBytes;
   static constexpr int kAccRegs = NB * 4;
+  static constexpr int kWavesWanted = WAVES_;
   static constexpr int kABits = 16, kWBits = WBITS;  // fp16 activations, packed weights
   static constexpr int kLaneBytes = WBITS * 4;       // packed bytes per lane per (channel block, k block)
   static constexpr int kBlockBytes = 64 * kLaneBytes;
-  static constexpr int kRing = WBITS == 8 ? 6 : 12;  // packed blocks in flight per wave (12 KB either way)
+  static constexpr int kRing = RING_;                // packed blocks in flight per wave (12 KB by default)
 
   struct WReg {
     int d[WBITS];
@@ -224,10 +227,16 @@ struct SkinnyWoTile {
     for (int nb = 0; nb < NB; ++nb) acc[nb] = v4f{0.f, 0.f, 0.f, 0.f};
     for (int kb = kb_lo; kb < kb_hi; kb += KP) {
       const int nk = min(KP, kb_hi - kb);
-      if (nk == 4) pass<4>(t, kb, m0, n0, nbv, lane, spatch, acc);
-      else if (nk == 3) pass<3>(t, kb, m0, n0, nbv, lane, spatch, acc);
-      else if (nk == 2) pass<2>(t, kb, m0, n0, nbv, lane, spatch, acc);
-      else pass<1>(t, kb, m0, n0, nbv, lane, spatch, acc);
+      if constexpr (KP >= 4) {
+        if (nk == 4) { pass<4>(t, kb, m0, n0, nbv, lane, spatch, acc); continue; }
+      }
+      if constexpr (KP >= 3) {
+        if (nk == 3) { pass<3>(t, kb, m0, n0, nbv, lane, spatch, acc); continue; }
+      }
+      if constexpr (KP >= 2) {
+        if (nk == 2) { pass<2>(t, kb, m0, n0, nbv, lane, spatch, acc); continue; }
+      }
+      pass<1>(t, kb, m0, n0, nbv, lane, spatch, acc);
     }
 
     // reduction over the 4 waves in a fixed order (wave 0 + 1 + 2 + 3), 16-channel blocks dealt round-robin to the waves
@@ -283,10 +292,11 @@ struct WoMfmaTile {
   static constexpr int WM = BN == 128 ? 2 : 1;  // waves along the tokens
   static constexpr int TM = BM / WM;            // tokens per wave
   static constexpr int MB = TM / 16;            // token blocks per wave
-  using Sk = SkinnyWoTile<WBITS, 128>;
+  using Sk = SkinnyWoTile<WBITS, 128>;  // (its packed-block loader and unpacker)
   static constexpr int kStageBytes = BM * 256;
   static constexpr int kLdsBytes = 2 * kStageBytes;
   static constexpr int kAccRegs = 16 * MB;
+  static constexpr int kWavesWanted = 2;
   static constexpr int kABits = 16, kWBits = WBITS;  // fp16 activations, packed weights
   static constexpr int kLaneBytes = Sk::kLaneBytes, kBlockBytes = Sk::kBlockBytes;
   static constexpr int kDma = kStageBytes / 1024 / kWaves;  // direct-to-LDS loads per wave per stage

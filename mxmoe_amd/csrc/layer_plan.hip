@@ -311,7 +311,7 @@ static int resolve_kernel(int kernel_id, const mxmoe_block_desc* h_desc, int et)
   };
   if (kernel_id < 0) {
     for (int i = 0; i < (int)reg.size() && kernel_id < 0; ++i)
-      if (reg[i].policy == Policy::Fused && covers(reg[i])) kernel_id = i;
+      if (reg[i].policy == Policy::Fused && reg[i].max_rows_hint == 0 && covers(reg[i])) kernel_id = i;  // (row counts are not known here: no few-row kernel)
     if (kernel_id < 0) {
       last_error() = "quant type not supported";
       return -1;

@@ -142,20 +142,23 @@ class TemplateGenerator:
         return _build.hipcc_build(self.files, Path(out))
 
 
-def build_kernel_source(tile_cfg, kname: str, kernel_type: KernelType = KernelType.Fused, deferred: bool = False):
+def build_kernel_source(tile_cfg, kname: str, kernel_type: KernelType = KernelType.Fused, deferred: bool = False, max_rows_hint: int = 0):
     """(declaration comment, translation unit) of one kernel; `tile_cfg` maps qcfg -> TileConfig or tuple of TileConfig.
-    `deferred`: the unit defines `register_<kname>()` instead of registering from a static initialiser."""
+    `deferred`: the unit defines `register_<kname>()` instead of registering from a static initialiser.  `max_rows_hint`: the kernel
+    is meant for problems of at most that many rows (the launcher's automatic choice prefers it when no problem has more)."""
     pairs = [(q, t) for q, item in tile_cfg.items() for t in _flat([item])]
     tiles = ", ".join(t.cpp_type() for _, t in pairs)
     comment = "; ".join(f"{q} if {BRANCH_CONDITION_MAP[q]} -> {t.to_str()}" for q, t in pairs)
-    defn = (KERNEL_DEFERRED_TEMPLATE if deferred else KERNEL_DEFINITION_TEMPLATE).substitute(KernelName=kname, Tiles=tiles, Comment=comment, Policy=POLICY[str(kernel_type)])
+    defn = (KERNEL_DEFERRED_TEMPLATE if deferred else KERNEL_DEFINITION_TEMPLATE).substitute(KernelName=kname, Tiles=tiles, Comment=comment, Policy=POLICY[str(kernel_type)],
+                                                                                                  Hint=f", {max_rows_hint}" if max_rows_hint else "")
     decl = f"//   {kname}: " + ", ".join(f"[{q}: ({t.BM},{t.BN},{t.BK}) ({t.WM},{t.WN},{t.WK}) {t.STAGE}]" for q, t in pairs)
     return decl, defn
 
 
-def _pick(arch: str, qcfg: str, *shapes, bf6: bool = False):
-    """Candidate tiles of `qcfg` with the given (BM, BN) shapes, in that order (`bf6`: the tiles on the 6-bit float path)."""
-    by_shape = {(t.BM, t.BN): t for t in get_possible_tile_list(arch, qcfg) if t.is_bf6() == bf6}
+def _pick(arch: str, qcfg: str, *shapes, bf6: bool = False, few_registers: bool = False):
+    """Candidate tiles of `qcfg` with the given (BM, BN) shapes, in that order (`bf6`: the tiles on the 6-bit float path;
+    `few_registers`: the few-token weight-only tiles in their few-register shape)."""
+    by_shape = {(t.BM, t.BN): t for t in get_possible_tile_list(arch, qcfg) if t.is_bf6() == bf6 and (t.is_skinny() and t.STAGE == 4) == few_registers}
     return tuple(by_shape[s] for s in shapes)
 
 
@@ -182,6 +185,10 @@ def default_kernel_specs(arch: str = "gfx950"):
         # tag 4, pack.pack_bf6_fragments).  Registered last: a caller that does not ask for them by name never gets them.
         # 8-bit weight-only formats in a kernel of their own (their tiles hold twice the packed registers of the 4-bit ones; a kernel
         # runs at the occupancy of its largest branch)
+        # the few-token tiles of the 4 / 3 / 2-bit weight-only formats alone: without the many-token tiles' registers three workgroups
+        # share a CU instead of two, which is what these latency-bound weight streams gain from (decode-sized batches)
+        ("groupgemm_hz_fused_wo_skinny", KernelType.Fused,
+         OrderedDict((f"w{b}a16_g128_asym", _pick(arch, f"w{b}a16_g128_asym", (16, 128), few_registers=True)) for b in (4, 3, 2))),
         ("groupgemm_hz_fused_wo8", KernelType.Fused, OrderedDict([("w8a16_g128_asym", _pick(arch, "w8a16_g128_asym", (16, 128), (128, 128)))])),
         # w8a8 in fp8 (e4m3 codes on both sides), next to w4a4
         ("groupgemm_hz_fused_wxax_e4m3", KernelType.Fused, OrderedDict([(w4, _pick(arch, w4, (128, 256), (64, 256), (32, 256))),
@@ -189,6 +196,10 @@ def default_kernel_specs(arch: str = "gfx950"):
         ("groupgemm_hz_fused_wxax_b6", KernelType.Fused, OrderedDict([(w4, _pick(arch, w4, (128, 256), (64, 256), (32, 256), bf6=True)), (w8, _pick(arch, w8, (128, 256), (64, 256), (32, 256)))])),
         ("groupgemm_hz_fused_all_b6", KernelType.Fused, everything_b6),
     ]
+
+
+# default kernels meant for problems of few rows only
+MAX_ROWS_HINT = {"groupgemm_hz_fused_wo_skinny": 64}
 
 
 def emit_default_library(out_dir: str | os.PathLike | None = None, arch: str = "gfx950") -> list:
@@ -205,7 +216,7 @@ def emit_default_library(out_dir: str | os.PathLike | None = None, arch: str = "
             t.validate()
         if not is_fusion_compatible(list(tile_cfg.values())):
             raise ValueError(f"{kname}: branches disagree on the wavefront count")
-        _decl, defn = build_kernel_source(tile_cfg, kname, ktype, deferred=True)
+        _decl, defn = build_kernel_source(tile_cfg, kname, ktype, deferred=True, max_rows_hint=MAX_ROWS_HINT.get(kname, 0))
         path = out_dir / f"default_{kname}.hip"
         if not path.exists() or path.read_text() != defn:
             path.write_text(defn)

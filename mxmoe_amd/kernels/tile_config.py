@@ -3,7 +3,7 @@
 `TileConfig` / `QConfig` / `NO_QUANT` keep the fields (and therefore the dataclass `repr`, which is the key of the
 kernel-profile table) of mxmoe/kernels/tile_config.py:122-286.  What changes is the meaning the hardware gives them:
 WM x WN x WK counts 64-lane wavefronts (always 4 per workgroup here), MMA names an MFMA instruction, STAGE is the number of
-LDS ring slots of the DMA pipeline (3 for the MFMA tiles; 2 = the register double buffer of the skinny tiles), and the candidate lists are those compiled for gfx950.
+LDS ring slots of the DMA pipeline (3 for the MFMA tiles; for the few-token weight-only tiles 2 names the 12-deep register ring with 4 k blocks per pass and 4 the few-register shape), and the candidate lists are those compiled for gfx950.
 """
 from __future__ import annotations
 
@@ -190,8 +190,8 @@ class TileConfig:
 
     def smem_bytes_tile(self):
         """LDS bytes of the tile as compiled (csrc/include/mxmoe_tiles.hpp, mxmoe_wo_tiles.hpp)."""
-        if self.is_skinny():
-            return 4 * (self.BN // 16) * (64 * 16 + 4 * 64)  # per-wave partial sums of the final reduction + (scale, zero) patches
+        if self.is_skinny():  # per-wave partial sums of the final reduction + (scale, zero) patches of one pass (4 k blocks, or 2)
+            return 4 * (self.BN // 16) * (64 * 16 + (2 if self.STAGE == 4 else 4) * 64)
         if self.is_weight_only():
             return 2 * self.BM * 256  # two stages of BM activation rows x one 128-wide k block
         if self.is_group_wa():
@@ -205,7 +205,8 @@ class TileConfig:
     def cpp_type(self) -> str:
         """The C++ tile type this descriptor instantiates."""
         if self.is_skinny():
-            return f"SkinnyWoTile<{self.QCFGB.QBITS}, {self.BN}>"
+            # STAGE 4: the few-register shape (2 k blocks per pass, 4 packed blocks in flight per wave, compiled for 3 waves per SIMD)
+            return f"SkinnyWoTile<{self.QCFGB.QBITS}, {self.BN}, 2, 4, 3>" if self.STAGE == 4 else f"SkinnyWoTile<{self.QCFGB.QBITS}, {self.BN}>"
         if self.is_weight_only():
             return f"WoMfmaTile<{self.QCFGB.QBITS}, {self.BM}, {self.BN}>"
         if self.is_bf6():
@@ -273,6 +274,8 @@ def get_possible_tile_list(arch: str, qcfg: str) -> list:
     mma = QCFG_TO_MMA[qcfg]
     if mma == "MFMA_F32_16x16x32_F16":
         skinny = [_with_q(TileConfig(BM=16, BN=bn, BK=128, WM=1, WN=4, WK=1, STAGE=2, MMA=mma), qcfg) for bn in (128, 64)]
+        if QCFG_MAP[qcfg].QCFGB.QBITS != 8:  # the few-register shape, for kernels made of few-token tiles alone (three workgroups per CU)
+            skinny.append(_with_q(TileConfig(BM=16, BN=128, BK=128, WM=1, WN=4, WK=1, STAGE=4, MMA=mma), qcfg))
         # (8-bit weights: the ring of packed blocks is twice as large, which leaves room for the 2 x 2 shape's accumulators only)
         shapes = ((128, 2, 2),) if QCFG_MAP[qcfg].QCFGB.QBITS == 8 else ((128, 2, 2), (256, 1, 4))
         big = [_with_q(TileConfig(BM=128, BN=bn, BK=128, WM=wm, WN=wn, WK=1, STAGE=2, MMA=mma), qcfg) for bn, wm, wn in shapes]

@@ -157,6 +157,10 @@ class MxMoELayer:
             kid = lib.mxmoe_plan_select_kernel(-1, h, et)
             if kid < 0:
                 raise RuntimeError(lib.mxmoe_last_error().decode())
+            if t <= 64:  # no problem can have more rows than there are tokens: a kernel made of few-token tiles alone, if one covers the formats
+                few = lib.mxmoe_find_kernel(b"groupgemm_hz_fused_wo_skinny")
+                if few >= 0 and lib.mxmoe_plan_select_kernel(few, h, et) == few:
+                    kid = few
             grid = lib.mxmoe_plan_grid_bound(kid, h, e_cnt, r_cap, shared_rows)
             if grid < 0:
                 raise RuntimeError(lib.mxmoe_last_error().decode())
