@@ -205,6 +205,12 @@ int mxmoe_plan_grid_bound(int kernel_id, const mxmoe_block_desc* h_desc, int num
 int mxmoe_plan_block(int kernel_id, const int64_t* d_recv_tokens_per_exp, int num_experts, int shared_rows, const mxmoe_block_desc* d_desc,
                      const mxmoe_block_desc* h_desc, const void* inp_store, const void* scale_store, void* out_store, void* d_plan, void* stream);
 int mxmoe_plan_layer(const mxmoe_plan_call* gate_up, const mxmoe_plan_call* down, const int64_t* d_recv_tokens_per_exp, int num_experts, int shared_rows, void* stream);
+/* mxmoe_build_permutation_inv and mxmoe_plan_layer in ONE launch, for decode-sized batches (num_tokens * topk <= 256, error 3 beyond):
+ * one workgroup builds the permutation while the others plan both blocks from counts they take from topk_ids themselves.  Same
+ * outputs as the two calls (no workspace is needed at this size). */
+int mxmoe_permute_plan_layer(const int32_t* topk_ids, int num_tokens, int topk, int num_experts, int32_t* dst_exp_sorted, int64_t* perm_indices, int64_t* src_slot,
+                             int64_t* recv_tokens_per_exp, int32_t* row_of_slot, const mxmoe_plan_call* gate_up, const mxmoe_plan_call* down, int shared_rows,
+                             void* stream);
 int mxmoe_group_gemm_planned(int kernel_id, const void* d_plan, int num_problems, int grid, void* stream);
 int mxmoe_quant_act_planned(const void* hidden, void* inp_store, void* scale_store, const int32_t* dst_exp_sorted, const int64_t* perm_indices, const void* d_plan,
                             int K, int rows_capacity, int num_tokens, int num_experts, int has_shared, int rotate, int had_k, int had_f, const float* had_signs,

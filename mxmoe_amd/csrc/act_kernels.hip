@@ -22,23 +22,13 @@
 #include "../../include/mxmoe_amd.h"
 #include "include/mxmoe_launch.hpp"
 #include "include/mxmoe_plan.hpp"
+#include "include/mxmoe_perm.hpp"
 
 namespace mxmoe {
 
 // ------------------------------------------------------------------------------------------------------------
 // Stable permutation by expert
 // ------------------------------------------------------------------------------------------------------------
-constexpr int kPermChunk = 256;  // flattened (token, slot) entries per single-wave workgroup
-
-// lanes of the wave that hold the same expert id as this lane (ids < 2^16)
-__device__ __forceinline__ uint64_t match_same(int e, int nbits) {
-  uint64_t m = ~0ull;
-  for (int b = 0; b < nbits; ++b) {
-    const uint64_t bal = __ballot((e >> b) & 1);
-    m &= ((e >> b) & 1) ? bal : ~bal;
-  }
-  return m;
-}
 
 __global__ void __launch_bounds__(64) perm_hist_kernel(const int32_t* __restrict__ ids, int total, int E, int32_t* __restrict__ hist /*[blocks][E]*/) {
   extern __shared__ int32_t cnt[];
@@ -54,16 +44,6 @@ __global__ void __launch_bounds__(64) perm_hist_kernel(const int32_t* __restrict
   }
   __syncthreads();
   for (int e = threadIdx.x; e < E; e += 64) hist[blockIdx.x * E + e] = cnt[e];
-}
-
-// inclusive scan of one value per lane across the wave
-__device__ __forceinline__ int wave_inclusive_scan(int v, int lane) {
-#pragma unroll
-  for (int o = 1; o < 64; o <<= 1) {
-    const int t = __shfl_up(v, o);
-    if (lane >= o) v += t;
-  }
-  return v;
 }
 
 // one single-wave workgroup per expert: exclusive scan of the expert's per-block counts (64 blocks per step); total -> recv
@@ -121,51 +101,12 @@ __global__ void __launch_bounds__(64) perm_scatter_kernel(const int32_t* __restr
 }
 
 // The three kernels above in one, for at most kPermChunk (token, slot) entries (decode-sized batches): one single-wave workgroup
-// counts, scans the experts and scatters, where three launches would cost more than their work.
+// counts, scans the experts and scatters, where three launches would cost more than their work (body: mxmoe_perm.hpp).
 __global__ void __launch_bounds__(64) perm_small_kernel(const int32_t* __restrict__ ids, int total, int E, int topk, int nbits, int64_t* __restrict__ recv,
                                                         int32_t* __restrict__ dst_exp_sorted, int64_t* __restrict__ perm, int64_t* __restrict__ src_slot,
                                                         int32_t* __restrict__ row_of_slot) {
   extern __shared__ int32_t run[];  // [E] counts, then next free rank per expert
-  const int lane = threadIdx.x;
-  for (int e = lane; e < E; e += 64) run[e] = 0;
-  __syncthreads();
-  for (int idx = lane; idx < total; idx += 64) {
-    const int e = ids[idx];
-    if (e >= 0 && e < E) atomicAdd(&run[e], 1);
-  }
-  __syncthreads();
-  int carry = 0;
-  for (int e0 = 0; e0 < E; e0 += 64) {
-    const int e = e0 + lane;
-    const int v = e < E ? run[e] : 0;
-    const int inc = wave_inclusive_scan(v, lane);
-    if (e < E) {
-      recv[e] = v;
-      run[e] = carry + inc - v;
-    }
-    carry += __shfl(inc, 63);
-  }
-  __syncthreads();
-  for (int i = 0; i < total; i += 64) {  // sub-chunks in order keep the sort stable
-    const int idx = i + lane;
-    const bool ok = idx < total;
-    int e = ok ? ids[idx] : -1;
-    if (e < 0 || e >= E) e = E;
-    const uint64_t same = match_same(e, nbits);
-    const int before = __popcll(same & ((1ull << lane) - 1));
-    int first = 0;
-    if (e < E) first = run[e];
-    __syncthreads();
-    if (e < E) {
-      const int pos = first + before;
-      dst_exp_sorted[pos] = e;
-      perm[pos] = idx / topk;
-      if (src_slot) src_slot[pos] = idx;
-      if (before == 0) run[e] = first + __popcll(same);
-    }
-    if (row_of_slot && ok) row_of_slot[idx] = e < E ? first + before : -1;
-    __syncthreads();
-  }
+  perm_small_body(ids, total, E, topk, nbits, recv, dst_exp_sorted, perm, src_slot, row_of_slot, run, true);
 }
 
 // ------------------------------------------------------------------------------------------------------------

@@ -11,6 +11,7 @@
 #include "../../include/mxmoe_amd.h"
 #include "include/mxmoe_launch.hpp"
 #include "include/mxmoe_plan.hpp"
+#include "include/mxmoe_perm.hpp"
 
 namespace mxmoe {
 
@@ -67,9 +68,8 @@ struct PlanPair {
   int chunks;  // launches per block
 };
 
-__global__ void __launch_bounds__(kPlanThreads) plan_block_kernel(const PlanPair pair) {
-  const PlanParams& p = pair.p[blockIdx.x / pair.chunks];  // one workgroup per launch of each block of the layer (gate_up, down): all only read the counts
-  const int chunk = blockIdx.x % pair.chunks;
+// `recv`: the tokens-per-expert counts (device memory, or LDS when the planning workgroup counted them itself).
+__device__ __forceinline__ void plan_block_body(const PlanParams& p, const int chunk, const int chunks, const int64_t* recv) {
   const int e0 = chunk * kMaxProblems;                       // first expert of this launch
   const int ecnt = min(kMaxProblems, p.Et - e0);             // experts of this launch
   __shared__ long s_tot[4][2];                       // per wave: rows, packed input, scales, output elements
@@ -89,7 +89,7 @@ __global__ void __launch_bounds__(kPlanThreads) plan_block_kernel(const PlanPair
   // what one expert occupies: rows, packed activation elements, scales, output elements (all in fp16 elements but the rows)
   auto footprint = [&](int x, long (&f)[4], int* tag_out, mxmoe_block_desc* d_out) {
     const mxmoe_block_desc d = p.desc[x];
-    const long rows = x < p.E ? (long)p.recv[x] : (long)p.shared_rows;
+    const long rows = x < p.E ? (long)recv[x] : (long)p.shared_rows;
     const int tag = act_tag_of(d.q), K = (int)d.K;
     const long qld = tag == 0 ? K : (tag == 1 || tag == 5 ? K / 2 : K / 4);  // fp16 elements per packed activation row (ref_bind.cu:491)
     const long sld = tag == 0 ? 0 : (tag == 3 ? K / 128 : 1);                // scales per row (ref_bind.cu:492)
@@ -260,7 +260,7 @@ __global__ void __launch_bounds__(kPlanThreads) plan_block_kernel(const PlanPair
   }
   if (e == 0) {
     // rows routed = sum over the routed experts of every launch: the last launch knows them all
-    if (chunk == pair.chunks - 1) misc[0] = s_base[4][0] + s_base[4][1] + s_routed[0] + s_routed[1];
+    if (chunk == chunks - 1) misc[0] = s_base[4][0] + s_base[4][1] + s_routed[0] + s_routed[1];
     if (chunk == 0 && p.Et == p.E) misc[1] = 0;
     int total = 0, wg = 0, np = 0, ne = 0, flat = 0;
     int last_tile0 = 0, last_wg0 = 0;  // of the phase being filled (kept here: reading them back from the table would wait for the store)
@@ -293,6 +293,42 @@ __global__ void __launch_bounds__(kPlanThreads) plan_block_kernel(const PlanPair
     fa->acc = nullptr;
     fa->sizes = sizes;
   }
+}
+
+__global__ void __launch_bounds__(kPlanThreads) plan_block_kernel(const PlanPair pair) {
+  // one workgroup per launch of each block of the layer (gate_up, down): all only read the counts
+  plan_block_body(pair.p[blockIdx.x / pair.chunks], blockIdx.x % pair.chunks, pair.chunks, pair.p[0].recv);
+}
+
+// Permutation and planning of a decode-sized batch (at most kPermChunk (token, slot) entries) in ONE launch: workgroup 0 builds the
+// permutation, the others plan the layer's launches from counts they take from the routed ids themselves (a few hundred ids: cheaper
+// than waiting for workgroup 0 in a second launch).  A forward of some tens of microseconds feels every launch it saves.
+struct PermSmallArgs {
+  const int32_t* ids;
+  int total, E, topk, nbits;
+  int64_t* recv;
+  int32_t* dst;
+  int64_t* perm;
+  int64_t* slot;
+  int32_t* row_of_slot;
+};
+__global__ void __launch_bounds__(kPlanThreads) perm_plan_small_kernel(const PermSmallArgs a, const PlanPair pair) {
+  extern __shared__ __align__(8) uint8_t pp_lds[];  // E int32 counters (workgroup 0) or E int64 counts (planning workgroups)
+  if (blockIdx.x == 0) {
+    perm_small_body(a.ids, a.total, a.E, a.topk, a.nbits, a.recv, a.dst, a.perm, a.slot, a.row_of_slot, reinterpret_cast<int32_t*>(pp_lds), threadIdx.x < 64);
+    return;
+  }
+  int64_t* counts = reinterpret_cast<int64_t*>(pp_lds);
+  unsigned long long* cnt = reinterpret_cast<unsigned long long*>(pp_lds);
+  for (int e = threadIdx.x; e < a.E; e += kPlanThreads) counts[e] = 0;
+  __syncthreads();
+  for (int i = threadIdx.x; i < a.total; i += kPlanThreads) {
+    const int e = a.ids[i];
+    if (e >= 0 && e < a.E) atomicAdd(&cnt[e], 1ull);
+  }
+  __syncthreads();
+  const int b = blockIdx.x - 1;
+  plan_block_body(pair.p[b / pair.chunks], b % pair.chunks, pair.chunks, counts);
 }
 
 // Kernel for the formats of `h_desc`, checked once on the host: every problem's format has a branch and its shape fits it.
@@ -493,6 +529,45 @@ int mxmoe_plan_layer(const mxmoe_plan_call* gate_up, const mxmoe_plan_call* down
     if (rc) return rc;
   }
   return launch_plan(pair, 2, stream);
+}
+
+int mxmoe_permute_plan_layer(const int32_t* topk_ids, int num_tokens, int topk, int num_experts, int32_t* dst_exp_sorted, int64_t* perm_indices, int64_t* src_slot,
+                             int64_t* recv_tokens_per_exp, int32_t* row_of_slot, const mxmoe_plan_call* gate_up, const mxmoe_plan_call* down, int shared_rows, void* stream) {
+  if (num_tokens <= 0 || topk <= 0 || num_experts <= 0 || num_experts > kMaxPlannedProblems || (long)num_tokens * topk > kPermChunk) {
+    last_error() = "the one-launch permutation + planning takes at most 256 (token, slot) entries: use mxmoe_build_permutation_inv and mxmoe_plan_layer";
+    return 3;
+  }
+  if (!topk_ids || !dst_exp_sorted || !perm_indices || !src_slot || !recv_tokens_per_exp || !gate_up || !down) {
+    last_error() = "null pointer";
+    return 5;
+  }
+  PlanPair pair;
+  const mxmoe_plan_call* c[2] = {gate_up, down};
+  for (int i = 0; i < 2; ++i) {
+    const int rc = fill_plan_params(pair.p[i], c[i]->kernel_id, recv_tokens_per_exp, num_experts, shared_rows, c[i]->d_desc, c[i]->h_desc, c[i]->inp_store, c[i]->scale_store,
+                                    c[i]->out_store, c[i]->d_plan);
+    if (rc) return rc;
+  }
+  pair.chunks = PlanLayout(pair.p[0].Et).chunks;
+  PermSmallArgs a;
+  a.ids = topk_ids;
+  a.total = num_tokens * topk;
+  a.E = num_experts;
+  a.topk = topk;
+  a.nbits = 1;
+  while ((1 << a.nbits) <= num_experts) ++a.nbits;  // ids 0..E (E = parked lanes)
+  a.recv = recv_tokens_per_exp;
+  a.dst = dst_exp_sorted;
+  a.perm = perm_indices;
+  a.slot = src_slot;
+  a.row_of_slot = row_of_slot;
+  hipLaunchKernelGGL(perm_plan_small_kernel, dim3(1 + 2 * pair.chunks), dim3(kPlanThreads), (size_t)num_experts * 8, (hipStream_t)stream, a, pair);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    last_error() = std::string("kernel launch failed: ") + hipGetErrorString(e);
+    return 4;
+  }
+  return 0;
 }
 
 int mxmoe_group_gemm_planned(int kernel_id, const void* d_plan, int num_problems, int grid, void* stream) {

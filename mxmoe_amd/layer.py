@@ -211,7 +211,7 @@ class MxMoELayer:
         Same kernels and results as `forward` + `combine`, but nothing here waits for the routing: the tables of both launches are
         derived from the tokens-per-expert counts by a planning kernel on the device (`mxmoe_plan_layer`: both blocks in one launch), the stores and plan
         buffers are allocated once per (tokens, top-k) for the worst case, and every launch argument is independent of the data.
-        The call only enqueues seven kernels (nine when more than 256 (token, slot) pairs are permuted; no synchronisation, no allocation after the first call when `out` is given), so it can
+        The call only enqueues six kernels (nine when more than 256 (token, slot) pairs are permuted; no synchronisation, no allocation after the first call when `out` is given), so it can
         be captured into a HIP graph.  Intermediate buffers belong to the layer and are reused by the next call of the same shape."""
         cfg, dev = self.cfg, self.device
         lib = _lib.load()
@@ -228,9 +228,13 @@ class MxMoELayer:
         final = out if out is not None else torch.empty((t, cfg.hidden), dtype=torch.float16, device=dev)
         assert final.shape == (t, cfg.hidden) and final.dtype == torch.float16 and final.is_contiguous()
         ck = lambda rc: _lib.check(lib, rc)  # noqa: E731
-        ck(lib.mxmoe_build_permutation_inv(ids.data_ptr(), t, topk, e_cnt, ps["dst"].data_ptr(), ps["perm"].data_ptr(), ps["slot"].data_ptr(), ps["recv"].data_ptr(),
-                                           ps["row_of_slot"].data_ptr(), ps["perm_ws"].data_ptr(), stream))
-        ck(lib.mxmoe_plan_layer(C.byref(ps["calls"][0]), C.byref(ps["calls"][1]), ps["recv"].data_ptr(), e_cnt, ps["shared_rows"], stream))
+        if ps["r_cap"] <= 256:  # decode-sized batch: permutation and planning in one launch
+            ck(lib.mxmoe_permute_plan_layer(ids.data_ptr(), t, topk, e_cnt, ps["dst"].data_ptr(), ps["perm"].data_ptr(), ps["slot"].data_ptr(), ps["recv"].data_ptr(),
+                                            ps["row_of_slot"].data_ptr(), C.byref(ps["calls"][0]), C.byref(ps["calls"][1]), ps["shared_rows"], stream))
+        else:
+            ck(lib.mxmoe_build_permutation_inv(ids.data_ptr(), t, topk, e_cnt, ps["dst"].data_ptr(), ps["perm"].data_ptr(), ps["slot"].data_ptr(), ps["recv"].data_ptr(),
+                                               ps["row_of_slot"].data_ptr(), ps["perm_ws"].data_ptr(), stream))
+            ck(lib.mxmoe_plan_layer(C.byref(ps["calls"][0]), C.byref(ps["calls"][1]), ps["recv"].data_ptr(), e_cnt, ps["shared_rows"], stream))
         hk, hf, _sg, sgp = ps["had1"]
         ck(lib.mxmoe_quant_act_planned(hidden.data_ptr(), b1["inp"].data_ptr(), b1["scale"].data_ptr(), ps["dst"].data_ptr(), ps["perm"].data_ptr(), b1["plan"].data_ptr(),
                                        cfg.hidden, ps["r_cap"], t, e_cnt, has_shared, cfg.rotate, hk, hf, sgp, stream))
