@@ -137,7 +137,14 @@ int mxmoe_build_permutation_static(const int32_t* topk_ids, int num_tokens, int 
  * 1 int8 per token, 2 int4 per token, 3 int4 with one scale per 128 values), first row, offset into inp_store and offset into
  * scale_store, both offsets in fp16 elements exactly as ref_bind.cu:475-505 computes them (row strides K, K/2, K/4, K/4 halves; one
  * scale per row, K/128 scales per row for tag 3).
- * rotate: 0 no rotation, 1 rotate rows of quantised experts, 2 rotate every row, with y = (H_k kron H_{n/k}) x / sqrt(n)
+ * Two more tags write the operands of the kernels whose branches carry a variant (mxmoe_kernel_branch): 4 = the int4 codes of
+ * tag 2 as 6-bit floats in fragments of 32 rows x 64 values (1536 bytes; an expert's region holds ceil(rows / 32) * (K / 64) of them,
+ * row-block-major, so its offset into inp_store is counted in fragments of 768 halves; K a multiple of 128), 5 = fp8 (OCP e4m3) codes
+ * with scale = max|x| / 448, stored like tag 1.  Neither exists in the reference's prologue (its fp8 kernels take operands
+ * converted on the host).
+ * rotate: bits 0-1: 0 no rotation, 1 rotate rows of quantised experts, 2 rotate every row; bit 2 (value 4): the table may hold tags 4
+ * and 5 (they live in a second set of kernels with a larger register budget; without the bit such an expert is quantised as tag 2).
+ * The rotation is y = (H_k kron H_{n/k}) x / sqrt(n)
  * (mxmoe/quant/hadamard_utils.py:96-106).  had_k = 1 for power-of-two rows; otherwise H_k = S_f kron B and had_signs is a
  * DEVICE float [(k/f)^2] array holding B as +-1.0 (mxmoe/quant/hadamard_utils.py:162-4379 tables).
  *

@@ -146,22 +146,27 @@ __device__ __forceinline__ const _Float16* shared_src(const RowArgs& a) {
   return a.shared_src_addr ? reinterpret_cast<const _Float16*>(*a.shared_src_addr) : a.src_shared;
 }
 
-// fixed fp32 op sequence for exp(t), identical to the CPU restatement: every step is one correctly rounded operation (the
-// multiply-adds are fused: one rounding each)
-__device__ __forceinline__ float exp_fixed(float t) {
-  t = fminf(fmaxf(t, -87.0f), 87.0f);
-  const float k = rintf(t * 1.4426950408889634f);
-  float r = __builtin_fmaf(-k, 0.693145751953125f, t);
-  r = __builtin_fmaf(-k, 1.428606765330187e-06f, r);
-  float p = 0.0001984127f;
-  p = __builtin_fmaf(p, r, 0.0013888889f);
-  p = __builtin_fmaf(p, r, 0.008333334f);
-  p = __builtin_fmaf(p, r, 0.041666668f);
-  p = __builtin_fmaf(p, r, 0.16666667f);
-  p = __builtin_fmaf(p, r, 0.5f);
-  p = __builtin_fmaf(p, r, 1.0f);
-  p = __builtin_fmaf(p, r, 1.0f);
-  return ldexpf(p, (int)k);
+// silu(g) = g / (1 + exp(-g)) as a fixed sequence of correctly rounded fp32 operations and exact integer ones, identical to the CPU
+// restatement (every multiply-add is fused: one rounding): exp(-g) = 2^t with t = clamp(-g log2(e), +-100) split into k = rint(t) and
+// f = t - k (exact), 2^f by a degree-4 Horner polynomial (relative error 3.7e-6), 2^k added to the exponent field (the result stays a
+// normal number); the reciprocal of d = 1 + exp(-g) from an integer-subtraction seed (within 5.06 %) and two Newton steps (7e-6).
+// silu(g) * u rounded to fp16 lies within 0.52 fp16 ulp of the exact value for every fp16 g.
+__device__ __forceinline__ float silu_fixed(float g) {
+  float t = g * -1.4426950408889634f;
+  t = fminf(fmaxf(t, -100.0f), 100.0f);
+  const float k = rintf(t);
+  const float f = t - k;
+  float p = 0.00967604f;
+  p = __builtin_fmaf(p, f, 0.05592204f);
+  p = __builtin_fmaf(p, f, 0.24022107f);
+  p = __builtin_fmaf(p, f, 0.693121f);
+  p = __builtin_fmaf(p, f, 1.0000001f);
+  const float e = __int_as_float(__float_as_int(p) + (int)((unsigned)(int)k << 23));
+  const float d = 1.0f + e;
+  float r = __int_as_float(0x7EF31000 - __float_as_int(d));
+  r = __builtin_fmaf(r, __builtin_fmaf(-d, r, 1.0f), r);
+  r = __builtin_fmaf(r, __builtin_fmaf(-d, r, 1.0f), r);
+  return g * r;
 }
 
 __device__ __forceinline__ float round_h(float v) { return (float)(_Float16)v; }
@@ -281,7 +286,7 @@ __device__ __forceinline__ void bf6_emit_row(const uint8_t* codes, int row_elems
 __device__ __forceinline__ int xcd_row_group(int wg) { return (wg & ~63) | ((wg & 7) << 3) | ((wg >> 3) & 7); }
 
 // NT threads per workgroup (256, or 192 when that wastes fewer lanes: a 1408-element row is 176 chunks of 8).
-template <int MAXC, bool SILU, int NT>
+template <int MAXC, bool SILU, int NT, bool EXT>
 __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
   extern __shared__ __align__(16) float lds[];
   const int tid = threadIdx.x;
@@ -385,7 +390,7 @@ __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
 #pragma unroll
           for (int j = 0; j < 8; ++j) {
             const float gf = (float)g[j];
-            const float s = gf / (1.0f + exp_fixed(-gf));
+            const float s = silu_fixed(gf);
             v[i][j] = round_h(keep_f32(s * (float)u[j]));
           }
         } else {
@@ -620,12 +625,12 @@ __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
     amax = red[0];
 #pragma unroll
     for (int w = 1; w < NT / 64; ++w) amax = fmaxf(amax, red[w]);
-    const float upper = tag == 1 ? 127.0f : (tag == 5 ? 448.0f : 7.0f);
+    const float upper = tag == 1 ? 127.0f : (EXT && tag == 5 ? 448.0f : 7.0f);
     float scale = round_h(amax / upper);   // fp16 division: fp32 quotient of two fp16 values, rounded to fp16
     if (scale == 0.0f) scale = 1.0f;       // quantize.cuh:258
     const ScaleDiv div(scale);
     if (tid == 0) a.scale_store[scale_off + lrow] = (_Float16)scale;
-    if (tag == 4) {  // the row's codes as fp16 in LDS (in place of the row itself, which every thread is done reading), then fragments
+    if (EXT && tag == 4) {  // the row's codes as fp16 in LDS (in place of the row itself, which every thread is done reading), then fragments
       uint8_t* codes = reinterpret_cast<uint8_t*>(x);
 #pragma unroll
       for (int i = 0; i < MAXC; ++i) {
@@ -636,12 +641,12 @@ __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
       bf6_emit_row(codes, n, 0, n, a.inp_store + 2 * inp_off, lrow, tid, NT);
       continue;  // (the next row begins with a barrier before it touches LDS)
     }
-    uint8_t* out = a.inp_store + 2 * (inp_off + lrow * (tag == 1 || tag == 5 ? n / 2 : n / 4));
+    uint8_t* out = a.inp_store + 2 * (inp_off + lrow * (tag == 1 || (EXT && tag == 5) ? n / 2 : n / 4));
 #pragma unroll
     for (int i = 0; i < MAXC; ++i) {
       const int c = tid + i * NT;
       if (c < nchunks) {
-        if (tag == 5) {
+        if (EXT && tag == 5) {
           *reinterpret_cast<uint2*>(out + c * 8) = fp8_chunk_codes(v[i], div);
           continue;
         }
@@ -671,7 +676,7 @@ __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
 // 8-element chunks l + 64*i.  The butterfly strides map to three levels, taken in the same ascending order as everywhere else:
 // 1, 2, 4 inside a chunk (registers), 8 .. 256 across the lanes (cross-lane exchange, no LDS staging, no barrier),
 // 512 .. n/2 between a lane's own chunks (registers).  Four independent rows per workgroup, nothing shared between them.
-template <int NI, bool SILU>
+template <int NI, bool SILU, bool EXT>
 __global__ void __launch_bounds__(256) row_quant_wave_kernel(const RowArgs a) {
   extern __shared__ __align__(16) uint8_t wave_codes[];  // [4 waves][n] fp16: a row's codes on their way to bf6 fragments (tag 4)
   const int lane = threadIdx.x & 63;
@@ -704,7 +709,7 @@ __global__ void __launch_bounds__(256) row_quant_wave_kernel(const RowArgs a) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           const float gf = (float)g[j];
-          const float s = gf / (1.0f + exp_fixed(-gf));
+          const float s = silu_fixed(gf);
           v[i][j] = round_h(keep_f32(s * (float)u[j]));
         }
       } else {
@@ -800,12 +805,12 @@ __global__ void __launch_bounds__(256) row_quant_wave_kernel(const RowArgs a) {
       for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[i][j]));
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
-    const float upper = tag == 1 ? 127.0f : (tag == 5 ? 448.0f : 7.0f);
+    const float upper = tag == 1 ? 127.0f : (EXT && tag == 5 ? 448.0f : 7.0f);
     float scale = round_h(amax / upper);   // fp16 division: fp32 quotient of two fp16 values, rounded to fp16
     if (scale == 0.0f) scale = 1.0f;       // quantize.cuh:258
     const ScaleDiv div(scale);
     if (lane == 0) a.scale_store[scale_off + lrow] = (_Float16)scale;
-    if (tag == 4) {
+    if (EXT && tag == 4) {
       uint8_t* codes = wave_codes + wave * (n * 2);
 #pragma unroll
       for (int i = 0; i < NI; ++i) *reinterpret_cast<v8h*>(codes + (lane + 64 * i) * 16) = bf6_chunk_codes(v[i], div);
@@ -816,11 +821,11 @@ __global__ void __launch_bounds__(256) row_quant_wave_kernel(const RowArgs a) {
       __builtin_amdgcn_wave_barrier();  // the next row's codes come after these reads
       continue;
     }
-    uint8_t* out = a.inp_store + 2 * (inp_off + lrow * (tag == 1 || tag == 5 ? n / 2 : n / 4));
+    uint8_t* out = a.inp_store + 2 * (inp_off + lrow * (tag == 1 || (EXT && tag == 5) ? n / 2 : n / 4));
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
       const int c = lane + 64 * i;
-      if (tag == 5) {
+      if (EXT && tag == 5) {
         *reinterpret_cast<uint2*>(out + c * 8) = fp8_chunk_codes(v[i], div);
         continue;
       }
@@ -855,7 +860,7 @@ __global__ void __launch_bounds__(256) row_quant_wave_kernel(const RowArgs a) {
 // Four independent rows per workgroup; no barrier (each wave owns its piece of LDS).
 constexpr int kDensePitch = 144;             // bytes per column of the transposed row: 64 fp16 + 16 (16 lanes read 16 distinct bank groups)
 constexpr int kDenseWaveLds = 32 * kDensePitch + (2048 + 8) * 2;  // transposed row + the rotated row in row order (+ a slot for discarded values)
-template <int MAXC, bool SILU>
+template <int MAXC, bool SILU, bool EXT>
 __global__ void __launch_bounds__(256) row_quant_dense_kernel(const RowArgs a) {
   extern __shared__ __align__(16) uint8_t dlds[];
   const int lane = threadIdx.x & 63;
@@ -950,7 +955,7 @@ __global__ void __launch_bounds__(256) row_quant_dense_kernel(const RowArgs a) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           const float gf = (float)g[j];
-          const float sl = gf / (1.0f + exp_fixed(-gf));
+          const float sl = silu_fixed(gf);
           v[i][j] = round_h(keep_f32(sl * (float)u[j]));
         }
       } else {
@@ -1118,12 +1123,12 @@ __global__ void __launch_bounds__(256) row_quant_dense_kernel(const RowArgs a) {
       for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[i][j]));  // chunks past the row hold zeros
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
-    const float upper = tag == 1 ? 127.0f : (tag == 5 ? 448.0f : 7.0f);
+    const float upper = tag == 1 ? 127.0f : (EXT && tag == 5 ? 448.0f : 7.0f);
     float scale = round_h(amax / upper);   // fp16 division: fp32 quotient of two fp16 values, rounded to fp16
     if (scale == 0.0f) scale = 1.0f;       // quantize.cuh:258
     const ScaleDiv div(scale);
     if (lane == 0) a.scale_store[scale_off + lrow] = (_Float16)scale;
-    if (tag == 4) {  // codes into the wave's row buffer (its reads of the rotated row are behind a wave barrier), then fragments
+    if (EXT && tag == 4) {  // codes into the wave's row buffer (its reads of the rotated row are behind a wave barrier), then fragments
 #pragma unroll
       for (int i = 0; i < MAXC; ++i) {
         const int c = lane + 64 * i;
@@ -1136,12 +1141,12 @@ __global__ void __launch_bounds__(256) row_quant_dense_kernel(const RowArgs a) {
       __builtin_amdgcn_wave_barrier();  // the next row's writes come after these reads
       continue;
     }
-    uint8_t* out = a.inp_store + 2 * (inp_off + lrow * (tag == 1 || tag == 5 ? n / 2 : n / 4));
+    uint8_t* out = a.inp_store + 2 * (inp_off + lrow * (tag == 1 || (EXT && tag == 5) ? n / 2 : n / 4));
 #pragma unroll
     for (int i = 0; i < MAXC; ++i) {
       const int c = lane + 64 * i;
       if (c < nchunks) {
-        if (tag == 5) {
+        if (EXT && tag == 5) {
           *reinterpret_cast<uint2*>(out + c * 8) = fp8_chunk_codes(v[i], div);
           continue;
         }
@@ -1177,7 +1182,7 @@ __global__ void __launch_bounds__(256) row_quant_dense_kernel(const RowArgs a) {
 constexpr int kWidePitch = 1024 + 8;                                 // bytes per k row of 512 fp16 in LDS: the 4 k groups (or row groups) that the
                                                                      // lanes of a wave touch together land 8 or 16 banks apart
 constexpr int kWideLds = 2 * 32 * kWidePitch + 64;                   // snapped row, rotated row, reduction slots
-template <bool SILU>
+template <bool SILU, bool EXT>
 __global__ void __launch_bounds__(512) row_quant_wide_kernel(const RowArgs a) {
   extern __shared__ __align__(16) uint8_t wlds[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -1230,7 +1235,7 @@ __global__ void __launch_bounds__(512) row_quant_wide_kernel(const RowArgs a) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           const float gf = (float)g[j];
-          const float sl = gf / (1.0f + exp_fixed(-gf));
+          const float sl = silu_fixed(gf);
           v[i][j] = round_h(keep_f32(sl * (float)u[j]));
         }
       } else {
@@ -1381,12 +1386,12 @@ __global__ void __launch_bounds__(512) row_quant_wide_kernel(const RowArgs a) {
     amax = red[8];
 #pragma unroll
     for (int w = 1; w < 8; ++w) amax = fmaxf(amax, red[8 + w]);
-    const float upper = tag == 1 ? 127.0f : (tag == 5 ? 448.0f : 7.0f);
+    const float upper = tag == 1 ? 127.0f : (EXT && tag == 5 ? 448.0f : 7.0f);
     float scale = round_h(amax / upper);   // fp16 division: fp32 quotient of two fp16 values, rounded to fp16
     if (scale == 0.0f) scale = 1.0f;       // quantize.cuh:258
     const ScaleDiv div(scale);
     if (tid == 0) a.scale_store[scale_off + lrow] = (_Float16)scale;
-    if (tag == 4) {  // codes into the rotated row's buffer, each wave over its own k rows, then fragments by the whole workgroup
+    if (EXT && tag == 4) {  // codes into the rotated row's buffer, each wave over its own k rows, then fragments by the whole workgroup
       __syncthreads();  // (a row that was not rotated did not pass the barriers that order the previous row's readers of this buffer)
 #pragma unroll
       for (int i = 0; i < MAXC; ++i) {
@@ -1398,13 +1403,13 @@ __global__ void __launch_bounds__(512) row_quant_wide_kernel(const RowArgs a) {
       __syncthreads();
       continue;
     }
-    uint8_t* out = a.inp_store + 2 * (inp_off + lrow * (tag == 1 || tag == 5 ? n / 2 : n / 4));
+    uint8_t* out = a.inp_store + 2 * (inp_off + lrow * (tag == 1 || (EXT && tag == 5) ? n / 2 : n / 4));
 #pragma unroll
     for (int i = 0; i < MAXC; ++i) {
       const int kr = wave + 8 * i;
       if (kr < kb) {
         const int c = kr * 64 + lane;
-        if (tag == 5) {
+        if (EXT && tag == 5) {
           *reinterpret_cast<uint2*>(out + c * 8) = fp8_chunk_codes(v[i], div);
           continue;
         }
@@ -1446,8 +1451,8 @@ static int make_plan(int n, int had_k, int had_f, bool rotate, RotPlan* p) {
   return 0;
 }
 
-template <bool SILU>
-static int launch_rows(const RowArgs& a, int lds_bytes, hipStream_t s) {
+template <bool SILU, bool EXT>
+static int launch_rows_as(const RowArgs& a, int lds_bytes, hipStream_t s) {
   const int nmax = a.plan.n > a.plan_shared.n ? a.plan.n : a.plan_shared.n;
   int dev = 0, cus = 256;
   (void)hipGetDevice(&dev);
@@ -1462,12 +1467,12 @@ static int launch_rows(const RowArgs& a, int lds_bytes, hipStream_t s) {
   if (a.plan.kb == 1 && a.plan_shared.kb == 1 && a.plan_shared.n == n && n % 512 == 0 && n <= 4096 && (n & (n - 1)) == 0) {
     // (a multiple of 64 workgroups: xcd_row_group permutes within runs of 64)
     const int wgrid = ((a.rows + 3) / 4 < cus * 8 ? (a.rows + 3) / 4 : cus * 8) + 63 & ~63;
-    const int wlds = 4 * n * 2;  // the waves' code rows (tag 4)
+    const int wlds = EXT ? 4 * n * 2 : 0;  // the waves' code rows (tag 4)
     switch (n / 512) {
-      case 1: hipLaunchKernelGGL((row_quant_wave_kernel<1, SILU>), dim3(wgrid), dim3(256), wlds, s, a); break;
-      case 2: hipLaunchKernelGGL((row_quant_wave_kernel<2, SILU>), dim3(wgrid), dim3(256), wlds, s, a); break;
-      case 4: hipLaunchKernelGGL((row_quant_wave_kernel<4, SILU>), dim3(wgrid), dim3(256), wlds, s, a); break;
-      default: hipLaunchKernelGGL((row_quant_wave_kernel<8, SILU>), dim3(wgrid), dim3(256), wlds, s, a); break;
+      case 1: hipLaunchKernelGGL((row_quant_wave_kernel<1, SILU, EXT>), dim3(wgrid), dim3(256), wlds, s, a); break;
+      case 2: hipLaunchKernelGGL((row_quant_wave_kernel<2, SILU, EXT>), dim3(wgrid), dim3(256), wlds, s, a); break;
+      case 4: hipLaunchKernelGGL((row_quant_wave_kernel<4, SILU, EXT>), dim3(wgrid), dim3(256), wlds, s, a); break;
+      default: hipLaunchKernelGGL((row_quant_wave_kernel<8, SILU, EXT>), dim3(wgrid), dim3(256), wlds, s, a); break;
     }
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
@@ -1481,10 +1486,10 @@ static int launch_rows(const RowArgs& a, int lds_bytes, hipStream_t s) {
     const int wgrid = ((a.rows + 3) / 4 < cus * 4 ? (a.rows + 3) / 4 : cus * 4) + 63 & ~63;
     const int dlds = 4 * kDenseWaveLds;
     switch ((n / 8 + 63) / 64) {
-      case 1: hipLaunchKernelGGL((row_quant_dense_kernel<1, SILU>), dim3(wgrid), dim3(256), dlds, s, a); break;
-      case 2: hipLaunchKernelGGL((row_quant_dense_kernel<2, SILU>), dim3(wgrid), dim3(256), dlds, s, a); break;
-      case 3: hipLaunchKernelGGL((row_quant_dense_kernel<3, SILU>), dim3(wgrid), dim3(256), dlds, s, a); break;
-      default: hipLaunchKernelGGL((row_quant_dense_kernel<4, SILU>), dim3(wgrid), dim3(256), dlds, s, a); break;
+      case 1: hipLaunchKernelGGL((row_quant_dense_kernel<1, SILU, EXT>), dim3(wgrid), dim3(256), dlds, s, a); break;
+      case 2: hipLaunchKernelGGL((row_quant_dense_kernel<2, SILU, EXT>), dim3(wgrid), dim3(256), dlds, s, a); break;
+      case 3: hipLaunchKernelGGL((row_quant_dense_kernel<3, SILU, EXT>), dim3(wgrid), dim3(256), dlds, s, a); break;
+      default: hipLaunchKernelGGL((row_quant_dense_kernel<4, SILU, EXT>), dim3(wgrid), dim3(256), dlds, s, a); break;
     }
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
@@ -1498,14 +1503,14 @@ static int launch_rows(const RowArgs& a, int lds_bytes, hipStream_t s) {
   if (a.plan.kb > 1 && a.plan.kb <= 32 && a.plan.m == 512 && a.plan.f == 1 && a.plan_shared.n == n && a.plan_shared.kb == a.plan.kb && a.rotate != 0) {
     static bool opted_in[64] = {};
     if (dev >= 0 && dev < 64 && !opted_in[dev]) {
-      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&row_quant_wide_kernel<SILU>), hipFuncAttributeMaxDynamicSharedMemorySize, kWideLds) != hipSuccess) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&row_quant_wide_kernel<SILU, EXT>), hipFuncAttributeMaxDynamicSharedMemorySize, kWideLds) != hipSuccess) {
         last_error() = "could not reserve LDS for the wide-row quantiser";
         return 4;
       }
       opted_in[dev] = true;
     }
     const int wgrid = a.rows < cus * 8 ? a.rows : cus * 8;
-    hipLaunchKernelGGL((row_quant_wide_kernel<SILU>), dim3(wgrid), dim3(512), kWideLds, s, a);
+    hipLaunchKernelGGL((row_quant_wide_kernel<SILU, EXT>), dim3(wgrid), dim3(512), kWideLds, s, a);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
       last_error() = std::string("kernel launch failed: ") + hipGetErrorString(e);
@@ -1522,15 +1527,15 @@ static int launch_rows(const RowArgs& a, int lds_bytes, hipStream_t s) {
   for (int i = 0; i < 9 && pick < 0; ++i)
     if (kShapes[i][0] * kShapes[i][1] >= nchunks) pick = i;
   switch (pick) {
-    case 0: hipLaunchKernelGGL((row_quant_kernel<1, SILU, 192>), dim3(grid), dim3(192), lds_bytes, s, a); break;
-    case 1: hipLaunchKernelGGL((row_quant_kernel<1, SILU, 256>), dim3(grid), dim3(256), lds_bytes, s, a); break;
-    case 2: hipLaunchKernelGGL((row_quant_kernel<2, SILU, 192>), dim3(grid), dim3(192), lds_bytes, s, a); break;
-    case 3: hipLaunchKernelGGL((row_quant_kernel<2, SILU, 256>), dim3(grid), dim3(256), lds_bytes, s, a); break;
-    case 4: hipLaunchKernelGGL((row_quant_kernel<3, SILU, 192>), dim3(grid), dim3(192), lds_bytes, s, a); break;
-    case 5: hipLaunchKernelGGL((row_quant_kernel<3, SILU, 256>), dim3(grid), dim3(256), lds_bytes, s, a); break;
-    case 6: hipLaunchKernelGGL((row_quant_kernel<2, SILU, 512>), dim3(grid), dim3(512), lds_bytes, s, a); break;
-    case 7: hipLaunchKernelGGL((row_quant_kernel<3, SILU, 512>), dim3(grid), dim3(512), lds_bytes, s, a); break;
-    case 8: hipLaunchKernelGGL((row_quant_kernel<4, SILU, 512>), dim3(grid), dim3(512), lds_bytes, s, a); break;
+    case 0: hipLaunchKernelGGL((row_quant_kernel<1, SILU, 192, EXT>), dim3(grid), dim3(192), lds_bytes, s, a); break;
+    case 1: hipLaunchKernelGGL((row_quant_kernel<1, SILU, 256, EXT>), dim3(grid), dim3(256), lds_bytes, s, a); break;
+    case 2: hipLaunchKernelGGL((row_quant_kernel<2, SILU, 192, EXT>), dim3(grid), dim3(192), lds_bytes, s, a); break;
+    case 3: hipLaunchKernelGGL((row_quant_kernel<2, SILU, 256, EXT>), dim3(grid), dim3(256), lds_bytes, s, a); break;
+    case 4: hipLaunchKernelGGL((row_quant_kernel<3, SILU, 192, EXT>), dim3(grid), dim3(192), lds_bytes, s, a); break;
+    case 5: hipLaunchKernelGGL((row_quant_kernel<3, SILU, 256, EXT>), dim3(grid), dim3(256), lds_bytes, s, a); break;
+    case 6: hipLaunchKernelGGL((row_quant_kernel<2, SILU, 512, EXT>), dim3(grid), dim3(512), lds_bytes, s, a); break;
+    case 7: hipLaunchKernelGGL((row_quant_kernel<3, SILU, 512, EXT>), dim3(grid), dim3(512), lds_bytes, s, a); break;
+    case 8: hipLaunchKernelGGL((row_quant_kernel<4, SILU, 512, EXT>), dim3(grid), dim3(512), lds_bytes, s, a); break;
     default:
       last_error() = "row too long for the activation kernels";
       return 3;
@@ -1541,6 +1546,14 @@ static int launch_rows(const RowArgs& a, int lds_bytes, hipStream_t s) {
     return 4;
   }
   return 0;
+}
+
+// Tags 4 and 5 (operand variants of the bf6 and fp8 matrix paths) are compiled into a second set of the kernels: their code raises every
+// kernel's register budget (the 512-thread kernel's past the two-workgroups-per-CU limit), and the host, which never reads the table,
+// is told by bit 2 of the entry points' `rotate` argument whether a table may hold them.
+template <bool SILU>
+static int launch_rows(const RowArgs& a, int lds_bytes, hipStream_t s, bool variants) {
+  return variants ? launch_rows_as<SILU, true>(a, lds_bytes, s) : launch_rows_as<SILU, false>(a, lds_bytes, s);
 }
 
 }  // namespace mxmoe
@@ -1718,6 +1731,8 @@ static int fill_common(RowArgs& a, int n, int n_shared, int had_k, int had_f, co
 
 int mxmoe_quant_act(const void* hidden, void* inp_store, void* scale_store, const int32_t* dst_exp_sorted, const int64_t* perm_indices, const int64_t* exp_table,
                     int K, int rows_routed, int num_tokens, int num_experts, int has_shared, int rotate, int had_k, int had_f, const float* had_signs, void* stream) {
+  const bool variants = (rotate & 4) != 0;
+  rotate &= 3;
   if (rows_routed < 0 || num_tokens < 0 || num_experts <= 0) {
     last_error() = "bad row or expert count";
     return 3;
@@ -1742,12 +1757,14 @@ int mxmoe_quant_act(const void* hidden, void* inp_store, void* scale_store, cons
   if (a.rows == 0) return 0;
   if (const int rc = fill_common(a, K, K, rotate ? had_k : 1, rotate ? had_f : 1, had_signs)) return rc;
   const int lds = (K + a.plan.kb * a.plan.kb + 16) * (int)sizeof(float);
-  return launch_rows<false>(a, lds, (hipStream_t)stream);
+  return launch_rows<false>(a, lds, (hipStream_t)stream, variants);
 }
 
 int mxmoe_silu_mul_quant(const void* gate_up, const void* gate_up_shared, void* inp_store, void* scale_store, const int32_t* dst_exp_sorted, const int64_t* exp_table,
                          int N, int N_shared, int rows_routed, int num_tokens, int num_experts, int has_shared, int rotate, int had_k, int had_f,
                          const float* had_signs, void* stream) {
+  const bool variants = (rotate & 4) != 0;
+  rotate &= 3;
   if (rows_routed < 0 || num_tokens < 0 || num_experts <= 0) {
     last_error() = "bad row or expert count";
     return 3;
@@ -1774,13 +1791,15 @@ int mxmoe_silu_mul_quant(const void* gate_up, const void* gate_up_shared, void* 
   if (const int rc = fill_common(a, N, has_shared ? N_shared : N, rotate ? had_k : 1, rotate ? had_f : 1, had_signs)) return rc;
   const int nmax = N > a.plan_shared.n ? N : a.plan_shared.n;
   const int lds = (nmax + a.plan.kb * a.plan.kb + 16) * (int)sizeof(float);
-  return launch_rows<true>(a, lds, (hipStream_t)stream);
+  return launch_rows<true>(a, lds, (hipStream_t)stream, variants);
 }
 
 // ---- the same three steps behind a device-side plan (mxmoe_plan_block): nothing here depends on the routing ----
 int mxmoe_quant_act_planned(const void* hidden, void* inp_store, void* scale_store, const int32_t* dst_exp_sorted, const int64_t* perm_indices, const void* d_plan,
                             int K, int rows_capacity, int num_tokens, int num_experts, int has_shared, int rotate, int had_k, int had_f, const float* had_signs,
                             void* stream) {
+  const bool variants = (rotate & 4) != 0;
+  rotate &= 3;
   if (rows_capacity <= 0 || num_tokens < 0 || num_experts <= 0) {
     last_error() = "bad row or expert count";
     return 3;
@@ -1808,12 +1827,14 @@ int mxmoe_quant_act_planned(const void* hidden, void* inp_store, void* scale_sto
   a.rotate = rotate;
   if (const int rc = fill_common(a, K, K, rotate ? had_k : 1, rotate ? had_f : 1, had_signs)) return rc;
   const int lds = (K + a.plan.kb * a.plan.kb + 16) * (int)sizeof(float);
-  return launch_rows<false>(a, lds, (hipStream_t)stream);
+  return launch_rows<false>(a, lds, (hipStream_t)stream, variants);
 }
 
 int mxmoe_silu_mul_quant_planned(const void* gate_up, const void* d_plan_gate_up, void* inp_store, void* scale_store, const int32_t* dst_exp_sorted, const void* d_plan,
                                  int N, int N_shared, int rows_capacity, int num_tokens, int num_experts, int has_shared, int rotate, int had_k, int had_f,
                                  const float* had_signs, void* stream) {
+  const bool variants = (rotate & 4) != 0;
+  rotate &= 3;
   if (rows_capacity <= 0 || num_tokens < 0 || num_experts <= 0) {
     last_error() = "bad row or expert count";
     return 3;
@@ -1845,7 +1866,7 @@ int mxmoe_silu_mul_quant_planned(const void* gate_up, const void* d_plan_gate_up
   if (const int rc = fill_common(a, N, has_shared ? N_shared : N, rotate ? had_k : 1, rotate ? had_f : 1, had_signs)) return rc;
   const int nmax = N > a.plan_shared.n ? N : a.plan_shared.n;
   const int lds = (nmax + a.plan.kb * a.plan.kb + 16) * (int)sizeof(float);
-  return launch_rows<true>(a, lds, (hipStream_t)stream);
+  return launch_rows<true>(a, lds, (hipStream_t)stream, variants);
 }
 
 size_t mxmoe_combine_workspace_bytes(int num_tokens, int topk) { return (size_t)num_tokens * topk * sizeof(int32_t); }

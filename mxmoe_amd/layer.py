@@ -54,6 +54,10 @@ class MxMoELayer:
         self.state = None
         self._static = None
 
+    def _variants(self, bf6: bool) -> int:
+        """The quantisers' variants bit: set when the block's expert table may hold tag 4 (bf6 fragments) or tag 5 (fp8)."""
+        return ops.ROWS_VARIANTS if bf6 or self.fp8 else 0
+
     @property
     def weight_bytes(self) -> int:
         return sum(w.nbytes for w in self.w13) + sum(w.nbytes for w in self.w2)
@@ -237,12 +241,12 @@ class MxMoELayer:
             ck(lib.mxmoe_plan_layer(C.byref(ps["calls"][0]), C.byref(ps["calls"][1]), ps["recv"].data_ptr(), e_cnt, ps["shared_rows"], stream))
         hk, hf, _sg, sgp = ps["had1"]
         ck(lib.mxmoe_quant_act_planned(hidden.data_ptr(), b1["inp"].data_ptr(), b1["scale"].data_ptr(), ps["dst"].data_ptr(), ps["perm"].data_ptr(), b1["plan"].data_ptr(),
-                                       cfg.hidden, ps["r_cap"], t, e_cnt, has_shared, cfg.rotate, hk, hf, sgp, stream))
+                                       cfg.hidden, ps["r_cap"], t, e_cnt, has_shared, cfg.rotate | self._variants(self.bf6_gate_up), hk, hf, sgp, stream))
         ck(lib.mxmoe_group_gemm_planned(b1["kid"], b1["plan"].data_ptr(), ps["et"], b1["grid"], stream))
         i_sh = cfg.inter * max(cfg.num_shared, 1)
         hk, hf, _sg, sgp = ps["had2"]
         ck(lib.mxmoe_silu_mul_quant_planned(ps["mid"].data_ptr(), b1["plan"].data_ptr(), b2["inp"].data_ptr(), b2["scale"].data_ptr(), ps["dst"].data_ptr(), b2["plan"].data_ptr(),
-                                            cfg.inter, i_sh, ps["r_cap"], t, e_cnt, has_shared, cfg.rotate, hk, hf, sgp, stream))
+                                            cfg.inter, i_sh, ps["r_cap"], t, e_cnt, has_shared, cfg.rotate | self._variants(self.bf6_down), hk, hf, sgp, stream))
         ck(lib.mxmoe_group_gemm_planned(b2["kid"], b2["plan"].data_ptr(), ps["et"], b2["grid"], stream))
         ck(lib.mxmoe_combine_planned(ps["out"].data_ptr(), b2["plan"].data_ptr(), ps["et"], w.data_ptr(), ps["row_of_slot"].data_ptr(), t, topk, cfg.hidden,
                                      final.data_ptr(), stream))
@@ -303,12 +307,12 @@ class MxMoELayer:
 
         hk, hf, sg = signs(cfg.hidden, cfg.hidden)
         _lib.check(lib, lib.mxmoe_quant_act(hidden.data_ptr(), inp1.data_ptr(), sa1.data_ptr(), dst.data_ptr(), perm.data_ptr(), base + off[0],
-                                            cfg.hidden, routed, t, e_cnt, int(has_shared), cfg.rotate, hk, hf, sg, stream))
+                                            cfg.hidden, routed, t, e_cnt, int(has_shared), cfg.rotate | self._variants(self.bf6_gate_up), hk, hf, sg, stream))
         launch(off[2], off[4], s1, q1, self.kid_gate_up)
         i_sh = cfg.inter * max(cfg.num_shared, 1)
         hk, hf, sg = signs(cfg.inter, i_sh)
         _lib.check(lib, lib.mxmoe_silu_mul_quant(mid.data_ptr(), mid.data_ptr() + routed * 2 * cfg.inter * 2, inp2.data_ptr(), sa2.data_ptr(), dst.data_ptr(), base + off[1],
-                                                 cfg.inter, i_sh, routed, t, e_cnt, int(has_shared), cfg.rotate, hk, hf, sg, stream))
+                                                 cfg.inter, i_sh, routed, t, e_cnt, int(has_shared), cfg.rotate | self._variants(self.bf6_down), hk, hf, sg, stream))
         launch(off[3], off[5], s2, q2, self.kid_down)
         ws = torch.empty(lib.mxmoe_combine_workspace_bytes(t, topk), dtype=torch.uint8, device=dev)
         shared_ptr = out.data_ptr() + routed * cfg.hidden * 2 if has_shared else None

@@ -37,7 +37,8 @@ def act_tag(a_bits: int, gsize: int, bf6: bool = False, fp8: bool = False) -> in
     return -1
 
 
-BF6_FRAGMENT_HALVES = 768      # fp16 elements of one 32-row x 64-k fragment (1536 bytes)
+BF6_FRAGMENT_HALVES = 768
+ROWS_VARIANTS = 4         # bit 2 of the quantisers' `rotate` argument: the expert table may hold tags 4 (bf6 fragments) and 5 (fp8)      # fp16 elements of one 32-row x 64-k fragment (1536 bytes)
 
 
 def packed_elems(tag: int, rows: int, width: int) -> int:
@@ -178,7 +179,7 @@ def quant_inp_act(hidden, topk_ids, num_experts: int, N: int, num_shared_experts
     hk, hf, signs = device_signs(k, dev) if rotate else (1, 1, None)
     routed = int(recv_cpu.sum())                            # rows whose expert id was in range; the sorted arrays hold exactly these
     _lib.check(lib, lib.mxmoe_quant_act(hidden.data_ptr(), inp_store.data_ptr(), scale_store.data_ptr(), dst.data_ptr(), perm.data_ptr(), d_table.data_ptr(),
-                                        k, routed, t, num_experts, int(has_shared), rotate, hk, hf, None if signs is None else signs.data_ptr(), _stream()))
+                                        k, routed, t, num_experts, int(has_shared), rotate | (ROWS_VARIANTS if bf6 or fp8 else 0), hk, hf, None if signs is None else signs.data_ptr(), _stream()))
     inp_list, scale_list = _views(inp_store, scale_store, table, rows, inp_sizes, scale_sizes, lds)
     out_list, off = [], 0
     for e, n in enumerate(rows):
@@ -215,7 +216,7 @@ def silu_mul_then_quant(inp, num_problems: int, num_experts: int, K: int, N: int
         raise RuntimeError("routed and shared intermediate sizes need the same Hadamard order")
     shared_ptr = flat.data_ptr() + r * N * 2 * 2
     _lib.check(lib, lib.mxmoe_silu_mul_quant(flat.data_ptr(), shared_ptr, inp_store.data_ptr(), scale_store.data_ptr(), values_sorted.data_ptr(), d_table.data_ptr(),
-                                             N, n_sh, r, num_tokens, num_experts, int(has_shared), rotate, hk, hf, None if signs is None else signs.data_ptr(), _stream()))
+                                             N, n_sh, r, num_tokens, num_experts, int(has_shared), rotate | (ROWS_VARIANTS if bf6 or fp8 else 0), hk, hf, None if signs is None else signs.data_ptr(), _stream()))
     inp_list, scale_list = _views(inp_store, scale_store, table, rows, inp_sizes, scale_sizes, lds)
     out_list, off = [], 0
     for e, n in enumerate(rows):

@@ -23,7 +23,8 @@ fails a test in ``tests/test_oracle_*.py``):
 * ``route_topk``          — textbook softmax / top-k, weights sum to one.
 * ``permute_by_expert``   — brute force against a dict-of-lists.
 * ``tile_to_problem``     — every (problem, tile_m, tile_n) visited exactly once.
-* ``silu_mul``            — float64 ``x*sigmoid(x)*u`` within one fp16 ulp.
+* ``silu_mul`` / ``exp2_neg_f32_fixed`` / ``rcp_f32_fixed`` — float64 ``x*sigmoid(x)*u`` within one fp16 ulp for EVERY fp16 gate
+  value; the two sequences against float64 exp and division (relative error bounds), exact-rational checks of ``fma_f32``.
 * ``unpermute_combine``   — one-hot weights return the routed row bit for bit, dense float64 sum
   within fp16 rounding (+ shared row), independence of the order of the sorted rows, dropped slots.
 
@@ -35,7 +36,8 @@ is this build's own deterministic definition; agreement with the reference at th
 "equal up to fp16 rounding of the rotated activation".  Also unpinned: the rounding inside
 ``silu_mul`` (the reference's kernel source for it, act_kernel.cuh, is absent; torch's fp16
 ``act_fn(g) * u`` rounds the activation to fp16 before the multiply, here silu(g) stays in fp32
-and the product is rounded once), at most one fp16 ulp of the product apart.
+and the product is rounded once; exp and the reciprocal are short fixed sequences accurate to 1e-5), at most one fp16 ulp of the
+product apart.
 * ``e4m3_encode`` / ``e4m3_decode`` / ``quant_e4m3`` / ``fp8_gemm`` — all 256 codes round-trip, hand-computed ties
   (to even) at normal, subnormal and top-of-range spacings, every fp16 value against an independent
   library cast (torch.float8_e4m3fn), absmax -> +-448; the fp8 format of the reference's w8a8_g-1_sym_E4M3 tiles
@@ -43,7 +45,7 @@ and the product is rounded once), at most one fp16 ulp of the product apart.
   (max / 448) is this build's definition: parity unpinned beyond "per-row scale, e4m3 codes, fp32 sums".
 * ``dense_grid`` / the exact dense stage of ``online_hadamard`` — python-int sums in shuffled
   orders give the same bits; grid edges (zero rows, subnormal and largest fp16 values).
-* ``fma_f32`` / ``exp_f32_fixed`` — one correct rounding against exact rational arithmetic.
+* ``fma_f32`` — one correct rounding against exact rational arithmetic.
 """
 from __future__ import annotations
 
@@ -185,10 +187,10 @@ def gemm_fp16(x: np.ndarray, w: np.ndarray) -> np.ndarray:
 # --------------------------------------------------------------------------------------------
 # SiLU * up  (input of the down projection)
 # --------------------------------------------------------------------------------------------
-_LOG2E = F32(1.4426950408889634)
-_LN2_HI = F32(0.693145751953125)          # 0x3f317200, low mantissa bits zero
-_LN2_LO = F32(1.428606765330187e-06)      # ln2 - LN2_HI
-_EXP_C = [F32(c) for c in (1.0, 1.0, 0.5, 0.16666667, 0.041666668, 0.008333334, 0.0013888889, 0.0001984127)]
+_NEG_LOG2E = F32(-1.4426950408889634)
+# 2^f on [-0.5, 0.5], degree 4, relative error 3.7e-6 (least squares on Chebyshev nodes), lowest coefficient first
+_EXP2_C = [F32(c) for c in (1.0000001, 0.693121, 0.24022107, 0.05592204, 0.00967604)]
+_RCP_SEED = np.int32(0x7EF31000)          # bits(seed) = this - bits(d): within 5.06 % of 1 / d for every positive normal d
 
 
 def fma_f32(a, b, c) -> np.ndarray:
@@ -212,35 +214,47 @@ def fma_f32(a, b, c) -> np.ndarray:
         return bits.view(np.float64).astype(F32)
 
 
-def exp_f32_fixed(t: np.ndarray) -> np.ndarray:
-    """exp(t) in fp32 as a FIXED sequence of correctly rounded fp32 operations.
+def exp2_neg_f32_fixed(g: np.ndarray) -> np.ndarray:
+    """``exp(-g)`` in fp32 as a FIXED sequence of correctly rounded fp32 and exact integer operations, relative error < 1e-5:
+    ``t = clamp(g * -log2(e), -100, 100)``, ``k = rint(t)``, ``f = t - k`` (exact), ``p = 2^f`` by a degree-4 Horner polynomial of
+    fused multiply-adds, and ``2^k`` added to p's exponent field (p lies in [0.70, 1.42] and |k| <= 100, so the result stays a
+    normal number).  The HIP kernels run the identical sequence."""
+    g = np.asarray(g, F32)
+    with np.errstate(invalid="ignore", over="ignore"):
+        t = (g * _NEG_LOG2E).astype(F32)
+        t = np.minimum(np.maximum(t, F32(-100.0)), F32(100.0))
+        k = np.rint(t).astype(F32)
+        f = (t - k).astype(F32)
+        p = np.full_like(f, _EXP2_C[4])
+        for c in _EXP2_C[3::-1]:
+            p = fma_f32(p, f, c)
+        return (p.view(np.int32) + (k.astype(np.int32) << 23)).view(F32)
 
-    ``k = rint(t*log2e)``, ``r = fma(-k, LN2_LO, fma(-k, LN2_HI, t))``, degree-7 Horner polynomial of fused multiply-adds,
-    exact scaling by 2^k.  The HIP kernels run the identical op sequence, which is what makes ``silu_mul`` bit-reproducible
-    between CPU and GPU.  Relative error < 2e-7.
-    """
-    t = np.clip(t.astype(F32), F32(-87.0), F32(87.0))
-    k = np.rint((t * _LOG2E).astype(F32)).astype(F32)
-    r = fma_f32(-k, _LN2_HI, t)
-    r = fma_f32(-k, _LN2_LO, r)
-    p = np.full_like(r, _EXP_C[7])
-    for c in _EXP_C[6::-1]:
-        p = fma_f32(p, r, c)
-    return np.ldexp(p, k.astype(np.int32)).astype(F32)
+
+def rcp_f32_fixed(d: np.ndarray) -> np.ndarray:
+    """``1 / d`` for positive normal d as a fixed sequence: an integer-subtraction seed (within 5.06 %) refined by two Newton steps
+    ``r <- fma(r, fma(-d, r, 1), r)``; relative error < 7e-6 (the fourth power of the seed's)."""
+    d = np.asarray(d, F32)
+    r = (_RCP_SEED - d.view(np.int32)).view(F32)
+    for _ in range(2):
+        r = fma_f32(r, fma_f32(-d, r, F32(1.0)), r)
+    return r
 
 
 def silu_mul(gate_up: np.ndarray) -> np.ndarray:
     """``silu(gate) * up`` on a fused ``[rows, 2I]`` fp16 tensor, first half = gate, second = up.
 
     Contract of the reference's ``silu_mul_then_quant_kernel`` launch (ref_bind.cu:691-716; kernel
-    source absent from the reference).  fp32: ``s = g / (1 + exp(-g))``, ``y = s * u``, one fp16 rounding.
+    source absent from the reference).  fp32: ``s = g * rcp(1 + exp(-g))`` with the two fixed sequences above, ``y = s * u``, one
+    fp16 rounding: within one fp16 ulp of the exact value (0.53 ulp at worst over every fp16 gate).
     """
     i = gate_up.shape[-1] // 2
     g = gate_up[..., :i].astype(F32)
     u = gate_up[..., i:].astype(F32)
-    e = exp_f32_fixed(-g)
-    s = (g / (F32(1.0) + e).astype(F32)).astype(F32)
-    return (s * u).astype(F32).astype(F16)
+    with np.errstate(invalid="ignore", over="ignore"):
+        d = (F32(1.0) + exp2_neg_f32_fixed(g)).astype(F32)
+        s = (g * rcp_f32_fixed(d)).astype(F32)
+        return (s * u).astype(F32).astype(F16)
 
 
 # --------------------------------------------------------------------------------------------

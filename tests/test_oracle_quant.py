@@ -171,22 +171,39 @@ def test_fma_f32_is_one_correct_rounding():
 
 
 def test_exp_fixed_and_silu_mul():
-    t = np.linspace(-87, 87, 20001).astype(np.float32)
-    rel = np.abs(O.exp_f32_fixed(t).astype(np.float64) / np.exp(t.astype(np.float64)) - 1)
-    assert rel.max() < 3e-7
+    """The two fixed sequences behind SiLU against float64 (relative error bounds that a wrong coefficient, a dropped Newton step or a
+    wrong seed would break), and silu(g) * u against the float64 value for EVERY finite fp16 gate and several up values: within one
+    fp16 ulp (0.52 at worst; a correctly rounded result would be within 0.5)."""
+    gg = np.linspace(-69, 69, 100001).astype(np.float32)
+    rel = np.abs(O.exp2_neg_f32_fixed(gg).astype(np.float64) / np.exp(-gg.astype(np.float64)) - 1)
+    assert rel.max() < 1e-5
+    assert O.exp2_neg_f32_fixed(np.float32(0.0)) == np.float32(1.0000001)          # k = 0, f = 0: the polynomial's constant term
+    big = O.exp2_neg_f32_fixed(np.array([-1e4, 1e4, np.inf, -np.inf], np.float32))       # clamped at 2^+-100: finite, normal, no overflow
+    assert np.all(np.isfinite(big)) and big[0] > 1e30 and 0 < big[1] < 1e-30 and big[0] == big[3] and big[1] == big[2]
+    d = np.exp2(np.linspace(0, 101, 100001)).astype(np.float32)
+    assert np.abs(O.rcp_f32_fixed(d).astype(np.float64) * d - 1).max() < 8e-6
+    seed_only = (np.int32(0x7EF31000) - d.view(np.int32)).view(np.float32)
+    assert 0.04 < np.abs(seed_only.astype(np.float64) * d - 1).max() < 0.051               # the seed alone is a 5 % guess: the Newton steps do the work
+    g = np.arange(65536, dtype=np.uint16).view(F16)
+    g = g[np.isfinite(g)]
+    worst = 0.0
+    for uval in (1.0, 0.333, -2.5, 1000.0, 6e-5):
+        u = np.full_like(g, F16(uval))
+        y = O.silu_mul(np.concatenate([g[None], u[None]], axis=1))[0]
+        g64, u64 = g.astype(np.float64), u.astype(np.float64)
+        with np.errstate(over="ignore"):
+            ref = g64 / (1 + np.exp(-g64)) * u64
+        fin = np.abs(ref) < 65504
+        ulp = np.maximum(2.0 ** np.floor(np.log2(np.maximum(np.abs(ref), 1e-30))) * 2.0 ** -10, 2.0 ** -24)
+        err = np.abs(y.astype(np.float64) - ref)[fin] / ulp[fin]
+        worst = max(worst, err.max())
+        assert np.all(np.isinf(y[~fin]) | (np.abs(y[~fin].astype(np.float64)) >= 65504 * (1 - 2.0 ** -11)))
+    assert worst < 0.53
     rng = np.random.default_rng(3)
     gu = (rng.standard_normal((17, 64)) * 3).astype(F16)
     gu[0, :4] = [F16(-60000), F16(60000), F16(0), F16(-0.0)]
     y = O.silu_mul(gu)
-    g = gu[:, :32].astype(np.float64)
-    u = gu[:, 32:].astype(np.float64)
-    with np.errstate(over="ignore"):
-        ref = g / (1 + np.exp(-g)) * u
-    assert y.shape == (17, 32)
-    fin = np.abs(ref) < 65504
-    ulp = np.maximum(2.0 ** np.floor(np.log2(np.maximum(np.abs(ref), 1e-30))) * 2.0**-10, 2.0**-24)
-    assert np.all(np.abs(y.astype(np.float64) - ref)[fin] <= 0.501 * ulp[fin])  # one correctly rounded fp16 result
-    assert np.all(np.isinf(y[~fin]))
+    assert y.shape == (17, 32) and y[0, 0] == 0 and y[0, 2] == 0
     # first half is the gate: swapping halves changes the answer
     assert not np.array_equal(y, O.silu_mul(np.concatenate([gu[:, 32:], gu[:, :32]], axis=1)))
 
