@@ -145,6 +145,12 @@ __device__ __forceinline__ bool row_exists(const RowArgs& a, int row) { return !
 __device__ __forceinline__ const _Float16* shared_src(const RowArgs& a) {
   return a.shared_src_addr ? reinterpret_cast<const _Float16*>(*a.shared_src_addr) : a.src_shared;
 }
+// Load of a value that no kernel of this launch writes (routing arrays, expert table), through the constant address space: with a
+// wave-uniform address it is a scalar load into scalar registers, off the vector register budget.
+template <class T>
+__device__ __forceinline__ T const_load(const T* p) {
+  return *(const __attribute__((address_space(4))) T*)(p);
+}
 
 // silu(g) = g / (1 + exp(-g)) as a fixed sequence of correctly rounded fp32 operations and exact integer ones, identical to the CPU
 // restatement (every multiply-add is fused: one rounding): exp(-g) = 2^t with t = clamp(-g log2(e), +-100) split into k = rint(t) and
@@ -170,6 +176,15 @@ __device__ __forceinline__ float silu_fixed(float g) {
 }
 
 __device__ __forceinline__ float round_h(float v) { return (float)(_Float16)v; }
+
+// Integer code of a value already clamped to the code range, as the low bits of a word: the addition of 1.5 * 2^23 rounds to an
+// integer by itself (to nearest, ties to even: rintf) and leaves its two's complement in the low mantissa bits.  push_code<BITS>
+// shifts a word of codes right by BITS and puts the new code on top: after 32 / BITS pushes the first code sits in the lowest bits.
+__device__ __forceinline__ unsigned code_word(float clamped) { return __float_as_uint(clamped + 12582912.0f); }
+template <int BITS>
+__device__ __forceinline__ unsigned push_code(unsigned w, unsigned code) {
+  return __builtin_amdgcn_alignbit(code, w, BITS);
+}
 
 // v / s in fp32 for fp16-valued v and s, given r = 1.0f / s: the rounded product v * r corrected once with its exact remainder.
 // With r the correctly rounded reciprocal this is the correctly rounded quotient, i.e. bit for bit what the division instruction
@@ -199,7 +214,7 @@ struct DenseGrid {
 };
 
 // Value of lane (l ^ M).  Distances 1 .. 8 stay inside a row of 16 lanes and are data-parallel-primitive moves in the vector ALU
-// (quad permutations; l ^ 4 = mirror of 8 lanes, then of 4; l ^ 8 = mirror of 16 lanes, then of 8); 16 and 32 go through the LDS
+// (quad permutations; l ^ 4 = mirror of 8 lanes, then of 4; l ^ 8 = a rotation of the row by 8); 16 and 32 go through the LDS
 // crossbar, whose throughput is what bounds this kernel once the arithmetic is trimmed.
 template <int M>
 __device__ __forceinline__ float lane_xor(float v) {
@@ -212,8 +227,7 @@ __device__ __forceinline__ float lane_xor(float v) {
     x = __builtin_amdgcn_update_dpp(0, x, 0x141, 0xF, 0xF, true);  // row_half_mirror: l ^ 7
     x = __builtin_amdgcn_update_dpp(0, x, 0x1B, 0xF, 0xF, true);   // quad_perm [3,2,1,0]: l ^ 3
   } else if constexpr (M == 8) {
-    x = __builtin_amdgcn_update_dpp(0, x, 0x140, 0xF, 0xF, true);  // row_mirror: l ^ 15
-    x = __builtin_amdgcn_update_dpp(0, x, 0x141, 0xF, 0xF, true);  // row_half_mirror: l ^ 7
+    x = __builtin_amdgcn_update_dpp(0, x, 0x128, 0xF, 0xF, true);  // row_ror:8: lane (l + 8) mod 16 = l ^ 8
   } else {
     return __shfl_xor(v, M);
   }
@@ -601,7 +615,7 @@ __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
 #pragma unroll
           for (int j = 0; j < 8; ++j) {
             const float r = round_h(div(v[i][j]));
-            w |= (unsigned)((int)rintf(fminf(fmaxf(r, -7.0f), 7.0f)) & 0xF) << (4 * j);
+            w = push_code<4>(w, code_word(fminf(fmaxf(r, -7.0f), 7.0f)));
           }
           *reinterpret_cast<unsigned*>(out + c * 4) = w;
         }
@@ -650,21 +664,24 @@ __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
           *reinterpret_cast<uint2*>(out + c * 8) = fp8_chunk_codes(v[i], div);
           continue;
         }
-        int q[8];
+        unsigned q[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           const float r = round_h(div(v[i][j]));
-          q[j] = (int)rintf(fminf(fmaxf(r, -upper), upper));
+          q[j] = code_word(fminf(fmaxf(r, -upper), upper));
         }
         if (tag == 1) {
-          uint2 w;
-          w.x = (q[0] & 0xFF) | ((q[1] & 0xFF) << 8) | ((q[2] & 0xFF) << 16) | ((unsigned)(q[3] & 0xFF) << 24);
-          w.y = (q[4] & 0xFF) | ((q[5] & 0xFF) << 8) | ((q[6] & 0xFF) << 16) | ((unsigned)(q[7] & 0xFF) << 24);
+          uint2 w{0, 0};
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            w.x = push_code<8>(w.x, q[j]);
+            w.y = push_code<8>(w.y, q[j + 4]);
+          }
           *reinterpret_cast<uint2*>(out + c * 8) = w;
         } else {
           unsigned w = 0;
 #pragma unroll
-          for (int j = 0; j < 8; ++j) w |= (unsigned)(q[j] & 0xF) << (4 * j);
+          for (int j = 0; j < 8; ++j) w = push_code<4>(w, q[j]);
           *reinterpret_cast<unsigned*>(out + c * 4) = w;
         }
       }
@@ -792,7 +809,7 @@ __global__ void __launch_bounds__(256) row_quant_wave_kernel(const RowArgs a) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           const float r = round_h(div(v[i][j]));
-          w |= (unsigned)((int)rintf(fminf(fmaxf(r, -7.0f), 7.0f)) & 0xF) << (4 * j);
+          w = push_code<4>(w, code_word(fminf(fmaxf(r, -7.0f), 7.0f)));
         }
         *reinterpret_cast<unsigned*>(out + c * 4) = w;
       }
@@ -829,21 +846,24 @@ __global__ void __launch_bounds__(256) row_quant_wave_kernel(const RowArgs a) {
         *reinterpret_cast<uint2*>(out + c * 8) = fp8_chunk_codes(v[i], div);
         continue;
       }
-      int q[8];
+      unsigned q[8];
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const float r = round_h(div(v[i][j]));
-        q[j] = (int)rintf(fminf(fmaxf(r, -upper), upper));
+        q[j] = code_word(fminf(fmaxf(r, -upper), upper));
       }
       if (tag == 1) {
-        uint2 w;
-        w.x = (q[0] & 0xFF) | ((q[1] & 0xFF) << 8) | ((q[2] & 0xFF) << 16) | ((unsigned)(q[3] & 0xFF) << 24);
-        w.y = (q[4] & 0xFF) | ((q[5] & 0xFF) << 8) | ((q[6] & 0xFF) << 16) | ((unsigned)(q[7] & 0xFF) << 24);
+        uint2 w{0, 0};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          w.x = push_code<8>(w.x, q[j]);
+          w.y = push_code<8>(w.y, q[j + 4]);
+        }
         *reinterpret_cast<uint2*>(out + c * 8) = w;
       } else {
         unsigned w = 0;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) w |= (unsigned)(q[j] & 0xF) << (4 * j);
+        for (int j = 0; j < 8; ++j) w = push_code<4>(w, q[j]);
         *reinterpret_cast<unsigned*>(out + c * 4) = w;
       }
     }
@@ -859,37 +879,39 @@ __global__ void __launch_bounds__(256) row_quant_wave_kernel(const RowArgs a) {
 // the quantise / pack / store code sees the same chunk-per-lane layout as in the other kernels and writes 16 bytes per lane.
 // Four independent rows per workgroup; no barrier (each wave owns its piece of LDS).
 constexpr int kDensePitch = 144;             // bytes per column of the transposed row: 64 fp16 + 16 (16 lanes read 16 distinct bank groups)
-constexpr int kDenseWaveLds = 32 * kDensePitch + (2048 + 8) * 2;  // transposed row + the rotated row in row order (+ a slot for discarded values)
+// LDS of a workgroup: B as matrix operands (one KiB per 16 x 32 block), then per wave the transposed row and the rotated row in row
+// order (+ a slot of 8 values for discarded ones)
+__host__ __device__ constexpr int dense_wave_lds(int n) { return 32 * kDensePitch + (n + 8) * 2; }
+__host__ __device__ constexpr int dense_lds(int n, int kb) { return ((kb + 15) >> 4) * ((kb + 31) >> 5) * 1024 + 4 * dense_wave_lds(n); }
 template <int MAXC, bool SILU, bool EXT>
 __global__ void __launch_bounds__(256) row_quant_dense_kernel(const RowArgs a) {
   extern __shared__ __align__(16) uint8_t dlds[];
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lm = lane & 15, lg = lane >> 4;
-  uint8_t* xt = dlds + wave * kDenseWaveLds;           // [32 columns][kDensePitch]
-  uint8_t* yrow = xt + 32 * kDensePitch;               // [n] fp16, then the discard slot
   const RotPlan pl = a.plan;
   const int n = pl.n, nchunks = n >> 3, kb = pl.kb;
   const int ksteps = (kb + 31) >> 5, mblocks = (kb + 15) >> 4;
-  // B as the first operand of v_mfma_f32_16x16x32_f16: lane holds row 16 mb + (lane & 15), k = 32 ks + 8 (lane >> 4) + 0..7
-  v8h bsign[4][2];
+  uint8_t* xt = dlds + mblocks * ksteps * 1024 + wave * dense_wave_lds(n);  // [32 columns][kDensePitch]
+  uint8_t* yrow = xt + 32 * kDensePitch;                                      // [n] fp16, then the discard slot
+  // B as the first operand of v_mfma_f32_16x16x32_f16: lane holds row 16 mb + (lane & 15), k = 32 ks + 8 (lane >> 4) + 0..7.  Kept in
+  // LDS (block (mb, ks) at (mb * ksteps + ks) KiB, 16 bytes per lane) and read per row: 32 registers fewer per lane.
+  for (int blkid = wave; blkid < mblocks * ksteps; blkid += 4) {
+    const int mb = blkid / ksteps, ks = blkid - mb * ksteps;
+    const int b = 16 * mb + lm;
+    v8h bs;
 #pragma unroll
-  for (int mb = 0; mb < 4; ++mb)
-#pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
-      const int b = 16 * mb + lm;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        // unconditional loads (index clamped into the table, the value dropped afterwards): all of them are in flight together
-        const int bp = 32 * ks + 8 * lg + i;
-        const float sv = a.signs[min(b, kb - 1) * kb + min(bp, kb - 1)];
-        bsign[mb][ks][i] = (b < kb && bp < kb) ? (_Float16)sv : (_Float16)0.0f;
-      }
+    for (int i = 0; i < 8; ++i) {
+      // unconditional loads (index clamped into the table, the value dropped afterwards): all of them are in flight together
+      const int bp = 32 * ks + 8 * lg + i;
+      const float sv = a.signs[min(b, kb - 1) * kb + min(bp, kb - 1)];
+      bs[i] = (b < kb && bp < kb) ? (_Float16)sv : (_Float16)0.0f;
     }
+    *reinterpret_cast<v8h*>(dlds + blkid * 1024 + lane * 16) = bs;
+  }
   // columns and k positions that no row ever writes must read as zero
   for (int i = lane; i < 32 * kDensePitch / 16; i += 64) reinterpret_cast<v4i*>(xt)[i] = v4i{0, 0, 0, 0};
-  asm volatile("" ::: "memory");
-  __builtin_amdgcn_wave_barrier();
+  __syncthreads();
 
   struct RowMeta {
     int tag;
@@ -898,19 +920,20 @@ __global__ void __launch_bounds__(256) row_quant_dense_kernel(const RowArgs a) {
     bool exists;
   };
   const _Float16* const src_shared = shared_src(a);
+  const int routed = a.routed_ptr ? (int)const_load(a.routed_ptr) : a.R;  // rows [routed, R) of a planned launch do not exist
   auto load_meta = [&](int row) {
     RowMeta m;
     const bool shared_row = row >= a.R;
-    m.exists = row_exists(a, row);
-    const int e = shared_row ? a.E : (m.exists ? a.dst_exp[row] : 0);
-    m.tag = (int)a.table[e];
-    m.lrow = shared_row ? row - a.R : row - a.table[a.Et + e];
-    m.inp_off = a.table[2 * a.Et + e];
-    m.scale_off = a.table[3 * a.Et + e];
+    m.exists = row < routed || shared_row;
+    const int e = shared_row ? a.E : (m.exists ? const_load(a.dst_exp + row) : 0);
+    m.tag = (int)const_load(a.table + e);
+    m.lrow = shared_row ? row - a.R : row - const_load(a.table + a.Et + e);
+    m.inp_off = const_load(a.table + 2 * a.Et + e);
+    m.scale_off = const_load(a.table + 3 * a.Et + e);
     if (SILU) {
       m.srow = shared_row ? src_shared + (long)(row - a.R) * 2 * n : a.src + (long)row * 2 * n;
     } else {
-      m.srow = (shared_row ? src_shared : a.src) + (shared_row ? (long)(row - a.R) : (m.exists ? (long)a.perm[row] : 0l)) * n;
+      m.srow = (shared_row ? src_shared : a.src) + (shared_row ? (long)(row - a.R) : (m.exists ? (long)const_load(a.perm + row) : 0l)) * n;
     }
     return m;
   };
@@ -923,35 +946,26 @@ __global__ void __launch_bounds__(256) row_quant_dense_kernel(const RowArgs a) {
     }
   };
   const int stride_rows = gridDim.x * 4;
+  // One row ahead: the bookkeeping of the next row (a chain of dependent loads) is fetched at the top of a row, its data as soon as
+  // this row's data has been turned into values, so the same registers hold both and the loads fly under the rotation and the stores.
   RowMeta next_meta;
-  v8h next_g[MAXC], next_u[MAXC];
+  v8h row_g[MAXC], row_u[MAXC];
   const int row0 = xcd_row_group(blockIdx.x) * 4 + wave;
   if (row0 < a.rows) {
     next_meta = load_meta(row0);
-    load_data(next_meta, next_g, next_u);
+    load_data(next_meta, row_g, row_u);
   }
   for (int row = row0; row < a.rows; row += stride_rows) {
     const RowMeta cur = next_meta;
-    v8h cur_g[MAXC], cur_u[MAXC];
-#pragma unroll
-    for (int i = 0; i < MAXC; ++i) {
-      cur_g[i] = next_g[i];
-      if (SILU) cur_u[i] = next_u[i];
-    }
-    if (row + stride_rows < a.rows) {  // the next row's bookkeeping and data are fetched under this row's arithmetic
-      next_meta = load_meta(row + stride_rows);
-      load_data(next_meta, next_g, next_u);
-    }
-    if (!cur.exists) continue;
-    const int tag = cur.tag;
-    const bool rot = a.rotate == 2 || (a.rotate == 1 && tag != 0);
+    const bool has_next = row + stride_rows < a.rows;
+    if (has_next) next_meta = load_meta(row + stride_rows);
     float v[MAXC][8];
 #pragma unroll
     for (int i = 0; i < MAXC; ++i) {
       const bool live = lane + 64 * i < nchunks;
-      const v8h g = cur_g[i];
+      const v8h g = row_g[i];
       if (SILU) {
-        const v8h u = cur_u[i];
+        const v8h u = row_u[i];
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           const float gf = (float)g[j];
@@ -967,6 +981,11 @@ __global__ void __launch_bounds__(256) row_quant_dense_kernel(const RowArgs a) {
         for (int j = 0; j < 8; ++j) v[i][j] = 0.0f;
       }
     }
+    if (has_next) load_data(next_meta, row_g, row_u);
+    if (!cur.exists) continue;
+    const int tag = cur.tag;
+    const bool rot = a.rotate == 2 || (a.rotate == 1 && tag != 0);
+
     if (rot) {
       // H_8 inside the chunk (strides 1, 2, 4), scale, round to fp16
       float mx = 0.0f;
@@ -1005,58 +1024,78 @@ __global__ void __launch_bounds__(256) row_quant_dense_kernel(const RowArgs a) {
       (void)to16;
       asm volatile("" ::: "memory");
       __builtin_amdgcn_wave_barrier();
-      // lane holds column col = 16 nb + (lane & 15), i.e. blk = 2 nb + ((lane >> 3) & 1), j = lane & 7, and rows
-      // b = 16 mb + 4 (lane >> 4) + r of every 16 x 16 block
-      v4f acc[4][2];
-#pragma unroll
-      for (int mb = 0; mb < 4; ++mb)
-#pragma unroll
-        for (int nb = 0; nb < 2; ++nb) acc[mb][nb] = v4f{0.f, 0.f, 0.f, 0.f};
-      const int ncols = pl.f > 2 ? 2 : 1;
-#pragma unroll
-      for (int ks = 0; ks < 2; ++ks) {
-        if (ks < ksteps) {
-#pragma unroll
-          for (int nb = 0; nb < 2; ++nb) {
-            if (nb < ncols) {
-              const v8h xf = *reinterpret_cast<const v8h*>(xt + (nb * 16 + lm) * kDensePitch + ks * 64 + lg * 16);
-#pragma unroll
-              for (int mb = 0; mb < 4; ++mb)
-                if (mb < mblocks) acc[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(bsign[mb][ks], xf, acc[mb][nb], 0, 0, 0);
-            }
-          }
-        }
-      }
-      // back to the row's scale, S_f butterflies across blk (bit 0 = lane bit 3, bit 1 = the column block; ascending), one rounding to
-      // fp16, and the value goes to its place in the row (values of rows or blocks that do not exist go to the discard slot)
+      // lane holds column col = 16 nb + (lane & 15), i.e. blk = 2 nb + ((lane >> 3) & 1), j = lane & 7, and rows b = 16 mb + 4 (lane >> 4) + r
+      // of every 16 x 16 block.  One block of 16 rows of B at a time (8 accumulator registers live, the second operand re-read
+      // from LDS), each followed by its way back: S_f butterflies across blk (bit 0 = lane bit 3, bit 1 = the column block;
+      // ascending), back to the row's scale (a power of two: exact wherever it is applied) with the one rounding to fp16, and the
+      // value goes to its place in the row (values of rows or blocks that do not exist go to the discard slot).  Compiled once per
+      // order f of the Sylvester factor, so that nothing in it branches on f.
       const float back = grid.from_grid * 16.0f;
-      const float sgn8 = (lane & 8) ? -1.0f : 1.0f;
-      const int blk0 = (lane >> 3) & 1, jj = lane & 7;
+      // (positions from a lane number the compiler must take as changing from row to row: otherwise it keeps every position of
+      // every row block in a register of its own for the whole kernel)
+      int lane_now = lane;
+      asm volatile("" : "+v"(lane_now));
+      auto dense_stage = [&](auto f_const) {
+        constexpr int F = decltype(f_const)::value;
+        constexpr int NCOLS = F > 2 ? 2 : 1;
+        const float sgn8 = (lane_now & 8) ? -1.0f : 1.0f;
+        const int blk0 = (lane_now >> 3) & 1, jj = lane_now & 7;
+        // row 16 mb + 4 (lane >> 4) + r of B exists, and the lane's column block too, when 16 mb + r < lim
+        const int lim = blk0 < F ? kb - 4 * (lane_now >> 4) : 0;
+        uint8_t* const y0 = yrow + 2 * (((blk0 * kb + 4 * (lane_now >> 4)) << 3) + jj);  // place of row block 0, r = 0, in the row
+        uint8_t* const y1 = y0 + 2 * ((2 * kb) << 3);                                      // the same, two column blocks on
+        uint8_t* const ydiscard = yrow + 2 * n;
+        constexpr int kStep = 2 * 8;  // bytes between the places of consecutive rows of B
 #pragma unroll
-      for (int mb = 0; mb < 4; ++mb) {
-        if (mb < mblocks) {
+        for (int mb = 0; mb < 4; ++mb) {
+          if (mb < mblocks) {
+            v4f acc[NCOLS];
 #pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            float t0 = acc[mb][0][r] * back, t1 = acc[mb][1][r] * back;
-            if (pl.f > 1) {
-              t0 = __builtin_fmaf(sgn8, t0, lane_xor<8>(t0));
-              if (pl.f > 2) {
-                t1 = __builtin_fmaf(sgn8, t1, lane_xor<8>(t1));
-                const float p = t0, q = t1;
-                t0 = p + q;
-                t1 = p - q;
+            for (int nb = 0; nb < NCOLS; ++nb) acc[nb] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+              if (ks < ksteps) {
+                const v8h bs = *reinterpret_cast<const v8h*>(dlds + (mb * ksteps + ks) * 1024 + lane * 16);
+#pragma unroll
+                for (int nb = 0; nb < NCOLS; ++nb) {
+                  const v8h xf = *reinterpret_cast<const v8h*>(xt + (nb * 16 + lm) * kDensePitch + ks * 64 + lg * 16);
+                  acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(bs, xf, acc[nb], 0, 0, 0);
+                }
               }
             }
-            const int b = 16 * mb + 4 * lg + r;
-            const bool ok0 = b < kb && blk0 < pl.f;
-            const int i0 = ok0 ? (((blk0 * kb + b) << 3) + jj) : 2048;
-            *reinterpret_cast<_Float16*>(yrow + i0 * 2) = (_Float16)t0;
-            if (pl.f > 2) {
-              const int i1 = b < kb ? ((((blk0 + 2) * kb + b) << 3) + jj) : 2048;
-              *reinterpret_cast<_Float16*>(yrow + i1 * 2) = (_Float16)t1;
+            // a block whose 16 rows all exist, in a column block that exists for every lane, needs no test per value
+            const bool whole = F > 1 && 16 * mb + 16 <= kb;
+            auto emit = [&](auto whole_const) {
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                constexpr bool kWhole = decltype(whole_const)::value;
+                const int off = (16 * mb + r) * kStep;
+                const bool ok = kWhole || 16 * mb + r < lim;
+                float t0 = acc[0][r], t1 = 0.0f;
+                if constexpr (F > 1) t0 = __builtin_fmaf(sgn8, t0, lane_xor<8>(t0));
+                if constexpr (F > 2) {
+                  t1 = acc[NCOLS - 1][r];
+                  t1 = __builtin_fmaf(sgn8, t1, lane_xor<8>(t1));
+                  const float p = t0, q = t1;
+                  t0 = p + q;
+                  t1 = p - q;
+                }
+                *reinterpret_cast<_Float16*>((ok ? y0 : ydiscard - off) + off) = (_Float16)(t0 * back);
+                if constexpr (F > 2) *reinterpret_cast<_Float16*>((ok ? y1 : ydiscard - off) + off) = (_Float16)(t1 * back);
+              }
+            };
+            if (whole) {
+              emit(std::true_type{});
+            } else {
+              emit(std::false_type{});
             }
           }
         }
+      };
+      switch (pl.f) {
+        case 1: dense_stage(std::integral_constant<int, 1>{}); break;
+        case 2: dense_stage(std::integral_constant<int, 2>{}); break;
+        default: dense_stage(std::integral_constant<int, 4>{}); break;
       }
       asm volatile("" ::: "memory");
       __builtin_amdgcn_wave_barrier();
@@ -1109,7 +1148,7 @@ __global__ void __launch_bounds__(256) row_quant_dense_kernel(const RowArgs a) {
 #pragma unroll
           for (int j = 0; j < 8; ++j) {
             const float r = round_h(div(v[i][j]));
-            w |= (unsigned)((int)rintf(fminf(fmaxf(r, -7.0f), 7.0f)) & 0xF) << (4 * j);
+            w = push_code<4>(w, code_word(fminf(fmaxf(r, -7.0f), 7.0f)));
           }
           *reinterpret_cast<unsigned*>(out + c * 4) = w;
         }
@@ -1150,21 +1189,24 @@ __global__ void __launch_bounds__(256) row_quant_dense_kernel(const RowArgs a) {
           *reinterpret_cast<uint2*>(out + c * 8) = fp8_chunk_codes(v[i], div);
           continue;
         }
-        int q[8];
+        unsigned q[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           const float r = round_h(div(v[i][j]));
-          q[j] = (int)rintf(fminf(fmaxf(r, -upper), upper));
+          q[j] = code_word(fminf(fmaxf(r, -upper), upper));
         }
         if (tag == 1) {
-          uint2 w;
-          w.x = (q[0] & 0xFF) | ((q[1] & 0xFF) << 8) | ((q[2] & 0xFF) << 16) | ((unsigned)(q[3] & 0xFF) << 24);
-          w.y = (q[4] & 0xFF) | ((q[5] & 0xFF) << 8) | ((q[6] & 0xFF) << 16) | ((unsigned)(q[7] & 0xFF) << 24);
+          uint2 w{0, 0};
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            w.x = push_code<8>(w.x, q[j]);
+            w.y = push_code<8>(w.y, q[j + 4]);
+          }
           *reinterpret_cast<uint2*>(out + c * 8) = w;
         } else {
           unsigned w = 0;
 #pragma unroll
-          for (int j = 0; j < 8; ++j) w |= (unsigned)(q[j] & 0xF) << (4 * j);
+          for (int j = 0; j < 8; ++j) w = push_code<4>(w, q[j]);
           *reinterpret_cast<unsigned*>(out + c * 4) = w;
         }
       }
@@ -1367,7 +1409,7 @@ __global__ void __launch_bounds__(512) row_quant_wide_kernel(const RowArgs a) {
 #pragma unroll
           for (int j = 0; j < 8; ++j) {
             const float r = round_h(div(v[i][j]));
-            w |= (unsigned)((int)rintf(fminf(fmaxf(r, -7.0f), 7.0f)) & 0xF) << (4 * j);
+            w = push_code<4>(w, code_word(fminf(fmaxf(r, -7.0f), 7.0f)));
           }
           *reinterpret_cast<unsigned*>(out + c * 4) = w;
         }
@@ -1413,21 +1455,24 @@ __global__ void __launch_bounds__(512) row_quant_wide_kernel(const RowArgs a) {
           *reinterpret_cast<uint2*>(out + c * 8) = fp8_chunk_codes(v[i], div);
           continue;
         }
-        int q[8];
+        unsigned q[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           const float r = round_h(div(v[i][j]));
-          q[j] = (int)rintf(fminf(fmaxf(r, -upper), upper));
+          q[j] = code_word(fminf(fmaxf(r, -upper), upper));
         }
         if (tag == 1) {
-          uint2 w;
-          w.x = (q[0] & 0xFF) | ((q[1] & 0xFF) << 8) | ((q[2] & 0xFF) << 16) | ((unsigned)(q[3] & 0xFF) << 24);
-          w.y = (q[4] & 0xFF) | ((q[5] & 0xFF) << 8) | ((q[6] & 0xFF) << 16) | ((unsigned)(q[7] & 0xFF) << 24);
+          uint2 w{0, 0};
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            w.x = push_code<8>(w.x, q[j]);
+            w.y = push_code<8>(w.y, q[j + 4]);
+          }
           *reinterpret_cast<uint2*>(out + c * 8) = w;
         } else {
           unsigned w = 0;
 #pragma unroll
-          for (int j = 0; j < 8; ++j) w |= (unsigned)(q[j] & 0xF) << (4 * j);
+          for (int j = 0; j < 8; ++j) w = push_code<4>(w, q[j]);
           *reinterpret_cast<unsigned*>(out + c * 4) = w;
         }
       }
@@ -1483,13 +1528,25 @@ static int launch_rows_as(const RowArgs& a, int lds_bytes, hipStream_t s) {
   }
   // table-driven factor times H_8, one size of row: one row per wave, dense stage on the matrix cores
   if (a.plan.kb > 1 && a.plan.m == 8 && a.plan.f <= 4 && a.plan.kb <= 64 && n <= 2048 && a.plan_shared.n == n && a.plan_shared.kb == a.plan.kb && a.rotate != 0) {
-    const int wgrid = ((a.rows + 3) / 4 < cus * 4 ? (a.rows + 3) / 4 : cus * 4) + 63 & ~63;
-    const int dlds = 4 * kDenseWaveLds;
+    const int dlds = dense_lds(n, a.plan.kb);
+    // as many workgroups as stay resident together (registers and LDS decide how many share a CU), each looping over its rows
+    auto launch = [&](auto kernel, int which) {
+      static int asked_lds[4][64] = {}, answer[4][64] = {};  // per kernel size and device: the last LDS size asked about
+      int per_cu = 0;
+      if (dev >= 0 && dev < 64 && asked_lds[which][dev] == dlds) {
+        per_cu = answer[which][dev];
+      } else {
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, dlds) != hipSuccess || per_cu < 1) per_cu = 2;
+        if (dev >= 0 && dev < 64) asked_lds[which][dev] = dlds, answer[which][dev] = per_cu;
+      }
+      const int wgrid = ((a.rows + 3) / 4 < cus * per_cu ? (a.rows + 3) / 4 : cus * per_cu) + 63 & ~63;  // (xcd_row_group: runs of 64)
+      hipLaunchKernelGGL(kernel, dim3(wgrid), dim3(256), dlds, s, a);
+    };
     switch ((n / 8 + 63) / 64) {
-      case 1: hipLaunchKernelGGL((row_quant_dense_kernel<1, SILU, EXT>), dim3(wgrid), dim3(256), dlds, s, a); break;
-      case 2: hipLaunchKernelGGL((row_quant_dense_kernel<2, SILU, EXT>), dim3(wgrid), dim3(256), dlds, s, a); break;
-      case 3: hipLaunchKernelGGL((row_quant_dense_kernel<3, SILU, EXT>), dim3(wgrid), dim3(256), dlds, s, a); break;
-      default: hipLaunchKernelGGL((row_quant_dense_kernel<4, SILU, EXT>), dim3(wgrid), dim3(256), dlds, s, a); break;
+      case 1: launch(row_quant_dense_kernel<1, SILU, EXT>, 0); break;
+      case 2: launch(row_quant_dense_kernel<2, SILU, EXT>, 1); break;
+      case 3: launch(row_quant_dense_kernel<3, SILU, EXT>, 2); break;
+      default: launch(row_quant_dense_kernel<4, SILU, EXT>, 3); break;
     }
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
