@@ -166,6 +166,16 @@ int mxmoe_silu_mul_quant(const void* gate_up, const void* gate_up_shared, void* 
  * expert id was dropped contribute nothing.  down_out [rows, K] fp16 are the rows of the down launch in sorted order,
  * shared_out [num_tokens, K] fp16 or NULL, topk_weights [num_tokens, topk] fp32, src_slot [rows] int64 as written by
  * mxmoe_build_permutation, out [num_tokens, K] fp16, all DEVICE pointers.  workspace: mxmoe_combine_workspace_bytes() bytes. */
+/* mxmoe_quant_act for power-of-two rows (K = 512, 1024, 2048 or 4096; error 3 otherwise), one token at a time instead of one
+ * destination row at a time: a token's row is read, rotated and quantised once per format among its destinations and stored to each,
+ * so top-k destinations of one format cost one rotation and one quantisation.  Same bytes in inp_store / scale_store as
+ * mxmoe_quant_act.  row_of_slot[t * topk + k] is the sorted row of slot k of token t, negative when that slot was dropped
+ * (mxmoe_build_permutation_inv, mxmoe_permute_plan_layer); exp_table as above, tags 0 - 3 (a planned block's table sits at
+ * mxmoe_plan_offset(1, problems) of its plan); topk <= 8; rotate 0, 1 or 2.  The reference quantises per destination row
+ * (ref_bind.cu:524-544). */
+int mxmoe_quant_act_tokens(const void* hidden, void* inp_store, void* scale_store, const int32_t* topk_ids, const int32_t* row_of_slot, const int64_t* exp_table,
+                           int K, int num_tokens, int topk, int num_experts, int has_shared, int rotate, void* stream);
+
 size_t mxmoe_combine_workspace_bytes(int num_tokens, int topk);
 int mxmoe_unpermute_combine(const void* down_out, const void* shared_out, const float* topk_weights, const int64_t* src_slot, int rows, int num_tokens, int topk,
                             int K, void* out, void* workspace, void* stream);

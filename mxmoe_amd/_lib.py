@@ -46,6 +46,7 @@ SIGNATURES = {
     "mxmoe_static_scratch_bytes": (C.c_size_t, []),
     "mxmoe_build_permutation_static": (_I, [_P, _I, _I, _I, _P, _P, _P, _P, _P]),
     "mxmoe_quant_act": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P]),
+    "mxmoe_quant_act_tokens": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]),
     "mxmoe_silu_mul_quant": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P]),
     "mxmoe_group_gemm_plan": (_I, [_I, C.POINTER(Dim3), C.POINTER(QParams), _I, C.POINTER(C.c_int32), C.POINTER(C.c_int32)]),
     "mxmoe_kernel_func": (_P, [_I]),

@@ -689,6 +689,56 @@ __global__ void __launch_bounds__(NT) row_quant_kernel(const RowArgs a) {
   }
 }
 
+// H_n x * scale for a row of n = 512 * NI values held by one wave (lane l: the NI chunks l + 64 i of 8 values), every level rounded
+// to fp32 in ascending order of stride and the scaled result rounded to fp16: strides 1, 2, 4 inside a chunk, 8 .. 256 across
+// lanes, 512 and up across the chunks of a lane.
+template <int NI>
+__device__ __forceinline__ void wave_rotate(float (&v)[NI][8], int lane, float scale) {
+#pragma unroll
+  for (int i = 0; i < NI; ++i)
+#pragma unroll
+    for (int h = 1; h < 8; h <<= 1)
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (!(j & h)) {
+          const float p = v[i][j], q = v[i][j + h];
+          v[i][j] = p + q;
+          v[i][j + h] = p - q;
+        }
+  auto lane_stage = [&](auto mc) {
+    constexpr int m = decltype(mc)::value;
+    // upper half of a pair: other - own, lower half: own + other; one fused multiply-add with own's sign, which rounds once
+    // exactly like the sum / difference (the product with +-1 is exact)
+    const float sgn = (lane & m) ? -1.0f : 1.0f;
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[i][j] = __builtin_fmaf(sgn, v[i][j], lane_xor<m>(v[i][j]));
+  };
+  lane_stage(std::integral_constant<int, 1>{});
+  lane_stage(std::integral_constant<int, 2>{});
+  lane_stage(std::integral_constant<int, 4>{});
+  lane_stage(std::integral_constant<int, 8>{});
+  lane_stage(std::integral_constant<int, 16>{});
+  lane_stage(std::integral_constant<int, 32>{});
+#pragma unroll
+  for (int hi = 1; hi < NI; hi <<= 1)
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+      if (!(i & hi)) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float p = v[i][j], q = v[i + hi][j];
+          v[i][j] = p + q;
+          v[i + hi][j] = p - q;
+        }
+      }
+#pragma unroll
+  for (int i = 0; i < NI; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[i][j] = round_h(keep_f32(v[i][j] * scale));
+}
+
 // One row per WAVE, for rows whose rotation is a pure Sylvester transform (n = 512 * NI, NI a power of two): lane l holds the NI
 // 8-element chunks l + 64*i.  The butterfly strides map to three levels, taken in the same ascending order as everywhere else:
 // 1, 2, 4 inside a chunk (registers), 8 .. 256 across the lanes (cross-lane exchange, no LDS staging, no barrier),
@@ -734,51 +784,7 @@ __global__ void __launch_bounds__(256) row_quant_wave_kernel(const RowArgs a) {
         for (int j = 0; j < 8; ++j) v[i][j] = (float)g[j];
       }
     }
-    if (rot) {
-#pragma unroll
-      for (int i = 0; i < NI; ++i)
-#pragma unroll
-        for (int h = 1; h < 8; h <<= 1)
-#pragma unroll
-          for (int j = 0; j < 8; ++j)
-            if (!(j & h)) {
-              const float p = v[i][j], q = v[i][j + h];
-              v[i][j] = p + q;
-              v[i][j + h] = p - q;
-            }
-      auto lane_stage = [&](auto mc) {
-        constexpr int m = decltype(mc)::value;
-        // upper half of a pair: other - own, lower half: own + other; one fused multiply-add with own's sign, which rounds once
-        // exactly like the sum / difference (the product with +-1 is exact)
-        const float sgn = (lane & m) ? -1.0f : 1.0f;
-#pragma unroll
-        for (int i = 0; i < NI; ++i)
-#pragma unroll
-          for (int j = 0; j < 8; ++j) v[i][j] = __builtin_fmaf(sgn, v[i][j], lane_xor<m>(v[i][j]));
-      };
-      lane_stage(std::integral_constant<int, 1>{});
-      lane_stage(std::integral_constant<int, 2>{});
-      lane_stage(std::integral_constant<int, 4>{});
-      lane_stage(std::integral_constant<int, 8>{});
-      lane_stage(std::integral_constant<int, 16>{});
-      lane_stage(std::integral_constant<int, 32>{});
-#pragma unroll
-      for (int hi = 1; hi < NI; hi <<= 1)
-#pragma unroll
-        for (int i = 0; i < NI; ++i)
-          if (!(i & hi)) {
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-              const float p = v[i][j], q = v[i + hi][j];
-              v[i][j] = p + q;
-              v[i + hi][j] = p - q;
-            }
-          }
-#pragma unroll
-      for (int i = 0; i < NI; ++i)
-#pragma unroll
-        for (int j = 0; j < 8; ++j) v[i][j] = round_h(keep_f32(v[i][j] * a.plan.scale));
-    }
+    if (rot) wave_rotate<NI>(v, lane, a.plan.scale);
     if (tag == 0) {
       _Float16* out = reinterpret_cast<_Float16*>(a.inp_store) + inp_off + lrow * n;
 #pragma unroll
@@ -865,6 +871,172 @@ __global__ void __launch_bounds__(256) row_quant_wave_kernel(const RowArgs a) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) w = push_code<4>(w, q[j]);
         *reinterpret_cast<unsigned*>(out + c * 4) = w;
+      }
+    }
+  }
+}
+
+// One TOKEN per wave, for the prologue of power-of-two rows (n = 512 * NI): a token's row is read, rotated and quantised once per
+// format among its destinations and stored to each of them, instead of once per destination row as in row_quant_wave_kernel
+// (top-k destinations of one format cost one rotation and one quantisation, not k).  Destinations: slot k of the token is sorted
+// row row_of_slot[t * topk + k] (negative: the slot's expert id was out of range) of expert ids[t * topk + k], plus, with a shared
+// expert, row t of expert E.  Same arithmetic per destination as the row kernels: the stored bytes are identical.  Tags 0 - 3.
+struct TokenArgs {
+  const _Float16* src;  // [T][n]
+  uint8_t* inp_store;
+  _Float16* scale_store;
+  const int32_t* ids;
+  const int32_t* row_of_slot;
+  const int64_t* table;  // [4][Et]: tag, start_row, inp_off, scale_off (offsets in fp16 elements)
+  int T, E, Et, topk, has_shared;
+  int rotate;  // 0 never, 1 rows of quantised experts, 2 every row
+  float scale;
+};
+constexpr int kTokenMaxTopk = 8;
+
+template <int NI>
+__global__ void __launch_bounds__(256) token_quant_wave_kernel(const TokenArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  constexpr int n = 512 * NI;
+  constexpr int KD = kTokenMaxTopk + 1;  // destinations at most: the slots, then the shared expert
+  const int ndst = a.topk + (a.has_shared ? 1 : 0);
+  const int stride = gridDim.x * 4;
+  for (int t = xcd_row_group(blockIdx.x) * 4 + wave; t < a.T; t += stride) {
+    // the destinations (wave-uniform: scalar loads, scalar registers)
+    int e_of[KD], tag_of[KD];
+    long lrow_of[KD];
+    unsigned present = 0;  // bit per tag among the destinations
+#pragma unroll
+    for (int k = 0; k < KD; ++k) {
+      e_of[k] = 0, tag_of[k] = -1, lrow_of[k] = 0;
+      if (k < ndst) {
+        const bool shared = k == a.topk;
+        const int r = shared ? t : const_load(a.row_of_slot + t * a.topk + k);
+        if (r >= 0) {
+          const int e = shared ? a.E : const_load(a.ids + t * a.topk + k);
+          e_of[k] = e;
+          tag_of[k] = (int)const_load(a.table + e);
+          lrow_of[k] = shared ? (long)t : (long)r - const_load(a.table + a.Et + e);
+          present |= 1u << tag_of[k];
+        }
+      }
+    }
+    if (present == 0) continue;
+    const _Float16* srow = a.src + (long)t * n;
+    float v[NI][8];
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const v8h g = *reinterpret_cast<const v8h*>(srow + (lane + 64 * i) * 8);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[i][j] = (float)g[j];
+    }
+    // fp16 copies (tag 0): of the row as it is unless every row is rotated
+    auto store_copies = [&]() {
+#pragma unroll
+      for (int k = 0; k < KD; ++k) {
+        if (k < ndst && tag_of[k] == 0) {
+          _Float16* out = reinterpret_cast<_Float16*>(a.inp_store) + const_load(a.table + 2 * a.Et + e_of[k]) + lrow_of[k] * n;
+#pragma unroll
+          for (int i = 0; i < NI; ++i) {
+            v8h o;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) o[j] = (_Float16)v[i][j];
+            *reinterpret_cast<v8h*>(out + (lane + 64 * i) * 8) = o;
+          }
+        }
+      }
+    };
+    if ((present & 1u) && a.rotate != 2) store_copies();
+    if ((present & ~1u) == 0 && a.rotate != 2) continue;
+    if (a.rotate != 0) wave_rotate<NI>(v, lane, a.scale);
+    if ((present & 1u) && a.rotate == 2) store_copies();
+    if (present & 0x8u) {  // tag 3: int4, one scale per 128 values = the 16 chunks held by an aligned group of 16 lanes
+      unsigned w[NI];
+      float gscale[NI];
+#pragma unroll
+      for (int i = 0; i < NI; ++i) {
+        float gmax = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) gmax = fmaxf(gmax, fabsf(v[i][j]));
+#pragma unroll
+        for (int o = 8; o > 0; o >>= 1) gmax = fmaxf(gmax, __shfl_xor(gmax, o));
+        float scale = round_h(gmax / 7.0f);
+        if (scale == 0.0f) scale = 1.0f;
+        const ScaleDiv div(scale);
+        gscale[i] = scale;
+        w[i] = 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float r = round_h(div(v[i][j]));
+          w[i] = push_code<4>(w[i], code_word(fminf(fmaxf(r, -7.0f), 7.0f)));
+        }
+      }
+#pragma unroll
+      for (int k = 0; k < KD; ++k) {
+        if (k < ndst && tag_of[k] == 3) {
+          uint8_t* out = a.inp_store + 2 * (const_load(a.table + 2 * a.Et + e_of[k]) + lrow_of[k] * (n / 4));
+          _Float16* sout = a.scale_store + const_load(a.table + 3 * a.Et + e_of[k]) + lrow_of[k] * (n >> 7);
+#pragma unroll
+          for (int i = 0; i < NI; ++i) {
+            const int c = lane + 64 * i;
+            if ((c & 15) == 0) sout[c >> 4] = (_Float16)gscale[i];
+            *reinterpret_cast<unsigned*>(out + c * 4) = w[i];
+          }
+        }
+      }
+    }
+    if ((present & 0x6u) == 0) continue;
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[i][j]));
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
+    if (present & 0x2u) {  // tag 1: int8 per token
+      float scale = round_h(amax / 127.0f);  // fp16 division: fp32 quotient of two fp16 values, rounded to fp16
+      if (scale == 0.0f) scale = 1.0f;       // quantize.cuh:258
+      const ScaleDiv div(scale);
+      uint2 w[NI];
+#pragma unroll
+      for (int i = 0; i < NI; ++i) {
+        w[i] = uint2{0, 0};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          w[i].x = push_code<8>(w[i].x, code_word(fminf(fmaxf(round_h(div(v[i][j])), -127.0f), 127.0f)));
+          w[i].y = push_code<8>(w[i].y, code_word(fminf(fmaxf(round_h(div(v[i][j + 4])), -127.0f), 127.0f)));
+        }
+      }
+#pragma unroll
+      for (int k = 0; k < KD; ++k) {
+        if (k < ndst && tag_of[k] == 1) {
+          uint8_t* out = a.inp_store + 2 * (const_load(a.table + 2 * a.Et + e_of[k]) + lrow_of[k] * (n / 2));
+          if (lane == 0) a.scale_store[const_load(a.table + 3 * a.Et + e_of[k]) + lrow_of[k]] = (_Float16)scale;
+#pragma unroll
+          for (int i = 0; i < NI; ++i) *reinterpret_cast<uint2*>(out + (lane + 64 * i) * 8) = w[i];
+        }
+      }
+    }
+    if (present & 0x4u) {  // tag 2: int4 per token
+      float scale = round_h(amax / 7.0f);
+      if (scale == 0.0f) scale = 1.0f;
+      const ScaleDiv div(scale);
+      unsigned w[NI];
+#pragma unroll
+      for (int i = 0; i < NI; ++i) {
+        w[i] = 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) w[i] = push_code<4>(w[i], code_word(fminf(fmaxf(round_h(div(v[i][j])), -7.0f), 7.0f)));
+      }
+#pragma unroll
+      for (int k = 0; k < KD; ++k) {
+        if (k < ndst && tag_of[k] == 2) {
+          uint8_t* out = a.inp_store + 2 * (const_load(a.table + 2 * a.Et + e_of[k]) + lrow_of[k] * (n / 4));
+          if (lane == 0) a.scale_store[const_load(a.table + 3 * a.Et + e_of[k]) + lrow_of[k]] = (_Float16)scale;
+#pragma unroll
+          for (int i = 0; i < NI; ++i) *reinterpret_cast<unsigned*>(out + (lane + 64 * i) * 4) = w[i];
+        }
       }
     }
   }
@@ -1849,6 +2021,59 @@ int mxmoe_silu_mul_quant(const void* gate_up, const void* gate_up_shared, void* 
   const int nmax = N > a.plan_shared.n ? N : a.plan_shared.n;
   const int lds = (nmax + a.plan.kb * a.plan.kb + 16) * (int)sizeof(float);
   return launch_rows<true>(a, lds, (hipStream_t)stream, variants);
+}
+
+int mxmoe_quant_act_tokens(const void* hidden, void* inp_store, void* scale_store, const int32_t* topk_ids, const int32_t* row_of_slot, const int64_t* exp_table,
+                           int K, int num_tokens, int topk, int num_experts, int has_shared, int rotate, void* stream) {
+  if (num_tokens < 0 || num_experts <= 0 || topk < 0 || topk > kTokenMaxTopk) {
+    last_error() = "bad token or expert count, or more than 8 slots per token";
+    return 3;
+  }
+  if (K < 512 || K > 4096 || (K & (K - 1))) {
+    last_error() = "the per-token prologue takes rows of 512, 1024, 2048 or 4096 values";
+    return 3;
+  }
+  if (rotate < 0 || rotate > 2) {
+    last_error() = "rotate is 0, 1 or 2 (tables with operand-variant tags go through mxmoe_quant_act)";
+    return 3;
+  }
+  if (!hidden || !inp_store || !exp_table || (topk > 0 && (!topk_ids || !row_of_slot))) {
+    last_error() = "null pointer";
+    return 5;
+  }
+  if (num_tokens == 0 || topk + has_shared == 0) return 0;
+  TokenArgs a{};
+  a.src = reinterpret_cast<const _Float16*>(hidden);
+  a.inp_store = reinterpret_cast<uint8_t*>(inp_store);
+  a.scale_store = reinterpret_cast<_Float16*>(scale_store);
+  a.ids = topk_ids;
+  a.row_of_slot = row_of_slot;
+  a.table = exp_table;
+  a.T = num_tokens;
+  a.E = num_experts;
+  a.Et = num_experts + (has_shared ? 1 : 0);
+  a.topk = topk;
+  a.has_shared = has_shared ? 1 : 0;
+  a.rotate = rotate;
+  a.scale = 1.0f / sqrtf((float)K);
+  int dev = 0, cus = 256;
+  (void)hipGetDevice(&dev);
+  (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+  // (a multiple of 64 workgroups: xcd_row_group permutes within runs of 64)
+  const int grid = ((num_tokens + 3) / 4 < cus * 8 ? (num_tokens + 3) / 4 : cus * 8) + 63 & ~63;
+  hipStream_t s = (hipStream_t)stream;
+  switch (K / 512) {
+    case 1: hipLaunchKernelGGL((token_quant_wave_kernel<1>), dim3(grid), dim3(256), 0, s, a); break;
+    case 2: hipLaunchKernelGGL((token_quant_wave_kernel<2>), dim3(grid), dim3(256), 0, s, a); break;
+    case 4: hipLaunchKernelGGL((token_quant_wave_kernel<4>), dim3(grid), dim3(256), 0, s, a); break;
+    default: hipLaunchKernelGGL((token_quant_wave_kernel<8>), dim3(grid), dim3(256), 0, s, a); break;
+  }
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    last_error() = std::string("kernel launch failed: ") + hipGetErrorString(e);
+    return 4;
+  }
+  return 0;
 }
 
 // ---- the same three steps behind a device-side plan (mxmoe_plan_block): nothing here depends on the routing ----

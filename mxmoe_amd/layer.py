@@ -205,6 +205,9 @@ class MxMoELayer:
             return hk, hf, sg, None if sg is None else sg.data_ptr()
 
         ps["had1"], ps["had2"] = signs(cfg.hidden, cfg.hidden), signs(cfg.inter, i_sh)
+        # power-of-two rows without operand variants: the prologue quantises a token once per format, not once per destination row
+        ps["per_token"] = ops.per_token_prologue(cfg.hidden, topk) and not self._variants(self.bf6_gate_up)
+        ps["table1"] = b1["plan"].data_ptr() + lib.mxmoe_plan_offset(1, et)
         cache[key] = ps
         return ps
 
@@ -240,8 +243,12 @@ class MxMoELayer:
                                                ps["row_of_slot"].data_ptr(), ps["perm_ws"].data_ptr(), stream))
             ck(lib.mxmoe_plan_layer(C.byref(ps["calls"][0]), C.byref(ps["calls"][1]), ps["recv"].data_ptr(), e_cnt, ps["shared_rows"], stream))
         hk, hf, _sg, sgp = ps["had1"]
-        ck(lib.mxmoe_quant_act_planned(hidden.data_ptr(), b1["inp"].data_ptr(), b1["scale"].data_ptr(), ps["dst"].data_ptr(), ps["perm"].data_ptr(), b1["plan"].data_ptr(),
-                                       cfg.hidden, ps["r_cap"], t, e_cnt, has_shared, cfg.rotate | self._variants(self.bf6_gate_up), hk, hf, sgp, stream))
+        if ps["per_token"]:
+            ck(lib.mxmoe_quant_act_tokens(hidden.data_ptr(), b1["inp"].data_ptr(), b1["scale"].data_ptr(), ids.data_ptr(), ps["row_of_slot"].data_ptr(), ps["table1"],
+                                          cfg.hidden, t, topk, e_cnt, has_shared, cfg.rotate, stream))
+        else:
+            ck(lib.mxmoe_quant_act_planned(hidden.data_ptr(), b1["inp"].data_ptr(), b1["scale"].data_ptr(), ps["dst"].data_ptr(), ps["perm"].data_ptr(), b1["plan"].data_ptr(),
+                                           cfg.hidden, ps["r_cap"], t, e_cnt, has_shared, cfg.rotate | self._variants(self.bf6_gate_up), hk, hf, sgp, stream))
         ck(lib.mxmoe_group_gemm_planned(b1["kid"], b1["plan"].data_ptr(), ps["et"], b1["grid"], stream))
         i_sh = cfg.inter * max(cfg.num_shared, 1)
         hk, hf, _sg, sgp = ps["had2"]

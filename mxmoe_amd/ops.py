@@ -94,9 +94,15 @@ def gg_permute_inp(hidden: torch.Tensor, topk_ids: torch.Tensor, E: int):
     return int((recv_cpu != 0).sum()), hidden.index_select(0, perm[:routed]), perm, recv_cpu
 
 
-def build_permutation(topk_ids: torch.Tensor, num_experts: int):
+def per_token_prologue(k: int, topk: int) -> bool:
+    """Shapes that mxmoe_quant_act_tokens takes: rows of 512 .. 4096 values, a power of two, at most 8 slots per token."""
+    return 512 <= k <= 4096 and k & (k - 1) == 0 and 0 < topk <= 8
+
+
+def build_permutation(topk_ids: torch.Tensor, num_experts: int, with_inverse: bool = False):
     """Stable sort of the flattened expert ids on the device -> (dst_exp_sorted int32 [R], perm_indices int64 [R],
-    src_slot int64 [R], recv_tokens_per_exp int64 [E] on the device)."""
+    src_slot int64 [R], recv_tokens_per_exp int64 [E] on the device); with `with_inverse` also row_of_slot int32 [R]: the sorted row
+    of every (token, slot), -1 where the expert id was out of range."""
     lib = _lib.load()
     ids = topk_ids.to(torch.int32).contiguous()
     t, k = ids.shape
@@ -107,6 +113,11 @@ def build_permutation(topk_ids: torch.Tensor, num_experts: int):
     slot = torch.empty(r, dtype=torch.int64, device=dev)
     recv = torch.empty(num_experts, dtype=torch.int64, device=dev)
     ws = torch.empty(lib.mxmoe_permute_workspace_bytes(r, num_experts), dtype=torch.uint8, device=dev)
+    if with_inverse:
+        inv = torch.empty(r, dtype=torch.int32, device=dev)
+        _lib.check(lib, lib.mxmoe_build_permutation_inv(ids.data_ptr(), t, k, num_experts, dst.data_ptr(), perm.data_ptr(), slot.data_ptr(), recv.data_ptr(),
+                                                        inv.data_ptr(), ws.data_ptr(), _stream()))
+        return dst, perm, slot, recv, inv
     _lib.check(lib, lib.mxmoe_build_permutation(ids.data_ptr(), t, k, num_experts, dst.data_ptr(), perm.data_ptr(), slot.data_ptr(), recv.data_ptr(), ws.data_ptr(), _stream()))
     return dst, perm, slot, recv
 
@@ -168,7 +179,9 @@ def quant_inp_act(hidden, topk_ids, num_experts: int, N: int, num_shared_experts
     t, k = hidden.shape
     topk = topk_ids.shape[1]
     has_shared = num_shared_experts > 0
-    dst, perm, _slot, recv = build_permutation(topk_ids, num_experts)
+    # power-of-two rows without operand variants: quantise a token once per format among its destinations, not once per destination row
+    per_token = per_token_prologue(k, topk) and not (bf6 or fp8)
+    dst, perm, _slot, recv, *inv = build_permutation(topk_ids, num_experts, with_inverse=per_token)
     recv_cpu = recv.cpu()                                   # one small D2H copy, as ref_bind.cu:451
     table, rows, inp_sizes, scale_sizes, lds, io, so = _offsets(recv_cpu, t, num_experts, has_shared, qparams_per_exp, k, k, bf6, fp8)
     dev = hidden.device
@@ -178,8 +191,14 @@ def quant_inp_act(hidden, topk_ids, num_experts: int, N: int, num_shared_experts
     d_table = table.to(dev)
     hk, hf, signs = device_signs(k, dev) if rotate else (1, 1, None)
     routed = int(recv_cpu.sum())                            # rows whose expert id was in range; the sorted arrays hold exactly these
-    _lib.check(lib, lib.mxmoe_quant_act(hidden.data_ptr(), inp_store.data_ptr(), scale_store.data_ptr(), dst.data_ptr(), perm.data_ptr(), d_table.data_ptr(),
-                                        k, routed, t, num_experts, int(has_shared), rotate | (ROWS_VARIANTS if bf6 or fp8 else 0), hk, hf, None if signs is None else signs.data_ptr(), _stream()))
+    if per_token:
+        ids32 = topk_ids.to(torch.int32).contiguous()
+        _lib.check(lib, lib.mxmoe_quant_act_tokens(hidden.data_ptr(), inp_store.data_ptr(), scale_store.data_ptr(), ids32.data_ptr(), inv[0].data_ptr(), d_table.data_ptr(),
+                                                   k, t, topk, num_experts, int(has_shared), rotate, _stream()))
+    else:
+        _lib.check(lib, lib.mxmoe_quant_act(hidden.data_ptr(), inp_store.data_ptr(), scale_store.data_ptr(), dst.data_ptr(), perm.data_ptr(), d_table.data_ptr(),
+                                            k, routed, t, num_experts, int(has_shared), rotate | (ROWS_VARIANTS if bf6 or fp8 else 0), hk, hf,
+                                            None if signs is None else signs.data_ptr(), _stream()))
     inp_list, scale_list = _views(inp_store, scale_store, table, rows, inp_sizes, scale_sizes, lds)
     out_list, off = [], 0
     for e, n in enumerate(rows):

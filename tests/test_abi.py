@@ -213,6 +213,11 @@ def test_prologue_entry_points_validate_on_the_host(lib):
     assert lib.mxmoe_quant_act(a, a, a, a, a, a, 256, -1, 2, 2, 0, 0, 1, 1, None, None) == 3
     assert lib.mxmoe_quant_act(a, a, a, a, a, a, 260, 4, 2, 2, 0, 0, 1, 1, None, None) == 3 and b"multiple of 8" in lib.mxmoe_last_error()
     assert lib.mxmoe_silu_mul_quant(a, None, a, a, a, a, 256, 256, 4, 2, 2, 1, 0, 1, 1, None, None) == 5
+    assert lib.mxmoe_quant_act_tokens(None, a, a, a, a, a, 2048, 4, 2, 2, 0, 0, None) == 5 and b"null" in lib.mxmoe_last_error()
+    assert lib.mxmoe_quant_act_tokens(a, a, a, a, a, a, 1408, 4, 2, 2, 0, 0, None) == 3 and b"512" in lib.mxmoe_last_error()
+    assert lib.mxmoe_quant_act_tokens(a, a, a, a, a, a, 2048, 4, 9, 2, 0, 0, None) == 3 and b"8 slots" in lib.mxmoe_last_error()
+    assert lib.mxmoe_quant_act_tokens(a, a, a, a, a, a, 2048, 4, 2, 2, 0, 4, None) == 3
+    assert lib.mxmoe_quant_act_tokens(a, a, a, a, a, a, 2048, 0, 2, 2, 0, 0, None) == 0      # no tokens: nothing to launch
     assert lib.mxmoe_silu_mul_quant(a, a, a, a, a, a, 1408, 1408, 4, 2, 2, 0, 1, 176, 4, None, None) == 3 and b"sign table" in lib.mxmoe_last_error()
     assert lib.mxmoe_permute_plan_layer(a, 200, 2, 8, a, a, a, a, a, a, a, 0, None) == 3 and b"256" in lib.mxmoe_last_error()   # larger batches: the two separate calls
     assert lib.mxmoe_permute_plan_layer(a, 4, 2, 8, a, a, a, a, a, None, a, 0, None) == 5

@@ -127,6 +127,52 @@ def test_quant_inp_act_bit_exact(k, rotate):
     assert p == len(inp_list)
 
 
+@pytest.mark.parametrize("k,topk,rotate,n_sh", [(2048, 8, 1, 1), (512, 1, 2, 0), (4096, 3, 1, 0), (1024, 4, 0, 1), (2048, 4, 2, 1)])
+def test_per_token_prologue_writes_the_same_bytes_as_the_per_row_one(k, topk, rotate, n_sh):
+    """mxmoe_quant_act_tokens (a token quantised once per format among its destinations) against mxmoe_quant_act (once per
+    destination row) over the same table: mixed formats (fp16 copies, int8, int4, int4 with group scales), expert ids out of range,
+    an expert without rows, up to 8 slots per token.  The stores must match byte for byte."""
+    from mxmoe_amd import _lib, ops
+
+    lib = _lib.load()
+    rng = np.random.default_rng(k + topk)
+    t, e = 70, 10
+    has_shared = n_sh > 0
+    x = torch.from_numpy(rng.standard_normal((t, k)).astype(F16)).to(DEV)
+    ids = _ids(rng, t, e, topk)
+    ids[ids == 6] = 7 if topk == 1 else e + 3                              # expert 6 gets no rows; with top-k > 1 its slots are dropped
+    ids[rng.random(ids.shape) < 0.1] = -1
+    d_ids = torch.from_numpy(ids).to(DEV)
+    fmts = [(4, 4, -1, True), (8, 8, -1, True), (16, 4, 128, False), (4, 4, 128, True), (16, 16, -1, True)]
+    qp = [fmts[i % len(fmts)] for i in range(e)] + [(8, 8, -1, True)]
+    dst, perm, _slot, recv, inv = ops.build_permutation(d_ids, e, with_inverse=True)
+    recv_cpu = recv.cpu()
+    table, _rows, _isz, _ssz, _lds, io, so = ops._offsets(recv_cpu, t, e, has_shared, qp, k, k)
+    d_table = table.to(DEV)
+    routed = int(recv_cpu.sum())
+    hk, hf, signs = ops.device_signs(k, DEV) if rotate else (1, 1, None)
+    stream = torch.cuda.current_stream().cuda_stream
+    stores = []
+    for which in range(2):
+        inp = torch.full((io,), 0x1234, dtype=torch.int16, device=DEV)
+        sc = torch.full((max(so, 1),), 0x1234, dtype=torch.int16, device=DEV)
+        if which == 0:
+            _lib.check(lib, lib.mxmoe_quant_act(x.data_ptr(), inp.data_ptr(), sc.data_ptr(), dst.data_ptr(), perm.data_ptr(), d_table.data_ptr(), k, routed, t, e,
+                                                int(has_shared), rotate, hk, hf, None if signs is None else signs.data_ptr(), stream))
+        else:
+            _lib.check(lib, lib.mxmoe_quant_act_tokens(x.data_ptr(), inp.data_ptr(), sc.data_ptr(), d_ids.data_ptr(), inv.data_ptr(), d_table.data_ptr(), k, t, topk, e,
+                                                       int(has_shared), rotate, stream))
+        torch.cuda.synchronize()
+        stores.append((inp.cpu().numpy(), sc.cpu().numpy()))
+    assert routed > 0 and (stores[0][0] != 0x1234).any()
+    assert np.array_equal(stores[0][0], stores[1][0])
+    assert np.array_equal(stores[0][1], stores[1][1])
+    # shapes the per-token entry point refuses
+    assert lib.mxmoe_quant_act_tokens(x.data_ptr(), inp.data_ptr(), sc.data_ptr(), d_ids.data_ptr(), inv.data_ptr(), d_table.data_ptr(), 1408, t, topk, e, 0, 1, stream) == 3
+    assert lib.mxmoe_quant_act_tokens(x.data_ptr(), inp.data_ptr(), sc.data_ptr(), d_ids.data_ptr(), inv.data_ptr(), d_table.data_ptr(), k, t, 9, e, 0, 1, stream) == 3
+    assert lib.mxmoe_quant_act_tokens(x.data_ptr(), inp.data_ptr(), sc.data_ptr(), d_ids.data_ptr(), inv.data_ptr(), d_table.data_ptr(), k, t, topk, e, 0, 5, stream) == 3
+
+
 @pytest.mark.parametrize("n,n_sh,rotate", [(1408, 2, 2), (2048, 0, 1), (14336, 0, 1), (512, 1, 0), (1408, 0, 1), (1408, 1, 2), (224, 0, 2), (96, 1, 1)])
 def test_silu_mul_then_quant_bit_exact(n, n_sh, rotate):
     from mxmoe_amd import ops
