@@ -374,11 +374,19 @@ inline double branch_cost(const BranchInfo& b) {
 constexpr int kMaxBranches = 32;
 struct PlanBranch {
   int fmt, BM, BN, k_multiple;
-  double cost;  // tile_cost
+  int bm_log2, bn_log2;  // of a tile dimension that is a power of two (the usual case: the planners shift instead of dividing), else -1
+  double cost;           // tile_cost
+  double cost_per_row;   // tile_cost / BM
 };
+// Tiles of size `dim` (2^`lg` when lg >= 0) that cover `x`.
+__host__ __device__ inline int tiles_over(int x, int dim, int lg) { return lg >= 0 ? (x + dim - 1) >> lg : (x + dim - 1) / dim; }
+constexpr int kNumFmts = (int)Fmt::UNSUPPORTED;
 struct PlanInfo {
   int nb;                    // branches
   int order[kMaxBranches];   // branch indices, most expensive tile first (branch_cost); ties keep the registration order
+  // the branches of one format as a list in registration order (-1 ends it): the planners look at no other branch
+  int first_of_fmt[kNumFmts];
+  int next_of_fmt[kMaxBranches];
   PlanBranch b[kMaxBranches];
 };
 
@@ -386,10 +394,10 @@ struct PlanInfo {
 __host__ __device__ inline int pick_branch(const PlanInfo& k, int f, int rows, int N) {
   int best = -1;
   double best_cost = 0;
-  for (int i = 0; i < k.nb; ++i) {
+  if (f < 0 || f >= kNumFmts) return -1;
+  for (int i = k.first_of_fmt[f]; i >= 0; i = k.next_of_fmt[i]) {
     const PlanBranch& b = k.b[i];
-    if (b.fmt != f) continue;
-    const double c = (double)((rows + b.BM - 1) / b.BM) * ((N + b.BN - 1) / b.BN) * b.cost;
+    const double c = (double)tiles_over(rows, b.BM, b.bm_log2) * tiles_over(N, b.BN, b.bn_log2) * b.cost;
     if (best < 0 || c < best_cost - 1e-9 || (c < best_cost + 1e-9 && b.BM > k.b[best].BM)) {
       best = i;
       best_cost = c;
@@ -408,10 +416,10 @@ struct Segment {
 __host__ __device__ inline int plan_segments(const PlanInfo& k, int f, int M, int N, Segment out[2]) {
   int big = -1;
   double big_unit = 0;
-  for (int i = 0; i < k.nb; ++i) {
+  if (f < 0 || f >= kNumFmts) return -1;
+  for (int i = k.first_of_fmt[f]; i >= 0; i = k.next_of_fmt[i]) {
     const PlanBranch& b = k.b[i];
-    if (b.fmt != f) continue;
-    const double unit = b.cost * ((N + b.BN - 1) / b.BN) / b.BM;  // cost per row of the problem
+    const double unit = b.cost_per_row * tiles_over(N, b.BN, b.bn_log2);  // cost per row of the problem
     if (big < 0 || unit < big_unit - 1e-12 || (unit < big_unit + 1e-12 && b.BM > k.b[big].BM)) {
       big = i;
       big_unit = unit;
@@ -421,10 +429,10 @@ __host__ __device__ inline int plan_segments(const PlanInfo& k, int f, int M, in
   if (M <= 0) return 0;
   auto cost_of = [&](int branch, int rows) {
     const PlanBranch& b = k.b[branch];
-    return (double)((rows + b.BM - 1) / b.BM) * ((N + b.BN - 1) / b.BN) * b.cost;
+    return (double)tiles_over(rows, b.BM, b.bm_log2) * tiles_over(N, b.BN, b.bn_log2) * b.cost;
   };
-  const int bm = k.b[big].BM;
-  const int full = (M / bm) * bm, rem = M - full;
+  const int bm = k.b[big].BM, bm_lg = k.b[big].bm_log2;
+  const int full = bm_lg >= 0 ? (M >> bm_lg) << bm_lg : (M / bm) * bm, rem = M - full;
   const int whole = pick_branch(k, f, M, N);
   if (rem == 0 || full == 0) {
     out[0] = Segment{0, M, whole};
@@ -442,7 +450,7 @@ __host__ __device__ inline int plan_segments(const PlanInfo& k, int f, int M, in
 
 __host__ __device__ inline int segment_tiles(const PlanInfo& k, const Segment& sg, int N) {
   const PlanBranch& b = k.b[sg.branch];
-  return ((sg.rows + b.BM - 1) / b.BM) * ((N + b.BN - 1) / b.BN);
+  return tiles_over(sg.rows, b.BM, b.bm_log2) * tiles_over(N, b.BN, b.bn_log2);
 }
 
 inline PlanInfo make_plan_info(const std::vector<BranchInfo>& branches) {
@@ -450,10 +458,26 @@ inline PlanInfo make_plan_info(const std::vector<BranchInfo>& branches) {
   std::memset(&k, 0, sizeof k);
   k.nb = std::min((int)branches.size(), kMaxBranches);
   for (int i = 0; i < k.nb; ++i) {
-    k.b[i] = PlanBranch{(int)branches[i].fmt, branches[i].BM, branches[i].BN, branches[i].k_multiple, tile_cost(branches[i])};
+    auto log2_of = [](int v) {
+      int lg = -1;
+      if (v > 0 && (v & (v - 1)) == 0)
+        for (lg = 0; (1 << lg) < v; ++lg) {}
+      return lg;
+    };
+    const double cost = tile_cost(branches[i]);
+    k.b[i] = PlanBranch{(int)branches[i].fmt, branches[i].BM, branches[i].BN, branches[i].k_multiple, log2_of(branches[i].BM), log2_of(branches[i].BN), cost,
+                        cost / branches[i].BM};
     k.order[i] = i;
   }
   std::stable_sort(k.order, k.order + k.nb, [&](int x, int y) { return branch_cost(branches[x]) > branch_cost(branches[y]); });
+  for (int f = 0; f < kNumFmts; ++f) k.first_of_fmt[f] = -1;
+  for (int i = k.nb - 1; i >= 0; --i) {
+    const int f = k.b[i].fmt;
+    k.next_of_fmt[i] = -1;
+    if (f < 0 || f >= kNumFmts) continue;
+    k.next_of_fmt[i] = k.first_of_fmt[f];
+    k.first_of_fmt[f] = i;
+  }
   return k;
 }
 

@@ -76,8 +76,19 @@ __device__ __forceinline__ void plan_block_body(const PlanParams& p, const int c
   __shared__ long s_base[5][2];                      // the same four, and the routed rows, summed over the experts before this launch
   __shared__ int s_cnt[kMaxBranches][2], s_til[kMaxBranches][2];  // per run-order rank and wave: entries, tiles
   __shared__ int s_cnt_long[kMaxBranches][2], s_til_long[kMaxBranches][2];  // ... of which belong to long-K problems
+  // the kernel's branch table, from the kernel arguments into LDS: the planning functions walk it entry by entry, and each step of
+  // such a walk through the argument segment costs a trip to the scalar cache
+  __shared__ PlanInfo info;
+  static_assert(sizeof(PlanInfo) % 4 == 0, "copied word by word");
+  for (int i = threadIdx.x; i < (int)(sizeof(PlanInfo) / 4); i += kPlanThreads) reinterpret_cast<int*>(&info)[i] = reinterpret_cast<const int*>(&p.info)[i];
   const int e = threadIdx.x, lane = e & 63, wave = e >> 6;
   const int ge = e0 + e;                             // this thread's expert
+  __shared__ unsigned s_used[2];                     // per wave: branches in use
+  if (e < kMaxBranches) {
+    s_cnt[e][0] = s_cnt[e][1] = s_til[e][0] = s_til[e][1] = 0;
+    s_cnt_long[e][0] = s_cnt_long[e][1] = s_til_long[e][0] = s_til_long[e][1] = 0;
+  }
+  if (e < 2) s_used[e] = 0;
   const bool mine = e < ecnt;
   const PlanLayout lay(p.Et);
   FusedArgs* fa = reinterpret_cast<FusedArgs*>(p.plan + chunk * kFusedArgsStride);
@@ -101,20 +112,25 @@ __device__ __forceinline__ void plan_block_body(const PlanParams& p, const int c
     if (tag_out) *tag_out = tag;
     if (d_out) *d_out = d;
   };
-  // experts before this launch
-  long base[5] = {0, 0, 0, 0, 0};
-  for (int x = e; x < e0; x += kPlanThreads) {
-    long f[4];
-    footprint(x, f, nullptr, nullptr);
+  // experts before this launch (none for the first: most blocks are one launch)
+  if (e0 > 0) {
+    long base[5] = {0, 0, 0, 0, 0};
+    for (int x = e; x < e0; x += kPlanThreads) {
+      long f[4];
+      footprint(x, f, nullptr, nullptr);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) base[i] += f[i];
-    if (x < p.E) base[4] += f[0];
-  }
+      for (int i = 0; i < 4; ++i) base[i] += f[i];
+      if (x < p.E) base[4] += f[0];
+    }
 #pragma unroll
-  for (int i = 0; i < 5; ++i) {
+    for (int i = 0; i < 5; ++i) {
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) base[i] += __shfl_xor(base[i], o);
-    if (lane == 0) s_base[i][wave] = base[i];
+      for (int o = 32; o > 0; o >>= 1) base[i] += __shfl_xor(base[i], o);
+      if (lane == 0) s_base[i][wave] = base[i];
+    }
+  } else if (lane == 0) {
+#pragma unroll
+    for (int i = 0; i < 5; ++i) s_base[i][wave] = 0;
   }
 
   long rows = 0, sld = 0;
@@ -156,16 +172,27 @@ __device__ __forceinline__ void plan_block_body(const PlanParams& p, const int c
   const bool long_k = mine && K > min(s_kmin[0], s_kmin[1]);
   // segments of this problem and, per branch in run order, this wave's entries and tiles
   Segment sg[2];
-  const int ns = mine ? plan_segments(p.info, fmt, (int)rows, N, sg) : 0;
+  const int ns = mine ? plan_segments(info, fmt, (int)rows, N, sg) : 0;
   int seg_tiles[2], seg_rank[2], seg_pos[2], seg_first[2];
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
-    seg_tiles[j] = j < ns ? segment_tiles(p.info, sg[j], N) : 0;
+    seg_tiles[j] = j < ns ? segment_tiles(info, sg[j], N) : 0;
     seg_rank[j] = -1;
     seg_pos[j] = seg_first[j] = 0;
   }
-  for (int r = 0; r < p.info.nb; ++r) {
-    const int b = p.info.order[r];
+  // branches that this wave's problems use at all (most branches of a kernel are not used by a given launch: their counters stay zero)
+  {
+    unsigned mask = 0;
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+      if (j < ns && seg_tiles[j] > 0) mask |= 1u << sg[j].branch;
+    if (mask) atomicOr(&s_used[wave], mask);
+  }
+  __builtin_amdgcn_wave_barrier();
+  const unsigned used = (unsigned)__builtin_amdgcn_readfirstlane((int)*(volatile unsigned*)&s_used[wave]);
+  for (int r = 0; r < info.nb; ++r) {
+    const int b = info.order[r];
+    if (!(used >> b & 1)) continue;
     int mine_tiles = 0, which = -1;
 #pragma unroll
     for (int j = 0; j < 2; ++j)
@@ -264,7 +291,7 @@ __device__ __forceinline__ void plan_block_body(const PlanParams& p, const int c
     if (chunk == 0 && p.Et == p.E) misc[1] = 0;
     int total = 0, wg = 0, np = 0, ne = 0, flat = 0;
     int last_tile0 = 0, last_wg0 = 0;  // of the phase being filled (kept here: reading them back from the table would wait for the store)
-    for (int r = 0; r < p.info.nb; ++r) {
+    for (int r = 0; r < info.nb; ++r) {
       const int tile0 = total;
       total += s_til[r][0] + s_til[r][1];
       ne += s_cnt[r][0] + s_cnt[r][1];
@@ -272,7 +299,7 @@ __device__ __forceinline__ void plan_block_body(const PlanParams& p, const int c
       if (np < kMaxPhases) {  // shapes beyond the phase table share the last phase
         fa->phase_tile0[np] = last_tile0 = tile0;
         fa->phase_wg0[np] = last_wg0 = wg;
-        if (p.info.b[p.info.order[r]].BM <= 16) flat |= 1 << np;
+        if (info.b[info.order[r]].BM <= 16) flat |= 1 << np;
         ++np;
       }
       wg = last_wg0 + (total - last_tile0 + kNumXcd - 1) / kNumXcd * kNumXcd;
