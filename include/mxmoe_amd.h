@@ -52,6 +52,15 @@ int mxmoe_kernel_branch(int kernel_id, int branch, int32_t out[8]);
  *   w4a4_g-1_sym      int4 [M,K/2] (even k low)  fragment blocks of int4 [N,K/2] (*) fp16 [M]        fp16 [N]
  *   w4a4_g128_sym     int4 [M,K/2] (even k low)  fragment blocks of int4 [N,K/2] (*) fp16 [M,K/128]  fp16 [K/128,N] (group-major)
  *   w{4,3,2}a16_g128  fp16 [M,K]                 packed [N/16][K/128][64][w dwords]  -               fp16 [N/16][K/128][16][2]
+ *   w8a16_g128        fp16 [M,K]                 packed [N/16][K/128][64][8 dwords]  -               fp16 [N/16][K/128][16][2]
+ *   w{8,4,3,2}a16_g-1 as the g128 rows: a channel's one (scale, zero) pair is stored once per group of 128
+ *
+ * Operand variants (kernels whose mxmoe_kernel_branch reports a variant in out[0] >> 8; chosen by name, never by kernel_id = -1):
+ *   w4a4_g-1_sym, variant 1 (bf6): As[p] = the int4 codes as 6-bit floats (e3m2) in fragments of 32 rows x 64 values, 1536 bytes each,
+ *     ceil(M/32) * (K/64) of them, row-block-major; Bs[p] = fragment blocks of the same 6-bit codes; scales as w4a4_g-1_sym; K a
+ *     multiple of 128, at least 256.  Results equal the integer kernels' bit for bit.
+ *   w8a8_g-1_sym, variant 2 (fp8, the reference's w8a8_g-1_sym_E4M3, mm_tile.cuh:696-697): As[p], Bs[p] = OCP e4m3 codes in the int8
+ *     layouts, scale = max|x| / 448.
  *
  * (*) weights of the integer formats are stored in MFMA fragment order: uint8 [ceil(N/32)][KB/64][2][64 lanes][16], KB = bytes per
  *     row; lane l of block (nb, ks, step) holds bytes ks*64 + (2*step + (l >> 5))*16 .. +16 of channel nb*32 + (l & 31), channels past N

@@ -1046,8 +1046,8 @@ __global__ void __launch_bounds__(256) token_quant_wave_kernel(const TokenArgs a
 // row is 176 x 8 with f = 4, kb = 44): lane l holds the chunks l + 64 i, a chunk being the 8 values of one k.  The Sylvester part
 // (H_8) stays inside a chunk.  The dense stage t[b][col] = sum_b' B[b][b'] q[b'][col] over the 8 f columns col = blk * 8 + j runs on the
 // matrix cores: the row, snapped to integers of at most 18 bits (DenseGrid) and divided by 16 so that every value is an fp16 number,
-// is written to LDS transposed ([col][b'], b' contiguous), B (+-1, zero padded) is the first operand held in registers for the
-// whole kernel, and the fp32 results are exact whatever order the hardware adds in.  Results return through LDS in row order, so
+// is written to LDS transposed ([col][b'], b' contiguous), B (+-1, zero padded) is the first operand, kept in LDS in operand order
+// and read block by block, and the fp32 results are exact whatever order the hardware adds in.  Results return through LDS in row order, so
 // the quantise / pack / store code sees the same chunk-per-lane layout as in the other kernels and writes 16 bytes per lane.
 // Four independent rows per workgroup; no barrier (each wave owns its piece of LDS).
 constexpr int kDensePitch = 144;             // bytes per column of the transposed row: 64 fp16 + 16 (16 lanes read 16 distinct bank groups)
