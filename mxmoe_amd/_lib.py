@@ -87,6 +87,9 @@ def load(path: str | Path | None = None) -> C.CDLL:
     """Load the library and attach the C-ABI signatures.  A generated library (`path` given) carries the GroupGEMM entry
     points only; the default library must export everything the header declares."""
     p = Path(path) if path is not None else LIB_PATH
+    hit = _cached.get(str(p))  # (as given: the operators come here on every call and should not walk the file system again)
+    if hit is not None:
+        return hit
     if not p.exists():
         raise RuntimeError(
             f"{p} is missing: build it with `python -m mxmoe_amd.build` (hipcc, gfx950). "
@@ -104,7 +107,7 @@ def load(path: str | Path | None = None) -> C.CDLL:
         fn = getattr(lib, name)
         fn.restype = res
         fn.argtypes = args
-    _cached[key] = lib
+    _cached[key] = _cached[str(p)] = lib
     return lib
 
 
