@@ -249,11 +249,11 @@ def test_layer_from_fake_quantised_weights_is_their_function(tmp_path):
     assert err2 > 3 * err, (err, err2)
 
 
-def _small_layer(num_shared=1, rotate=1, bf6=False):
+def _small_layer(num_shared=1, rotate=1, bf6=False, hidden=256, topk=2):
     from mxmoe_amd import synth
     from mxmoe_amd.layer import MxMoELayer
 
-    cfg = synth.MoEConfig("t", "test", 6, 2, 256, 1408, 96, num_shared=num_shared, rotate=rotate)
+    cfg = synth.MoEConfig("t", "test", 6, topk, hidden, 1408, 96, num_shared=num_shared, rotate=rotate)
     g = synth.W4A4G128
     fm = [(synth.W4A4, synth.W8A8), (synth.W8A8, synth.W4A4), (g, g), (synth.W4A16, synth.W3A16), (synth.FP16, synth.FP16), (synth.W4A4, synth.W4A4),
           (synth.W8A8, synth.W8A8)][: 6 + (1 if num_shared else 0)]
@@ -299,6 +299,25 @@ def test_planned_forward_equals_the_host_planned_one(num_shared):
     assert np.array_equal(ptrs[1], gu.b_ptr) and np.array_equal(ptrs[3], gu.sb_ptr)
     assert np.array_equal(ptrs[2], np.where(gu.sld > 0, b1["scale"].data_ptr() + 2 * bt.table[3], 0))
     assert misc[1] == (ptrs[4][-1] if num_shared else 0)
+
+
+@pytest.mark.parametrize("hidden,topk,rotate", [(512, 2, 1), (1024, 5, 2), (512, 3, 0)])
+def test_planned_forward_with_the_per_token_prologue_equals_the_per_row_one(hidden, topk, rotate):
+    """Power-of-two rows: the planned forward quantises its input once per token and format (mxmoe_quant_act_tokens), the forward
+    with host tables once per destination row (mxmoe_quant_act); every format in one layer, a shared expert, some expert ids out
+    of range.  Identical outputs."""
+    from mxmoe_amd import synth
+
+    cfg, layer = _small_layer(1, rotate, hidden=hidden, topk=topk)
+    hidden_t = synth.make_hidden(cfg)
+    ids, w = synth.make_routing(cfg)
+    ids[3, 0] = cfg.num_experts + 1
+    ids[7, topk - 1] = -2
+    assert layer._planned_setup(cfg.tokens, cfg.topk)["per_token"]
+    got = layer(hidden_t, ids, w).clone()
+    want = layer.call_with_host_tables(hidden_t, ids, w)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
 
 
 def test_device_planner_writes_the_host_launchers_tile_tables():
