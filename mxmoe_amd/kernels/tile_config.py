@@ -36,6 +36,10 @@ TYPE_TO_BITS = {
 # 8 / 4 / 2 bits with both group sizes; 3 bits is this library's addition)
 WEIGHT_ONLY_QCFG = [f"w{w}a16_g{g}_{s}" for w in (8, 4, 3, 2) for g in (128, -1) for s in ("sym", "asym")]
 
+# The reference's "_accfp16" names (fp16 accumulators in its mma instructions, tile_config.py:41,50-56): the matrix instructions of
+# gfx950 accumulate fp16 products in fp32 only, so these names are accepted and built as the fp32-accumulating tiles of the base format.
+ACCFP16_ALIASES = {"fp16_accfp16": "fp16", **{f"{q}_accfp16": q for q in WEIGHT_ONLY_QCFG}}
+
 SUPPORTED_QCFG = [
     "fp16",
     "w8a8_g-1_sym",
@@ -43,6 +47,7 @@ SUPPORTED_QCFG = [
     "w4a4_g-1_sym",
     "w4a4_g128_sym",
     *WEIGHT_ONLY_QCFG,
+    *ACCFP16_ALIASES,
 ]
 
 # (M, N, K) of one MFMA instruction
@@ -70,6 +75,7 @@ QCFG_TO_MMA = {
     "w4a4_g128_sym": "MFMA_I32_32x32x32_I8_FROM_I4",
     **{q: "MFMA_F32_16x16x32_F16" for q in WEIGHT_ONLY_QCFG},
 }
+QCFG_TO_MMA.update({alias: QCFG_TO_MMA[base] for alias, base in ACCFP16_ALIASES.items()})
 
 
 @dataclasses.dataclass
@@ -261,6 +267,7 @@ QCFG_MAP = {
     "w4a4_g128_sym": TileConfig(QCFGA=QCFG_W4A4_G128, QCFGB=QCFG_W4A4_G128),
     **{k: TileConfig(QCFGB=build_qcfgb_from_str(k)) for k in WEIGHT_ONLY_QCFG},
 }
+QCFG_MAP.update({alias: QCFG_MAP[base] for alias, base in ACCFP16_ALIASES.items()})
 
 
 def _with_q(t: TileConfig, qcfg: str) -> TileConfig:

@@ -104,6 +104,13 @@ def test_template_generator_product_and_sources(tmp_path):
             'WxAxTile<Op::I8, 64, 256>>("groupgemm_ms_launch_0", Policy::MultiStream)') in (tmp_path / "sets" / "ms_launch_0.hip").read_text()
     with pytest.raises(ValueError, match="Unsupported qcfg"):
         TemplateGenerator("gfx950", ["w1a16_g128_sym"])
+    # the reference's fp16-accumulate names are accepted and built as the base format's (fp32-accumulating) tiles
+    for alias, base in (("w4a16_g128_asym_accfp16", "w4a16_g128_asym"), ("fp16_accfp16", "fp16"), ("w2a16_g-1_sym_accfp16", "w2a16_g-1_sym")):
+        assert tile_config.get_info_from_qcfg_str(alias) == tile_config.get_info_from_qcfg_str(base)
+        assert [t.cpp_type() for t in tile_config.get_possible_tile_list("gfx950", alias)] == [t.cpp_type() for t in tile_config.get_possible_tile_list("gfx950", base)]
+    ga = TemplateGenerator("gfx950", ["w4a16_g128_asym_accfp16"], KernelType.Fused, out_dir=tmp_path / "acc")
+    ga.generate_source_code()
+    assert "SkinnyWoTile<4, 128" in (tmp_path / "acc" / "hz_fused_0.hip").read_text()
 
 
 def test_default_library_is_generator_output(tmp_path, lib):
