@@ -259,6 +259,13 @@ class MxMoELayer:
                                      final.data_ptr(), stream))
         return final
 
+    def capture(self, tokens: int, topk: int | None = None) -> "CapturedForward":
+        """The planned forward for a fixed (tokens, top-k) shape, captured into a HIP graph: write the inputs into the returned
+        object's `hidden`, `topk_ids`, `topk_weights` tensors, call `replay()`, read `out`.  Nothing in the forward depends on the
+        routing at enqueue time, so one capture serves every routing; a replay has no per-kernel launch gaps (decode-sized batches
+        gain most: 0.105 against 0.12 ms for DeepSeek-V2-Lite at 32 tokens)."""
+        return CapturedForward(self, tokens, self.cfg.topk if topk is None else topk)
+
     def call_with_host_tables(self, hidden: torch.Tensor, topk_ids: torch.Tensor, topk_weights: torch.Tensor) -> torch.Tensor:
         """The whole MoE MLP with the tables of both launches built on the HOST (what the reference's operators do), `(hidden [T, K] fp16, topk_ids [T, k] int32, topk_weights [T, k] fp32) -> [T, K] fp16`: what a serving
         framework's fused-MoE operator computes after routing (permute, quantise, gate_up, SiLU * up, down, un-permute + combine).
@@ -357,3 +364,27 @@ class MxMoELayer:
                 c += 2 * m * n
             out[name] = {"weights": w, "activations": a, "outputs": c, "total": w + a + c}
         return out
+
+
+class CapturedForward:
+    """`MxMoELayer.__call__` for one shape as a HIP graph over static input and output tensors."""
+
+    def __init__(self, layer: MxMoELayer, tokens: int, topk: int):
+        dev = layer.device
+        self.hidden = torch.zeros((tokens, layer.cfg.hidden), dtype=torch.float16, device=dev)
+        self.topk_ids = torch.zeros((tokens, topk), dtype=torch.int32, device=dev)
+        self.topk_weights = torch.zeros((tokens, topk), dtype=torch.float32, device=dev)
+        self.out = torch.empty((tokens, layer.cfg.hidden), dtype=torch.float16, device=dev)
+        side = torch.cuda.Stream(device=dev)  # (default priority)
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):  # one eager run: every buffer of this shape exists before the capture
+            layer(self.hidden, self.topk_ids, self.topk_weights, out=self.out)
+        torch.cuda.current_stream().wait_stream(side)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph, stream=side):
+            layer(self.hidden, self.topk_ids, self.topk_weights, out=self.out)
+        self._layer = layer  # the graph's kernels read the layer's buffers
+
+    def replay(self) -> torch.Tensor:
+        self.graph.replay()
+        return self.out

@@ -574,3 +574,19 @@ def test_planned_forward_replays_from_a_graph():
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(out, want), f"replay {replay}"
+    # the same through the layer's own capture object
+    cap = layer.capture(cfg.tokens)
+    for replay in range(2):
+        gen.manual_seed(200 + replay)
+        new_ids = torch.stack([torch.randperm(cfg.num_experts, generator=gen)[: cfg.topk] for _ in range(cfg.tokens)]).to(torch.int32)
+        new_w = torch.rand(cfg.tokens, cfg.topk, generator=gen)
+        new_h = torch.randn(cfg.tokens, cfg.hidden, generator=gen).half()
+        layer.forward(new_h, new_ids)
+        want = layer.combine(new_w).clone()
+        cap.hidden.copy_(new_h.cuda())
+        cap.topk_ids.copy_(new_ids.cuda())
+        cap.topk_weights.copy_(new_w.cuda())
+        torch.cuda.synchronize()
+        got = cap.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), f"captured replay {replay}"
