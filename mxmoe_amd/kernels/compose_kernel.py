@@ -169,7 +169,8 @@ def default_kernel_specs(arch: str = "gfx950"):
     wo_big = OrderedDict((f"w{b}a16_g128_asym", _pick(arch, f"w{b}a16_g128_asym", (128, 256))) for b in (4, 3, 2))
     wo_all = OrderedDict((q, wo[q] + wo_big[q]) for q in wo)
     everything = OrderedDict([(w4, _pick(arch, w4, (128, 256), (32, 256))), (w8, _pick(arch, w8, (128, 256), (32, 256))),
-                              ("fp16", _pick(arch, "fp16", (128, 256), (32, 256))), *wo_all.items(), ("w4a4_g128_sym", _pick(arch, "w4a4_g128_sym", (64, 256)))])
+                              ("fp16", _pick(arch, "fp16", (128, 256), (32, 256))), *wo_all.items(), ("w4a4_g128_sym", _pick(arch, "w4a4_g128_sym", (64, 256))),
+                              ("w8a16_g128_asym", _pick(arch, "w8a16_g128_asym", (16, 128), (128, 128)))])
     everything_b6 = OrderedDict(everything)
     everything_b6[w4] = _pick(arch, w4, (128, 256), (32, 256), bf6=True)
     return [

@@ -41,7 +41,8 @@ def pack_wxax_fragments(rows: torch.Tensor) -> torch.Tensor:
     (The reference's `pack_wxax` / `permute_weight`, quantize.cuh:318-381,424-475, play the same role for ldmatrix.)"""
     r = rows.contiguous().view(torch.uint8)
     n, kb = r.shape
-    assert kb % 64 == 0, "K must fill whole 64-byte slices"
+    if kb % 64:
+        raise ValueError(f"K must fill whole 64-byte slices of packed codes (128 int4 or 64 int8 values): a row of {kb} bytes does not")
     n32 = (n + 31) // 32
     if n32 * 32 != n:
         r = torch.cat([r, torch.zeros((n32 * 32 - n, kb), dtype=torch.uint8, device=r.device)])

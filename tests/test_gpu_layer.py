@@ -89,7 +89,8 @@ def test_mixed_layer_with_shared_expert_within_tolerance():
     from mxmoe_amd import synth
 
     cfg = synth.MoEConfig("t", "test", 4, 2, 256, 1408, 16, num_shared=2, rotate=0)
-    fm = [(synth.W4A16, synth.W3A16), (synth.W3A16, synth.W4A16), (synth.FP16, synth.FP16), (synth.W4A16, synth.W4A16), (synth.W4A16, synth.W3A16)]
+    w8a16, w4a16_pc = (16, 8, 128, False), (16, 4, -1, True)   # 8-bit weights; 4-bit weights with one scale per channel
+    fm = [(synth.W4A16, synth.W3A16), (w8a16, synth.W4A16), (synth.FP16, w8a16), (w4a16_pc, synth.W4A16), (synth.W4A16, synth.W3A16)]
     for r in _run(cfg, fm):
         assert _rel(r["g_mid"], r["mid"]) <= 1e-2, f"gate_up, expert {r['e']}"
         # the down input differs in the last fp16 bit from the oracle's, so compare the end result at the stated tolerance
