@@ -173,6 +173,7 @@ def default_kernel_specs(arch: str = "gfx950"):
                               ("w8a16_g128_asym", _pick(arch, "w8a16_g128_asym", (16, 128), (128, 128)))])
     everything_b6 = OrderedDict(everything)
     everything_b6[w4] = _pick(arch, w4, (128, 256), (32, 256), bf6=True)
+    everything_e4m3 = OrderedDict(("w8a8_g-1_sym_E4M3" if q == w8 else q, _pick(arch, "w8a8_g-1_sym_E4M3", (128, 256), (32, 256)) if q == w8 else t) for q, t in everything.items())
     return [
         ("groupgemm_hz_fused_wxax", KernelType.Fused, OrderedDict([(w4, _pick(arch, w4, (128, 256), (64, 256), (32, 256))), (w8, _pick(arch, w8, (128, 256), (64, 256), (32, 256)))])),
         ("groupgemm_hz_fused_fp16", KernelType.Fused, OrderedDict([("fp16", _pick(arch, "fp16", (128, 256), (64, 256), (32, 256)))])),
@@ -196,6 +197,7 @@ def default_kernel_specs(arch: str = "gfx950"):
                                                                          ("w8a8_g-1_sym_E4M3", _pick(arch, "w8a8_g-1_sym_E4M3", (128, 256), (64, 256), (32, 256)))])),
         ("groupgemm_hz_fused_wxax_b6", KernelType.Fused, OrderedDict([(w4, _pick(arch, w4, (128, 256), (64, 256), (32, 256), bf6=True)), (w8, _pick(arch, w8, (128, 256), (64, 256), (32, 256)))])),
         ("groupgemm_hz_fused_all_b6", KernelType.Fused, everything_b6),
+        ("groupgemm_hz_fused_all_e4m3", KernelType.Fused, everything_e4m3),
     ]
 
 

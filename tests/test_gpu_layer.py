@@ -459,6 +459,29 @@ def test_layer_with_w8a8_blocks_in_fp8():
         p += 1
 
 
+def test_fp8_blocks_next_to_every_other_format():
+    """fp8=True in a layer that also holds fp16, weight-only and group-quantised blocks (kernel groupgemm_hz_fused_all_e4m3): the three
+    forms of the forward agree bit for bit, and the result is within 1e-1 (of the largest output) of the same layer with int8 w8a8
+    blocks: e4m3 keeps 3 mantissa bits where int8 keeps up to 7, so the two formats of the same block differ by a few per cent."""
+    from mxmoe_amd import _lib, synth
+    from mxmoe_amd.layer import MxMoELayer
+
+    cfg = synth.MoEConfig("t", "test", 6, 3, 512, 1408, 70, num_shared=1, rotate=1)
+    fm = [(synth.W8A8, synth.W4A16), (synth.FP16, synth.W8A8), (synth.W4A4G128, synth.W8A8), ((16, 8, 128, False), synth.W4A4), (synth.W8A8, synth.W8A8),
+          (synth.W3A16, synth.W2A16), (synth.W8A8, synth.W8A8)]
+    weights = [synth.expert_weights(cfg, e) for e in range(7)]
+    layer = MxMoELayer(cfg, formats=fm, weights=weights, fp8=True)
+    lib = _lib.load()
+    assert lib.mxmoe_kernel_name(layer.kid_gate_up).decode().endswith("groupgemm_hz_fused_all_e4m3")
+    hidden = synth.make_hidden(cfg)
+    ids, w = synth.make_routing(cfg)
+    layer.forward(hidden, ids)
+    want = layer.combine(w).clone()
+    assert torch.equal(layer(hidden, ids, w), want) and torch.equal(layer.call_with_host_tables(hidden, ids, w), want)
+    ref = MxMoELayer(cfg, formats=fm, weights=weights)(hidden, ids, w)
+    assert _rel(want.float().cpu().numpy(), ref.float().cpu().numpy()) <= 1e-1
+
+
 def test_planned_forward_of_more_experts_than_one_launch_holds():
     """130 routed experts and a shared one: each block runs as two launches (experts 0 .. 119, then the rest), planned on the device
     chunk by chunk; the result equals the stepwise operators' (whose host launcher splits long problem lists the same way) and the
