@@ -21,7 +21,7 @@ PEAK = {"int8": 5000.0, "fp16": 2500.0, "fp6": 10100.0, "hbm": 8000.0}  # MI355X
 
 # HBM bytes per launch of the dominant (gate_up) kernel, from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE runs scaled by the
 # same counters on a plain 256 MiB copy (summaries: profiles/fused_group_gemm_<workload>.txt, profiles/counter_calibration_copy_256MiB.txt)
-TRAFFIC = {"c1": 729899884, "c2": 556661594, "c3": 684746679, "c4": 201769125, "c5": 5836590038}
+TRAFFIC = {"c1": 729899884, "c2": 556661594, "c3": 684746679, "c4": 201769125, "c5": 5813884599}
 
 
 def build_layer(name: str, tokens: int | None, bf6=False):
