@@ -61,6 +61,9 @@ int mxmoe_kernel_branch(int kernel_id, int branch, int32_t out[8]);
  *     multiple of 128, at least 256.  Results equal the integer kernels' bit for bit.
  *   w8a8_g-1_sym, variant 2 (fp8, the reference's w8a8_g-1_sym_E4M3, mm_tile.cuh:696-697): As[p], Bs[p] = OCP e4m3 codes in the int8
  *     layouts, scale = max|x| / 448.
+ *   fp16, variant 3 (bfloat16, the reference's bf16, tile_config.py:42): As[p], Bs[p] and Cs[p] hold bfloat16 numbers in the fp16
+ *     layouts; fp32 accumulation, one rounding (to nearest even) to bfloat16.  GroupGEMM entry points only: the layer forward's
+ *     activation step computes in fp16.
  *
  * (*) weights of the integer formats are stored in MFMA fragment order: uint8 [ceil(N/32)][KB/64][2][64 lanes][16], KB = bytes per
  *     row; lane l of block (nb, ks, step) holds bytes ks*64 + (2*step + (l >> 5))*16 .. +16 of channel nb*32 + (l & 31), channels past N

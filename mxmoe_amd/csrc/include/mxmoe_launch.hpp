@@ -255,7 +255,7 @@ struct BranchInfo {
   // never chosen automatically: the caller names it, because only the caller knows what its operands hold.
   int variant = 0;
 };
-constexpr int kVariantBf6 = 1, kVariantFp8 = 2;
+constexpr int kVariantBf6 = 1, kVariantFp8 = 2, kVariantBf16 = 3;
 
 template <class T>
 struct BranchOf;
@@ -264,7 +264,8 @@ struct BranchOf<MfmaTile<OP, BM, BN, WGM, WGN>> {
   static BranchInfo get() {
     using T = MfmaTile<OP, BM, BN, WGM, WGN>;
     const Fmt f = OP == Op::I8 ? Fmt::W8A8 : (OP == Op::I4 ? Fmt::W4A4 : Fmt::FP16);
-    return BranchInfo{f, BM, BN, T::BK, WGM, WGN, T::kLdsBytes, T::BK, 0};
+    // bfloat16 problems carry the QParams of fp16 ones (16 / 16 bits): which of the two a kernel computes is the kernel's variant
+    return BranchInfo{f, BM, BN, T::BK, WGM, WGN, T::kLdsBytes, T::BK, 0, 0, OP == Op::BF16 ? kVariantBf16 : 0};
   }
 };
 template <int BM>
@@ -573,7 +574,8 @@ int register_fused(const char* fn_name, Policy policy = Policy::Fused, int max_r
   std::string n;
   for (const auto& b : k.branches) {
     char buf[160];
-    snprintf(buf, sizeof buf, "[%s%s: (%d,%d,%d) (%d,%d,1) 2], ", fmt_name(b.fmt, b.fmt == Fmt::W8A8 || b.fmt == Fmt::W4A4), b.variant == kVariantFp8 ? "_E4M3" : "", b.BM, b.BN,
+    snprintf(buf, sizeof buf, "[%s%s: (%d,%d,%d) (%d,%d,1) 2], ", b.variant == kVariantBf16 ? "bf16" : fmt_name(b.fmt, b.fmt == Fmt::W8A8 || b.fmt == Fmt::W4A4),
+             b.variant == kVariantFp8 ? "_E4M3" : "", b.BM, b.BN,
              b.BK, b.WGM, b.WGN);
     n += buf;
     k.lds_bytes = std::max(k.lds_bytes, b.lds_bytes);

@@ -38,7 +38,7 @@ constexpr int kThreads = 256;  // workgroup size shared by every fused branch
 constexpr int kWaves = 4;
 constexpr int kRowBytes = 64;  // bytes of one operand row held in LDS per pipeline stage
 
-enum class Op { I8, I4, F16, F8 };  // F8: OCP e4m3 codes on the fp8 matrix instruction, fp32 accumulators
+enum class Op { I8, I4, F16, F8, BF16 };  // F8: OCP e4m3 codes on the fp8 matrix instruction, fp32 accumulators; BF16: bfloat16 operands and outputs
 
 // What one problem looks like to a tile.
 struct TileArgs {
@@ -164,6 +164,21 @@ struct OpTraits<Op::F8> {
   using Acc = v16f;
   static constexpr int kBitsPerElem = 8;
 };
+template <>
+struct OpTraits<Op::BF16> {
+  using Acc = v16f;
+  static constexpr int kBitsPerElem = 16;
+};
+// operands and outputs are floating-point numbers of 16 bits (no scales, fp32 accumulators written out after one rounding)
+template <Op OP>
+constexpr bool kFloat16Op = OP == Op::F16 || OP == Op::BF16;
+
+// fp32 -> bfloat16 bits, round to nearest even (NaN stays a quiet NaN)
+__device__ __forceinline__ unsigned short bf16_bits(float x) {
+  unsigned u = __float_as_uint(x);
+  u += 0x7FFFu + ((u >> 16) & 1u);
+  return x != x ? (unsigned short)0x7FC0 : (unsigned short)(u >> 16);
+}
 
 // A BM x BN output tile computed by WGM x WGN waves with 32x32 MFMA blocks.
 template <Op OP, int BM_, int BN_, int WGM_, int WGN_>
@@ -283,6 +298,9 @@ struct MfmaTile {
       } else if constexpr (OP == Op::I4) {
         c = __builtin_amdgcn_mfma_i32_32x32x32_i8(b[0], a[0], c, 0, 0, 0);
         c = __builtin_amdgcn_mfma_i32_32x32x32_i8(b[1], a[1], c, 0, 0, 0);
+      } else if constexpr (OP == Op::BF16) {
+        typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+        c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, b[0]), __builtin_bit_cast(v8bf, a[0]), c, 0, 0, 0);
       } else {
         c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, b[0]), __builtin_bit_cast(v8h, a[0]), c, 0, 0, 0);
       }
@@ -376,7 +394,7 @@ struct MfmaTile {
     // the slowest wave
     float s_a[FM];
     v4h s_b[FN][4];
-    if constexpr (OP != Op::F16) {
+    if constexpr (!kFloat16Op<OP>) {
 #pragma unroll
       for (int i = 0; i < FM; ++i) {
         const int m = min(m0 + wm * TM + i * 32 + lrow, M - 1);
@@ -403,7 +421,7 @@ struct MfmaTile {
             const int m = m0 + wm * TM + i * 32 + lrow, n = n0 + wn * TN + j * 32 + (r / 4) * 8 + nq + (r & 3);
             const auto v = acc[i][j][r];
             int a;
-            if constexpr (OP == Op::F16) a = __builtin_bit_cast(int, (float)v); else a = (int)v;
+            if constexpr (kFloat16Op<OP>) a = __builtin_bit_cast(int, (float)v); else a = (int)v;
             if constexpr (OP == Op::I4) a >>= 8;  // exact
             if (m < M && n < N) gstore<int>(t.acc_dump + (long)m * N + n, a);
           }
@@ -432,6 +450,9 @@ struct MfmaTile {
             if constexpr (OP == Op::F16) {
 #pragma unroll
               for (int e = 0; e < 4; ++e) o[e] = (_Float16)acc[i][j][q * 4 + e];
+            } else if constexpr (OP == Op::BF16) {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) o[e] = __builtin_bit_cast(_Float16, bf16_bits(acc[i][j][q * 4 + e]));
             } else {
 #pragma unroll
               for (int e = 0; e < 4; ++e) {

@@ -369,6 +369,8 @@ static int resolve_kernel(int kernel_id, const mxmoe_block_desc* h_desc, int et)
       // a kernel's w4a4 tiles take packed int4 rows or bf6 fragments, never both: the descriptor says which the block will get
       if (f == (int)Fmt::W4A4 && kernel_takes_bf6(k) != wants_bf6(h_desc[i].q)) return false;
       if (f == (int)Fmt::W8A8 && (kernel_variant(k, Fmt::W8A8) == kVariantFp8) != wants_fp8(h_desc[i].q)) return false;
+      // 16-bit float blocks of a layer are fp16 (the activation step between the launches computes in fp16): no bfloat16 kernel here
+      if (f == (int)Fmt::FP16 && kernel_variant(k, Fmt::FP16) != 0) return false;
     }
     return true;
   };

@@ -83,9 +83,11 @@ def bench_func(fn, warmup: int = 20, iters: int = 50, max_warm_s: float = 10.0) 
     return {"min": ts[0], "max": ts[-1], "mean": sum(trim) / len(trim), "median": ts[len(ts) // 2]}
 
 
-def make_problem(entry: dict, gen: torch.Generator, device="cuda", keep_ref: bool = False, bf6: bool = False, fp8: bool = False) -> dict:
+def make_problem(entry: dict, gen: torch.Generator, device="cuda", keep_ref: bool = False, bf6: bool = False, fp8: bool = False, bf16: bool = False) -> dict:
     """Random fp16 operands for one workload entry, quantised and packed for its format (QInput::from_fp16).  `bf6`: w4a4 operands as
-    bf6 fragments, the layout of the kernels whose w4a4 tiles run on the 6-bit float matrix path (`kernel_takes_bf6`)."""
+    bf6 fragments, the layout of the kernels whose w4a4 tiles run on the 6-bit float matrix path (`kernel_takes_bf6`).  `bf16`: the
+    16-bit float problems hold bfloat16 numbers (kernels whose dense tiles run the bf16 matrix instruction); their tensors keep the
+    fp16 dtype as a container of the bits (`.view(torch.bfloat16)` reads them)."""
     m, n, k = entry["shape"]
     qp = (entry["a_bits"], entry["w_bits"], entry["gsize"], bool(entry["sym"]))
     if gen is None:  # values drawn on the device (timing-only problems)
@@ -95,6 +97,13 @@ def make_problem(entry: dict, gen: torch.Generator, device="cuda", keep_ref: boo
         a = (torch.rand(m, k, generator=gen, dtype=torch.float32) * 2 - 1).to(torch.float16).to(device)
         b = (torch.rand(n, k, generator=gen, dtype=torch.float32) * 2 - 1).to(torch.float16).to(device)
     fp8 = fp8 and qp[:3] == (8, 8, -1)
+    if bf16 and qp[0] >= 16 and qp[1] >= 16:
+        a, b = a.to(torch.bfloat16), b.to(torch.bfloat16)
+        prob = {"size": (m, n, k), "q": qp, "A": a.view(torch.float16), "sa": None, "B": b.view(torch.float16), "sb": None,
+                "C": torch.zeros(m, n, dtype=torch.float16, device=device), "bf16": True}
+        if keep_ref:
+            prob["a16"], prob["b16"] = a, b
+        return prob
     pw = quantize_and_pack(b, qp, bf6=bf6, fp8=fp8)
     prob = {"size": (m, n, k), "q": qp, "B": pw.data, "sb": pw.scale, "C": torch.zeros(m, n, dtype=torch.float16, device=device)}
     if qp[0] < 16:
@@ -128,6 +137,13 @@ def kernel_takes_fp8(lib, kid: int) -> bool:
     from .ops import kernel_variants
 
     return kernel_variants(lib, kid).get(1) == 2
+
+
+def kernel_takes_bf16(lib, kid: int) -> bool:
+    """Whether kernel `kid` computes its 16-bit float problems in bfloat16."""
+    from .ops import kernel_variants
+
+    return kernel_variants(lib, kid).get(0) == 3
 
 
 def _launch_of(probs, lib, kernel_id=-1) -> GroupGemmLaunch:
@@ -195,11 +211,12 @@ def bench_one_case(entries, lib=None, mode: str = "bench", filters=(), out_file:
         if filters and not any(f in name for f in filters):
             continue
         mine = probs
-        want = (kernel_takes_bf6(lib, kid) and any(p["q"][:3] == (4, 4, -1) for p in probs), kernel_takes_fp8(lib, kid) and any(p["q"][:3] == (8, 8, -1) for p in probs))
+        want = (kernel_takes_bf6(lib, kid) and any(p["q"][:3] == (4, 4, -1) for p in probs), kernel_takes_fp8(lib, kid) and any(p["q"][:3] == (8, 8, -1) for p in probs),
+                kernel_takes_bf16(lib, kid) and any(p["q"][0] >= 16 and p["q"][1] >= 16 for p in probs))
         if any(want):
             if want not in variants:
                 gen.manual_seed(42)
-                variants[want] = [make_problem(e, gen, keep_ref=(mode == "check"), bf6=want[0], fp8=want[1]) for e in entries if e["shape"][0] > 0]
+                variants[want] = [make_problem(e, gen, keep_ref=(mode == "check"), bf6=want[0], fp8=want[1], bf16=want[2]) for e in entries if e["shape"][0] > 0]
             mine = variants[want]
         g = _launch_of(mine, lib, kid)
         try:
@@ -211,7 +228,8 @@ def bench_one_case(entries, lib=None, mode: str = "bench", filters=(), out_file:
             torch.cuda.synchronize()
             for p in mine:
                 ref = (p["a16"].float() @ p["b16"].float().T)
-                err = (p["C"].float() - ref).abs().max().item() if p["size"][0] else 0.0
+                got = p["C"].view(torch.bfloat16) if p.get("bf16") else p["C"]
+                err = (got.float() - ref).abs().max().item() if p["size"][0] else 0.0
                 tol = 1.0 if p["q"][1] >= 16 else float("inf")  # test_utils.h:71 — meaningful for fp16 only, as in the reference
                 print(f"{name}: problem {p['size']} {p['q']} max abs err vs fp16 reference {err:.4f}{' FAIL' if err > tol else ''}")
             continue

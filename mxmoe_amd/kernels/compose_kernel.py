@@ -43,7 +43,8 @@ def _gen_condition(qcfg: str) -> str:
     return f"(a_bits == {a} && w_bits == {w} && gsize == {g} && sym == {'true' if sym else 'false'})"
 
 
-BRANCH_CONDITION_MAP = {"fp16": "(a_bits == 16 && w_bits == 16)", **{k: _gen_condition(k) for k in SUPPORTED_QCFG if k != "fp16"}}
+BRANCH_CONDITION_MAP = {"fp16": "(a_bits == 16 && w_bits == 16)", "bf16": "(a_bits == 16 && w_bits == 16)",
+                        **{k: _gen_condition(k) for k in SUPPORTED_QCFG if k not in ("fp16", "bf16")}}
 
 GEN_DIR = Path(__file__).resolve().parent.parent / "csrc" / "generated"
 
@@ -198,6 +199,8 @@ def default_kernel_specs(arch: str = "gfx950"):
         ("groupgemm_hz_fused_wxax_b6", KernelType.Fused, OrderedDict([(w4, _pick(arch, w4, (128, 256), (64, 256), (32, 256), bf6=True)), (w8, _pick(arch, w8, (128, 256), (64, 256), (32, 256)))])),
         ("groupgemm_hz_fused_all_b6", KernelType.Fused, everything_b6),
         ("groupgemm_hz_fused_all_e4m3", KernelType.Fused, everything_e4m3),
+        # bfloat16 operands and outputs (the reference's "bf16"): the QParams of fp16 problems, so by name only
+        ("groupgemm_hz_fused_bf16", KernelType.Fused, OrderedDict([("bf16", _pick(arch, "bf16", (128, 256), (64, 256), (32, 256)))])),
     ]
 
 

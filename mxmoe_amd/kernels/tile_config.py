@@ -42,6 +42,7 @@ ACCFP16_ALIASES = {"fp16_accfp16": "fp16", **{f"{q}_accfp16": q for q in WEIGHT_
 
 SUPPORTED_QCFG = [
     "fp16",
+    "bf16",  # bfloat16 operands and outputs, fp32 accumulation (tile_config.py:42): the QParams of fp16, told apart by the kernel (a variant)
     "w8a8_g-1_sym",
     "w8a8_g-1_sym_E4M3",  # fp8 (OCP e4m3) codes on both sides, fp32 accumulation (tile_config.py:45)
     "w4a4_g-1_sym",
@@ -53,6 +54,7 @@ SUPPORTED_QCFG = [
 # (M, N, K) of one MFMA instruction
 MMA_SHAPE = {
     "MFMA_F32_32x32x16_F16": (32, 32, 16),
+    "MFMA_F32_32x32x16_BF16": (32, 32, 16),
     "MFMA_I32_32x32x32_I8": (32, 32, 32),
     "MFMA_I32_32x32x32_I8_FROM_I4": (32, 32, 32),  # int4 operands widened to int8 (16*v) in registers
     "MFMA_F32_16x16x32_F16": (16, 16, 32),
@@ -61,14 +63,15 @@ MMA_SHAPE = {
     "MFMA_F32_32x32x64_BF6_FROM_I4": (32, 32, 64),
     "MFMA_F32_32x32x16_FP8": (32, 32, 16),
 }
-MMA_TO_ACC_TYPE = {"MFMA_F32_32x32x16_F16": "float", "MFMA_I32_32x32x32_I8": "int32_t", "MFMA_I32_32x32x32_I8_FROM_I4": "int32_t", "MFMA_F32_16x16x32_F16": "float",
+MMA_TO_ACC_TYPE = {"MFMA_F32_32x32x16_F16": "float", "MFMA_F32_32x32x16_BF16": "float", "MFMA_I32_32x32x32_I8": "int32_t", "MFMA_I32_32x32x32_I8_FROM_I4": "int32_t", "MFMA_F32_16x16x32_F16": "float",
                    "MFMA_F32_32x32x64_BF6_FROM_I4": "float", "MFMA_F32_32x32x16_FP8": "float"}
-MMA_TO_INP_TYPE = {"MFMA_F32_32x32x16_F16": "half", "MFMA_I32_32x32x32_I8": "int8_t", "MFMA_I32_32x32x32_I8_FROM_I4": "int4_t", "MFMA_F32_16x16x32_F16": "half",
+MMA_TO_INP_TYPE = {"MFMA_F32_32x32x16_F16": "half", "MFMA_F32_32x32x16_BF16": "bfloat16", "MFMA_I32_32x32x32_I8": "int8_t", "MFMA_I32_32x32x32_I8_FROM_I4": "int4_t", "MFMA_F32_16x16x32_F16": "half",
                    "MFMA_F32_32x32x64_BF6_FROM_I4": "int4_t", "MFMA_F32_32x32x16_FP8": "fp8e4m3"}
 BF6_MMA = "MFMA_F32_32x32x64_BF6_FROM_I4"
 
 QCFG_TO_MMA = {
     "fp16": "MFMA_F32_32x32x16_F16",
+    "bf16": "MFMA_F32_32x32x16_BF16",
     "w8a8_g-1_sym": "MFMA_I32_32x32x32_I8",
     "w8a8_g-1_sym_E4M3": "MFMA_F32_32x32x16_FP8",
     "w4a4_g-1_sym": "MFMA_I32_32x32x32_I8_FROM_I4",
@@ -217,10 +220,10 @@ class TileConfig:
             return f"WoMfmaTile<{self.QCFGB.QBITS}, {self.BM}, {self.BN}>"
         if self.is_bf6():
             return f"Bf6Tile<{self.BM}>"
-        op = {"MFMA_F32_32x32x16_F16": "Op::F16", "MFMA_I32_32x32x32_I8": "Op::I8", "MFMA_I32_32x32x32_I8_FROM_I4": "Op::I4", "MFMA_F32_32x32x16_FP8": "Op::F8"}[self.MMA]
+        op = {"MFMA_F32_32x32x16_F16": "Op::F16", "MFMA_F32_32x32x16_BF16": "Op::BF16", "MFMA_I32_32x32x32_I8": "Op::I8", "MFMA_I32_32x32x32_I8_FROM_I4": "Op::I4", "MFMA_F32_32x32x16_FP8": "Op::F8"}[self.MMA]
         if self.is_group_wa():
             return f"WxAxGTile<{self.BM}>"
-        if op != "Op::F16":
+        if op not in ("Op::F16", "Op::BF16"):
             return f"WxAxTile<{op}, {self.BM}, {self.BN}>"
         return f"MfmaTile<{op}, {self.BM}, {self.BN}, {self.WM}, {self.WN}>"
 
@@ -235,18 +238,18 @@ class TileConfig:
             if (self.BN, self.BK, self.WM, self.WN, self.WK, self.STAGE) != (256, 64, 1, 4, 1, 4) or self.BM not in (32, 64, 128):
                 raise ValueError(f"{self!r}: bf6 tiles are BM x 256 x 64 with 1 x 4 waves and 4 stages, BM in 32 / 64 / 128")
             return
-        k_elems = {"MFMA_F32_32x32x16_F16": 32, "MFMA_I32_32x32x32_I8": 64, "MFMA_I32_32x32x32_I8_FROM_I4": 128, "MFMA_F32_32x32x16_FP8": 64}[self.MMA]
+        k_elems = {"MFMA_F32_32x32x16_F16": 32, "MFMA_F32_32x32x16_BF16": 32, "MFMA_I32_32x32x32_I8": 64, "MFMA_I32_32x32x32_I8_FROM_I4": 128, "MFMA_F32_32x32x16_FP8": 64}[self.MMA]
         if self.BK != k_elems or self.STAGE != 3 or self.WK != 1 or (self.BM // self.WM) % 32 or (self.BN // self.WN) % 32:
             raise ValueError(f"{self!r}: unsupported shape for {self.MMA} (BK must be {k_elems}, STAGE 3, wave tile a multiple of 32x32)")
         if self.is_group_wa() and self.BM not in (32, 64):
             raise ValueError(f"{self!r}: group-quantised int4 tiles are 32 x 256 or 64 x 256 (two sets of accumulators)")
-        if self.MMA != "MFMA_F32_32x32x16_F16" and ((self.WM, self.WN) != (1, 4) or self.BN != 256 or self.BM not in (32, 64, 128)):
+        if self.MMA not in ("MFMA_F32_32x32x16_F16", "MFMA_F32_32x32x16_BF16") and ((self.WM, self.WN) != (1, 4) or self.BN != 256 or self.BM not in (32, 64, 128)):
             raise ValueError(f"{self!r}: integer tiles are BM x 256 with 1 x 4 waves (each wave streams its own 64 weight channels), BM in 32 / 64 / 128")
 
 
 def get_info_from_qcfg_str(qcfg: str):
     """'w4a4_g-1_sym' -> (w_bits, a_bits, gsize, sym)   (tile_config.py:288-294)."""
-    if qcfg.startswith("fp16"):
+    if qcfg.startswith("fp16") or qcfg == "bf16":
         return 16, 16, -1, True
     s = qcfg.split("_")
     wbits = int(s[0].split("a")[0].split("w")[1])
@@ -261,6 +264,7 @@ def build_qcfgb_from_str(qcfg: str) -> QConfig:
 
 QCFG_MAP = {
     "fp16": TileConfig(),
+    "bf16": TileConfig(),
     "w8a8_g-1_sym": TileConfig(QCFGA=QCFG_W8A8, QCFGB=QCFG_W8A8),
     "w8a8_g-1_sym_E4M3": TileConfig(QCFGA=QCFG_W8A8_E4M3, QCFGB=QCFG_W8A8_E4M3),
     "w4a4_g-1_sym": TileConfig(QCFGA=QCFG_W4A4, QCFGB=QCFG_W4A4),
@@ -287,8 +291,8 @@ def get_possible_tile_list(arch: str, qcfg: str) -> list:
         shapes = ((128, 2, 2),) if QCFG_MAP[qcfg].QCFGB.QBITS == 8 else ((128, 2, 2), (256, 1, 4))
         big = [_with_q(TileConfig(BM=128, BN=bn, BK=128, WM=wm, WN=wn, WK=1, STAGE=2, MMA=mma), qcfg) for bn, wm, wn in shapes]
         return skinny + big
-    bk = {"MFMA_F32_32x32x16_F16": 32, "MFMA_I32_32x32x32_I8": 64, "MFMA_I32_32x32x32_I8_FROM_I4": 128, "MFMA_F32_32x32x16_FP8": 64}[mma]
-    if mma == "MFMA_F32_32x32x16_F16":
+    bk = {"MFMA_F32_32x32x16_F16": 32, "MFMA_F32_32x32x16_BF16": 32, "MFMA_I32_32x32x32_I8": 64, "MFMA_I32_32x32x32_I8_FROM_I4": 128, "MFMA_F32_32x32x16_FP8": 64}[mma]
+    if mma in ("MFMA_F32_32x32x16_F16", "MFMA_F32_32x32x16_BF16"):
         shapes = [(128, 256, 2, 2), (64, 256, 1, 4), (32, 256, 1, 4), (128, 128, 2, 2), (256, 128, 2, 2)]
     elif qcfg == "w4a4_g128_sym":
         shapes = [(64, 256, 1, 4), (32, 256, 1, 4)]

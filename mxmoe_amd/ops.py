@@ -49,7 +49,7 @@ def packed_elems(tag: int, rows: int, width: int) -> int:
 
 
 def kernel_variants(lib, kid: int) -> dict:
-    """{format id: operand variant} of kernel `kid`'s branches that take a variant (1 bf6 fragments, 2 fp8 e4m3 codes)."""
+    """{format id: operand variant} of kernel `kid`'s branches that take a variant (1 bf6 fragments, 2 fp8 e4m3 codes, 3 bfloat16)."""
     import ctypes as C
 
     out, res = (C.c_int32 * 8)(), {}
@@ -60,10 +60,11 @@ def kernel_variants(lib, kid: int) -> dict:
     return res
 
 
-def select_kernel(qparams, bf6: bool = False, fp8: bool = False, lib=None) -> int:
+def select_kernel(qparams, bf6: bool = False, fp8: bool = False, lib=None, bf16: bool = False) -> int:
     """Registry index of the first fused kernel with a tile for every format in `qparams` whose operand variants are exactly the ones
-    asked for: w4a4 operands as bf6 fragments (`bf6`), w8a8 operands as fp8 e4m3 codes (`fp8`).  -1 (the launcher's own choice) when
-    none is asked for; kernels with variants are never chosen automatically, since the launcher cannot see what the operands hold."""
+    asked for: w4a4 operands as bf6 fragments (`bf6`), w8a8 operands as fp8 e4m3 codes (`fp8`), 16-bit float problems in bfloat16
+    (`bf16`).  -1 (the launcher's own choice) when none is asked for; kernels with variants are never chosen automatically, since the
+    launcher cannot see what the operands hold."""
     lib = lib or _lib.load()
     qs = sorted({tuple(int(v) for v in q) for q in qparams})
     want = {}
@@ -71,11 +72,13 @@ def select_kernel(qparams, bf6: bool = False, fp8: bool = False, lib=None) -> in
         want[2] = 1
     if fp8 and (8, 8, -1, 1) in qs:
         want[1] = 2
+    if bf16 and any(q[0] >= 16 and q[1] >= 16 for q in qs):
+        want[0] = 3
     if not want:
         return -1
     sizes = (_lib.Dim3 * len(qs))(*[_lib.Dim3(1, 256, 256) for _ in qs])
     hq = (_lib.QParams * len(qs))(*[_lib.QParams(a, w, g, 1 if s else 0) for (a, w, g, s) in qs])
-    fmt_ids = {(4, 4, -1): 2, (8, 8, -1): 1}
+    fmt_ids = {(4, 4, -1): 2, (8, 8, -1): 1, (16, 16, -1): 0}
     mine = {fmt_ids[q[:3]] for q in qs if q[:3] in fmt_ids}
     for kid in range(lib.mxmoe_num_kernels()):
         if lib.mxmoe_kernel_policy(kid) != 0:

@@ -43,6 +43,8 @@ product apart.
   library cast (torch.float8_e4m3fn), absmax -> +-448; the fp8 format of the reference's w8a8_g-1_sym_E4M3 tiles
   has no quantiser in the reference (only the matrix instruction, mm_tile.cuh:696-697), so its scale rule
   (max / 448) is this build's definition: parity unpinned beyond "per-row scale, e4m3 codes, fp32 sums".
+* ``bf16_round`` / ``bf16_bits`` / ``gemm_bf16`` — hand-computed ties (to even) on both sides of a binade, every float32 of a
+  random sample against an independent library cast (torch.bfloat16), round trip through the bits.
 * ``dense_grid`` / the exact dense stage of ``online_hadamard`` — python-int sums in shuffled
   orders give the same bits; grid edges (zero rows, subnormal and largest fp16 values).
 * ``fma_f32`` — one correct rounding against exact rational arithmetic.
@@ -182,6 +184,32 @@ def gemm_fakequant(xq: np.ndarray, wq: np.ndarray) -> np.ndarray:
 def gemm_fp16(x: np.ndarray, w: np.ndarray) -> np.ndarray:
     """fp16 x fp16 -> fp32 accumulate -> fp16 (cta_gemm.cuh:8-107); float64 here, compared at 1e-2."""
     return gemm_fakequant(x, w)
+
+
+def bf16_round(x: np.ndarray) -> np.ndarray:
+    """float32 -> nearest bfloat16 (ties to even), returned as float32 values: the type of the reference's ``bf16`` tiles
+    (tile_config.py:42, MMA_BF16_FP32: bf16 operands, fp32 accumulators, bf16 outputs).  numpy has no bfloat16, so the rounding is done
+    on the bit pattern: add half of the dropped 16 bits' unit, plus the kept part's lowest bit minus one for the tie."""
+    u = np.ascontiguousarray(x, dtype=F32).view(np.uint32).astype(np.uint64)
+    r = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16) << 16
+    out = (r & 0xFFFFFFFF).astype(np.uint32).view(F32)
+    return np.where(np.isnan(x), F32(np.nan), out).astype(F32)
+
+
+def bf16_bits(x: np.ndarray) -> np.ndarray:
+    """The 16-bit storage of ``bf16_round(x)`` (upper half of the float32 pattern)."""
+    return (bf16_round(x).view(np.uint32) >> 16).astype(np.uint16)
+
+
+def bf16_from_bits(b: np.ndarray) -> np.ndarray:
+    return (np.ascontiguousarray(b, dtype=np.uint16).astype(np.uint32) << 16).view(F32)
+
+
+def gemm_bf16(x: np.ndarray, w: np.ndarray) -> np.ndarray:
+    """bf16 x bf16 -> fp32 accumulate -> bf16 (cta_gemm.cuh:8-107 with the bf16 matrix instruction): ``x``, ``w`` hold bf16 values as
+    float32; float64 sum, rounded to float32 and then to bf16 (compared at 1e-2, like the fp16 GEMM: the hardware's order of additions
+    is its own)."""
+    return bf16_round((x.astype(np.float64) @ w.astype(np.float64).T).astype(F32))
 
 
 # --------------------------------------------------------------------------------------------

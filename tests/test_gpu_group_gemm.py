@@ -244,6 +244,51 @@ def test_fp16_group_gemm():
         assert _rel(out, p["ref"]) <= 2e-3                                 # fp32 accumulation: far inside the tolerance
 
 
+def test_bf16_group_gemm():
+    """The reference's `bf16` format (tile_config.py:42): bfloat16 operands and outputs on v_mfma_f32_32x32x16_bf16, kernel
+    groupgemm_hz_fused_bf16 (chosen by name: its problems carry the QParams of fp16 ones).  Ragged problems within 1e-2 of the oracle,
+    and small-integer operands, whose sums are exact whatever the order, bit for bit, ties of the output rounding included."""
+    from mxmoe_amd import _lib, ops
+    from mxmoe_amd.group_gemm import GroupGemmLaunch
+
+    lib = _lib.load()
+    kid = ops.select_kernel([(16, 16, -1, True)], bf16=True)
+    assert lib.mxmoe_kernel_name(kid).decode().endswith("groupgemm_hz_fused_bf16") and ops.kernel_variants(lib, kid) == {0: 3}
+    rng = np.random.default_rng(21)
+    sizes = [(200, 264, 96), (1, 8, 32), (0, 64, 64), (33, 512, 1408), (129, 40, 2048)]
+    As, Bs, Cs, refs = [], [], [], []
+    for (m, n, k) in sizes:
+        a = O.bf16_round(rng.standard_normal((m, k)).astype(np.float32))
+        b = O.bf16_round((rng.standard_normal((n, k)) * 0.05).astype(np.float32))
+        As.append(torch.from_numpy(O.bf16_bits(a).view(np.int16)).view(torch.float16).to(DEV))
+        Bs.append(torch.from_numpy(O.bf16_bits(b).view(np.int16)).view(torch.float16).to(DEV))
+        Cs.append(torch.full((m, n), float("nan"), dtype=torch.float16, device=DEV))
+        refs.append(O.gemm_bf16(a, b))
+    # exact case: integers up to 16 against 0 / 1 weights, and rows whose sums are the ties 257 -> 256 and 259 -> 260
+    m, n, k = 64, 32, 64
+    a = rng.integers(-16, 17, (m, k)).astype(np.float32)
+    b = rng.integers(0, 2, (n, k)).astype(np.float32)
+    a[0, :] = 0; a[0, 0], a[0, 1] = 256, 1
+    a[1, :] = 0; a[1, 0], a[1, 1] = 258, 1
+    b[:, 0] = b[:, 1] = 1
+    As.append(torch.from_numpy(O.bf16_bits(a).view(np.int16)).view(torch.float16).to(DEV))
+    Bs.append(torch.from_numpy(O.bf16_bits(b).view(np.int16)).view(torch.float16).to(DEV))
+    Cs.append(torch.zeros((m, n), dtype=torch.float16, device=DEV))
+    sizes.append((m, n, k))
+    exact = O.bf16_round((a.astype(np.float64) @ b.astype(np.float64).T).astype(np.float32))
+    assert exact[0, 0] == 256.0 and exact[1, 0] == 260.0
+    g = GroupGemmLaunch(As, Bs, None, None, Cs, sizes, [(16, 16, -1, True)] * len(sizes), kernel_id=kid, lib=lib)
+    g.run()
+    torch.cuda.synchronize()
+    for c, ref, sz in zip(Cs[:-1], refs, sizes):
+        if sz[0] == 0:
+            continue
+        got = c.view(torch.bfloat16).float().cpu().numpy()
+        assert np.isfinite(got).all() and _rel(got, ref) <= 1e-2, sz
+    got = O.bf16_from_bits(Cs[-1].cpu().numpy().view(np.uint16))
+    assert np.array_equal(got.view(np.uint32), exact.view(np.uint32))
+
+
 def test_weight_only_skinny():
     from mxmoe_amd.weights import quantize_and_pack
 

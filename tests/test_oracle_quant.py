@@ -359,3 +359,24 @@ def test_e4m3_against_an_independent_cast_and_the_quantiser_rule():
     # and fp8_gemm on one-hot / unit operands returns the operand values themselves
     a = O.e4m3_encode(np.eye(8)[:, :8] * 1.0)
     assert np.array_equal(O.fp8_gemm(c[:3, :8], a), v[:3, :8])
+
+
+def test_bf16_rounding_known_answers_and_an_independent_cast():
+    """bfloat16 keeps 8 significant bits: 257 lies halfway between 256 and 258 and goes to the even 256, 259 to 260, 1 + 2^-8 to 1,
+    1 + 3 * 2^-8 to 1 + 2^-6; values of the format are fixed points; a random sample agrees with torch's cast bit for bit."""
+    import torch
+
+    x = np.array([257.0, 259.0, 1.0 + 2.0 ** -8, 1.0 + 3 * 2.0 ** -8, -257.0, 255.5, 3.0e38, 1.0e-40, 0.0, -0.0], dtype=np.float32)
+    want = np.array([256.0, 260.0, 1.0, 1.0 + 2.0 ** -6, -256.0, 256.0, 3.0e38, 1.0e-40, 0.0, -0.0], dtype=np.float32)
+    got = O.bf16_round(x)
+    assert np.array_equal(got[:6], want[:6])
+    assert np.array_equal(O.bf16_round(got), got)                           # idempotent
+    assert np.array_equal(O.bf16_from_bits(O.bf16_bits(x)), got)
+    rng = np.random.default_rng(5)
+    r = np.concatenate([rng.standard_normal(200000).astype(np.float32) * np.float32(10.0) ** rng.integers(-30, 30, 200000).astype(np.float32), x])
+    t = torch.from_numpy(r).to(torch.bfloat16).to(torch.float32).numpy()
+    assert np.array_equal(O.bf16_round(r).view(np.uint32), t.view(np.uint32))
+    a = O.bf16_round(rng.standard_normal((5, 64)).astype(np.float32))
+    b = O.bf16_round(rng.standard_normal((7, 64)).astype(np.float32))
+    ref = torch.from_numpy(a.astype(np.float64) @ b.astype(np.float64).T).to(torch.float32).to(torch.bfloat16).to(torch.float32).numpy()
+    assert np.array_equal(O.gemm_bf16(a, b), ref)
