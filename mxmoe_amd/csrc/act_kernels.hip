@@ -1399,7 +1399,8 @@ constexpr int kWideLds = 2 * 32 * kWidePitch + 64;                   // snapped 
 template <bool SILU, bool EXT>
 __global__ void __launch_bounds__(512) row_quant_wide_kernel(const RowArgs a) {
   extern __shared__ __align__(16) uint8_t wlds[];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // in a scalar register: "is k row wave + 8 i live" is then a scalar branch
   const int lm = lane & 15, lg = lane >> 4;
   uint8_t* xt = wlds;                                   // [32 k rows][kWidePitch]: the snapped row
   uint8_t* yrow = xt + 32 * kWidePitch;                 // [32 rows][kWidePitch]: the rotated row
@@ -1437,34 +1438,38 @@ __global__ void __launch_bounds__(512) row_quant_wide_kernel(const RowArgs a) {
     } else {
       srow = (shared_row ? src_shared : a.src) + (shared_row ? (long)(row - a.R) : (long)a.perm[row]) * n;
     }
+    // A k row past kb (the last of a wave's four when kb is not a multiple of 8: waves 4 .. 7 of a 28-row view) costs nothing: the
+    // whole wave skips its loads, its SiLU and its butterflies, and the slot holds zeros.
     float v[MAXC][8];
 #pragma unroll
     for (int i = 0; i < MAXC; ++i) {
       const int kr = wave + 8 * i;
-      const bool live = kr < kb;
-      const int c = min(kr, kb - 1) * 64 + lane;  // chunk index in the row
-      const v8h g = *reinterpret_cast<const v8h*>(srow + c * 8);
-      if (SILU) {
-        const v8h u = *reinterpret_cast<const v8h*>(srow + n + c * 8);
+      if (kr < kb) {
+        const int c = kr * 64 + lane;  // chunk index in the row
+        const v8h g = *reinterpret_cast<const v8h*>(srow + c * 8);
+        if (SILU) {
+          const v8h u = *reinterpret_cast<const v8h*>(srow + n + c * 8);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const float gf = (float)g[j];
-          const float sl = silu_fixed(gf);
-          v[i][j] = round_h(keep_f32(sl * (float)u[j]));
+          for (int j = 0; j < 8; ++j) {
+            const float gf = (float)g[j];
+            const float sl = silu_fixed(gf);
+            v[i][j] = round_h(keep_f32(sl * (float)u[j]));
+          }
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) v[i][j] = (float)g[j];
         }
       } else {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) v[i][j] = (float)g[j];
-      }
-      if (!live) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) v[i][j] = 0.0f;
       }
     }
     if (rot) {
       // H_512 along each k row: strides 1, 2, 4 inside the chunk, 8 .. 256 across the lanes (ascending)
+      float mx = 0.0f;
 #pragma unroll
-      for (int i = 0; i < MAXC; ++i)
+      for (int i = 0; i < MAXC; ++i) {
+        if (wave + 8 * i >= kb) continue;
 #pragma unroll
         for (int h = 1; h < 8; h <<= 1)
 #pragma unroll
@@ -1474,28 +1479,24 @@ __global__ void __launch_bounds__(512) row_quant_wide_kernel(const RowArgs a) {
               v[i][j] = p + q;
               v[i][j + h] = p - q;
             }
-      auto lane_stage = [&](auto mc) {
-        constexpr int m = decltype(mc)::value;
-        const float sgn = (lane & m) ? -1.0f : 1.0f;
-#pragma unroll
-        for (int i = 0; i < MAXC; ++i)
+        auto lane_stage = [&](auto mc) {
+          constexpr int m = decltype(mc)::value;
+          const float sgn = (lane & m) ? -1.0f : 1.0f;
 #pragma unroll
           for (int j = 0; j < 8; ++j) v[i][j] = __builtin_fmaf(sgn, v[i][j], lane_xor<m>(v[i][j]));
-      };
-      lane_stage(std::integral_constant<int, 1>{});
-      lane_stage(std::integral_constant<int, 2>{});
-      lane_stage(std::integral_constant<int, 4>{});
-      lane_stage(std::integral_constant<int, 8>{});
-      lane_stage(std::integral_constant<int, 16>{});
-      lane_stage(std::integral_constant<int, 32>{});
-      float mx = 0.0f;
-#pragma unroll
-      for (int i = 0; i < MAXC; ++i)
+        };
+        lane_stage(std::integral_constant<int, 1>{});
+        lane_stage(std::integral_constant<int, 2>{});
+        lane_stage(std::integral_constant<int, 4>{});
+        lane_stage(std::integral_constant<int, 8>{});
+        lane_stage(std::integral_constant<int, 16>{});
+        lane_stage(std::integral_constant<int, 32>{});
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           v[i][j] = round_h(keep_f32(v[i][j] * pl.scale));
           mx = fmaxf(mx, fabsf(v[i][j]));
         }
+      }
 #pragma unroll
       for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
       if (lane == 0) red[wave] = mx;
@@ -1539,9 +1540,10 @@ __global__ void __launch_bounds__(512) row_quant_wide_kernel(const RowArgs a) {
 #pragma unroll
       for (int i = 0; i < MAXC; ++i) {
         const int kr = wave + 8 * i;
-        const v8h y = *reinterpret_cast<const v8h*>(yrow + min(kr, kb - 1) * kWidePitch + lane * 16);
+        if (kr >= kb) continue;  // (still zeros)
+        const v8h y = *reinterpret_cast<const v8h*>(yrow + kr * kWidePitch + lane * 16);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) v[i][j] = kr < kb ? (float)y[j] : 0.0f;
+        for (int j = 0; j < 8; ++j) v[i][j] = (float)y[j];
       }
     }
 
@@ -1566,6 +1568,7 @@ __global__ void __launch_bounds__(512) row_quant_wide_kernel(const RowArgs a) {
 #pragma unroll
       for (int i = 0; i < MAXC; ++i) {
         const int kr = wave + 8 * i;
+        if (kr >= kb) continue;
         const int c = kr * 64 + lane;
         float gmax = 0.0f;
 #pragma unroll
@@ -1575,16 +1578,14 @@ __global__ void __launch_bounds__(512) row_quant_wide_kernel(const RowArgs a) {
         float scale = round_h(gmax / 7.0f);
         if (scale == 0.0f) scale = 1.0f;
         const ScaleDiv div(scale);
-        if (kr < kb) {
-          if ((c & 15) == 0) sout[c >> 4] = (_Float16)scale;
-          unsigned w = 0;
+        if ((c & 15) == 0) sout[c >> 4] = (_Float16)scale;
+        unsigned w = 0;
 #pragma unroll
-          for (int j = 0; j < 8; ++j) {
-            const float r = round_h(div(v[i][j]));
-            w = push_code<4>(w, code_word(fminf(fmaxf(r, -7.0f), 7.0f)));
-          }
-          *reinterpret_cast<unsigned*>(out + c * 4) = w;
+        for (int j = 0; j < 8; ++j) {
+          const float r = round_h(div(v[i][j]));
+          w = push_code<4>(w, code_word(fminf(fmaxf(r, -7.0f), 7.0f)));
         }
+        *reinterpret_cast<unsigned*>(out + c * 4) = w;
       }
       continue;
     }
