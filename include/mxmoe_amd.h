@@ -114,6 +114,17 @@ int mxmoe_group_gemm_plan_tables(int kernel_id, const mxmoe_dim3* h_sizes, const
  * kernels call to find their tile is the one evaluated here. */
 int mxmoe_group_gemm_plan_tile_map(int kernel_id, const mxmoe_dim3* h_sizes, const mxmoe_qparams* h_q, int problem_count, int grid, int32_t* tile_of_wg);
 
+/* ---- routing: what the models' gates compute between the router's logits and this layer (mxmoe/quant/moe_tracer.py:79-86:
+ *      F.softmax(router_logits, dim=1, dtype=float) -> torch.topk -> optional division by the sum of the k weights) ----
+ *
+ * router_logits [num_tokens, num_experts] (device) as fp16 (logits_dtype 0), fp32 (1) or bf16 (2).  Writes topk_ids [num_tokens, topk]
+ * int32 and topk_weights [num_tokens, topk] fp32 in order of decreasing probability; equal probabilities go to the lower expert id
+ * first (torch.topk leaves that order open).  probability = exp(x - max) / sum in fp32; renormalise != 0 divides the k weights by
+ * their sum (Mixtral; Qwen-MoE and DeepSeek-V2-Lite keep the plain probabilities).  1 <= topk <= min(num_experts, 64),
+ * num_experts <= 4096, error 3 otherwise; num_tokens = 0 is a no-op. */
+int mxmoe_route_topk(const void* router_logits, int logits_dtype, int num_tokens, int num_experts, int topk, int renormalise, int32_t* topk_ids,
+                     float* topk_weights, void* stream);
+
 /* ---- token permutation: replaces gg_permute_inp and the sort / bincount prologue of quant_inp_act
  *      (mxmoe/kernels/src/ref_bind.cu:47-64, 449-453) ----
  *

@@ -41,6 +41,7 @@ SIGNATURES = {
     "mxmoe_group_gemm": (_I, [_I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, C.POINTER(Dim3), _P, C.POINTER(QParams), _I, _P, _P]),
     "mxmoe_permute_workspace_bytes": (C.c_size_t, [_I, _I]),
     "mxmoe_build_permutation": (_I, [_P, _I, _I, _I, _P, _P, _P, _P, _P, _P]),
+    "mxmoe_route_topk": (_I, [_P, _I, _I, _I, _I, _I, _P, _P, _P]),
     "mxmoe_build_permutation_inv": (_I, [_P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P]),
     "mxmoe_combine_planned": (_I, [_P, _P, _I, _P, _P, _I, _I, _I, _P, _P]),
     "mxmoe_static_scratch_bytes": (C.c_size_t, []),

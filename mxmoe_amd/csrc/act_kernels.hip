@@ -110,6 +110,86 @@ __global__ void __launch_bounds__(64) perm_small_kernel(const int32_t* __restric
 }
 
 // ------------------------------------------------------------------------------------------------------------
+// Routing: router logits -> (top-k expert ids, top-k weights)
+// ------------------------------------------------------------------------------------------------------------
+// What the models' gates compute in front of the layer (mxmoe/quant/moe_tracer.py:79-86: softmax over the experts in fp32, top-k of
+// the probabilities, optionally divided by their sum).  One wave per token, four tokens per workgroup; a token's probabilities sit in
+// the wave's slice of LDS (entry e belongs to lane e mod 64: no lane reads what another wrote), and every one of the k rounds takes
+// the largest remaining (probability, lowest index first) by a wave-wide maximum of a 64-bit key.
+struct RouteArgs {
+  const void* logits;  // [T][E]
+  int dtype;           // 0 fp16, 1 fp32, 2 bf16
+  int T, E, topk, renorm;
+  int32_t* ids;        // [T][topk]
+  float* weights;      // [T][topk]
+};
+
+__device__ __forceinline__ float route_logit(const RouteArgs& a, long i) {
+  if (a.dtype == 1) return reinterpret_cast<const float*>(a.logits)[i];
+  if (a.dtype == 0) return (float)reinterpret_cast<const _Float16*>(a.logits)[i];
+  return __uint_as_float((unsigned)reinterpret_cast<const uint16_t*>(a.logits)[i] << 16);
+}
+
+__global__ void __launch_bounds__(256) route_topk_kernel(const RouteArgs a) {
+  extern __shared__ float route_lds[];  // [4][E]
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int t = blockIdx.x * 4 + wave;
+  if (t >= a.T) return;  // (no workgroup barrier below)
+  float* p = route_lds + wave * a.E;
+  const long base = (long)t * a.E;
+  float mx = -INFINITY;
+  for (int e = lane; e < a.E; e += 64) {
+    const float x = route_logit(a, base + e);
+    p[e] = x;
+    mx = fmaxf(mx, x);
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+  float sum = 0.0f;
+  for (int e = lane; e < a.E; e += 64) {
+    const float v = expf(p[e] - mx);
+    p[e] = v;
+    sum += v;
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
+  for (int e = lane; e < a.E; e += 64) p[e] = p[e] / sum;
+  int my_id = 0;
+  float my_w = 0.0f, wsum = 0.0f;
+  for (int r = 0; r < a.topk; ++r) {
+    // key = (probability bits, ~index): probabilities are not negative, so their bit patterns order like the values (a NaN sorts
+    // above every number); a taken entry holds -1 and gets the key 0, which loses against every live entry
+    unsigned long long key = 0;
+    for (int e = lane; e < a.E; e += 64) {
+      const float v = p[e];
+      const unsigned long long k = v == -1.0f ? 0ull : ((unsigned long long)(__float_as_uint(v) & 0x7FFFFFFFu) << 32) | (0xFFFFFFFFu - (unsigned)e);
+      key = k > key ? k : key;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const unsigned lo = __shfl_xor((unsigned)key, o), hi = __shfl_xor((unsigned)(key >> 32), o);
+      const unsigned long long other = ((unsigned long long)hi << 32) | lo;
+      key = other > key ? other : key;
+    }
+    const int idx = (int)(0xFFFFFFFFu - (unsigned)key);
+    const float val = p[idx];  // (read before the owner's write below: the same value for every lane)
+    __builtin_amdgcn_wave_barrier();
+    if ((idx & 63) == lane) p[idx] = -1.0f;
+    __builtin_amdgcn_wave_barrier();
+    wsum += val;
+    if (lane == r) {
+      my_id = idx;
+      my_w = val;
+    }
+  }
+  if (lane < a.topk) {
+    a.ids[(long)t * a.topk + lane] = my_id;
+    a.weights[(long)t * a.topk + lane] = a.renorm ? my_w / wsum : my_w;
+  }
+}
+
+// ------------------------------------------------------------------------------------------------------------
 // Row kernels
 // ------------------------------------------------------------------------------------------------------------
 struct RotPlan {
@@ -1878,6 +1958,35 @@ static int check_permutation_args(const int32_t* topk_ids, int num_tokens, int t
   if (!topk_ids || !dst_exp_sorted || !perm_indices || !src_slot || !recv_tokens_per_exp) {
     last_error() = "null pointer";
     return 5;
+  }
+  return 0;
+}
+
+int mxmoe_route_topk(const void* router_logits, int logits_dtype, int num_tokens, int num_experts, int topk, int renormalise, int32_t* topk_ids,
+                     float* topk_weights, void* stream) {
+  if (num_tokens < 0 || num_experts <= 0 || num_experts > 4096 || topk <= 0 || topk > num_experts || topk > 64 || logits_dtype < 0 || logits_dtype > 2) {
+    last_error() = "routing takes 1..4096 experts, top-k of at most min(experts, 64), logits as fp16 (0), fp32 (1) or bf16 (2)";
+    return 3;
+  }
+  if (num_tokens == 0) return 0;
+  if (!router_logits || !topk_ids || !topk_weights) {
+    last_error() = "null pointer";
+    return 5;
+  }
+  RouteArgs a;
+  a.logits = router_logits;
+  a.dtype = logits_dtype;
+  a.T = num_tokens;
+  a.E = num_experts;
+  a.topk = topk;
+  a.renorm = renormalise != 0;
+  a.ids = topk_ids;
+  a.weights = topk_weights;
+  hipLaunchKernelGGL(route_topk_kernel, dim3((num_tokens + 3) / 4), dim3(256), (size_t)4 * num_experts * sizeof(float), (hipStream_t)stream, a);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    last_error() = std::string("kernel launch failed: ") + hipGetErrorString(e);
+    return 4;
   }
   return 0;
 }

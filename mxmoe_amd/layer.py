@@ -259,12 +259,28 @@ class MxMoELayer:
                                      final.data_ptr(), stream))
         return final
 
-    def capture(self, tokens: int, topk: int | None = None) -> "CapturedForward":
+    def forward_from_logits(self, hidden: torch.Tensor, router_logits: torch.Tensor, topk: int | None = None, renormalise: bool = False,
+                            out: torch.Tensor | None = None) -> torch.Tensor:
+        """`(hidden [T, K] fp16, router_logits [T, E] fp16 / fp32 / bf16) -> [T, K] fp16`: the routing kernel (softmax, top-k, optional
+        renormalisation: `mxmoe_route_topk`) in front of `__call__`.  The ids and weights land in buffers the layer keeps per shape,
+        so this too enqueues kernels only and can be captured."""
+        t = hidden.shape[0]
+        topk = self.cfg.topk if topk is None else topk
+        assert router_logits.shape == (t, self.cfg.num_experts)
+        ps = self._planned_setup(t, topk)
+        if "route_ids" not in ps:
+            ps["route_ids"] = torch.empty((t, topk), dtype=torch.int32, device=self.device)
+            ps["route_w"] = torch.empty((t, topk), dtype=torch.float32, device=self.device)
+        ops.route_topk(router_logits.to(self.device), topk, renormalise, out_ids=ps["route_ids"], out_weights=ps["route_w"])
+        return self(hidden, ps["route_ids"], ps["route_w"], out=out)
+
+    def capture(self, tokens: int, topk: int | None = None, logits_dtype: torch.dtype | None = None, renormalise: bool = False) -> "CapturedForward":
         """The planned forward for a fixed (tokens, top-k) shape, captured into a HIP graph: write the inputs into the returned
         object's `hidden`, `topk_ids`, `topk_weights` tensors, call `replay()`, read `out`.  Nothing in the forward depends on the
         routing at enqueue time, so one capture serves every routing; a replay has no per-kernel launch gaps (decode-sized batches
-        gain most: 0.105 against 0.12 ms for DeepSeek-V2-Lite at 32 tokens)."""
-        return CapturedForward(self, tokens, self.cfg.topk if topk is None else topk)
+        gain most: 0.105 against 0.12 ms for DeepSeek-V2-Lite at 32 tokens).  With `logits_dtype` the graph starts at the router's
+        logits instead (`forward_from_logits`): the input is then `router_logits` [tokens, experts] of that dtype."""
+        return CapturedForward(self, tokens, self.cfg.topk if topk is None else topk, logits_dtype, renormalise)
 
     def call_with_host_tables(self, hidden: torch.Tensor, topk_ids: torch.Tensor, topk_weights: torch.Tensor) -> torch.Tensor:
         """The whole MoE MLP with the tables of both launches built on the HOST (what the reference's operators do), `(hidden [T, K] fp16, topk_ids [T, k] int32, topk_weights [T, k] fp32) -> [T, K] fp16`: what a serving
@@ -369,20 +385,25 @@ class MxMoELayer:
 class CapturedForward:
     """`MxMoELayer.__call__` for one shape as a HIP graph over static input and output tensors."""
 
-    def __init__(self, layer: MxMoELayer, tokens: int, topk: int):
+    def __init__(self, layer: MxMoELayer, tokens: int, topk: int, logits_dtype: torch.dtype | None = None, renormalise: bool = False):
         dev = layer.device
         self.hidden = torch.zeros((tokens, layer.cfg.hidden), dtype=torch.float16, device=dev)
-        self.topk_ids = torch.zeros((tokens, topk), dtype=torch.int32, device=dev)
-        self.topk_weights = torch.zeros((tokens, topk), dtype=torch.float32, device=dev)
         self.out = torch.empty((tokens, layer.cfg.hidden), dtype=torch.float16, device=dev)
+        if logits_dtype is None:
+            self.topk_ids = torch.zeros((tokens, topk), dtype=torch.int32, device=dev)
+            self.topk_weights = torch.zeros((tokens, topk), dtype=torch.float32, device=dev)
+            run = lambda: layer(self.hidden, self.topk_ids, self.topk_weights, out=self.out)  # noqa: E731
+        else:
+            self.router_logits = torch.zeros((tokens, layer.cfg.num_experts), dtype=logits_dtype, device=dev)
+            run = lambda: layer.forward_from_logits(self.hidden, self.router_logits, topk, renormalise, out=self.out)  # noqa: E731
         side = torch.cuda.Stream(device=dev)  # (default priority)
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):  # one eager run: every buffer of this shape exists before the capture
-            layer(self.hidden, self.topk_ids, self.topk_weights, out=self.out)
+            run()
         torch.cuda.current_stream().wait_stream(side)
         self.graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(self.graph, stream=side):
-            layer(self.hidden, self.topk_ids, self.topk_weights, out=self.out)
+            run()
         self._layer = layer  # the graph's kernels read the layer's buffers
 
     def replay(self) -> torch.Tensor:

@@ -102,6 +102,26 @@ def per_token_prologue(k: int, topk: int) -> bool:
     return 512 <= k <= 4096 and k & (k - 1) == 0 and 0 < topk <= 8
 
 
+_LOGIT_DTYPES = {torch.float16: 0, torch.float32: 1, torch.bfloat16: 2}
+
+
+def route_topk(router_logits: torch.Tensor, topk: int, renormalise: bool = False, out_ids: torch.Tensor | None = None, out_weights: torch.Tensor | None = None):
+    """Router logits [T, E] (fp16, fp32 or bf16, on the device) -> (topk_ids int32 [T, k], topk_weights fp32 [T, k]): softmax over the
+    experts in fp32, the k largest probabilities in decreasing order (equal ones: lower expert id first), divided by their sum when
+    `renormalise` (mxmoe/quant/moe_tracer.py:79-86).  `out_ids` / `out_weights` receive the result when given (no allocation)."""
+    lib = _lib.load()
+    if router_logits.dtype not in _LOGIT_DTYPES:
+        raise ValueError(f"router logits of dtype {router_logits.dtype}: fp16, fp32 or bf16 expected")
+    logits = router_logits.contiguous()
+    t, e = logits.shape
+    dev = logits.device
+    ids = out_ids if out_ids is not None else torch.empty((t, topk), dtype=torch.int32, device=dev)
+    w = out_weights if out_weights is not None else torch.empty((t, topk), dtype=torch.float32, device=dev)
+    assert ids.shape == (t, topk) and ids.dtype == torch.int32 and ids.is_contiguous() and w.shape == (t, topk) and w.dtype == torch.float32 and w.is_contiguous()
+    _lib.check(lib, lib.mxmoe_route_topk(logits.data_ptr(), _LOGIT_DTYPES[logits.dtype], t, e, topk, int(bool(renormalise)), ids.data_ptr(), w.data_ptr(), _stream()))
+    return ids, w
+
+
 def build_permutation(topk_ids: torch.Tensor, num_experts: int, with_inverse: bool = False):
     """Stable sort of the flattened expert ids on the device -> (dst_exp_sorted int32 [R], perm_indices int64 [R],
     src_slot int64 [R], recv_tokens_per_exp int64 [E] on the device); with `with_inverse` also row_of_slot int32 [R]: the sorted row

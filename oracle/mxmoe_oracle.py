@@ -20,7 +20,8 @@ fails a test in ``tests/test_oracle_*.py``):
 * ``had_table``           — H H^T = K I and all entries +-1.
 * ``online_hadamard``     — dense kron(H_K, H_{n/K}) / sqrt(n) in float64.
 * ``had_factor``          — kron(S_f, B) rebuilt and compared with the table.
-* ``route_topk``          — textbook softmax / top-k, weights sum to one.
+* ``route_topk``          — textbook softmax / top-k in float64, weights sum to one; hand-computed probabilities (logits = ln of
+  small integers), equal logits in index order, torch.softmax + torch.topk as an independent library routine.
 * ``permute_by_expert``   — brute force against a dict-of-lists.
 * ``tile_to_problem``     — every (problem, tile_m, tile_n) visited exactly once.
 * ``silu_mul`` / ``exp2_neg_f32_fixed`` / ``rcp_f32_fixed`` — float64 ``x*sigmoid(x)*u`` within one fp16 ulp for EVERY fp16 gate
@@ -433,15 +434,19 @@ def matmul_hadU_f64(x: np.ndarray) -> np.ndarray:
 # --------------------------------------------------------------------------------------------
 # Routing, permutation, offsets
 # --------------------------------------------------------------------------------------------
-def route_topk(logits: np.ndarray, topk: int):
-    """moe_tracer.py:79-86: ``softmax(logits, fp32) -> topk -> renormalise``.  Returns (ids int32 [T,k], weights fp32)."""
+def route_topk(logits: np.ndarray, topk: int, renormalise: bool = True):
+    """moe_tracer.py:79-86: ``softmax(logits, fp32) -> topk -> (optionally) renormalise``.  Returns (ids int32 [T,k], weights fp32).
+
+    Equal probabilities go to the lower expert id first (torch.topk leaves that order open).  ``renormalise`` divides the k weights
+    by their sum (Mixtral's ``norm_topk_prob``); without it the weights are the plain probabilities (Qwen-MoE, DeepSeek-V2-Lite)."""
     z = logits.astype(F32)
     z = z - z.max(axis=1, keepdims=True)
     p = np.exp(z)
     p = p / p.sum(axis=1, keepdims=True)
     ids = np.argsort(-p, axis=1, kind="stable")[:, :topk]
     w = np.take_along_axis(p, ids, axis=1)
-    w = w / w.sum(axis=1, keepdims=True)
+    if renormalise:
+        w = w / w.sum(axis=1, keepdims=True)
     return ids.astype(np.int32), w.astype(F32)
 
 

@@ -222,6 +222,11 @@ def test_prologue_entry_points_validate_on_the_host(lib):
     assert lib.mxmoe_permute_plan_layer(a, 200, 2, 8, a, a, a, a, a, a, a, 0, None) == 3 and b"256" in lib.mxmoe_last_error()   # larger batches: the two separate calls
     assert lib.mxmoe_permute_plan_layer(a, 4, 2, 8, a, a, a, a, a, None, a, 0, None) == 5
     assert lib.mxmoe_build_permutation(None, 4, 2, 8, a, a, a, a, a, None) == 5
+    assert lib.mxmoe_route_topk(a, 1, 4, 8, 9, 0, a, a, None) == 3 and b"top-k" in lib.mxmoe_last_error()      # k > experts
+    assert lib.mxmoe_route_topk(a, 1, 4, 5000, 2, 0, a, a, None) == 3
+    assert lib.mxmoe_route_topk(a, 3, 4, 8, 2, 0, a, a, None) == 3                                              # unknown dtype
+    assert lib.mxmoe_route_topk(a, 1, 4, 8, 2, 0, None, a, None) == 5
+    assert lib.mxmoe_route_topk(None, 1, 0, 8, 2, 0, None, None, None) == 0                                     # no tokens: nothing to launch
     assert lib.mxmoe_build_permutation(a, 0, 2, 8, a, a, a, a, a, None) == 3
 
 

@@ -16,6 +16,31 @@ def test_route_topk_textbook():
     assert np.allclose(w.sum(1), 1, atol=1e-6)
 
 
+def test_route_topk_known_answers_ties_and_library_routine():
+    import torch
+
+    # probabilities 0.1, 0.4, 0.2, 0.3 by construction: logits = ln(1, 4, 2, 3) + any constant
+    logits = (np.log(np.array([[1.0, 4.0, 2.0, 3.0]])) + 5.0).astype(np.float32)
+    ids, w = O.route_topk(logits, 2, renormalise=False)
+    assert ids.tolist() == [[1, 3]] and np.allclose(w, [[0.4, 0.3]], rtol=1e-6)
+    ids, w = O.route_topk(logits, 2, renormalise=True)
+    assert ids.tolist() == [[1, 3]] and np.allclose(w, [[4 / 7, 3 / 7]], rtol=1e-6)
+    ids, w = O.route_topk(logits, 4, renormalise=False)
+    assert ids.tolist() == [[1, 3, 2, 0]] and np.allclose(w.sum(), 1.0, rtol=1e-6)
+    # equal logits: lower expert id first
+    ids, w = O.route_topk(np.array([[0.5, 2.0, 2.0, -1.0, 2.0]], np.float32), 3, renormalise=True)
+    assert ids.tolist() == [[1, 2, 4]] and np.allclose(w, 1 / 3, rtol=1e-6)
+    # an independent library routine on logits without ties
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((200, 60)).astype(np.float32) * 3
+    for renorm in (False, True):
+        ids, w = O.route_topk(x, 4, renormalise=renorm)
+        tw, ti = torch.topk(torch.softmax(torch.from_numpy(x), dim=1, dtype=torch.float32), 4, dim=-1)
+        if renorm:
+            tw = tw / tw.sum(dim=-1, keepdim=True)
+        assert np.array_equal(ids, ti.numpy()) and np.allclose(w, tw.numpy(), rtol=1e-5)
+
+
 def test_permutation_bruteforce_and_stability():
     rng = np.random.default_rng(1)
     E, T, k = 7, 40, 3
