@@ -251,6 +251,14 @@ int mxmoe_plan_layer(const mxmoe_plan_call* gate_up, const mxmoe_plan_call* down
 int mxmoe_permute_plan_layer(const int32_t* topk_ids, int num_tokens, int topk, int num_experts, int32_t* dst_exp_sorted, int64_t* perm_indices, int64_t* src_slot,
                              int64_t* recv_tokens_per_exp, int32_t* row_of_slot, const mxmoe_plan_call* gate_up, const mxmoe_plan_call* down, int shared_rows,
                              void* stream);
+/* The same pair of calls in TWO launches for larger batches: the experts are counted per chunk of 256 (token, slot) entries, then one
+ * launch scatters the chunks and, in further workgroups that do not wait for them, plans both blocks from the same counts (the two
+ * separate calls take four launches).  `workspace`: mxmoe_permute_workspace_bytes(num_tokens * topk, num_experts) bytes of device
+ * scratch.  Takes batches with ceil(num_tokens * topk / 256) * num_experts <= 16384 (8192 tokens x top-4 over 60 experts: 7680),
+ * error 3 beyond; at most 256 entries it is mxmoe_permute_plan_layer. */
+int mxmoe_permute_plan_layer_ws(const int32_t* topk_ids, int num_tokens, int topk, int num_experts, int32_t* dst_exp_sorted, int64_t* perm_indices, int64_t* src_slot,
+                                int64_t* recv_tokens_per_exp, int32_t* row_of_slot, const mxmoe_plan_call* gate_up, const mxmoe_plan_call* down, int shared_rows,
+                                void* workspace, void* stream);
 int mxmoe_group_gemm_planned(int kernel_id, const void* d_plan, int num_problems, int grid, void* stream);
 int mxmoe_quant_act_planned(const void* hidden, void* inp_store, void* scale_store, const int32_t* dst_exp_sorted, const int64_t* perm_indices, const void* d_plan,
                             int K, int rows_capacity, int num_tokens, int num_experts, int has_shared, int rotate, int had_k, int had_f, const float* had_signs,

@@ -63,6 +63,7 @@ SIGNATURES = {
     "mxmoe_plan_block": (_I, [_I, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P]),
     "mxmoe_plan_layer": (_I, [_P, _P, _P, _I, _I, _P]),
     "mxmoe_permute_plan_layer": (_I, [_P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _P]),
+    "mxmoe_permute_plan_layer_ws": (_I, [_P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P]),
     "mxmoe_group_gemm_planned": (_I, [_I, _P, _I, _I, _P]),
     "mxmoe_quant_act_planned": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P]),
     "mxmoe_silu_mul_quant_planned": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P]),

@@ -30,7 +30,7 @@ namespace mxmoe {
 // Stable permutation by expert
 // ------------------------------------------------------------------------------------------------------------
 
-__global__ void __launch_bounds__(64) perm_hist_kernel(const int32_t* __restrict__ ids, int total, int E, int32_t* __restrict__ hist /*[blocks][E]*/) {
+__global__ void __launch_bounds__(64) perm_hist_kernel(const int32_t* __restrict__ ids, int total, int E, int32_t* __restrict__ hist, int stride /*0: [blocks][E]; else [E][stride]*/) {
   extern __shared__ int32_t cnt[];
   for (int e = threadIdx.x; e < E; e += 64) cnt[e] = 0;
   __syncthreads();
@@ -43,7 +43,7 @@ __global__ void __launch_bounds__(64) perm_hist_kernel(const int32_t* __restrict
     }
   }
   __syncthreads();
-  for (int e = threadIdx.x; e < E; e += 64) hist[blockIdx.x * E + e] = cnt[e];
+  for (int e = threadIdx.x; e < E; e += 64) hist[stride ? (long)e * stride + blockIdx.x : (long)blockIdx.x * E + e] = cnt[e];
 }
 
 // one single-wave workgroup per expert: exclusive scan of the expert's per-block counts (64 blocks per step); total -> recv
@@ -61,43 +61,15 @@ __global__ void __launch_bounds__(64) perm_scan_kernel(int32_t* __restrict__ his
 }
 
 __global__ void __launch_bounds__(64) perm_scatter_kernel(const int32_t* __restrict__ ids, int total, int E, int topk, int nbits, const int32_t* __restrict__ hist,
-                                                          const int64_t* __restrict__ recv, int32_t* __restrict__ dst_exp_sorted, int64_t* __restrict__ perm,
+                                                          int raw, int64_t* __restrict__ recv, int32_t* __restrict__ dst_exp_sorted, int64_t* __restrict__ perm,
                                                           int64_t* __restrict__ src_slot, int32_t* __restrict__ row_of_slot) {
   extern __shared__ int32_t run[];  // next free rank per expert for this block
-  {  // first row of every expert = exclusive scan of the per-expert totals, plus this block's offset inside the expert
-    int carry = 0;
-    for (int e0 = 0; e0 < E; e0 += 64) {
-      const int e = e0 + (int)threadIdx.x;
-      const int v = e < E ? (int)recv[e] : 0;
-      const int inc = wave_inclusive_scan(v, threadIdx.x);
-      if (e < E) run[e] = carry + inc - v + hist[blockIdx.x * E + e];
-      carry += __shfl(inc, 63);
-    }
-  }
-  __syncthreads();
-  const int lane = threadIdx.x;
-  const int base = blockIdx.x * kPermChunk;
-  for (int i = 0; i < kPermChunk; i += 64) {  // sub-chunks in order keep the sort stable
-    const int idx = base + i + lane;
-    const bool ok = idx < total;
-    int e = ok ? ids[idx] : -1;
-    if (e < 0 || e >= E) e = E;  // parked on a dummy id, never written
-    const uint64_t same = match_same(e, nbits);
-    const int before = __popcll(same & ((1ull << lane) - 1));
-    int first = 0;
-    if (e < E) first = run[e];
-    __syncthreads();
-    if (e < E) {
-      const int pos = first + before;
-      dst_exp_sorted[pos] = e;
-      perm[pos] = idx / topk;
-      if (src_slot) src_slot[pos] = idx;
-      if (before == 0) run[e] = first + __popcll(same);
-    }
-    // the inverse map (sorted row of every (token, slot); -1 where the expert id was out of range), for the combine
-    if (row_of_slot && ok) row_of_slot[idx] = e < E ? first + before : -1;
-    __syncthreads();
-  }
+  perm_scatter_body(ids, total, E, topk, nbits, hist, (int)gridDim.x, (int)blockIdx.x, raw != 0, recv, dst_exp_sorted, perm, src_slot, row_of_slot, run, true);
+}
+
+void launch_perm_hist(const int32_t* ids, int total, int E, int32_t* hist, bool expert_major, hipStream_t stream) {
+  const int blocks = (total + kPermChunk - 1) / kPermChunk;
+  hipLaunchKernelGGL(perm_hist_kernel, dim3(blocks), dim3(64), (size_t)E * sizeof(int32_t), stream, ids, total, E, hist, expert_major ? perm_hist_stride(blocks) : 0);
 }
 
 // The three kernels above in one, for at most kPermChunk (token, slot) entries (decode-sized batches): one single-wave workgroup
@@ -1922,7 +1894,7 @@ extern "C" {
 
 size_t mxmoe_permute_workspace_bytes(int total, int num_experts) {
   const size_t blocks = (size_t)(total + kPermChunk - 1) / kPermChunk;
-  return (blocks * num_experts + num_experts) * sizeof(int32_t);
+  return ((size_t)perm_hist_stride((int)blocks) * num_experts + num_experts) * sizeof(int32_t);
 }
 
 static int build_permutation_impl(const int32_t* topk_ids, int num_tokens, int topk, int num_experts, int32_t* dst_exp_sorted, int64_t* perm_indices,
@@ -1936,9 +1908,12 @@ static int build_permutation_impl(const int32_t* topk_ids, int num_tokens, int t
     hipLaunchKernelGGL(perm_small_kernel, dim3(1), dim3(64), lds, s, topk_ids, total, num_experts, topk, nbits, recv_tokens_per_exp, dst_exp_sorted, perm_indices, src_slot,
                        row_of_slot);
   } else {
-    hipLaunchKernelGGL(perm_hist_kernel, dim3(blocks), dim3(64), lds, s, topk_ids, total, num_experts, hist);
-    hipLaunchKernelGGL(perm_scan_kernel, dim3(num_experts), dim3(64), 0, s, hist, blocks, num_experts, recv_tokens_per_exp);
-    hipLaunchKernelGGL(perm_scatter_kernel, dim3(blocks), dim3(64), lds, s, topk_ids, total, num_experts, topk, nbits, hist, recv_tokens_per_exp, dst_exp_sorted,
+    // few workgroups and experts: the scatter workgroups sum the counts they need themselves, which saves the scan launch
+    // (the 16-byte loads of that path need an aligned workspace; any other goes the three-launch way)
+    const int raw = (long)blocks * num_experts <= kPermFusedScanMax && (reinterpret_cast<uintptr_t>(hist) & 15) == 0;
+    launch_perm_hist(topk_ids, total, num_experts, hist, raw != 0, s);
+    if (!raw) hipLaunchKernelGGL(perm_scan_kernel, dim3(num_experts), dim3(64), 0, s, hist, blocks, num_experts, recv_tokens_per_exp);
+    hipLaunchKernelGGL(perm_scatter_kernel, dim3(blocks), dim3(64), lds, s, topk_ids, total, num_experts, topk, nbits, hist, raw, recv_tokens_per_exp, dst_exp_sorted,
                        perm_indices, src_slot, row_of_slot);
   }
   const hipError_t e = hipGetLastError();

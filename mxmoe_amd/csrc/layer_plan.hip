@@ -358,6 +358,38 @@ __global__ void __launch_bounds__(kPlanThreads) perm_plan_small_kernel(const Per
   plan_block_body(pair.p[b / pair.chunks], b % pair.chunks, pair.chunks, counts);
 }
 
+// The same for larger batches, after perm_hist_kernel has counted the experts per chunk of kPermChunk entries: the first `blocks`
+// workgroups scatter their chunk (each summing the counts it needs: perm_scatter_body with raw counts), the others plan the
+// layer's launches from the column sums of the same histogram.  Neither waits for the other, so the forward's serial head is two
+// launches (count, scatter + plan) instead of four (count, scan, scatter, plan).
+struct PermScatterArgs {
+  const int32_t* ids;
+  int total, E, topk, nbits, blocks;
+  const int32_t* hist;
+  int64_t* recv;
+  int32_t* dst;
+  int64_t* perm;
+  int64_t* slot;
+  int32_t* row_of_slot;
+};
+__global__ void __launch_bounds__(kPlanThreads) perm_scatter_plan_kernel(const PermScatterArgs a, const PlanPair pair) {
+  extern __shared__ __align__(8) uint8_t pp_lds[];  // E int32 ranks (scatter workgroups) or E int64 counts (planning workgroups)
+  if ((int)blockIdx.x < a.blocks) {
+    perm_scatter_body(a.ids, a.total, a.E, a.topk, a.nbits, a.hist, a.blocks, (int)blockIdx.x, true, a.recv, a.dst, a.perm, a.slot, a.row_of_slot,
+                      reinterpret_cast<int32_t*>(pp_lds), threadIdx.x < 64);
+    return;
+  }
+  int64_t* counts = reinterpret_cast<int64_t*>(pp_lds);
+  for (int e = threadIdx.x; e < a.E; e += kPlanThreads) {
+    int v, before;
+    perm_hist_row_sums(a.hist + (long)e * perm_hist_stride(a.blocks), a.blocks, 0, &v, &before);
+    counts[e] = v;
+  }
+  __syncthreads();
+  const int b = blockIdx.x - a.blocks;
+  plan_block_body(pair.p[b / pair.chunks], b % pair.chunks, pair.chunks, counts);
+}
+
 // Kernel for the formats of `h_desc`, checked once on the host: every problem's format has a branch and its shape fits it.
 static int resolve_kernel(int kernel_id, const mxmoe_block_desc* h_desc, int et) {
   auto& reg = registry();
@@ -591,6 +623,58 @@ int mxmoe_permute_plan_layer(const int32_t* topk_ids, int num_tokens, int topk, 
   a.slot = src_slot;
   a.row_of_slot = row_of_slot;
   hipLaunchKernelGGL(perm_plan_small_kernel, dim3(1 + 2 * pair.chunks), dim3(kPlanThreads), (size_t)num_experts * 8, (hipStream_t)stream, a, pair);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    last_error() = std::string("kernel launch failed: ") + hipGetErrorString(e);
+    return 4;
+  }
+  return 0;
+}
+
+int mxmoe_permute_plan_layer_ws(const int32_t* topk_ids, int num_tokens, int topk, int num_experts, int32_t* dst_exp_sorted, int64_t* perm_indices, int64_t* src_slot,
+                                int64_t* recv_tokens_per_exp, int32_t* row_of_slot, const mxmoe_plan_call* gate_up, const mxmoe_plan_call* down, int shared_rows,
+                                void* workspace, void* stream) {
+  if (num_tokens > 0 && topk > 0 && (long)num_tokens * topk <= kPermChunk)
+    return mxmoe_permute_plan_layer(topk_ids, num_tokens, topk, num_experts, dst_exp_sorted, perm_indices, src_slot, recv_tokens_per_exp, row_of_slot, gate_up, down,
+                                    shared_rows, stream);
+  const long total = (long)num_tokens * topk;
+  const long blocks = (total + kPermChunk - 1) / kPermChunk;
+  if (num_tokens <= 0 || topk <= 0 || num_experts <= 0 || num_experts > kMaxPlannedProblems || blocks * num_experts > kPermFusedScanMax) {
+    last_error() = "the two-launch permutation + planning takes batches whose (chunks of 256 entries) x experts is at most 16384: use mxmoe_build_permutation_inv and mxmoe_plan_layer";
+    return 3;
+  }
+  if (!topk_ids || !dst_exp_sorted || !perm_indices || !src_slot || !recv_tokens_per_exp || !gate_up || !down || !workspace) {
+    last_error() = "null pointer";
+    return 5;
+  }
+  if (reinterpret_cast<uintptr_t>(workspace) & 15) {
+    last_error() = "the workspace of the two-launch permutation + planning must be 16-byte aligned";
+    return 3;
+  }
+  PlanPair pair;
+  const mxmoe_plan_call* c[2] = {gate_up, down};
+  for (int i = 0; i < 2; ++i) {
+    const int rc = fill_plan_params(pair.p[i], c[i]->kernel_id, recv_tokens_per_exp, num_experts, shared_rows, c[i]->d_desc, c[i]->h_desc, c[i]->inp_store, c[i]->scale_store,
+                                    c[i]->out_store, c[i]->d_plan);
+    if (rc) return rc;
+  }
+  pair.chunks = PlanLayout(pair.p[0].Et).chunks;
+  PermScatterArgs a;
+  a.ids = topk_ids;
+  a.total = (int)total;
+  a.E = num_experts;
+  a.topk = topk;
+  a.nbits = 1;
+  while ((1 << a.nbits) <= num_experts) ++a.nbits;  // ids 0..E (E = parked lanes)
+  a.blocks = (int)blocks;
+  a.hist = reinterpret_cast<const int32_t*>(workspace);
+  a.recv = recv_tokens_per_exp;
+  a.dst = dst_exp_sorted;
+  a.perm = perm_indices;
+  a.slot = src_slot;
+  a.row_of_slot = row_of_slot;
+  launch_perm_hist(topk_ids, a.total, num_experts, reinterpret_cast<int32_t*>(workspace), true, (hipStream_t)stream);
+  hipLaunchKernelGGL(perm_scatter_plan_kernel, dim3(a.blocks + 2 * pair.chunks), dim3(kPlanThreads), (size_t)num_experts * 8, (hipStream_t)stream, a, pair);
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     last_error() = std::string("kernel launch failed: ") + hipGetErrorString(e);

@@ -218,7 +218,7 @@ class MxMoELayer:
         Same kernels and results as `forward` + `combine`, but nothing here waits for the routing: the tables of both launches are
         derived from the tokens-per-expert counts by a planning kernel on the device (`mxmoe_plan_layer`: both blocks in one launch), the stores and plan
         buffers are allocated once per (tokens, top-k) for the worst case, and every launch argument is independent of the data.
-        The call only enqueues six kernels (nine when more than 256 (token, slot) pairs are permuted; no synchronisation, no allocation after the first call when `out` is given), so it can
+        The call only enqueues six kernels (seven when more than 256 (token, slot) pairs are permuted, nine beyond what `mxmoe_permute_plan_layer_ws` takes; no synchronisation, no allocation after the first call when `out` is given), so it can
         be captured into a HIP graph.  Intermediate buffers belong to the layer and are reused by the next call of the same shape."""
         cfg, dev = self.cfg, self.device
         lib = _lib.load()
@@ -238,6 +238,10 @@ class MxMoELayer:
         if ps["r_cap"] <= 256:  # decode-sized batch: permutation and planning in one launch
             ck(lib.mxmoe_permute_plan_layer(ids.data_ptr(), t, topk, e_cnt, ps["dst"].data_ptr(), ps["perm"].data_ptr(), ps["slot"].data_ptr(), ps["recv"].data_ptr(),
                                             ps["row_of_slot"].data_ptr(), C.byref(ps["calls"][0]), C.byref(ps["calls"][1]), ps["shared_rows"], stream))
+        elif -(-ps["r_cap"] // 256) * e_cnt <= 16384:  # count, then scatter and plan side by side in one launch
+            ck(lib.mxmoe_permute_plan_layer_ws(ids.data_ptr(), t, topk, e_cnt, ps["dst"].data_ptr(), ps["perm"].data_ptr(), ps["slot"].data_ptr(), ps["recv"].data_ptr(),
+                                               ps["row_of_slot"].data_ptr(), C.byref(ps["calls"][0]), C.byref(ps["calls"][1]), ps["shared_rows"],
+                                               ps["perm_ws"].data_ptr(), stream))
         else:
             ck(lib.mxmoe_build_permutation_inv(ids.data_ptr(), t, topk, e_cnt, ps["dst"].data_ptr(), ps["perm"].data_ptr(), ps["slot"].data_ptr(), ps["recv"].data_ptr(),
                                                ps["row_of_slot"].data_ptr(), ps["perm_ws"].data_ptr(), stream))

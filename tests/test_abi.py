@@ -221,6 +221,8 @@ def test_prologue_entry_points_validate_on_the_host(lib):
     assert lib.mxmoe_silu_mul_quant(a, a, a, a, a, a, 1408, 1408, 4, 2, 2, 0, 1, 176, 4, None, None) == 3 and b"sign table" in lib.mxmoe_last_error()
     assert lib.mxmoe_permute_plan_layer(a, 200, 2, 8, a, a, a, a, a, a, a, 0, None) == 3 and b"256" in lib.mxmoe_last_error()   # larger batches: the two separate calls
     assert lib.mxmoe_permute_plan_layer(a, 4, 2, 8, a, a, a, a, a, None, a, 0, None) == 5
+    assert lib.mxmoe_permute_plan_layer_ws(a, 100000, 8, 256, a, a, a, a, a, a, a, 0, a, None) == 3 and b"16384" in lib.mxmoe_last_error()
+    assert lib.mxmoe_permute_plan_layer_ws(a, 2000, 2, 8, a, a, a, a, a, a, a, 0, None, None) == 5             # no workspace
     assert lib.mxmoe_build_permutation(None, 4, 2, 8, a, a, a, a, a, None) == 5
     assert lib.mxmoe_route_topk(a, 1, 4, 8, 9, 0, a, a, None) == 3 and b"top-k" in lib.mxmoe_last_error()      # k > experts
     assert lib.mxmoe_route_topk(a, 1, 4, 5000, 2, 0, a, a, None) == 3

@@ -505,6 +505,62 @@ def test_planned_forward_of_more_experts_than_one_launch_holds():
         ids[::5, 1] = cfg.num_experts + 3                                # second round: some slots belong to experts held elsewhere
 
 
+@pytest.mark.parametrize("experts,tokens", [(6, 700), (130, 500)])
+def test_two_launch_permutation_and_planning_writes_what_the_separate_calls_write(experts, tokens):
+    """mxmoe_permute_plan_layer_ws (count; scatter + plan side by side) against mxmoe_build_permutation_inv + mxmoe_plan_layer (four
+    launches) on the same buffers: identical permutation, counts, inverse map and plan buffers, with dropped ids; the forward that
+    uses it equals the stepwise operators' result."""
+    import ctypes as C
+
+    from mxmoe_amd import _lib, synth
+    from mxmoe_amd.layer import MxMoELayer
+
+    cfg = synth.MoEConfig("t", "test", experts, 3, 256, 512, tokens, num_shared=1, rotate=1, formats=(synth.W4A4, synth.W8A8, synth.FP16), format_probs=(0.4, 0.4, 0.2))
+    layer = MxMoELayer(cfg)
+    hidden = synth.make_hidden(cfg)
+    ids, w = synth.make_routing(cfg)
+    ids = ids.clone()
+    ids[::7, 2] = experts + 1                                            # dropped slots
+    ids[3, 0] = -1
+    layer.forward(hidden, ids)
+    want = layer.combine(w).clone()
+    got = layer(hidden, ids, w)                                          # (more than 256 entries: the two-launch head)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+    lib = _lib.load()
+    ps = layer._planned_setup(tokens, cfg.topk)
+    assert ps["r_cap"] > 256 and -(-ps["r_cap"] // 256) * experts <= 16384
+    names = ("dst", "perm", "slot", "recv", "row_of_slot")
+    routed = int(((ids >= 0) & (ids < experts)).sum())
+    snap = {k: ps[k].clone() for k in names}
+    plans = [ps["b1"]["plan"].clone(), ps["b2"]["plan"].clone()]
+    for k in names:
+        ps[k].fill_(-3)
+    ps["b1"]["plan"].zero_()
+    ps["b2"]["plan"].zero_()
+    stream = torch.cuda.current_stream().cuda_stream
+    d_ids = ids.to("cuda").to(torch.int32).contiguous()
+    _lib.check(lib, lib.mxmoe_build_permutation_inv(d_ids.data_ptr(), tokens, cfg.topk, experts, ps["dst"].data_ptr(), ps["perm"].data_ptr(), ps["slot"].data_ptr(),
+                                                    ps["recv"].data_ptr(), ps["row_of_slot"].data_ptr(), ps["perm_ws"].data_ptr(), stream))
+    _lib.check(lib, lib.mxmoe_plan_layer(C.byref(ps["calls"][0]), C.byref(ps["calls"][1]), ps["recv"].data_ptr(), experts, ps["shared_rows"], stream))
+    torch.cuda.synchronize()
+    assert int(ps["recv"].sum()) == routed
+    for k in ("recv", "row_of_slot"):
+        assert torch.equal(ps[k], snap[k]), k
+    for k in ("dst", "perm", "slot"):                                    # rows past the routed ones are not written by either
+        assert torch.equal(ps[k][:routed], snap[k][:routed]), k
+    et = ps["et"]
+    first, last = lib.mxmoe_plan_offset(1, et), lib.mxmoe_plan_offset(4, et) + 12 * et
+    for now, before in zip((ps["b1"]["plan"], ps["b2"]["plan"]), plans):
+        a, b = now.cpu().numpy(), before.cpu().numpy()
+        assert np.array_equal(a[:56], b[:56])                               # the header's pointers (same buffers on both sides)
+        ai, bi = a[56:].view(np.int32), b[56:].view(np.int32)               # offset, entries, tiles, phases; phase_tile0[9]; phase_wg0[9]; flat; entries
+        ne, nph = int(bi[1]), int(bi[3])
+        assert ne > 0 and np.array_equal(ai[:4], bi[:4]) and np.array_equal(ai[4:5 + nph], bi[4:5 + nph]) and np.array_equal(ai[13:14 + nph], bi[13:14 + nph])
+        assert ai[22] == bi[22] and np.array_equal(ai[23:23 + 4 * ne], bi[23:23 + 4 * ne])
+        assert np.array_equal(a[first:last], b[first:last])                 # table, pointer arrays, row counts, sizes
+
+
 def test_single_block_planning_writes_what_the_paired_launch_writes():
     """mxmoe_plan_block (one block per launch) against mxmoe_plan_layer (both blocks of the layer in one launch): identical plan
     buffers for the same counts."""

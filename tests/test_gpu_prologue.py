@@ -19,7 +19,7 @@ def test_permutation_matches_oracle_and_is_stable():
     from mxmoe_amd import ops
 
     rng = np.random.default_rng(0)
-    for (t, e, k) in [(1, 4, 2), (37, 7, 3), (300, 60, 4), (2048, 64, 6), (513, 8, 2)]:
+    for (t, e, k) in [(1, 4, 2), (37, 7, 3), (300, 60, 4), (2048, 64, 6), (513, 8, 2), (12000, 64, 6)]:   # (the last: beyond the scan-less path)
         ids = _ids(rng, t, e, k)
         if e > 5:
             ids[ids == 3] = 5 if k == 1 else ids[ids == 3]                  # keep ids valid
@@ -40,7 +40,7 @@ def test_permutation_with_inverse_map_small_and_large_and_dropped_ids():
     lib = _lib.load()
     rng = np.random.default_rng(3)
     stream = torch.cuda.current_stream().cuda_stream
-    for (t, e, k) in [(1, 4, 2), (32, 64, 6), (42, 7, 6), (43, 7, 6), (64, 4, 4), (65, 4, 4), (700, 60, 4)]:
+    for (t, e, k) in [(1, 4, 2), (32, 64, 6), (42, 7, 6), (43, 7, 6), (64, 4, 4), (65, 4, 4), (700, 60, 4), (3000, 256, 8)]:   # (the last: with the scan kernel)
         ids = _ids(rng, t, e, k)
         ids[rng.random(ids.shape) < 0.15] = e + 2                            # dropped entries
         if t > 3:
