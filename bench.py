@@ -132,6 +132,22 @@ def roofline_of(cfg, layer, up_ms: float, dn_ms: float):
     return tuple(roofline_entry(cfg, layer, n) for n in names)
 
 
+def roofline_step(cfg, layer, ms: float) -> dict:
+    """The whole step (both launches back to back on one stream, `ms` per step by the bench's own clock) against the same peak as
+    its launches: ops of both over the step time, or algorithmic bytes of both for the few-token weight-only layers."""
+    st = layer.state
+    by = layer.algorithmic_bytes()
+    fmts = {q[:2] for plan in (st["gg1"], st["gg2"]) for q in plan.qparams}
+    if cfg.tokens * cfg.topk / cfg.num_experts >= 128:
+        peak = PEAK["fp16"] if all(a >= 16 for a, _ in fmts) else PEAK["int8"]
+        ach = layer.gemm_ops() / (ms * 1e-3) / 1e12
+        return {"bound": "mfma", "achieved": round(ach, 2), "peak": peak, "unit": "TFLOP/s", "frac": round(ach / peak, 4), "step_us": round(ms * 1e3, 2)}
+    total = by["gate_up"]["total"] + by["down"]["total"]
+    ach = total / (ms * 1e-3) / 1e9
+    return {"bound": "hbm", "achieved": round(ach, 1), "peak": PEAK["hbm"], "unit": "GB/s", "frac": round(ach / PEAK["hbm"], 4), "step_us": round(ms * 1e3, 2),
+            "algorithmic_bytes": total}
+
+
 def cpu_baseline(cfg, budget_s: float = 20.0):
     """The fake-quant path (per expert: fake_quant(x) @ fake_quant(W13)^T -> SiLU*up -> fake_quant(.) @ fake_quant(W2)^T,
     fp16 storage, fp32 matmul) from the CPU oracle, on as many experts of this workload as fit the time budget."""
@@ -248,6 +264,7 @@ def run_workload(name: str, steps: int, warmup: int, tokens=None, whole: bool = 
         "gate_up_us": round(up * 1e3, 2), "down_us": round(dn * 1e3, 2),
         "gate_up_tops": round(st["gg1"].ops / (up * 1e-3) / 1e12, 2), "down_tops": round(st["gg2"].ops / (dn * 1e-3) / 1e12, 2),
         "ops": ops, "whole_layer": time_whole_layer(cfg, layer) if whole else None, "roofline": roof[0], "roofline_other_launch": roof[1],
+        "roofline_step": roofline_step(cfg, layer, ms),
     }
 
 
@@ -324,7 +341,7 @@ def main() -> int:
         "config": {"workload": f"{args.workload}: {cfg.description}", "experts": cfg.num_experts, "topk": cfg.topk, "hidden": cfg.hidden,
                    "intermediate": cfg.inter, "tokens": cfg.tokens, "formats": fm, "step": "gate_up GroupGEMM launch + down GroupGEMM launch"},
         "roofline": main_res["roofline"],
-        "detail": {**{k: main_res[k] for k in ("gate_up_us", "down_us", "gate_up_tops", "down_tops", "ops", "whole_layer", "roofline_other_launch")},
+        "detail": {**{k: main_res[k] for k in ("gate_up_us", "down_us", "gate_up_tops", "down_tops", "ops", "whole_layer", "roofline_other_launch", "roofline_step")},
                    "w4a4_path": args.w4a4_path, "other_w4a4_path": alt},
         "also": also,
     }
