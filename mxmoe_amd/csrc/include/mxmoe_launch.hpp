@@ -291,10 +291,10 @@ struct BranchOf<Bf6Tile<BM>> {
     return BranchInfo{Fmt::W4A4, BM, T::BN, T::BK, 1, 4, T::kLdsBytes, 128, 0, 256, kVariantBf6};
   }
 };
-template <int WBITS, int BN, int KP, int RING, int WAVES>
-struct BranchOf<SkinnyWoTile<WBITS, BN, KP, RING, WAVES>> {
+template <int WBITS, int BN, int KP, int RING, int WAVES, int MB>
+struct BranchOf<SkinnyWoTile<WBITS, BN, KP, RING, WAVES, MB>> {
   static BranchInfo get() {
-    using T = SkinnyWoTile<WBITS, BN, KP, RING, WAVES>;
+    using T = SkinnyWoTile<WBITS, BN, KP, RING, WAVES, MB>;
     return BranchInfo{WBITS == 8 ? Fmt::W8A16 : WBITS == 4 ? Fmt::W4A16 : WBITS == 3 ? Fmt::W3A16 : Fmt::W2A16, T::BM, BN, 128, 1, 4, T::kLdsBytes, 128, 0};
   }
 };
@@ -353,10 +353,10 @@ inline double tile_cost(const BranchInfo& b) {
       {Fmt::W4A4, 128, 256, 1.00}, {Fmt::W4A4, 64, 256, 0.58}, {Fmt::W4A4, 32, 256, 0.48},
       {Fmt::W8A8, 128, 256, 1.00}, {Fmt::W8A8, 64, 256, 0.74}, {Fmt::W8A8, 32, 256, 0.56},
       {Fmt::FP16, 128, 256, 1.00}, {Fmt::FP16, 64, 256, 0.69}, {Fmt::FP16, 32, 256, 0.53}, {Fmt::FP16, 128, 128, 0.57}, {Fmt::FP16, 256, 128, 1.09},
-      {Fmt::W4A16, 16, 128, 0.37}, {Fmt::W4A16, 16, 64, 0.20}, {Fmt::W4A16, 128, 128, 1.00}, {Fmt::W4A16, 128, 256, 1.50},
-      {Fmt::W3A16, 16, 128, 0.31}, {Fmt::W3A16, 16, 64, 0.20}, {Fmt::W3A16, 128, 128, 1.00}, {Fmt::W3A16, 128, 256, 1.50},
-      {Fmt::W2A16, 16, 128, 0.25}, {Fmt::W2A16, 16, 64, 0.20}, {Fmt::W2A16, 128, 128, 1.00}, {Fmt::W2A16, 128, 256, 1.50},
-      {Fmt::W8A16, 16, 128, 0.60}, {Fmt::W8A16, 16, 64, 0.35}, {Fmt::W8A16, 128, 128, 1.00},
+      {Fmt::W4A16, 16, 128, 0.37}, {Fmt::W4A16, 16, 64, 0.20}, {Fmt::W4A16, 32, 128, 0.42}, {Fmt::W4A16, 128, 128, 1.00}, {Fmt::W4A16, 128, 256, 1.50},
+      {Fmt::W3A16, 16, 128, 0.31}, {Fmt::W3A16, 16, 64, 0.20}, {Fmt::W3A16, 32, 128, 0.36}, {Fmt::W3A16, 128, 128, 1.00}, {Fmt::W3A16, 128, 256, 1.50},
+      {Fmt::W2A16, 16, 128, 0.25}, {Fmt::W2A16, 16, 64, 0.20}, {Fmt::W2A16, 32, 128, 0.30}, {Fmt::W2A16, 128, 128, 1.00}, {Fmt::W2A16, 128, 256, 1.50},
+      {Fmt::W8A16, 16, 128, 0.60}, {Fmt::W8A16, 16, 64, 0.35}, {Fmt::W8A16, 32, 128, 0.66}, {Fmt::W8A16, 128, 128, 1.00},
       {Fmt::W4A4G128, 64, 256, 1.00}, {Fmt::W4A4G128, 32, 256, 0.60},
   };
   for (const Row& r : table)
@@ -379,6 +379,9 @@ struct PlanBranch {
   double cost;           // tile_cost
   double cost_per_row;   // tile_cost / BM
 };
+// A phase of such tiles keeps the plain workgroup order (no XCD remap): the few-token weight-only tiles stream their own weights
+// and share nothing but a few rows of activations with their neighbours.
+__host__ __device__ inline bool flat_phase(const PlanBranch& b) { return b.BM <= 16 || (is_weight_only((Fmt)b.fmt) && b.BM < 128); }
 // Tiles of size `dim` (2^`lg` when lg >= 0) that cover `x`.
 __host__ __device__ inline int tiles_over(int x, int dim, int lg) { return lg >= 0 ? (x + dim - 1) >> lg : (x + dim - 1) / dim; }
 constexpr int kNumFmts = (int)Fmt::UNSUPPORTED;
@@ -635,10 +638,17 @@ inline int auto_kernel_for(const mxmoe_qparams* h_q, int count, long max_rows) {
   }
   return plain;
 }
+// (A few-row kernel runs 16-row tiles: it is meant for lists whose problems mostly fit one such tile.  When more than a quarter of
+// the non-empty problems need several, the kernels that also hold the 32-row few-token tile do better, whatever the largest count.)
 inline int auto_kernel(const mxmoe_dim3* h_sizes, const mxmoe_qparams* h_q, int count) {
   long max_rows = 0;
-  for (int i = 0; i < count; ++i) max_rows = std::max(max_rows, (long)h_sizes[i].x);
-  return auto_kernel_for(h_q, count, max_rows);
+  int live = 0, over = 0;
+  for (int i = 0; i < count; ++i) {
+    max_rows = std::max(max_rows, (long)h_sizes[i].x);
+    live += h_sizes[i].x > 0;
+    over += h_sizes[i].x > 16;
+  }
+  return auto_kernel_for(h_q, count, 4 * over > live ? -1 : max_rows);
 }
 
 // K a multiple of the tile's K step, N a multiple of 8 (16 for the weight-only layouts)
@@ -701,7 +711,7 @@ inline int build_fused_tables(const FusedKernel& k, const mxmoe_dim3* h_sizes, c
     if (np < kMaxPhases) {
       a.phase_tile0[np] = tile0;
       a.phase_wg0[np] = wg;
-      if (pi.b[b].BM <= 16) a.phase_flat |= 1 << np;
+      if (flat_phase(pi.b[b])) a.phase_flat |= 1 << np;
       ++np;
     }
     const int p0 = a.phase_tile0[np - 1];

@@ -33,18 +33,21 @@
 namespace mxmoe {
 
 // KP: k blocks (128 wide) per pass of a wave, whose activations live in registers; RING: packed weight blocks in flight per wave;
-// WAVES: waves per SIMD a kernel made of such tiles alone is compiled for (fewer registers per wave, more workgroups per CU).
-template <int WBITS_, int BN_, int KP_ = 4, int RING_ = (WBITS_ == 8 ? 6 : 12), int WAVES_ = 2>
+// WAVES: waves per SIMD a kernel made of such tiles alone is compiled for (fewer registers per wave, more workgroups per CU);
+// MB: blocks of 16 tokens per tile.  Every unpacked weight operand is multiplied into all MB token blocks, so an expert with 17 .. 32
+// tokens still streams its weights once (two 16-token tiles stream them twice, the second time out of L2 at best, and take nearly
+// twice as long); the activations of a pass and the partial sums take MB times the registers, which is why KP shrinks as MB grows.
+template <int WBITS_, int BN_, int KP_ = 4, int RING_ = (WBITS_ == 8 ? 6 : 12), int WAVES_ = 2, int MB_ = 1>
 struct SkinnyWoTile {
-  static constexpr int WBITS = WBITS_, BM = 16, BN = BN_;
+  static constexpr int WBITS = WBITS_, MB = MB_, BM = 16 * MB_, BN = BN_;
   static_assert(WBITS == 8 || WBITS == 4 || WBITS == 3 || WBITS == 2, "w8 / w4 / w3 / w2");
   static_assert(BN % 64 == 0, "the final reduction deals 16-channel blocks to 4 waves");
   static constexpr int NB = BN / 16;                 // 16-channel blocks per tile
   static constexpr int KP = KP_;                     // k blocks (128 wide) per pass of a wave: their activations live in registers
-  static constexpr int kRedBytes = kWaves * NB * 64 * 16;  // per-wave partial sums for the final reduction
+  static constexpr int kRedBytes = kWaves * NB * MB * 64 * 16;  // per-wave partial sums for the final reduction
   static constexpr int kScaleBytes = NB * KP * 64;         // per-wave patch of (scale, zero) pairs of one pass
   static constexpr int kLdsBytes = kRedBytes + kWaves * kScaleBytes;
-  static constexpr int kAccRegs = NB * 4;
+  static constexpr int kAccRegs = NB * MB * 4;
   static constexpr int kWavesWanted = WAVES_;
   static constexpr int kABits = 16, kWBits = WBITS;  // fp16 activations, packed weights
   static constexpr int kLaneBytes = WBITS * 4;       // packed bytes per lane per (channel block, k block)
@@ -135,7 +138,7 @@ struct SkinnyWoTile {
   //   s * (sum_k x[k] * (q[k] + bias[k])  -  sum_k x[k] * bias[k])  +  z * sum_k x[k]
   // where the first sum comes from 4 MFMAs on the biased weights and the other two from MFMAs of x against constant operands.
   template <int NKB>
-  __device__ static __forceinline__ void pass(const TileArgs& t, int kb0, int m0, int n0, int nbv, int lane, uint8_t* __restrict__ spatch, v4f (&acc)[NB]) {
+  __device__ static __forceinline__ void pass(const TileArgs& t, int kb0, int m0, int n0, int nbv, int lane, uint8_t* __restrict__ spatch, v4f (&acc)[NB][MB]) {
     const int K = t.K, KB = K / 128;
     const int lm = lane & 15, lg = lane >> 4;
     const v8h ones = {(_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f};
@@ -151,17 +154,18 @@ struct SkinnyWoTile {
 #pragma unroll
     for (int q = 0; q < kRing && q < Q; ++q) wr[q] = w_of(q);
     __builtin_amdgcn_sched_barrier(0);
-    // activations: lane holds row lm, k = 128*(kb0 + s) + 32*lg + 8*j + 0..7
-    v8h xf[NKB][4];
-    {
-      const int m = m0 + lm;
+    // activations: lane holds row lm of each token block, k = 128*(kb0 + s) + 32*lg + 8*j + 0..7
+    v8h xf[MB][NKB][4];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+      const int m = m0 + mb * 16 + lm;
       const _Float16* xr = reinterpret_cast<const _Float16*>(t.A) + (long)(m < t.M ? m : 0) * K + kb0 * 128 + lg * 32;
 #pragma unroll
       for (int s = 0; s < NKB; ++s)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const v4i v = gload<v4i>(xr + s * 128 + j * 8);
-          xf[s][j] = m < t.M ? __builtin_bit_cast(v8h, v) : v8h{};
+          xf[mb][s][j] = m < t.M ? __builtin_bit_cast(v8h, v) : v8h{};
         }
     }
     // (scale, zero) pairs of the pass: 64 bytes per block, NKB consecutive blocks per channel block -> LDS [nb][s][64 B]
@@ -181,16 +185,18 @@ struct SkinnyWoTile {
       if (c < Q * 4) *reinterpret_cast<v4i*>(spatch + c * 16) = sv[i];
     }
 
-    v4f sx[NKB], sxb[NKB];  // per k block: sum of x, sum of x * bias  (row = any channel, column = token)
+    v4f sx[MB][NKB], sxb[MB][NKB];  // per token block and k block: sum of x, sum of x * bias  (row = any channel, column = token)
 #pragma unroll
-    for (int s = 0; s < NKB; ++s) {
-      sx[s] = sxb[s] = v4f{0.f, 0.f, 0.f, 0.f};
+    for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        sx[s] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, xf[s][j], sx[s], 0, 0, 0);
-        sxb[s] = __builtin_amdgcn_mfma_f32_16x16x32_f16(bias, xf[s][j], sxb[s], 0, 0, 0);
+      for (int s = 0; s < NKB; ++s) {
+        sx[mb][s] = sxb[mb][s] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          sx[mb][s] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, xf[mb][s][j], sx[mb][s], 0, 0, 0);
+          sxb[mb][s] = __builtin_amdgcn_mfma_f32_16x16x32_f16(bias, xf[mb][s][j], sxb[mb][s], 0, 0, 0);
+        }
       }
-    }
     static_for<Q>([&](auto qc) {
       constexpr int q = decltype(qc)::value;
       constexpr int nb = q / NKB, s = q % NKB;
@@ -199,11 +205,15 @@ struct SkinnyWoTile {
       if constexpr (q + kRing < Q) wr[q % kRing] = w_of(q + kRing);
       const v8h s8 = __builtin_bit_cast(v8h, *reinterpret_cast<const v4i*>(spatch + q * 64 + lg * 16));  // (scale, zero) of channels 4*lg .. 4*lg+3
       __builtin_amdgcn_sched_barrier(0);  // the refill is issued here, kRing blocks ahead of its use, not where the scheduler likes it
-      v4f part = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int j = 0; j < 4; ++j) part = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf[j], xf[s][j], part, 0, 0, 0);
+      for (int mb = 0; mb < MB; ++mb) {
+        v4f part = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int e = 0; e < 4; ++e) acc[nb][e] = __builtin_fmaf(part[e] - sxb[s][e], (float)s8[2 * e], __builtin_fmaf(sx[s][e], (float)s8[2 * e + 1], acc[nb][e]));
+        for (int j = 0; j < 4; ++j) part = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf[j], xf[mb][s][j], part, 0, 0, 0);
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          acc[nb][mb][e] = __builtin_fmaf(part[e] - sxb[mb][s][e], (float)s8[2 * e], __builtin_fmaf(sx[mb][s][e], (float)s8[2 * e + 1], acc[nb][mb][e]));
+      }
       __builtin_amdgcn_sched_barrier(0);
     });
   }
@@ -222,9 +232,11 @@ struct SkinnyWoTile {
     const int KW = (KB + kWaves - 1) / kWaves;
     const int kb_lo = min(KB, wave * KW), kb_hi = min(KB, kb_lo + KW);
     uint8_t* spatch = smem + kRedBytes + wave * kScaleBytes;
-    v4f acc[NB];
+    v4f acc[NB][MB];
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) acc[nb] = v4f{0.f, 0.f, 0.f, 0.f};
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) acc[nb][mb] = v4f{0.f, 0.f, 0.f, 0.f};
     for (int kb = kb_lo; kb < kb_hi; kb += KP) {
       const int nk = min(KP, kb_hi - kb);
       if constexpr (KP >= 4) {
@@ -242,30 +254,35 @@ struct SkinnyWoTile {
     // reduction over the 4 waves in a fixed order (wave 0 + 1 + 2 + 3), 16-channel blocks dealt round-robin to the waves
     v4f* red = reinterpret_cast<v4f*>(smem);
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) red[(wave * NB + nb) * 64 + lane] = acc[nb];
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) red[((wave * NB + nb) * MB + mb) * 64 + lane] = acc[nb][mb];
     __syncthreads();
-    const int m = m0 + lm;
 #pragma unroll
     for (int r = 0; r < NB / kWaves; ++r) {
       const int nb = wave + kWaves * r;
-      v4f sum = red[nb * 64 + lane];
 #pragma unroll
-      for (int w = 1; w < kWaves; ++w) {
-        const v4f p = red[(w * NB + nb) * 64 + lane];
+      for (int mb = 0; mb < MB; ++mb) {
+        const int m = m0 + mb * 16 + lm;
+        v4f sum = red[(nb * MB + mb) * 64 + lane];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) sum[e] += p[e];
-      }
-      if (m < M && nb < nbv) {
-        const int n = n0 + nb * 16 + lg * 4;
-        v4h o;
+        for (int w = 1; w < kWaves; ++w) {
+          const v4f p = red[((w * NB + nb) * MB + mb) * 64 + lane];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) o[e] = (_Float16)sum[e];
-        gstore<v4h>(t.C + (long)m * N + n, o);
-        if (t.acc_dump) {
+          for (int e = 0; e < 4; ++e) sum[e] += p[e];
+        }
+        if (m < M && nb < nbv) {
+          const int n = n0 + nb * 16 + lg * 4;
+          v4h o;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const float f = sum[e];  // a copy: a bit cast applied to a vector element reads element 0
-            gstore<int>(t.acc_dump + (long)m * N + n + e, __float_as_int(f));
+          for (int e = 0; e < 4; ++e) o[e] = (_Float16)sum[e];
+          gstore<v4h>(t.C + (long)m * N + n, o);
+          if (t.acc_dump) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const float f = sum[e];  // a copy: a bit cast applied to a vector element reads element 0
+              gstore<int>(t.acc_dump + (long)m * N + n + e, __float_as_int(f));
+            }
           }
         }
       }

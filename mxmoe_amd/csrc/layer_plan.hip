@@ -299,7 +299,7 @@ __device__ __forceinline__ void plan_block_body(const PlanParams& p, const int c
       if (np < kMaxPhases) {  // shapes beyond the phase table share the last phase
         fa->phase_tile0[np] = last_tile0 = tile0;
         fa->phase_wg0[np] = last_wg0 = wg;
-        if (info.b[info.order[r]].BM <= 16) flat |= 1 << np;
+        if (flat_phase(info.b[info.order[r]])) flat |= 1 << np;
         ++np;
       }
       wg = last_wg0 + (total - last_tile0 + kNumXcd - 1) / kNumXcd * kNumXcd;

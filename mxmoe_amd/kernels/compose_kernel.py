@@ -166,12 +166,12 @@ def _pick(arch: str, qcfg: str, *shapes, bf6: bool = False, few_registers: bool 
 def default_kernel_specs(arch: str = "gfx950"):
     """The kernels of libmxmoe_amd.so: (function name, kernel type, {qcfg: shape set}) in registry order."""
     w4, w8 = "w4a4_g-1_sym", "w8a8_g-1_sym"
-    wo = OrderedDict((f"w{b}a16_g128_asym", _pick(arch, f"w{b}a16_g128_asym", (16, 128))) for b in (4, 3, 2))
+    wo = OrderedDict((f"w{b}a16_g128_asym", _pick(arch, f"w{b}a16_g128_asym", (16, 128), (32, 128))) for b in (4, 3, 2))
     wo_big = OrderedDict((f"w{b}a16_g128_asym", _pick(arch, f"w{b}a16_g128_asym", (128, 256))) for b in (4, 3, 2))
     wo_all = OrderedDict((q, wo[q] + wo_big[q]) for q in wo)
     everything = OrderedDict([(w4, _pick(arch, w4, (128, 256), (32, 256))), (w8, _pick(arch, w8, (128, 256), (32, 256))),
                               ("fp16", _pick(arch, "fp16", (128, 256), (32, 256))), *wo_all.items(), ("w4a4_g128_sym", _pick(arch, "w4a4_g128_sym", (64, 256))),
-                              ("w8a16_g128_asym", _pick(arch, "w8a16_g128_asym", (16, 128), (128, 128)))])
+                              ("w8a16_g128_asym", _pick(arch, "w8a16_g128_asym", (16, 128), (32, 128), (128, 128)))])
     everything_b6 = OrderedDict(everything)
     everything_b6[w4] = _pick(arch, w4, (128, 256), (32, 256), bf6=True)
     everything_e4m3 = OrderedDict(("w8a8_g-1_sym_E4M3" if q == w8 else q, _pick(arch, "w8a8_g-1_sym_E4M3", (128, 256), (32, 256)) if q == w8 else t) for q, t in everything.items())
@@ -192,7 +192,7 @@ def default_kernel_specs(arch: str = "gfx950"):
         # share a CU instead of two, which is what these latency-bound weight streams gain from (decode-sized batches)
         ("groupgemm_hz_fused_wo_skinny", KernelType.Fused,
          OrderedDict((f"w{b}a16_g128_asym", _pick(arch, f"w{b}a16_g128_asym", (16, 128), few_registers=True)) for b in (4, 3, 2))),
-        ("groupgemm_hz_fused_wo8", KernelType.Fused, OrderedDict([("w8a16_g128_asym", _pick(arch, "w8a16_g128_asym", (16, 128), (128, 128)))])),
+        ("groupgemm_hz_fused_wo8", KernelType.Fused, OrderedDict([("w8a16_g128_asym", _pick(arch, "w8a16_g128_asym", (16, 128), (32, 128), (128, 128)))])),
         # w8a8 in fp8 (e4m3 codes on both sides), next to w4a4
         ("groupgemm_hz_fused_wxax_e4m3", KernelType.Fused, OrderedDict([(w4, _pick(arch, w4, (128, 256), (64, 256), (32, 256))),
                                                                          ("w8a8_g-1_sym_E4M3", _pick(arch, "w8a8_g-1_sym_E4M3", (128, 256), (64, 256), (32, 256)))])),

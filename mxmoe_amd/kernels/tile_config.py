@@ -184,7 +184,7 @@ class TileConfig:
         return self.MMA == "MFMA_F32_16x16x32_F16"
 
     def is_skinny(self) -> bool:
-        return self.is_weight_only() and self.BM == 16
+        return self.is_weight_only() and self.BM in (16, 32)
 
     def is_bf6(self) -> bool:
         """int4 operands handed over as bf6 fragments (both activations and weights; the quantisers write them, tag 4)."""
@@ -200,7 +200,8 @@ class TileConfig:
     def smem_bytes_tile(self):
         """LDS bytes of the tile as compiled (csrc/include/mxmoe_tiles.hpp, mxmoe_wo_tiles.hpp)."""
         if self.is_skinny():  # per-wave partial sums of the final reduction + (scale, zero) patches of one pass (4 k blocks, or 2)
-            return 4 * (self.BN // 16) * (64 * 16 + (2 if self.STAGE == 4 else 4) * 64)
+            kp = 2 if self.STAGE == 4 or self.BM == 32 else 4
+            return 4 * (self.BN // 16) * (64 * 16 * (self.BM // 16) + kp * 64)
         if self.is_weight_only():
             return 2 * self.BM * 256  # two stages of BM activation rows x one 128-wide k block
         if self.is_group_wa():
@@ -214,6 +215,8 @@ class TileConfig:
     def cpp_type(self) -> str:
         """The C++ tile type this descriptor instantiates."""
         if self.is_skinny():
+            if self.BM == 32:  # two blocks of 16 tokens against every unpacked weight: 2 k blocks per pass, 8 (8-bit: 4) packed blocks in flight
+                return f"SkinnyWoTile<{self.QCFGB.QBITS}, {self.BN}, 2, {4 if self.QCFGB.QBITS == 8 else 8}, 2, 2>"
             # STAGE 4: the few-register shape (2 k blocks per pass, 4 packed blocks in flight per wave, compiled for 3 waves per SIMD)
             return f"SkinnyWoTile<{self.QCFGB.QBITS}, {self.BN}, 2, 4, 3>" if self.STAGE == 4 else f"SkinnyWoTile<{self.QCFGB.QBITS}, {self.BN}>"
         if self.is_weight_only():
@@ -231,8 +234,8 @@ class TileConfig:
         if self.num_warps != 4:
             raise ValueError(f"{self!r}: gfx950 tiles use 4 wavefronts per workgroup")
         if self.is_weight_only():
-            if self.BK != 128 or not ((self.BM == 16 and self.BN % 64 == 0 and (self.WM, self.WN) == (1, 4)) or (self.BM, self.BN, self.WM, self.WN) in ((128, 128, 2, 2), (128, 256, 1, 4))):
-                raise ValueError(f"{self!r}: weight-only tiles are 16 x (64k) x 128 (1 x 4 waves), 128 x 128 x 128 (2 x 2 waves) or 128 x 256 x 128 (1 x 4 waves)")
+            if self.BK != 128 or not ((self.BM in (16, 32) and self.BN % 64 == 0 and (self.WM, self.WN) == (1, 4)) or (self.BM, self.BN, self.WM, self.WN) in ((128, 128, 2, 2), (128, 256, 1, 4))):
+                raise ValueError(f"{self!r}: weight-only tiles are 16 or 32 x (64k) x 128 (1 x 4 waves), 128 x 128 x 128 (2 x 2 waves) or 128 x 256 x 128 (1 x 4 waves)")
             return
         if self.is_bf6():
             if (self.BN, self.BK, self.WM, self.WN, self.WK, self.STAGE) != (256, 64, 1, 4, 1, 4) or self.BM not in (32, 64, 128):
@@ -285,6 +288,7 @@ def get_possible_tile_list(arch: str, qcfg: str) -> list:
     mma = QCFG_TO_MMA[qcfg]
     if mma == "MFMA_F32_16x16x32_F16":
         skinny = [_with_q(TileConfig(BM=16, BN=bn, BK=128, WM=1, WN=4, WK=1, STAGE=2, MMA=mma), qcfg) for bn in (128, 64)]
+        skinny.append(_with_q(TileConfig(BM=32, BN=128, BK=128, WM=1, WN=4, WK=1, STAGE=2, MMA=mma), qcfg))  # experts with 17 .. 32 (.. 64) tokens
         if QCFG_MAP[qcfg].QCFGB.QBITS != 8:  # the few-register shape, for kernels made of few-token tiles alone (three workgroups per CU)
             skinny.append(_with_q(TileConfig(BM=16, BN=128, BK=128, WM=1, WN=4, WK=1, STAGE=4, MMA=mma), qcfg))
         # (8-bit weights: the ring of packed blocks is twice as large, which leaves room for the 2 x 2 shape's accumulators only)

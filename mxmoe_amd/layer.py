@@ -161,7 +161,7 @@ class MxMoELayer:
             kid = lib.mxmoe_plan_select_kernel(-1, h, et)
             if kid < 0:
                 raise RuntimeError(lib.mxmoe_last_error().decode())
-            if t <= 64:  # no problem can have more rows than there are tokens: a kernel made of few-token tiles alone, if one covers the formats
+            if t <= 64 and t * topk <= 12 * e_cnt:  # few tokens, and on average well under one 16-row tile per expert: a kernel made of 16-row few-token tiles alone, if one covers the formats
                 few = lib.mxmoe_find_kernel(b"groupgemm_hz_fused_wo_skinny")
                 if few >= 0 and lib.mxmoe_plan_select_kernel(few, h, et) == few:
                     kid = few

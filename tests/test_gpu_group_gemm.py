@@ -309,6 +309,49 @@ def test_weight_only_skinny():
         assert _rel(out, p["ref"]) <= 1e-2, (p["size"], p["q"], _rel(out, p["ref"]))
 
 
+def test_weight_only_tiles_of_32_tokens():
+    """Experts with 17 .. 32 tokens (and the 33 .. 64 that two such tiles cover) run the few-token tile with two blocks of 16 tokens
+    per unpacked weight.  Its sums are formed in the same order as the 16-token tile's, so the outputs equal those of the kernel made
+    of 16-token tiles bit for bit, besides staying within 1e-2 of the fake-quant path; ragged channel counts, K = 1408 (waves with 3, 3,
+    3 and 2 k blocks), every bit width, per-channel scales."""
+    import ctypes as C
+
+    from mxmoe_amd import _lib
+    from mxmoe_amd.weights import quantize_and_pack
+
+    lib = _lib.load()
+    rng = np.random.default_rng(17)
+    cases = {"groupgemm_hz_fused_wo": [(17, 2816, 2048, 4, 128, False), (32, 144, 256, 3, 128, True), (31, 2048, 1408, 4, -1, False), (24, 160, 384, 2, 128, True),
+                                        (32, 5632, 2048, 4, 128, False), (47, 256, 1408, 3, 128, False), (20, 128, 128, 2, -1, False), (3, 256, 256, 4, 128, False)],
+             "groupgemm_hz_fused_wo8": [(17, 256, 2048, 8, 128, False), (32, 2816, 1408, 8, -1, True), (25, 144, 256, 8, 128, True), (9, 128, 128, 8, 128, False)]}
+    for kernel, shapes in cases.items():
+        probs = []
+        for (m, n, k, bits, gs, sym) in shapes:
+            x = rng.standard_normal((m, k)).astype(F16)
+            w = (rng.standard_normal((n, k)) * 0.02).astype(F16)
+            pw = quantize_and_pack(torch.from_numpy(w), (16, bits, gs, sym))
+            q, s_, z = O.quant_minmax(w, bits, gs, sym)
+            ref = O.gemm_fakequant(x, O.dequant(q, s_, z, gs))
+            probs.append(dict(A=torch.from_numpy(x).to(DEV), B=pw.data.to(DEV), sb=pw.scale.to(DEV), ref=ref, size=(m, n, k), q=(16, bits, gs, sym)))
+        kid = lib.mxmoe_find_kernel(kernel.encode())
+        assert kid >= 0
+        g, outs, _ = _launch(probs, kernel_id=kid, dump=False)
+        _, branches, _ = g.plan()
+        info = (C.c_int32 * 8)()
+        bms = []
+        for b in branches:
+            assert lib.mxmoe_kernel_branch(kid, b, info) == 0
+            bms.append(info[1])
+        assert 32 in bms and 16 in bms, bms                                # the new tile is in use, next to the 16-token one
+        for p, out in zip(probs, outs):
+            assert np.isfinite(out).all() and _rel(out, p["ref"]) <= 1e-2, (p["size"], p["q"], _rel(out, p["ref"]))
+        if kernel.endswith("_wo"):                                         # the same problems through 16-token tiles only
+            few = lib.mxmoe_find_kernel(b"groupgemm_hz_fused_wo_skinny")
+            _, outs16, _ = _launch(probs, kernel_id=few, dump=False)
+            for p, a, b in zip(probs, outs, outs16):
+                assert np.array_equal(a.view(np.uint16), b.view(np.uint16)), p["size"]
+
+
 def test_weight_only_many_tokens():
     """Experts with many tokens run the 128 x 256 dequantise-to-fp16 MFMA tile (and the remainder rows the skinny one); channel
     counts that leave one or two of its four waves without channels are among the cases."""
