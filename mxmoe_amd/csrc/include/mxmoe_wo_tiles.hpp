@@ -387,9 +387,15 @@ struct WoMfmaTile {
       }
       asm volatile("" ::: "memory");
       const v8h bias = Sk::bias8();
-      // one k block; PAR = parity of kb, a compile-time constant so that the ring slots are fixed registers
-      auto step = [&](auto parc, int kb) {
+      // token blocks of this wave that hold rows of the problem: a tile of a problem with at most half of BM rows left (an expert
+      // with a few dozen tokens, a short last row tile) runs a second copy of the loop that leaves out the fragment reads and
+      // matrix instructions of the upper half, which would only multiply zeros; such a tile is then bound by its weight stream
+      // rather than by 128 rows of arithmetic
+      const int mbv = __builtin_amdgcn_readfirstlane(max(0, min(MB, (a_rows - wm * TM + 15) / 16)));
+      // one k block; PAR = parity of kb, a compile-time constant so that the ring slots are fixed registers; LIVE: token blocks computed
+      auto step = [&](auto parc, int kb, auto livec) {
         constexpr int st = decltype(parc)::value;
+        constexpr int LIVE = decltype(livec)::value;
         // the activation stage of this k block has landed: the only younger loads are the 8 ring refills of the last iteration
         // (or the 8 ring loads of the prologue)
         vm_wait<8>();
@@ -401,7 +407,7 @@ struct WoMfmaTile {
         for (int j = 0; j < 4; ++j) {
           v8h xf[MB];
 #pragma unroll
-          for (int mb = 0; mb < MB; ++mb) xf[mb] = __builtin_bit_cast(v8h, lds_x(st, mb, j));
+          for (int mb = 0; mb < LIVE; ++mb) xf[mb] = __builtin_bit_cast(v8h, lds_x(st, mb, j));
 #pragma unroll
           for (int nb = 0; nb < 4; ++nb) {
             v8h wf[4];
@@ -411,7 +417,7 @@ struct WoMfmaTile {
             const v8h z8 = {sz[1], sz[1], sz[1], sz[1], sz[1], sz[1], sz[1], sz[1]};
             const v8h w8 = __builtin_elementwise_fma(wf[j] - bias, s8, z8);  // exact q, then fma(q, scale, zero) in fp16
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb) acc[nb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w8, xf[mb], acc[nb][mb], 0, 0, 0);
+            for (int mb = 0; mb < LIVE; ++mb) acc[nb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w8, xf[mb], acc[nb][mb], 0, 0, 0);
           }
           // keeps the scheduler from starting the next sub-block's unpacking and fragment reads early: that costs no time (the
           // other wave of the SIMD fills the gap) and without it the 3-bit tile runs out of registers
@@ -423,10 +429,18 @@ struct WoMfmaTile {
           sr[base + nb] = s_of(nb, kb + 2);
         }
       };
+      if (mbv > MB / 2) {
 #pragma unroll 1
-      for (int kb = 0; kb < KB; kb += 2) {
-        step(std::integral_constant<int, 0>{}, kb);
-        if (kb + 1 < KB) step(std::integral_constant<int, 1>{}, kb + 1);
+        for (int kb = 0; kb < KB; kb += 2) {
+          step(std::integral_constant<int, 0>{}, kb, std::integral_constant<int, MB>{});
+          if (kb + 1 < KB) step(std::integral_constant<int, 1>{}, kb + 1, std::integral_constant<int, MB>{});
+        }
+      } else {
+#pragma unroll 1
+        for (int kb = 0; kb < KB; kb += 2) {
+          step(std::integral_constant<int, 0>{}, kb, std::integral_constant<int, MB / 2>{});
+          if (kb + 1 < KB) step(std::integral_constant<int, 1>{}, kb + 1, std::integral_constant<int, MB / 2>{});
+        }
       }
     }
     vm_wait<0>();
