@@ -310,8 +310,8 @@ def test_weight_only_skinny():
 
 
 def test_weight_only_tiles_of_32_tokens():
-    """Experts with 17 .. 32 tokens (and the 33 .. 64 that two such tiles cover) run the few-token tile with two blocks of 16 tokens
-    per unpacked weight.  Its sums are formed in the same order as the 16-token tile's, so the outputs equal those of the kernel made
+    """Experts with 17 .. 32 tokens run the few-token tile with two blocks of 16 tokens per unpacked weight (from 33 tokens on the
+    planner weighs two such tiles against the 128-token tile).  Its sums are formed in the same order as the 16-token tile's, so the outputs equal those of the kernel made
     of 16-token tiles bit for bit, besides staying within 1e-2 of the fake-quant path; ragged channel counts, K = 1408 (waves with 3, 3,
     3 and 2 k blocks), every bit width, per-channel scales."""
     import ctypes as C
@@ -349,7 +349,8 @@ def test_weight_only_tiles_of_32_tokens():
             few = lib.mxmoe_find_kernel(b"groupgemm_hz_fused_wo_skinny")
             _, outs16, _ = _launch(probs, kernel_id=few, dump=False)
             for p, a, b in zip(probs, outs, outs16):
-                assert np.array_equal(a.view(np.uint16), b.view(np.uint16)), p["size"]
+                if p["size"][0] <= 32:    # (more rows go to the 128-token tile, which rounds every dequantised weight to fp16: other last bits)
+                    assert np.array_equal(a.view(np.uint16), b.view(np.uint16)), p["size"]
 
 
 def test_weight_only_many_tokens():
