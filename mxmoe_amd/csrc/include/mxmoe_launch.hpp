@@ -355,9 +355,9 @@ inline double tile_cost(const BranchInfo& b) {
       {Fmt::W4A4, 128, 256, 1.00}, {Fmt::W4A4, 64, 256, 0.58}, {Fmt::W4A4, 32, 256, 0.48},
       {Fmt::W8A8, 128, 256, 1.00}, {Fmt::W8A8, 64, 256, 0.74}, {Fmt::W8A8, 32, 256, 0.56},
       {Fmt::FP16, 128, 256, 1.00}, {Fmt::FP16, 64, 256, 0.69}, {Fmt::FP16, 32, 256, 0.53}, {Fmt::FP16, 128, 128, 0.57}, {Fmt::FP16, 256, 128, 1.09},
-      {Fmt::W4A16, 16, 128, 0.37}, {Fmt::W4A16, 16, 64, 0.20}, {Fmt::W4A16, 32, 128, 0.42}, {Fmt::W4A16, 128, 128, 1.00}, {Fmt::W4A16, 128, 256, 1.50},
-      {Fmt::W3A16, 16, 128, 0.31}, {Fmt::W3A16, 16, 64, 0.20}, {Fmt::W3A16, 32, 128, 0.42}, {Fmt::W3A16, 128, 128, 1.00}, {Fmt::W3A16, 128, 256, 1.50},
-      {Fmt::W2A16, 16, 128, 0.25}, {Fmt::W2A16, 16, 64, 0.20}, {Fmt::W2A16, 32, 128, 0.42}, {Fmt::W2A16, 128, 128, 1.00}, {Fmt::W2A16, 128, 256, 1.50},
+      {Fmt::W4A16, 16, 128, 0.37}, {Fmt::W4A16, 16, 64, 0.20}, {Fmt::W4A16, 32, 128, 0.50}, {Fmt::W4A16, 128, 128, 1.00}, {Fmt::W4A16, 128, 256, 1.50},
+      {Fmt::W3A16, 16, 128, 0.31}, {Fmt::W3A16, 16, 64, 0.20}, {Fmt::W3A16, 32, 128, 0.50}, {Fmt::W3A16, 128, 128, 1.00}, {Fmt::W3A16, 128, 256, 1.50},
+      {Fmt::W2A16, 16, 128, 0.25}, {Fmt::W2A16, 16, 64, 0.20}, {Fmt::W2A16, 32, 128, 0.50}, {Fmt::W2A16, 128, 128, 1.00}, {Fmt::W2A16, 128, 256, 1.50},
       {Fmt::W8A16, 16, 128, 0.60}, {Fmt::W8A16, 16, 64, 0.35}, {Fmt::W8A16, 32, 128, 0.66}, {Fmt::W8A16, 128, 128, 1.00},
       {Fmt::W4A4G128, 64, 256, 1.00}, {Fmt::W4A4G128, 32, 256, 0.60},
   };
