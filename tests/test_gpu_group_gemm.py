@@ -322,7 +322,8 @@ def test_weight_only_tiles_of_32_tokens():
     lib = _lib.load()
     rng = np.random.default_rng(17)
     cases = {"groupgemm_hz_fused_wo": [(17, 2816, 2048, 4, 128, False), (32, 144, 256, 3, 128, True), (31, 2048, 1408, 4, -1, False), (24, 160, 384, 2, 128, True),
-                                        (32, 5632, 2048, 4, 128, False), (47, 256, 1408, 3, 128, False), (20, 128, 128, 2, -1, False), (3, 256, 256, 4, 128, False)],
+                                        (32, 5632, 2048, 4, 128, False), (47, 256, 1408, 3, 128, False), (20, 128, 128, 2, -1, False), (3, 256, 256, 4, 128, False),
+                                        (20, 256, 14336, 4, 128, False)],   # (the last: 14 passes per wave)
              "groupgemm_hz_fused_wo8": [(17, 256, 2048, 8, 128, False), (32, 2816, 1408, 8, -1, True), (25, 144, 256, 8, 128, True), (9, 128, 128, 8, 128, False)]}
     for kernel, shapes in cases.items():
         probs = []
